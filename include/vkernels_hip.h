@@ -1,0 +1,200 @@
+/*
+ * vkernels_hip.h — C ABI of libvkernels_hip.so, the MI355X (gfx950) build of
+ * the fused MXFP4 Mixture-of-Experts path.
+ *
+ * The entry points keep the names, argument order and conventions of the
+ * reference's device ABI (src/c/vkernels/capi/hip_capi.hpp) so that a caller
+ * that binds the reference's library — the ctypes loader in
+ * src/python/vkernels/vllm_experts.py:388-459, the harness in
+ * tests/python/test_mxfp4_serving_parity.py:200-225 — binds this one
+ * unchanged.  Entry points marked "additive" have no counterpart in the
+ * reference and follow the same conventions.
+ *
+ * Conventions (src/c/vkernels/capi/hip_capi.hpp:24-40):
+ *   - every pointer is caller-owned DEVICE memory unless stated otherwise;
+ *   - launchers enqueue work on `stream` (NULL = the default stream) and
+ *     return at once: no allocation, no synchronisation, safe to capture in a
+ *     HIP graph;
+ *   - launchers that return void report launch errors through
+ *     hipGetLastError() after the caller synchronises;
+ *   - launchers that return int validate their arguments on the host and
+ *     return VK_OK or a VK_ERROR_* code; the message of the last failure on
+ *     the calling thread is available from vk_last_error().
+ */
+#ifndef VKERNELS_HIP_H_
+#define VKERNELS_HIP_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Status codes.  Replaces src/c/vkernels/capi/capi.hpp:41-47. */
+enum {
+  VK_OK = 0,
+  VK_ERROR_INVALID_ARGUMENT = 1,
+  VK_ERROR_OUT_OF_RANGE = 2,
+  VK_ERROR_UNSUPPORTED = 3,
+  VK_ERROR_INTERNAL = 4
+};
+
+/* Activation tags.  Replaces MoEActivation,
+ * src/c/vkernels/kernels/moe_fused.hpp:47-50. */
+enum { VK_MOE_SWIGLU = 0, VK_MOE_SITU = 1 };
+
+/* Library version string.  Replaces src/c/vkernels/capi/capi.hpp:54. */
+const char* vk_version(void);
+
+/* 0: this build has no CUDA path.  Replaces capi.hpp:57. */
+int vk_has_cuda(void);
+
+/* Thread-local message / code of the most recent failing call on this
+ * thread ("" / VK_OK if none).  Replaces capi.hpp:60-63. */
+const char* vk_last_error(void);
+int vk_last_error_code(void);
+
+/* Set the thread-local error state.  Replaces capi.hpp:68. */
+void vk_set_last_error(int code, const char* message);
+
+/* Release memory returned by the library (nothing in this ABI allocates; kept
+ * so that bindings that import the symbol still load).  Replaces capi.hpp:71. */
+void vk_free(void* p);
+
+/* Upper bound on the padded row count EM for (M, top_k, block_size,
+ * num_experts): (ceil(M*top_k/block_size) + num_experts) * block_size; the
+ * size to give sorted_ids (and /block_size for expert_ids).  Host arithmetic
+ * only.  Replaces vk_moe_align_block_size_max_em,
+ * src/c/vkernels/capi/capi.hpp:537-539 (capi_moe.cpp:110-117). */
+size_t vk_moe_align_block_size_max_em(int32_t M, int32_t top_k,
+                                      int32_t block_size, int32_t num_experts);
+
+/*
+ * Fused MXFP4 MoE layer: gate/up grouped GEMM with inline E2M1 x ue8m0
+ * dequantisation, bias, SwiGLU or SiTU epilogue (one bf16 rounding) into
+ * act_scratch, then the down grouped GEMM, bias, routing weight and
+ * accumulation into out.
+ * Replaces vk_hip_fused_moe_mxfp4, src/c/vkernels/capi/hip_capi.hpp:99-108
+ * (src/c/vkernels/capi/hip_capi.cpp:40-57).
+ *
+ *   A           [M, hidden]            bf16 bit patterns
+ *   w13         [E, 2*ispp, hidden/2]  packed E2M1, gate rows [0,ispp), up
+ *                                      rows [ispp,2*ispp), low nibble = even k
+ *   w13_scale   [E, 2*ispp, hidden/32] ue8m0
+ *   w2          [E, hidden, ispp/2]    packed E2M1
+ *   w2_scale    [E, hidden, ispp/32]   ue8m0
+ *   topk_ids    [M, top_k]             routing table (not read; kept for ABI)
+ *   topk_w      [M, top_k]             routing weights, read as topk_w[flat]
+ *   act_scratch [EM, ispp]             bf16, indexed by sorted row; rows of
+ *                                      padding are left untouched
+ *   out         [M, hidden]            fp32; the caller zero-initialises it
+ *                                      and the call ACCUMULATES into it
+ *   sorted_ids  [EM]                   flat index token*top_k+sel per sorted
+ *                                      row; entries >= M*top_k are padding
+ *   expert_ids  [EM/block_size]        expert of each block; < 0 = skip
+ *   EM          padded row count the two arrays were built for (may be the
+ *               host's upper bound; padding blocks/rows are skipped)
+ *   block_size  the alignment sorted_ids/expert_ids were built with; any
+ *               positive multiple of 16
+ *   hidden, ispp multiples of 64
+ */
+void vk_hip_fused_moe_mxfp4(
+    const uint16_t* A, const uint8_t* w13, const uint8_t* w13_scale,
+    const uint8_t* w2, const uint8_t* w2_scale,
+    const int32_t* topk_ids, const float* topk_w,
+    uint16_t* act_scratch, float* out,
+    int M, int hidden, int ispp, int top_k,
+    const int32_t* sorted_ids, const int32_t* expert_ids,
+    int EM, float swiglu_limit,
+    int activation, float beta, float linear_beta,
+    const float* b13, const float* b2, int block_size, void* stream);
+
+/*
+ * Additive: the two stages of vk_hip_fused_moe_mxfp4 as separate launches,
+ * for callers that place work between them (a tensor-parallel all-reduce, a
+ * profiler's events).  Device counterparts of the reference's stage split,
+ * src/c/vkernels/kernels/moe_fused.hpp:103-125, with the activation fused
+ * into the first stage and the combine into the second; calling one after the
+ * other on a stream is exactly vk_hip_fused_moe_mxfp4.  Arguments as there.
+ */
+void vk_hip_moe_gateup_mxfp4(
+    const uint16_t* A, const uint8_t* w13, const uint8_t* w13_scale,
+    uint16_t* act_scratch, int M, int hidden, int ispp, int top_k,
+    const int32_t* sorted_ids, const int32_t* expert_ids, int EM,
+    float swiglu_limit, int activation, float beta, float linear_beta,
+    const float* b13, int block_size, void* stream);
+
+void vk_hip_moe_down_mxfp4(
+    const uint16_t* act, const uint8_t* w2, const uint8_t* w2_scale,
+    const float* topk_w, float* out, int M, int hidden, int ispp, int top_k,
+    const int32_t* sorted_ids, const int32_t* expert_ids, int EM,
+    const float* b2, int block_size, void* stream);
+
+/*
+ * On-device alignment of the routing table: stable bucket of the flat indices
+ * by (local) expert, each expert padded to a multiple of block_size.
+ * Replaces vk_hip_moe_align_block_size,
+ * src/c/vkernels/capi/hip_capi.hpp:148-153 (hip_capi.cpp:66-95).
+ *
+ *   topk_ids    [M*top_k]       global expert ids; ids outside
+ *                               [0,num_experts) are skipped
+ *   expert_map  [num_experts]   global -> local (-1 = skip), or NULL (1:1)
+ *   local_n                     experts on this rank (<= num_experts)
+ *   max_EM                      host upper bound on EM, multiple of
+ *                               block_size, > 0
+ *   sorted_ids  [max_EM]        all entries written; padding = M*top_k
+ *   expert_ids  [max_EM/block_size] all entries written; padding = -1
+ *   out_EM      [1]             padded row count, at least one block
+ *
+ * Unlike the reference there is no M*top_k <= 1024 limit: any size runs on
+ * the device and VK_ERROR_UNSUPPORTED is only returned for num_experts beyond
+ * VK_HIP_ALIGN_MAX_EXPERTS.
+ */
+#define VK_HIP_ALIGN_MAX_EXPERTS 1024
+int vk_hip_moe_align_block_size(
+    const int32_t* topk_ids, const int32_t* expert_map,
+    int32_t M, int32_t top_k, int32_t block_size,
+    int32_t num_experts, int32_t local_n, int32_t max_EM,
+    int32_t* sorted_ids, int32_t* expert_ids, int32_t* out_EM,
+    void* stream);
+
+/*
+ * Additive: softmax -> top-k -> renormalise router, one wavefront per token.
+ * Follows the conventions of vk_hip_moe_align_block_size; the semantics are
+ * those of src/python/vkernels/torch_ops/tokenspeed_amd/routing.py:59-157
+ * without bias and with scaling factor 1: p = softmax(logits) in fp32, top_k
+ * arg-max picks of p with ties to the lowest expert index, weights p[ids],
+ * divided by their sum when renormalize != 0 (a zero sum divides by 1).
+ *
+ *   logits    [T, E]      fp32
+ *   topk_ids  [T, top_k]  int32, selection order (descending probability)
+ *   topk_w    [T, top_k]  fp32
+ *   E <= VK_HIP_ROUTE_MAX_EXPERTS, 1 <= top_k <= min(E, VK_HIP_ROUTE_MAX_TOPK)
+ */
+#define VK_HIP_ROUTE_MAX_EXPERTS 1024
+#define VK_HIP_ROUTE_MAX_TOPK 32
+int vk_hip_moe_route_topk(const float* logits, int32_t T, int32_t E,
+                          int32_t top_k, int32_t renormalize,
+                          int32_t* topk_ids, float* topk_w, void* stream);
+
+/*
+ * Additive: dequantise an [N, K] tile of packed weights to bf16 with the
+ * same device routine the GEMM kernels use, written transposed as [K][N].
+ * Device counterpart of dequant_weight_tile,
+ * src/c/vkernels/kernels/moe_fused.hpp:217-235 (moe_fused.cpp:141-174), for
+ * bit-exact checks of the weight decode.  group_size must be 32.
+ * fast != 0 selects the hardware-conversion path the GEMM kernels take for
+ * ordinary tiles (valid for finite codes and scale bytes 3..252); fast == 0
+ * the exact integer path they fall back to.
+ */
+int vk_hip_dequant_weight_tile(const uint8_t* packed, const uint8_t* scale,
+                               uint16_t* out_bf16, int32_t N, int32_t K,
+                               int32_t group_size, int32_t stride_packed,
+                               int32_t stride_scale_n, int32_t stride_scale_k,
+                               int32_t fast, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* VKERNELS_HIP_H_ */

@@ -1,0 +1,196 @@
+// hip_capi.cpp — the extern "C" surface of libvkernels_hip.so (declared in
+// include/vkernels_hip.h).  Host-side argument checks and error state only;
+// the kernels live in the moe_*.hip translation units.
+#include "vkernels_hip.h"
+
+#include <hip/hip_runtime.h>
+
+#include <string>
+
+#include "vk_internal.hpp"
+
+namespace {
+
+thread_local std::string g_last_error;
+thread_local int g_last_error_code = VK_OK;
+
+int fail(int code, const char* message) {
+  vk_set_last_error(code, message);
+  return code;
+}
+
+}  // namespace
+
+extern "C" {
+
+const char* vk_version(void) { return "0.1.0"; }
+
+int vk_has_cuda(void) { return 0; }
+
+const char* vk_last_error(void) { return g_last_error.c_str(); }
+
+int vk_last_error_code(void) { return g_last_error_code; }
+
+void vk_set_last_error(int code, const char* message) {
+  g_last_error_code = code;
+  g_last_error = message != nullptr ? message : "";
+}
+
+void vk_free(void* p) { free(p); }
+
+size_t vk_moe_align_block_size_max_em(int32_t M, int32_t top_k,
+                                      int32_t block_size,
+                                      int32_t num_experts) {
+  if (block_size <= 0) return 0;
+  const int32_t n = M * top_k;
+  const int32_t max_em = ((n + block_size - 1) / block_size + num_experts) * block_size;
+  return max_em > 0 ? static_cast<size_t>(max_em) : 0;
+}
+
+namespace {
+
+// Shared contract check of the three layer entry points.  They return void
+// like the reference's launcher; a violation is recorded for vk_last_error()
+// and nothing is launched.
+bool layer_args_ok(const char* who, bool need13, bool need2, const vk::FusedMoeArgs& a) {
+  const char* why = nullptr;
+  if (a.sorted_ids == nullptr || a.expert_ids == nullptr || a.act == nullptr)
+    why = "buffers must not be null";
+  else if (need13 && (a.A == nullptr || a.w13 == nullptr || a.w13_scale == nullptr))
+    why = "buffers must not be null";
+  else if (need2 && (a.w2 == nullptr || a.w2_scale == nullptr || a.topk_w == nullptr ||
+                     a.out == nullptr))
+    why = "buffers must not be null";
+  else if (a.hidden <= 0 || a.ispp <= 0 || a.hidden % 64 != 0 || a.ispp % 64 != 0)
+    why = "hidden and ispp must be positive multiples of 64";
+  else if (a.top_k <= 0)
+    why = "top_k must be positive";
+  else if (a.block_size <= 0 || a.block_size % 16 != 0 || a.EM % a.block_size != 0)
+    why = "block_size must be a multiple of 16 and divide EM";
+  if (why == nullptr) return true;
+  vk_set_last_error(VK_ERROR_INVALID_ARGUMENT, (std::string(who) + ": " + why).c_str());
+  return false;
+}
+
+}  // namespace
+
+void vk_hip_fused_moe_mxfp4(
+    const uint16_t* A, const uint8_t* w13, const uint8_t* w13_scale,
+    const uint8_t* w2, const uint8_t* w2_scale,
+    const int32_t* topk_ids, const float* topk_w,
+    uint16_t* act_scratch, float* out,
+    int M, int hidden, int ispp, int top_k,
+    const int32_t* sorted_ids, const int32_t* expert_ids,
+    int EM, float swiglu_limit,
+    int activation, float beta, float linear_beta,
+    const float* b13, const float* b2, int block_size, void* stream) {
+  (void)topk_ids;
+  if (M <= 0 || EM <= 0) return;  // nothing routed: out is left as it is
+  vk::FusedMoeArgs a{};
+  a.A = A; a.w13 = w13; a.w13_scale = w13_scale; a.w2 = w2; a.w2_scale = w2_scale;
+  a.topk_w = topk_w; a.act = act_scratch; a.out = out;
+  a.sorted_ids = sorted_ids; a.expert_ids = expert_ids; a.b13 = b13; a.b2 = b2;
+  a.M = M; a.hidden = hidden; a.ispp = ispp; a.top_k = top_k; a.EM = EM;
+  a.block_size = block_size; a.swiglu_limit = swiglu_limit; a.beta = beta;
+  a.linear_beta = linear_beta; a.activation = activation;
+  if (!layer_args_ok("vk_hip_fused_moe_mxfp4", true, true, a)) return;
+  vk::launch_fused_moe(a, static_cast<hipStream_t>(stream));
+}
+
+void vk_hip_moe_gateup_mxfp4(
+    const uint16_t* A, const uint8_t* w13, const uint8_t* w13_scale,
+    uint16_t* act_scratch, int M, int hidden, int ispp, int top_k,
+    const int32_t* sorted_ids, const int32_t* expert_ids, int EM,
+    float swiglu_limit, int activation, float beta, float linear_beta,
+    const float* b13, int block_size, void* stream) {
+  if (M <= 0 || EM <= 0) return;
+  vk::FusedMoeArgs a{};
+  a.A = A; a.w13 = w13; a.w13_scale = w13_scale; a.act = act_scratch;
+  a.sorted_ids = sorted_ids; a.expert_ids = expert_ids; a.b13 = b13;
+  a.M = M; a.hidden = hidden; a.ispp = ispp; a.top_k = top_k; a.EM = EM;
+  a.block_size = block_size; a.swiglu_limit = swiglu_limit; a.beta = beta;
+  a.linear_beta = linear_beta; a.activation = activation;
+  if (!layer_args_ok("vk_hip_moe_gateup_mxfp4", true, false, a)) return;
+  vk::launch_moe_gateup(a, static_cast<hipStream_t>(stream));
+}
+
+void vk_hip_moe_down_mxfp4(
+    const uint16_t* act, const uint8_t* w2, const uint8_t* w2_scale,
+    const float* topk_w, float* out, int M, int hidden, int ispp, int top_k,
+    const int32_t* sorted_ids, const int32_t* expert_ids, int EM,
+    const float* b2, int block_size, void* stream) {
+  if (M <= 0 || EM <= 0) return;
+  vk::FusedMoeArgs a{};
+  a.w2 = w2; a.w2_scale = w2_scale; a.topk_w = topk_w;
+  a.act = const_cast<uint16_t*>(act); a.out = out;
+  a.sorted_ids = sorted_ids; a.expert_ids = expert_ids; a.b2 = b2;
+  a.M = M; a.hidden = hidden; a.ispp = ispp; a.top_k = top_k; a.EM = EM;
+  a.block_size = block_size;
+  if (!layer_args_ok("vk_hip_moe_down_mxfp4", false, true, a)) return;
+  vk::launch_moe_down(a, static_cast<hipStream_t>(stream));
+}
+
+int vk_hip_moe_align_block_size(
+    const int32_t* topk_ids, const int32_t* expert_map,
+    int32_t M, int32_t top_k, int32_t block_size,
+    int32_t num_experts, int32_t local_n, int32_t max_EM,
+    int32_t* sorted_ids, int32_t* expert_ids, int32_t* out_EM,
+    void* stream) {
+  if (block_size <= 0)
+    return fail(VK_ERROR_INVALID_ARGUMENT, "block_size must be positive");
+  if (M < 0 || top_k < 0 || num_experts < 0 || local_n < 0 || max_EM < 0)
+    return fail(VK_ERROR_INVALID_ARGUMENT, "sizes must be non-negative");
+  if (max_EM == 0 || (max_EM % block_size) != 0)
+    return fail(VK_ERROR_INVALID_ARGUMENT, "max_EM must be a positive multiple of block_size");
+  if (local_n > num_experts)
+    return fail(VK_ERROR_INVALID_ARGUMENT, "local_n must not exceed num_experts");
+  if (out_EM == nullptr || sorted_ids == nullptr || expert_ids == nullptr)
+    return fail(VK_ERROR_INVALID_ARGUMENT, "sorted_ids/expert_ids/out_EM must not be null");
+  if (M > 0 && top_k > 0 && topk_ids == nullptr)
+    return fail(VK_ERROR_INVALID_ARGUMENT, "topk_ids must not be null");
+  const long long n = static_cast<long long>(M) * static_cast<long long>(top_k);
+  if (n > 0x7FFFFFFFll)
+    return fail(VK_ERROR_OUT_OF_RANGE, "M*top_k does not fit in int32");
+  if (local_n > VK_HIP_ALIGN_MAX_EXPERTS)
+    return fail(VK_ERROR_UNSUPPORTED, "more local experts than VK_HIP_ALIGN_MAX_EXPERTS");
+  vk::launch_align(topk_ids, expert_map, static_cast<int>(n), block_size, num_experts,
+                   local_n, max_EM, sorted_ids, expert_ids, out_EM,
+                   static_cast<hipStream_t>(stream));
+  return VK_OK;
+}
+
+int vk_hip_moe_route_topk(const float* logits, int32_t T, int32_t E,
+                          int32_t top_k, int32_t renormalize,
+                          int32_t* topk_ids, float* topk_w, void* stream) {
+  if (T < 0 || E <= 0 || top_k <= 0)
+    return fail(VK_ERROR_INVALID_ARGUMENT, "T must be >= 0, E and top_k positive");
+  if (top_k > E)
+    return fail(VK_ERROR_INVALID_ARGUMENT, "top_k must not exceed E");
+  if (E > VK_HIP_ROUTE_MAX_EXPERTS || top_k > VK_HIP_ROUTE_MAX_TOPK)
+    return fail(VK_ERROR_UNSUPPORTED, "E or top_k beyond the router's limits");
+  if (T == 0) return VK_OK;
+  if (logits == nullptr || topk_ids == nullptr || topk_w == nullptr)
+    return fail(VK_ERROR_INVALID_ARGUMENT, "logits/topk_ids/topk_w must not be null");
+  vk::launch_route_topk(logits, T, E, top_k, renormalize, topk_ids, topk_w,
+                        static_cast<hipStream_t>(stream));
+  return VK_OK;
+}
+
+int vk_hip_dequant_weight_tile(const uint8_t* packed, const uint8_t* scale,
+                               uint16_t* out_bf16, int32_t N, int32_t K,
+                               int32_t group_size, int32_t stride_packed,
+                               int32_t stride_scale_n, int32_t stride_scale_k,
+                               int32_t fast, void* stream) {
+  if (group_size != 32)
+    return fail(VK_ERROR_UNSUPPORTED, "group_size must be 32");
+  if (N < 0 || K < 0 || K % 32 != 0)
+    return fail(VK_ERROR_INVALID_ARGUMENT, "N must be >= 0 and K a multiple of 32");
+  if (N == 0 || K == 0) return VK_OK;
+  if (packed == nullptr || scale == nullptr || out_bf16 == nullptr)
+    return fail(VK_ERROR_INVALID_ARGUMENT, "packed/scale/out_bf16 must not be null");
+  vk::launch_dequant_tile(packed, scale, out_bf16, N, K, stride_packed, stride_scale_n,
+                          stride_scale_k, fast, static_cast<hipStream_t>(stream));
+  return VK_OK;
+}
+
+}  // extern "C"

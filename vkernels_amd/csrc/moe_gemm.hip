@@ -1,0 +1,410 @@
+// moe_gemm.hip — the two grouped GEMMs of the fused MXFP4 MoE layer.
+//
+//   stage 0  act[r, 0:I]   = bf16(act_fn(A[tok(r)] . W13[e, 0:I]^T  + b13,
+//                                        A[tok(r)] . W13[e, I:2I]^T + b13))
+//   stage 1  out[tok(r), :] += (act[r] . W2[e]^T + b2) * topk_w[flat(r)]
+//
+// for every sorted row r of every block whose expert_ids entry e is >= 0
+// (reference semantics: src/c/vkernels/kernels/moe_fused.cpp:235-564).
+//
+// Weight-streaming design.  The weights dominate the bytes (4.25 bits per
+// weight against a handful of activation rows per expert), so the kernels
+// are organised around reading every weight byte of an active expert once,
+// in 16-byte pieces, straight into the register layout of the MFMA operand:
+//
+//   * a run = the consecutive blocks of one expert; the workgroup of the
+//     run's first block does the whole run, later blocks exit at once, so
+//     an expert's weights are streamed once however many rows it has;
+//   * a wavefront owns NT weight tiles of 16 rows each (stage 0: NT/2 gate
+//     tiles and the NT/2 up tiles of the same columns, so the activation is
+//     fused; stage 1: NT consecutive tiles) and walks the whole K dimension;
+//   * weights sit on the A side of v_mfma_f32_16x16x32_bf16: lane (n, q) =
+//     (lane % 16, lane / 16) holds row n, so one global_load_dwordx4 of that
+//     lane brings the 32 codes of one scale group, enough for four MFMAs;
+//     quad q of a K step of 128 takes group 4*step + q, so a wavefront reads
+//     64 contiguous bytes of each of its 16 rows per step;
+//   * dequantisation is exact: the codes are turned into the bf16 value the
+//     reference computes (see mxfp4.hpp) and multiplied by bf16 activations
+//     with fp32 accumulation, as the reference does;
+//   * the activation rows (up to MT tiles of 16 rows per pass) are staged by
+//     the whole workgroup through LDS in MFMA-operand order, one 256-wide K
+//     chunk at a time, prefetched through registers;
+//   * stage 1 adds into `out` with hardware fp32 atomics, as the ABI
+//     requires `out` to be accumulated into.
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "moe_heuristics.hpp"
+#include "mxfp4.hpp"
+#include "vk_internal.hpp"
+
+namespace vk {
+namespace {
+
+constexpr int kKStep = 128;    // K per MFMA group of four (one scale group per quad)
+constexpr int kKChunk = 256;   // K staged through LDS per barrier pair
+constexpr int kStepsPerChunk = kKChunk / kKStep;
+
+struct GemmArgs {
+  const uint16_t* A;        // stage 0: activations [M, K]; stage 1: act [EM, K]
+  const uint8_t* W;         // [E, rows_w, K/2]
+  const uint8_t* Ws;        // [E, rows_w, K/32]
+  const int32_t* sorted_ids;
+  const int32_t* expert_ids;
+  const float* topk_w;      // stage 1
+  const float* bias;        // b13 [E, 2I] or b2 [E, H], may be null
+  uint16_t* act;            // stage 0 output [EM, I]
+  float* out;               // stage 1 output [M, H]
+  int n_flat;               // M * top_k
+  int top_k;
+  int K;                    // hidden (stage 0) or ispp (stage 1)
+  int ncols;                // ispp (stage 0) or hidden (stage 1)
+  int num_blocks;
+  int block_size;
+  float swiglu_limit, beta, linear_beta;
+  int activation;
+};
+
+__device__ __forceinline__ float act_value(int activation, float g, float u,
+                                           float limit, float beta,
+                                           float linear_beta) {
+  if (activation == 1) {
+    const float sig = 1.0f / (1.0f + expf(-g));
+    const float gate_out = beta * tanhf(g / beta) * sig;
+    const float up_out = linear_beta > 0.0f ? linear_beta * tanhf(u / linear_beta) : u;
+    return gate_out * up_out;
+  }
+  if (limit > 0.0f) {
+    if (g > limit) g = limit;
+    if (u > limit) u = limit;
+    if (u < -limit) u = -limit;
+  }
+  return (g / (1.0f + expf(-g))) * u;
+}
+
+__device__ __forceinline__ bf16x8 as_bf16x8(u32x4 v) {
+  union { u32x4 u; bf16x8 b; } c;
+  c.u = v;
+  return c.b;
+}
+
+// WAVES wavefronts per workgroup, NT weight tiles per wavefront, MT row tiles
+// per pass.  STAGE 0 = gate/up + activation, 1 = down + combine.
+template <int STAGE, int WAVES, int NT, int MT>
+__global__ __launch_bounds__(64 * WAVES) void stream_gemm_kernel(GemmArgs p) {
+  constexpr int kThreads = 64 * WAVES;
+  constexpr int kItemsPerChunk = MT * 16 * (kKChunk / 8);  // 16-byte pieces of A
+  constexpr int kItems = (kItemsPerChunk + kThreads - 1) / kThreads;
+
+  // A operand fragments of one chunk: [MT][steps][4 d][64 lanes] x 16 bytes.
+  __shared__ u32x4 a_lds[MT * kStepsPerChunk * 4 * 64];
+  __shared__ int row_src[MT * 16];   // A row to read for each tile row, -1 = none
+  __shared__ int row_flat[MT * 16];  // flat index of each tile row, -1 = padding
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int ln = lane & 15;  // weight row within a tile / token within a row tile
+  const int lq = lane >> 4;  // quad
+
+  // ---- run of blocks owned by this workgroup -----------------------------
+  const int b0 = blockIdx.y;
+  const int e = p.expert_ids[b0];
+  if (e < 0) return;
+  if (b0 > 0 && p.expert_ids[b0 - 1] == e) return;
+  int run_blocks = 1;
+  while (b0 + run_blocks < p.num_blocks && p.expert_ids[b0 + run_blocks] == e) ++run_blocks;
+  const int run_row0 = b0 * p.block_size;
+  const int run_tiles = run_blocks * (p.block_size / 16);
+
+  // ---- weight tiles owned by this wavefront --------------------------------
+  const int K = p.K;
+  const int groups = K / 32;
+  const int row_bytes = K / 2;
+  const int units = STAGE == 0 ? p.ncols / (8 * NT) : p.ncols / (16 * NT);
+  const int unit = blockIdx.x * WAVES + wave;
+  const bool wave_active = unit < units;
+  const int rows_w = STAGE == 0 ? 2 * p.ncols : p.ncols;
+  const uint8_t* w_rows[NT];
+  const uint8_t* s_rows[NT];
+  int col0[NT];  // first output column of each tile (stage 0: gate column)
+#pragma unroll
+  for (int t = 0; t < NT; ++t) {
+    int row;
+    if (STAGE == 0) {
+      const int half = t / (NT / 2), tt = t % (NT / 2);
+      col0[t] = unit * (8 * NT) + tt * 16;
+      row = half * p.ncols + col0[t] + ln;
+    } else {
+      col0[t] = unit * (16 * NT) + t * 16;
+      row = col0[t] + ln;
+    }
+    if (!wave_active) row = 0;
+    const size_t r = (size_t)e * (size_t)rows_w + (size_t)row;
+    w_rows[t] = p.W + r * (size_t)row_bytes;
+    s_rows[t] = p.Ws + r * (size_t)groups;
+  }
+
+  const int n_chunks = (K + kKChunk - 1) / kKChunk;
+
+  for (int tile0 = 0; tile0 < run_tiles; tile0 += MT) {
+    // ---- rows of this pass ------------------------------------------------
+    __syncthreads();  // previous pass done with row_src / a_lds
+    for (int i = tid; i < MT * 16; i += kThreads) {
+      const int tile = tile0 + i / 16;
+      int flat = -1, src = -1;
+      if (tile < run_tiles) {
+        const int r = run_row0 + tile * 16 + (i & 15);
+        const int f = p.sorted_ids[r];
+        if (f >= 0 && f < p.n_flat) {
+          flat = f;
+          src = STAGE == 0 ? f / p.top_k : r;
+        }
+      }
+      row_flat[i] = flat;
+      row_src[i] = src;
+    }
+    __syncthreads();
+    bool tile_live[MT];
+    bool any_live = false;
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+      tile_live[mt] = __ballot(lane < 16 && row_flat[mt * 16 + (lane & 15)] >= 0) != 0ull;
+      any_live |= tile_live[mt];
+    }
+    if (!any_live) continue;  // uniform over the workgroup
+
+    // ---- A staging bookkeeping: item -> (tile, row, 8-wide k piece) -------
+    // item = (mt * 32 + piece) * 16 + row; piece = step*16 + q*4 + d.
+    const uint16_t* a_src[kItems];
+    int a_dst[kItems];
+    int a_k[kItems];
+#pragma unroll
+    for (int it = 0; it < kItems; ++it) {
+      const int item = tid + it * kThreads;
+      a_src[it] = nullptr;
+      a_dst[it] = 0;
+      a_k[it] = 0;
+      if (item < kItemsPerChunk) {
+        const int row = item & 15;
+        const int piece = (item >> 4) & 31;
+        const int mt = item >> 9;
+        const int step = piece >> 4, q = (piece >> 2) & 3, d = piece & 3;
+        const int src = row_src[mt * 16 + row];
+        a_dst[it] = ((mt * kStepsPerChunk + step) * 4 + d) * 64 + q * 16 + row;
+        a_k[it] = step * kKStep + q * 32 + d * 8;
+        if (src >= 0) a_src[it] = p.A + (size_t)src * (size_t)K;
+      }
+    }
+
+    u32x4 a_reg[kItems];
+    auto load_a = [&](int chunk) {
+#pragma unroll
+      for (int it = 0; it < kItems; ++it) {
+        const int k = chunk * kKChunk + a_k[it];
+        u32x4 v = {0u, 0u, 0u, 0u};
+        if (a_src[it] != nullptr && k < K)
+          v = *reinterpret_cast<const u32x4*>(a_src[it] + k);
+        a_reg[it] = v;
+      }
+    };
+    auto store_a = [&]() {
+#pragma unroll
+      for (int it = 0; it < kItems; ++it)
+        if (tid + it * kThreads < kItemsPerChunk) a_lds[a_dst[it]] = a_reg[it];
+    };
+
+    // ---- weight registers of one chunk ------------------------------------
+    u32x4 w_reg[kStepsPerChunk][NT];
+    uint32_t s_reg[kStepsPerChunk][NT];
+    auto load_w = [&](int chunk, u32x4 (&w)[kStepsPerChunk][NT],
+                      uint32_t (&s)[kStepsPerChunk][NT]) {
+#pragma unroll
+      for (int st = 0; st < kStepsPerChunk; ++st) {
+        const int g = (chunk * kStepsPerChunk + st) * 4 + lq;
+        const bool ok = wave_active && g < groups;
+#pragma unroll
+        for (int t = 0; t < NT; ++t) {
+          u32x4 v = {0u, 0u, 0u, 0u};
+          uint32_t sc = 127u;
+          if (ok) {
+            v = *reinterpret_cast<const u32x4*>(w_rows[t] + (size_t)g * 16);
+            sc = s_rows[t][g];
+          }
+          w[st][t] = v;
+          s[st][t] = sc;
+        }
+      }
+    };
+
+    f32x4 acc[NT][MT];
+#pragma unroll
+    for (int t = 0; t < NT; ++t)
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) acc[t][mt] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+    load_a(0);
+    load_w(0, w_reg, s_reg);
+
+    for (int chunk = 0; chunk < n_chunks; ++chunk) {
+      __syncthreads();  // everyone is done reading the previous chunk
+      store_a();
+      __syncthreads();
+      if (chunk + 1 < n_chunks) load_a(chunk + 1);
+
+      // Move this chunk's weights out of the prefetch registers and start
+      // the next chunk's loads before the arithmetic.
+      u32x4 w_cur[kStepsPerChunk][NT];
+      uint32_t s_cur[kStepsPerChunk][NT];
+#pragma unroll
+      for (int st = 0; st < kStepsPerChunk; ++st)
+#pragma unroll
+        for (int t = 0; t < NT; ++t) {
+          w_cur[st][t] = w_reg[st][t];
+          s_cur[st][t] = s_reg[st][t];
+        }
+      if (chunk + 1 < n_chunks) load_w(chunk + 1, w_reg, s_reg);
+
+#pragma unroll
+      for (int st = 0; st < kStepsPerChunk; ++st) {
+        // Fast conversion is valid only for finite codes and mid-range scales.
+        bool slow = false;
+#pragma unroll
+        for (int t = 0; t < NT; ++t) {
+          slow |= !scale_fast_ok(s_cur[st][t]);
+          slow |= (fp4x8_nonfinite(w_cur[st][t][0]) | fp4x8_nonfinite(w_cur[st][t][1]) |
+                   fp4x8_nonfinite(w_cur[st][t][2]) | fp4x8_nonfinite(w_cur[st][t][3])) != 0u;
+        }
+        const bool wave_slow = __ballot(slow) != 0ull;
+#pragma unroll
+        for (int d = 0; d < 4; ++d) {
+          bf16x8 wf[NT];
+          if (!wave_slow) {
+#pragma unroll
+            for (int t = 0; t < NT; ++t)
+              wf[t] = as_bf16x8(dequant8_fast(w_cur[st][t][d], scale_half_f32(s_cur[st][t])));
+          } else {
+#pragma unroll
+            for (int t = 0; t < NT; ++t)
+              wf[t] = as_bf16x8(dequant8_exact(w_cur[st][t][d], s_cur[st][t]));
+          }
+#pragma unroll
+          for (int mt = 0; mt < MT; ++mt) {
+            if (!tile_live[mt]) continue;
+            const bf16x8 af = as_bf16x8(a_lds[((mt * kStepsPerChunk + st) * 4 + d) * 64 + lane]);
+#pragma unroll
+            for (int t = 0; t < NT; ++t)
+              acc[t][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[t], af, acc[t][mt], 0, 0, 0);
+          }
+        }
+      }
+    }
+
+    // ---- epilogue -----------------------------------------------------------
+    // acc[t][mt][r] = C[weight row 4*lq + r of tile t][row ln of row tile mt]
+    if (!wave_active) continue;
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+      if (!tile_live[mt]) continue;
+      const int flat = row_flat[mt * 16 + ln];
+      if (flat < 0) continue;
+      const int srow = run_row0 + (tile0 + mt) * 16 + ln;
+      if (STAGE == 0) {
+#pragma unroll
+        for (int t = 0; t < NT / 2; ++t) {
+          const int c = col0[t] + 4 * lq;
+          uint32_t packed[2];
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            float g = acc[t][mt][r];
+            float u = acc[t + NT / 2][mt][r];
+            if (p.bias != nullptr) {
+              const float* b = p.bias + (size_t)e * (size_t)(2 * p.ncols);
+              g += b[c + r];
+              u += b[p.ncols + c + r];
+            }
+            const uint32_t v = f32_to_bf16_bits(
+                act_value(p.activation, g, u, p.swiglu_limit, p.beta, p.linear_beta));
+            if (r & 1) packed[r >> 1] |= v << 16;
+            else packed[r >> 1] = v;
+          }
+          uint2 st2 = make_uint2(packed[0], packed[1]);
+          *reinterpret_cast<uint2*>(p.act + (size_t)srow * (size_t)p.ncols + c) = st2;
+        }
+      } else {
+        const float w = p.topk_w[flat];
+        float* orow = p.out + (size_t)(flat / p.top_k) * (size_t)p.ncols;
+#pragma unroll
+        for (int t = 0; t < NT; ++t) {
+          const int c = col0[t] + 4 * lq;
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            float v = acc[t][mt][r];
+            if (p.bias != nullptr) v += p.bias[(size_t)e * (size_t)p.ncols + c + r];
+            unsafeAtomicAdd(orow + c + r, v * w);
+          }
+        }
+      }
+    }
+  }
+}
+
+template <int STAGE>
+void launch_stage(const GemmArgs& g, hipStream_t stream) {
+  constexpr int WAVES = 4, NT = 4, MT = 4;
+  const int units = STAGE == 0 ? g.ncols / (8 * NT) : g.ncols / (16 * NT);
+  const dim3 grid((units + WAVES - 1) / WAVES, g.num_blocks);
+  hipLaunchKernelGGL((stream_gemm_kernel<STAGE, WAVES, NT, MT>), grid, dim3(64 * WAVES), 0,
+                     stream, g);
+}
+
+GemmArgs common_args(const FusedMoeArgs& a) {
+  GemmArgs g{};
+  g.sorted_ids = a.sorted_ids;
+  g.expert_ids = a.expert_ids;
+  g.topk_w = a.topk_w;
+  g.act = a.act;
+  g.out = a.out;
+  g.n_flat = a.M * a.top_k;
+  g.top_k = a.top_k;
+  g.num_blocks = a.EM / a.block_size;
+  g.block_size = a.block_size;
+  g.swiglu_limit = a.swiglu_limit;
+  g.beta = a.beta;
+  g.linear_beta = a.linear_beta;
+  g.activation = a.activation;
+  return g;
+}
+
+}  // namespace
+
+void launch_moe_gateup(const FusedMoeArgs& a, hipStream_t stream) {
+  if (a.M <= 0 || a.EM <= 0 || a.block_size <= 0) return;
+  GemmArgs g = common_args(a);
+  g.A = a.A;
+  g.W = a.w13;
+  g.Ws = a.w13_scale;
+  g.bias = a.b13;
+  g.K = a.hidden;
+  g.ncols = a.ispp;
+  launch_stage<0>(g, stream);
+}
+
+void launch_moe_down(const FusedMoeArgs& a, hipStream_t stream) {
+  if (a.M <= 0 || a.EM <= 0 || a.block_size <= 0) return;
+  GemmArgs g = common_args(a);
+  g.A = a.act;
+  g.W = a.w2;
+  g.Ws = a.w2_scale;
+  g.bias = a.b2;
+  g.K = a.ispp;
+  g.ncols = a.hidden;
+  launch_stage<1>(g, stream);
+}
+
+void launch_fused_moe(const FusedMoeArgs& a, hipStream_t stream) {
+  launch_moe_gateup(a, stream);
+  launch_moe_down(a, stream);
+}
+
+}  // namespace vk

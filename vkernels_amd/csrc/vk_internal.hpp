@@ -1,0 +1,46 @@
+// vk_internal.hpp — launchers shared between the kernel translation units and
+// the C ABI.  Not part of the public interface.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace vk {
+
+void launch_route_topk(const float* logits, int T, int E, int top_k,
+                       int renormalize, int32_t* topk_ids, float* topk_w,
+                       hipStream_t stream);
+
+void launch_align(const int32_t* topk_ids, const int32_t* expert_map, int N,
+                  int block_size, int num_experts, int local_n, int max_EM,
+                  int32_t* sorted_ids, int32_t* expert_ids, int32_t* out_em,
+                  hipStream_t stream);
+
+void launch_dequant_tile(const uint8_t* packed, const uint8_t* scale,
+                         uint16_t* out_bf16, int N, int K, int stride_packed,
+                         int stride_scale_n, int stride_scale_k, int fast,
+                         hipStream_t stream);
+
+struct FusedMoeArgs {
+  const uint16_t* A;
+  const uint8_t* w13;
+  const uint8_t* w13_scale;
+  const uint8_t* w2;
+  const uint8_t* w2_scale;
+  const float* topk_w;
+  uint16_t* act;
+  float* out;
+  const int32_t* sorted_ids;
+  const int32_t* expert_ids;
+  const float* b13;
+  const float* b2;
+  int M, hidden, ispp, top_k, EM, block_size;
+  float swiglu_limit, beta, linear_beta;
+  int activation;
+};
+
+void launch_fused_moe(const FusedMoeArgs& a, hipStream_t stream);
+void launch_moe_gateup(const FusedMoeArgs& a, hipStream_t stream);
+void launch_moe_down(const FusedMoeArgs& a, hipStream_t stream);
+
+}  // namespace vk
