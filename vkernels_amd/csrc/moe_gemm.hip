@@ -33,6 +33,7 @@
 //     requires `out` to be accumulated into.
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+#include <stdlib.h>
 
 #include "moe_heuristics.hpp"
 #include "mxfp4.hpp"
@@ -86,6 +87,368 @@ __device__ __forceinline__ bf16x8 as_bf16x8(u32x4 v) {
   union { u32x4 u; bf16x8 b; } c;
   c.u = v;
   return c.b;
+}
+
+
+// Epilogue of one 16-row activation tile: acc[t][r] = C[weight row 4*lq + r of
+// tile t][activation row ln].  Stage 0 applies bias + activation to the
+// (gate, up) pairs and stores bf16; stage 1 applies bias and the routing
+// weight and adds into `out`.
+template <int STAGE, int NT>
+__device__ __forceinline__ void epilogue_tile(const GemmArgs& p, int e, const f32x4 (&acc)[NT],
+                                              const int (&col0)[NT], int flat, int srow, int lq) {
+  if (STAGE == 0) {
+#pragma unroll
+    for (int t = 0; t < NT / 2; ++t) {
+      const int c = col0[t] + 4 * lq;
+      uint32_t packed[2];
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        float g = acc[t][r];
+        float u = acc[t + NT / 2][r];
+        if (p.bias != nullptr) {
+          const float* b = p.bias + (size_t)e * (size_t)(2 * p.ncols);
+          g += b[c + r];
+          u += b[p.ncols + c + r];
+        }
+        const uint32_t v = f32_to_bf16_bits(
+            act_value(p.activation, g, u, p.swiglu_limit, p.beta, p.linear_beta));
+        if (r & 1) packed[r >> 1] |= v << 16;
+        else packed[r >> 1] = v;
+      }
+      *reinterpret_cast<uint2*>(p.act + (size_t)srow * (size_t)p.ncols + c) =
+          make_uint2(packed[0], packed[1]);
+    }
+  } else {
+    const float w = p.topk_w[flat];
+    float* orow = p.out + (size_t)(flat / p.top_k) * (size_t)p.ncols;
+#pragma unroll
+    for (int t = 0; t < NT; ++t) {
+      const int c = col0[t] + 4 * lq;
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        float v = acc[t][r];
+        if (p.bias != nullptr) v += p.bias[(size_t)e * (size_t)p.ncols + c + r];
+        unsafeAtomicAdd(orow + c + r, v * w);
+      }
+    }
+  }
+}
+
+// Weight rows, scale rows and first output column of the NT tiles of `unit`.
+template <int STAGE, int NT>
+__device__ __forceinline__ void unit_tiles(const GemmArgs& p, int e, int unit, int ln,
+                                           const uint8_t* (&w_rows)[NT],
+                                           const uint8_t* (&s_rows)[NT], int (&col0)[NT]) {
+  const int rows_w = STAGE == 0 ? 2 * p.ncols : p.ncols;
+#pragma unroll
+  for (int t = 0; t < NT; ++t) {
+    int row;
+    if (STAGE == 0) {
+      const int half = t / (NT / 2), tt = t % (NT / 2);
+      col0[t] = unit * (8 * NT) + tt * 16;
+      row = half * p.ncols + col0[t] + ln;
+    } else {
+      col0[t] = unit * (16 * NT) + t * 16;
+      row = col0[t] + ln;
+    }
+    const size_t r = (size_t)e * (size_t)rows_w + (size_t)row;
+    w_rows[t] = p.W + r * (size_t)(p.K / 2);
+    s_rows[t] = p.Ws + r * (size_t)(p.K / 32);
+  }
+}
+
+// ---------------------------------------------------------------------------
+// Decode kernel ("resident"): one workgroup per compute unit, the activation
+// rows of a run resident in LDS for the whole K dimension, no barrier inside
+// the K loop.
+//
+// The launch has as many workgroups as the device has compute units.  Every
+// workgroup lists the runs (consecutive blocks of one expert), flattens
+// (run, weight unit) into one index space and takes an equal contiguous
+// slice of it, so the weight bytes are spread evenly over the compute units
+// whatever the number of active experts.  For each run its slice touches,
+// and each 16-row pass of that run, the workgroup stages the 16 activation
+// rows, all of K, into LDS in MFMA-operand order (read coalesced, 256 bytes
+// of a row per 16 lanes; at most nsteps x 4 KiB, 92 KiB for K = 2880); then
+// each wavefront streams the weight tiles of its units from HBM through a
+// D-deep register pipeline, 64 bytes of each of its 16 rows per step, and
+// takes the activation operand with conflict-free ds_read_b128.
+//
+// LDS layout of the operand of K step ks, MFMA d (one 1 KiB plane): lane L
+// reads its 16 bytes at slot L ^ (4 d).  The XOR makes the staging stores of
+// 16 consecutive lanes (4 rows x 4 consecutive pieces of 64 bytes) fall into
+// 16 different bank groups.
+// ---------------------------------------------------------------------------
+constexpr int kMaxRuns = 1024;  // runs the resident kernel can list in LDS
+
+// Reference-exact slow path: one K step at a time, integer-exact
+// dequantisation.  Taken by a wavefront only after its fast pass met an
+// inf/NaN code or a scale byte outside [3, 252].
+template <int NT>
+__device__ __forceinline__ void resident_exact_pass(const uint8_t* const (&w_rows)[NT],
+                                                    const uint8_t* const (&s_rows)[NT],
+                                                    const u32x4* a_lds, int groups, int lane,
+                                                    f32x4 (&acc)[NT]) {
+  const int lq = lane >> 4;
+#pragma unroll
+  for (int t = 0; t < NT; ++t) acc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll 1
+  for (int ks = 0; ks * 4 < groups; ++ks) {
+    const int g = ks * 4 + lq;
+    const bool ok = g < groups;
+#pragma unroll 1
+    for (int d = 0; d < 4; ++d) {
+      const u32x4 av = a_lds[(ks * 4 + d) * 64 + (lane ^ (4 * d))];
+#pragma unroll
+      for (int t = 0; t < NT; ++t) {
+        uint32_t x = 0u, sc = 127u;
+        if (ok) {
+          x = *reinterpret_cast<const uint32_t*>(w_rows[t] + (size_t)g * 16 + d * 4);
+          sc = s_rows[t][g];
+        }
+        acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(dequant8_exact(x, sc)),
+                                                         as_bf16x8(av), acc[t], 0, 0, 0);
+      }
+    }
+  }
+}
+
+// S = number of wavefronts that share one unit, each taking 1/S of the K
+// steps; their partial sums meet in LDS.  With S > 1 a round of the unit
+// loop keeps all WAVES wavefronts busy on WAVES / S units, which evens out
+// the tail of a slice whose unit count is not a multiple of WAVES.
+template <int STAGE, int WAVES, int NT, int D, int S>
+__global__ __launch_bounds__(64 * WAVES) void stream_resident_kernel(GemmArgs p) {
+  constexpr int kSlots = WAVES / S;  // units per round
+  extern __shared__ u32x4 a_lds[];   // [nsteps][4][64], then the partial sums
+  __shared__ int run_block0[kMaxRuns];
+  __shared__ int n_runs_sh;
+  __shared__ int row_flat[16];
+  __shared__ int bad_sh[WAVES];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int ln = lane & 15;
+  const int lq = lane >> 4;
+  const int part = wave / kSlots;  // which share of K
+  const int slot = wave % kSlots;
+
+  const int K = p.K;
+  const int groups = K / 32;
+  const int nsteps = (groups + 3) / 4;  // K steps, the last one possibly partial
+  const int nfull = groups / 4;
+  const int units = STAGE == 0 ? p.ncols / (8 * NT) : p.ncols / (16 * NT);
+  // full K steps of this wavefront's share; the last share also takes the
+  // partial step, if there is one
+  const int ks_begin = nfull * part / S;
+  const int ks_end = nfull * (part + 1) / S;
+  const int n_mine = ks_end - ks_begin;
+  const int last = n_mine > 0 ? ks_end - 1 : 0;
+  const int nmain = n_mine / D;
+  const bool takes_tail = part == S - 1 && nfull * 4 < groups;
+  f32x4* red = reinterpret_cast<f32x4*>(a_lds + (size_t)nsteps * 256);  // [S-1][kSlots][NT][64]
+
+  // ---- list the runs (first block of every run, in order) -----------------
+  if (wave == 0) {
+    int n = 0;
+    for (int base = 0; base < p.num_blocks; base += 64) {
+      const int b = base + lane;
+      bool leader = false;
+      if (b < p.num_blocks) {
+        const int e = p.expert_ids[b];
+        leader = e >= 0 && (b == 0 || p.expert_ids[b - 1] != e);
+      }
+      const unsigned long long m = __ballot(leader);
+      if (leader) {
+        const int idx = n + (int)__popcll(m & ((1ull << lane) - 1ull));
+        if (idx < kMaxRuns) run_block0[idx] = b;
+      }
+      n += (int)__popcll(m);
+    }
+    if (lane == 0) n_runs_sh = n < kMaxRuns ? n : kMaxRuns;
+  }
+  __syncthreads();
+  const int n_runs = n_runs_sh;
+  const long long total = (long long)n_runs * units;
+  const long long per_wg = (total + gridDim.x - 1) / gridDim.x;
+  const long long s0 = (long long)blockIdx.x * per_wg;
+  const long long s1 = s0 + per_wg < total ? s0 + per_wg : total;
+  if (s0 >= s1) return;  // uniform over the workgroup
+
+  struct Stage {
+    u32x4 w[NT];
+    uint32_t s[NT];  // four scale bytes of the step; this lane uses byte lq
+  };
+
+  for (int r = (int)(s0 / units); r <= (int)((s1 - 1) / units); ++r) {
+    const long long base_slot = (long long)r * units;
+    const int u0 = (int)((s0 > base_slot ? s0 : base_slot) - base_slot);
+    const int u1 = (int)((s1 < base_slot + units ? s1 : base_slot + units) - base_slot);
+    const int b0 = run_block0[r];
+    const int e = p.expert_ids[b0];
+    int run_blocks = 1;
+    while (b0 + run_blocks < p.num_blocks && p.expert_ids[b0 + run_blocks] == e) ++run_blocks;
+    const int run_row0 = b0 * p.block_size;
+    const int run_tiles = run_blocks * (p.block_size / 16);
+
+    for (int tile = 0; tile < run_tiles; ++tile) {
+      // ---- rows of this pass ------------------------------------------------
+      __syncthreads();  // previous pass is done with row_flat and a_lds
+      if (tid < 16) {
+        const int f = p.sorted_ids[run_row0 + tile * 16 + tid];
+        row_flat[tid] = (f >= 0 && f < p.n_flat) ? f : -1;
+      }
+      __syncthreads();
+      bool any = false;
+#pragma unroll
+      for (int j = 0; j < 16; ++j) any |= row_flat[j] >= 0;
+      if (!any) continue;  // uniform
+
+      // ---- stage the 16 rows, all of K, in operand order --------------------
+      // Lane (j, d) = (lane / 4, lane % 4) copies piece d of quad q of K step
+      // ks of row j; 4 lanes read 64 contiguous bytes.  Loads first, stores
+      // after, so that the copies of one wavefront are all in flight together.
+      {
+        constexpr int kMaxIter = 10;  // WAVES * kMaxIter >= nsteps * 4 (checked by the launcher)
+        const int d = lane & 3;
+        const int j = lane >> 2;
+        const int f = row_flat[j];
+        const uint16_t* src =
+            p.A + (size_t)(f >= 0 ? (STAGE == 0 ? f / p.top_k : run_row0 + tile * 16 + j) : 0) *
+                      (size_t)K;
+        u32x4 v[kMaxIter];
+#pragma unroll
+        for (int it = 0; it < kMaxIter; ++it) {
+          const int pq = wave + it * WAVES;
+          const int k = (pq >> 2) * kKStep + (pq & 3) * 32 + d * 8;
+          v[it] = u32x4{0u, 0u, 0u, 0u};
+          if (pq < nsteps * 4 && k < K && f >= 0) v[it] = *reinterpret_cast<const u32x4*>(src + k);
+        }
+#pragma unroll
+        for (int it = 0; it < kMaxIter; ++it) {
+          const int pq = wave + it * WAVES;
+          if (pq < nsteps * 4)
+            a_lds[((pq >> 2) * 4 + d) * 64 + (((pq & 3) * 16 + j) ^ (4 * d))] = v[it];
+        }
+      }
+      __syncthreads();
+
+      const int my_flat = row_flat[ln];
+      const int srow = run_row0 + tile * 16 + ln;
+
+      // ---- rounds of kSlots units ---------------------------------------------
+      for (int ub = u0; ub < u1; ub += kSlots) {
+        const int unit = ub + slot;
+        const bool active = unit < u1;
+        const uint8_t* w_rows[NT];
+        const uint8_t* s_rows[NT];
+        int col0[NT];
+        unit_tiles<STAGE, NT>(p, e, active ? unit : u0, ln, w_rows, s_rows, col0);
+
+        auto load = [&](Stage& st, int ks) {
+          const size_t g = (size_t)(ks * 4 + lq);
+#pragma unroll
+          for (int t = 0; t < NT; ++t) {
+            st.w[t] = *reinterpret_cast<const u32x4*>(w_rows[t] + g * 16);
+            __builtin_memcpy(&st.s[t], s_rows[t] + ks * 4, 4);
+          }
+        };
+
+        f32x4 acc[NT];
+#pragma unroll
+        for (int t = 0; t < NT; ++t) acc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+        uint32_t bad = 0u;
+
+        auto compute = [&](const Stage& st, int ks) {
+          float sc[NT];
+#pragma unroll
+          for (int t = 0; t < NT; ++t) {
+            const uint32_t sb = (st.s[t] >> (8 * lq)) & 0xFFu;
+            bad |= (uint32_t)!scale_fast_ok(sb);
+            bad |= fp4x8_nonfinite(st.w[t][0]) | fp4x8_nonfinite(st.w[t][1]) |
+                   fp4x8_nonfinite(st.w[t][2]) | fp4x8_nonfinite(st.w[t][3]);
+            sc[t] = scale_half_f32(sb);
+          }
+#pragma unroll
+          for (int d = 0; d < 4; ++d) {
+            const bf16x8 af = as_bf16x8(a_lds[(ks * 4 + d) * 64 + (lane ^ (4 * d))]);
+#pragma unroll
+            for (int t = 0; t < NT; ++t)
+              acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+                  as_bf16x8(dequant8_fast(st.w[t][d], sc[t])), af, acc[t], 0, 0, 0);
+          }
+        };
+
+        if (active) {
+          if (n_mine > 0) {
+            Stage st[D];
+#pragma unroll
+            for (int i = 0; i < D; ++i) load(st[i], min(ks_begin + i, last));
+            for (int it = 0; it < nmain; ++it) {
+#pragma unroll
+              for (int i = 0; i < D; ++i) {
+                compute(st[i], ks_begin + it * D + i);
+                load(st[i], min(ks_begin + (it + 1) * D + i, last));
+              }
+            }
+            const int rem = n_mine - nmain * D;
+#pragma unroll
+            for (int i = 0; i < D - 1; ++i)
+              if (i < rem) compute(st[i], ks_begin + nmain * D + i);
+          }
+          if (takes_tail) {
+            // last, partial K step: quads past the end contribute zeros
+            Stage st;
+            const int g = nfull * 4 + lq;
+            const bool ok = g < groups;
+#pragma unroll
+            for (int t = 0; t < NT; ++t) {
+              st.w[t] = u32x4{0u, 0u, 0u, 0u};
+              st.s[t] = 127u << (8 * lq);
+              if (ok) {
+                st.w[t] = *reinterpret_cast<const u32x4*>(w_rows[t] + (size_t)g * 16);
+                st.s[t] = (uint32_t)s_rows[t][g] << (8 * lq);
+              }
+            }
+            compute(st, nfull);
+          }
+        }
+        bool wave_bad = __ballot(bad != 0u) != 0ull;
+
+        if (S > 1) {
+          // partial sums of the other shares meet in LDS
+          __syncthreads();  // the previous round's sums have been read
+          if (part > 0 && active) {
+#pragma unroll
+            for (int t = 0; t < NT; ++t)
+              red[(((part - 1) * kSlots + slot) * NT + t) * 64 + lane] = acc[t];
+          }
+          if (lane == 0) bad_sh[wave] = wave_bad ? 1 : 0;
+          __syncthreads();
+          if (part == 0 && active) {
+#pragma unroll
+            for (int o = 1; o < S; ++o) {
+#pragma unroll
+              for (int t = 0; t < NT; ++t) {
+                const f32x4 v = red[(((o - 1) * kSlots + slot) * NT + t) * 64 + lane];
+                acc[t][0] += v[0];
+                acc[t][1] += v[1];
+                acc[t][2] += v[2];
+                acc[t][3] += v[3];
+              }
+              wave_bad |= bad_sh[o * kSlots + slot] != 0;
+            }
+          }
+        }
+        if (part == 0 && active) {
+          if (wave_bad) resident_exact_pass<NT>(w_rows, s_rows, a_lds, groups, lane, acc);
+          if (my_flat >= 0) epilogue_tile<STAGE, NT>(p, e, acc, col0, my_flat, srow, lq);
+        }
+      }
+    }
+  }
 }
 
 // WAVES wavefronts per workgroup, NT weight tiles per wavefront, MT row tiles
@@ -349,8 +712,63 @@ __global__ __launch_bounds__(64 * WAVES) void stream_gemm_kernel(GemmArgs p) {
   }
 }
 
+int env_int(const char* name, int fallback) {
+  const char* v = getenv(name);
+  return (v != nullptr && *v != 0) ? atoi(v) : fallback;
+}
+
+int num_compute_units() {
+  static const int cus = [] {
+    int dev = 0, n = 0;
+    if (hipGetDevice(&dev) != hipSuccess) return 256;
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0)
+      return 256;
+    return n;
+  }();
+  return cus;
+}
+
+constexpr size_t kResidentLdsLimit = 144 * 1024;  // dynamic LDS the resident kernel may ask for
+
+template <int STAGE, int WAVES, int NT, int D, int S>
+void launch_resident(const GemmArgs& g, size_t lds, hipStream_t stream) {
+  auto* kern = stream_resident_kernel<STAGE, WAVES, NT, D, S>;
+  static const bool configured = [kern] {
+    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                              hipFuncAttributeMaxDynamicSharedMemorySize,
+                              (int)kResidentLdsLimit);
+    return true;
+  }();
+  (void)configured;
+  const int wgs = env_int("VK_MOE_WGS", num_compute_units());
+  hipLaunchKernelGGL(kern, dim3(wgs), dim3(64 * WAVES), lds, stream, g);
+}
+
 template <int STAGE>
 void launch_stage(const GemmArgs& g, hipStream_t stream) {
+  const MoeTile tile = pick_moe_tile(g.n_flat, g.K, g.ncols);
+  int variant = env_int("VK_MOE_VARIANT", tile.variant);
+  const int nt = env_int("VK_MOE_NT", tile.nt);
+  const int depth = env_int("VK_MOE_DEPTH", tile.depth);
+  const int waves = env_int("VK_MOE_WAVES", tile.waves);
+  const int split = env_int("VK_MOE_SPLIT", tile.split);
+  const int nsteps = (g.K / 32 + 3) / 4;
+  // operand planes + partial sums of the K-split
+  const size_t resident_lds = (size_t)nsteps * 4096 +
+                              (size_t)(split - 1) * (waves / split) * nt * 1024;
+  if (resident_lds > kResidentLdsLimit || g.num_blocks > kMaxRuns || nsteps * 4 > waves * 10)
+    variant = kMoeVariantLds;
+  if (variant == kMoeVariantResident) {
+#define VK_RESIDENT(W_, NT_, D_, S_) \
+  if (waves == W_ && nt == NT_ && depth == D_ && split == S_) \
+    return launch_resident<STAGE, W_, NT_, D_, S_>(g, resident_lds, stream)
+    VK_RESIDENT(16, 2, 3, 1); VK_RESIDENT(16, 2, 2, 2); VK_RESIDENT(16, 2, 3, 2);
+    VK_RESIDENT(16, 2, 4, 2); VK_RESIDENT(16, 2, 2, 4); VK_RESIDENT(16, 2, 3, 4);
+    VK_RESIDENT(8, 2, 4, 1); VK_RESIDENT(8, 2, 4, 2); VK_RESIDENT(8, 2, 6, 2); VK_RESIDENT(8, 2, 3, 2);
+    VK_RESIDENT(8, 4, 3, 2); VK_RESIDENT(8, 4, 2, 2); VK_RESIDENT(16, 4, 2, 2);
+#undef VK_RESIDENT
+    return launch_resident<STAGE, 16, 2, 3, 2>(g, (size_t)nsteps * 4096 + 8 * 2 * 1024, stream);
+  }
   constexpr int WAVES = 4, NT = 4, MT = 4;
   const int units = STAGE == 0 ? g.ncols / (8 * NT) : g.ncols / (16 * NT);
   const dim3 grid((units + WAVES - 1) / WAVES, g.num_blocks);

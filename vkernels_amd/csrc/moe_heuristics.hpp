@@ -1,4 +1,4 @@
-// moe_heuristics.hpp — tile shapes of the MoE grouped GEMMs for gfx950.
+// moe_heuristics.hpp — launch shapes of the MoE grouped GEMMs for gfx950.
 //
 // Same role as the GEMM candidate table of the reference
 // (src/c/vkernels/kernels/common/heuristics.hpp:20-61), which has no MoE
@@ -8,10 +8,27 @@
 
 namespace vk {
 
+enum { kMoeVariantLds = 0, kMoeVariantResident = 2 };
+
 struct MoeTile {
-  int waves;  // wavefronts per workgroup
-  int nt;     // 16-row weight tiles per wavefront
-  int mt;     // 16-row activation tiles per pass
+  int variant;  // kMoeVariantResident: one workgroup per compute unit, the
+                // activation rows of a run resident in LDS (decode);
+                // kMoeVariantLds: activation rows staged through LDS chunk by chunk
+  int waves;    // wavefronts per workgroup
+  int nt;       // 16-row weight tiles per wavefront
+  int depth;    // K steps in flight per wavefront (resident variant)
+  int split;    // wavefronts sharing the K steps of one unit (resident variant)
 };
+
+// n_flat = tokens * top_k routed rows in the call, K / ncols the GEMM's
+// reduction and output widths.  The number of experts is not known to the
+// launcher, so the split is on the routed rows alone: a decode batch leaves
+// most experts with at most one 16-row tile.
+inline MoeTile pick_moe_tile(int n_flat, int K, int ncols) {
+  (void)K;
+  (void)ncols;
+  if (n_flat <= 512) return MoeTile{kMoeVariantResident, 16, 2, 3, 1};
+  return MoeTile{kMoeVariantLds, 4, 4, 0, 1};
+}
 
 }  // namespace vk
