@@ -45,6 +45,9 @@ def parse_args():
     ap.add_argument("--weight-sets", type=int, default=0, help="0 = enough to exceed 1 GiB")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--block-size", type=int, default=0)
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also run a 512 MiB device copy three times, so that a profiler's "
+                         "FETCH_SIZE / WRITE_SIZE counters can be scaled by a kernel of known traffic")
     return ap.parse_args()
 
 
@@ -202,6 +205,12 @@ def main():
             "down_kernel_gbs": down_bytes / (down_avg * 1e-3) / 1e9,
         },
     }
+    if args.copy_calibration:
+        src = torch.empty(512 << 20, dtype=torch.uint8, device=dev).fill_(1)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
     if not args.no_cpu:
         line["cpu_baseline"] = cpu_baseline(cfg, T, seed)
     print(json.dumps(line))
