@@ -35,6 +35,8 @@
 #include <stdint.h>
 #include <stdlib.h>
 
+#include <type_traits>
+
 #include "moe_heuristics.hpp"
 #include "mxfp4.hpp"
 #include "vk_internal.hpp"
@@ -80,7 +82,8 @@ __device__ __forceinline__ float act_value(int activation, float g, float u,
     if (u > limit) u = limit;
     if (u < -limit) u = -limit;
   }
-  return (g / (1.0f + expf(-g))) * u;
+  // v_exp_f32 / v_rcp_f32: about 1 ulp each, far inside the bf16 rounding that follows
+  return (g * __builtin_amdgcn_rcpf(1.0f + __expf(-g))) * u;
 }
 
 __device__ __forceinline__ bf16x8 as_bf16x8(u32x4 v) {
@@ -182,6 +185,9 @@ __device__ __forceinline__ void unit_tiles(const GemmArgs& p, int e, int unit, i
 // ---------------------------------------------------------------------------
 constexpr int kMaxRuns = 1024;  // runs the resident kernel can list in LDS
 
+__device__ unsigned long long g_dbg_times[16 * 32];
+#define VK_DBG_T(slot) do { if (blockIdx.x == 3 && lane == 0 && (slot) < 32) g_dbg_times[wave * 32 + (slot)] = clock64(); } while (0)
+
 // Reference-exact slow path: one K step at a time, integer-exact
 // dequantisation.  Taken by a wavefront only after its fast pass met an
 // inf/NaN code or a scale byte outside [3, 252].
@@ -218,7 +224,7 @@ __device__ __forceinline__ void resident_exact_pass(const uint8_t* const (&w_row
 // steps; their partial sums meet in LDS.  With S > 1 a round of the unit
 // loop keeps all WAVES wavefronts busy on WAVES / S units, which evens out
 // the tail of a slice whose unit count is not a multiple of WAVES.
-template <int STAGE, int WAVES, int NT, int D, int S>
+template <int STAGE, int WAVES, int NT, int D, int S, int DBG = 0>
 __global__ __launch_bounds__(64 * WAVES) void stream_resident_kernel(GemmArgs p) {
   constexpr int kSlots = WAVES / S;  // units per round
   extern __shared__ u32x4 a_lds[];   // [nsteps][4][64], then the partial sums
@@ -250,6 +256,8 @@ __global__ __launch_bounds__(64 * WAVES) void stream_resident_kernel(GemmArgs p)
   const bool takes_tail = part == S - 1 && nfull * 4 < groups;
   f32x4* red = reinterpret_cast<f32x4*>(a_lds + (size_t)nsteps * 256);  // [S-1][kSlots][NT][64]
 
+  int dbg_slot = 0;
+  VK_DBG_T(dbg_slot++);
   // ---- list the runs (first block of every run, in order) -----------------
   if (wave == 0) {
     int n = 0;
@@ -270,6 +278,7 @@ __global__ __launch_bounds__(64 * WAVES) void stream_resident_kernel(GemmArgs p)
     if (lane == 0) n_runs_sh = n < kMaxRuns ? n : kMaxRuns;
   }
   __syncthreads();
+  VK_DBG_T(dbg_slot++);
   const int n_runs = n_runs_sh;
   const long long total = (long long)n_runs * units;
   const long long per_wg = (total + gridDim.x - 1) / gridDim.x;
@@ -279,8 +288,11 @@ __global__ __launch_bounds__(64 * WAVES) void stream_resident_kernel(GemmArgs p)
 
   struct Stage {
     u32x4 w[NT];
-    uint32_t s[NT];  // four scale bytes of the step; this lane uses byte lq
   };
+  // scale bytes of this wavefront's current unit: [NT][16 rows][groups]
+  const int sc_tile_bytes = 16 * groups;
+  uint8_t* sc_lds = reinterpret_cast<uint8_t*>(a_lds + (size_t)nsteps * 256) +
+                    (size_t)(S - 1) * kSlots * NT * 1024 + (size_t)wave * NT * sc_tile_bytes;
 
   for (int r = (int)(s0 / units); r <= (int)((s1 - 1) / units); ++r) {
     const long long base_slot = (long long)r * units;
@@ -311,29 +323,33 @@ __global__ __launch_bounds__(64 * WAVES) void stream_resident_kernel(GemmArgs p)
       // ks of row j; 4 lanes read 64 contiguous bytes.  Loads first, stores
       // after, so that the copies of one wavefront are all in flight together.
       {
-        constexpr int kMaxIter = 10;  // WAVES * kMaxIter >= nsteps * 4 (checked by the launcher)
+        constexpr int kBatch = 4;  // copies in flight per lane
         const int d = lane & 3;
         const int j = lane >> 2;
         const int f = row_flat[j];
         const uint16_t* src =
             p.A + (size_t)(f >= 0 ? (STAGE == 0 ? f / p.top_k : run_row0 + tile * 16 + j) : 0) *
                       (size_t)K;
-        u32x4 v[kMaxIter];
+        for (int pq0 = wave; pq0 < nsteps * 4 && DBG < 3; pq0 += WAVES * kBatch) {
+          u32x4 v[kBatch];
 #pragma unroll
-        for (int it = 0; it < kMaxIter; ++it) {
-          const int pq = wave + it * WAVES;
-          const int k = (pq >> 2) * kKStep + (pq & 3) * 32 + d * 8;
-          v[it] = u32x4{0u, 0u, 0u, 0u};
-          if (pq < nsteps * 4 && k < K && f >= 0) v[it] = *reinterpret_cast<const u32x4*>(src + k);
-        }
+          for (int it = 0; it < kBatch; ++it) {
+            const int pq = pq0 + it * WAVES;
+            const int k = (pq >> 2) * kKStep + (pq & 3) * 32 + d * 8;
+            v[it] = u32x4{0u, 0u, 0u, 0u};
+            if (pq < nsteps * 4 && k < K && f >= 0) v[it] = *reinterpret_cast<const u32x4*>(src + k);
+          }
 #pragma unroll
-        for (int it = 0; it < kMaxIter; ++it) {
-          const int pq = wave + it * WAVES;
-          if (pq < nsteps * 4)
-            a_lds[((pq >> 2) * 4 + d) * 64 + (((pq & 3) * 16 + j) ^ (4 * d))] = v[it];
+          for (int it = 0; it < kBatch; ++it) {
+            const int pq = pq0 + it * WAVES;
+            if (pq < nsteps * 4)
+              a_lds[((pq >> 2) * 4 + d) * 64 + (((pq & 3) * 16 + j) ^ (4 * d))] = v[it];
+          }
         }
       }
+      VK_DBG_T(dbg_slot++);
       __syncthreads();
+      VK_DBG_T(dbg_slot++);
 
       const int my_flat = row_flat[ln];
       const int srow = run_row0 + tile * 16 + ln;
@@ -347,13 +363,24 @@ __global__ __launch_bounds__(64 * WAVES) void stream_resident_kernel(GemmArgs p)
         int col0[NT];
         unit_tiles<STAGE, NT>(p, e, active ? unit : u0, ln, w_rows, s_rows, col0);
 
-        auto load = [&](Stage& st, int ks) {
-          const size_t g = (size_t)(ks * 4 + lq);
+        // The unit's scale bytes (16 rows x groups, contiguous per tile) come in
+        // with a few coalesced 16-byte loads instead of one load per K step.
+        if (active && DBG < 5) {
 #pragma unroll
           for (int t = 0; t < NT; ++t) {
-            st.w[t] = *reinterpret_cast<const u32x4*>(w_rows[t] + g * 16);
-            __builtin_memcpy(&st.s[t], s_rows[t] + ks * 4, 4);
+            const uint8_t* src = s_rows[t] - (size_t)ln * groups;
+            for (int off = lane * 16; off < sc_tile_bytes; off += 1024)
+              *reinterpret_cast<u32x4*>(sc_lds + t * sc_tile_bytes + off) =
+                  *reinterpret_cast<const u32x4*>(src + off);
           }
+        }
+
+        auto load = [&](Stage& st, int ks) {
+          if (DBG == 2 && ks > 3) return;  // diagnosis: no weight traffic in steady state
+          const size_t g = (size_t)(ks * 4 + lq);
+#pragma unroll
+          for (int t = 0; t < NT; ++t)
+            st.w[t] = *reinterpret_cast<const u32x4*>(w_rows[t] + g * 16);
         };
 
         f32x4 acc[NT];
@@ -361,11 +388,20 @@ __global__ __launch_bounds__(64 * WAVES) void stream_resident_kernel(GemmArgs p)
         for (int t = 0; t < NT; ++t) acc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
         uint32_t bad = 0u;
 
-        auto compute = [&](const Stage& st, int ks) {
+        auto compute = [&](const Stage& st, int ks, auto tail) {
+          if (DBG == 1 || DBG >= 3) {  // diagnosis: consume the data without dequant / LDS / MFMA
+#pragma unroll
+            for (int t = 0; t < NT; ++t)
+              acc[t][0] += __uint_as_float((st.w[t][0] ^ st.w[t][1] ^ st.w[t][2] ^ st.w[t][3]) & 0x3FFFFFFFu);
+            return;
+          }
           float sc[NT];
+          const int g = ks * 4 + lq;
 #pragma unroll
           for (int t = 0; t < NT; ++t) {
-            const uint32_t sb = (st.s[t] >> (8 * lq)) & 0xFFu;
+            const uint32_t sb = (!decltype(tail)::value || g < groups)
+                                    ? (uint32_t)sc_lds[t * sc_tile_bytes + ln * groups + g]
+                                    : 127u;
             bad |= (uint32_t)!scale_fast_ok(sb);
             bad |= fp4x8_nonfinite(st.w[t][0]) | fp4x8_nonfinite(st.w[t][1]) |
                    fp4x8_nonfinite(st.w[t][2]) | fp4x8_nonfinite(st.w[t][3]);
@@ -389,16 +425,19 @@ __global__ __launch_bounds__(64 * WAVES) void stream_resident_kernel(GemmArgs p)
             for (int it = 0; it < nmain; ++it) {
 #pragma unroll
               for (int i = 0; i < D; ++i) {
-                compute(st[i], ks_begin + it * D + i);
+                compute(st[i], ks_begin + it * D + i, std::false_type{});
                 load(st[i], min(ks_begin + (it + 1) * D + i, last));
+                // keep the scheduler from pulling the next step's conversions
+                // up here: that only lengthens live ranges until they spill
+                __builtin_amdgcn_sched_barrier(0);
               }
             }
             const int rem = n_mine - nmain * D;
 #pragma unroll
             for (int i = 0; i < D - 1; ++i)
-              if (i < rem) compute(st[i], ks_begin + nmain * D + i);
+              if (i < rem) compute(st[i], ks_begin + nmain * D + i, std::false_type{});
           }
-          if (takes_tail) {
+          if (takes_tail && DBG < 6) {
             // last, partial K step: quads past the end contribute zeros
             Stage st;
             const int g = nfull * 4 + lq;
@@ -406,13 +445,9 @@ __global__ __launch_bounds__(64 * WAVES) void stream_resident_kernel(GemmArgs p)
 #pragma unroll
             for (int t = 0; t < NT; ++t) {
               st.w[t] = u32x4{0u, 0u, 0u, 0u};
-              st.s[t] = 127u << (8 * lq);
-              if (ok) {
-                st.w[t] = *reinterpret_cast<const u32x4*>(w_rows[t] + (size_t)g * 16);
-                st.s[t] = (uint32_t)s_rows[t][g] << (8 * lq);
-              }
+              if (ok) st.w[t] = *reinterpret_cast<const u32x4*>(w_rows[t] + (size_t)g * 16);
             }
-            compute(st, nfull);
+            compute(st, nfull, std::true_type{});
           }
         }
         bool wave_bad = __ballot(bad != 0u) != 0ull;
@@ -442,10 +477,13 @@ __global__ __launch_bounds__(64 * WAVES) void stream_resident_kernel(GemmArgs p)
             }
           }
         }
+        VK_DBG_T(dbg_slot++);
         if (part == 0 && active) {
           if (wave_bad) resident_exact_pass<NT>(w_rows, s_rows, a_lds, groups, lane, acc);
-          if (my_flat >= 0) epilogue_tile<STAGE, NT>(p, e, acc, col0, my_flat, srow, lq);
+          if (DBG >= 4) { if (my_flat == 12345678) { float sum = 0.f; for (int t = 0; t < NT; ++t) sum += acc[t][0]; p.act[lane] = (uint16_t)sum; } }
+          else if (my_flat >= 0) epilogue_tile<STAGE, NT>(p, e, acc, col0, my_flat, srow, lq);
         }
+        VK_DBG_T(dbg_slot++);
       }
     }
   }
@@ -728,11 +766,11 @@ int num_compute_units() {
   return cus;
 }
 
-constexpr size_t kResidentLdsLimit = 144 * 1024;  // dynamic LDS the resident kernel may ask for
+constexpr size_t kResidentLdsLimit = 152 * 1024;  // dynamic LDS the resident kernel may ask for
 
-template <int STAGE, int WAVES, int NT, int D, int S>
+template <int STAGE, int WAVES, int NT, int D, int S, int DBG = 0>
 void launch_resident(const GemmArgs& g, size_t lds, hipStream_t stream) {
-  auto* kern = stream_resident_kernel<STAGE, WAVES, NT, D, S>;
+  auto* kern = stream_resident_kernel<STAGE, WAVES, NT, D, S, DBG>;
   static const bool configured = [kern] {
     (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                               hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -755,10 +793,18 @@ void launch_stage(const GemmArgs& g, hipStream_t stream) {
   const int nsteps = (g.K / 32 + 3) / 4;
   // operand planes + partial sums of the K-split
   const size_t resident_lds = (size_t)nsteps * 4096 +
-                              (size_t)(split - 1) * (waves / split) * nt * 1024;
-  if (resident_lds > kResidentLdsLimit || g.num_blocks > kMaxRuns || nsteps * 4 > waves * 10)
+                              (size_t)(split - 1) * (waves / split) * nt * 1024 +
+                              (size_t)waves * nt * 16 * (g.K / 32);
+  if (resident_lds > kResidentLdsLimit || g.num_blocks > kMaxRuns || nsteps * 4 > 128)
     variant = kMoeVariantLds;
   if (variant == kMoeVariantResident) {
+    const int dbg = env_int("VK_MOE_DBG", 0);
+    if (dbg == 1) return launch_resident<STAGE, 16, 2, 3, 1, 1>(g, resident_lds, stream);
+    if (dbg == 2) return launch_resident<STAGE, 16, 2, 3, 1, 2>(g, resident_lds, stream);
+    if (dbg == 3) return launch_resident<STAGE, 16, 2, 3, 1, 3>(g, resident_lds, stream);
+    if (dbg == 4) return launch_resident<STAGE, 16, 2, 3, 1, 4>(g, resident_lds, stream);
+    if (dbg == 5) return launch_resident<STAGE, 16, 2, 3, 1, 5>(g, resident_lds, stream);
+    if (dbg == 6) return launch_resident<STAGE, 16, 2, 3, 1, 6>(g, resident_lds, stream);
 #define VK_RESIDENT(W_, NT_, D_, S_) \
   if (waves == W_ && nt == NT_ && depth == D_ && split == S_) \
     return launch_resident<STAGE, W_, NT_, D_, S_>(g, resident_lds, stream)
@@ -766,8 +812,11 @@ void launch_stage(const GemmArgs& g, hipStream_t stream) {
     VK_RESIDENT(16, 2, 4, 2); VK_RESIDENT(16, 2, 2, 4); VK_RESIDENT(16, 2, 3, 4);
     VK_RESIDENT(8, 2, 4, 1); VK_RESIDENT(8, 2, 4, 2); VK_RESIDENT(8, 2, 6, 2); VK_RESIDENT(8, 2, 3, 2);
     VK_RESIDENT(8, 4, 3, 2); VK_RESIDENT(8, 4, 2, 2); VK_RESIDENT(16, 4, 2, 2);
+    VK_RESIDENT(8, 2, 3, 1); VK_RESIDENT(8, 2, 6, 1); VK_RESIDENT(8, 2, 8, 1);
+    VK_RESIDENT(8, 4, 2, 1); VK_RESIDENT(8, 4, 3, 1); VK_RESIDENT(8, 4, 4, 1);
+    VK_RESIDENT(12, 2, 3, 1); VK_RESIDENT(12, 2, 4, 1); VK_RESIDENT(12, 2, 6, 1);
 #undef VK_RESIDENT
-    return launch_resident<STAGE, 16, 2, 3, 2>(g, (size_t)nsteps * 4096 + 8 * 2 * 1024, stream);
+    variant = kMoeVariantLds;
   }
   constexpr int WAVES = 4, NT = 4, MT = 4;
   const int units = STAGE == 0 ? g.ncols / (8 * NT) : g.ncols / (16 * NT);
@@ -795,6 +844,10 @@ GemmArgs common_args(const FusedMoeArgs& a) {
 }
 
 }  // namespace
+
+extern "C" void vk_hip_debug_read_times(unsigned long long* host) {
+  (void)hipMemcpyFromSymbol(host, HIP_SYMBOL(g_dbg_times), sizeof(unsigned long long) * 16 * 32);
+}
 
 void launch_moe_gateup(const FusedMoeArgs& a, hipStream_t stream) {
   if (a.M <= 0 || a.EM <= 0 || a.block_size <= 0) return;
