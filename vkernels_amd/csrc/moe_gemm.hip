@@ -164,7 +164,7 @@ __device__ __forceinline__ void unit_tiles(const GemmArgs& p, int e, int unit, i
 // ---------------------------------------------------------------------------
 // Decode kernel ("resident"): one workgroup per compute unit, the activation
 // rows of a run resident in LDS for the whole K dimension, no barrier inside
-// the K loop.
+// the K loop, and every wavefront's weight loads one uninterrupted stream.
 //
 // The launch has as many workgroups as the device has compute units.  Every
 // workgroup lists the runs (consecutive blocks of one expert), flattens
@@ -172,25 +172,28 @@ __device__ __forceinline__ void unit_tiles(const GemmArgs& p, int e, int unit, i
 // slice of it, so the weight bytes are spread evenly over the compute units
 // whatever the number of active experts.  For each run its slice touches,
 // and each 16-row pass of that run, the workgroup stages the 16 activation
-// rows, all of K, into LDS in MFMA-operand order (read coalesced, 256 bytes
-// of a row per 16 lanes; at most nsteps x 4 KiB, 92 KiB for K = 2880); then
-// each wavefront streams the weight tiles of its units from HBM through a
-// D-deep register pipeline, 64 bytes of each of its 16 rows per step, and
-// takes the activation operand with conflict-free ds_read_b128.
+// rows, all of K, into LDS in MFMA-operand order (read coalesced; at most
+// nsteps x 4 KiB, 92 KiB for K = 2880).  Wavefront w then takes units
+// w, w + WAVES, ... of the slice and walks their K steps as ONE sequence:
+// a D-deep register pipeline of 16-byte-per-lane weight loads whose cursor
+// runs ahead of the arithmetic and crosses from one unit into the next, so
+// that neither the epilogue of a unit nor the start of the next one leaves
+// the memory pipe empty.  The scale bytes of a unit (16 rows x K/32,
+// contiguous per tile) are fetched with a few coalesced loads while the
+// previous unit streams and parked in a per-wavefront LDS region.
 //
 // LDS layout of the operand of K step ks, MFMA d (one 1 KiB plane): lane L
 // reads its 16 bytes at slot L ^ (4 d).  The XOR makes the staging stores of
 // 16 consecutive lanes (4 rows x 4 consecutive pieces of 64 bytes) fall into
-// 16 different bank groups.
+// 16 different bank groups.  Planes past K are zero, which is what makes the
+// last, partial K step need no masking of the weight side.
 // ---------------------------------------------------------------------------
 constexpr int kMaxRuns = 1024;  // runs the resident kernel can list in LDS
-
-__device__ unsigned long long g_dbg_times[16 * 32];
-#define VK_DBG_T(slot) do { if (blockIdx.x == 3 && lane == 0 && (slot) < 32) g_dbg_times[wave * 32 + (slot)] = clock64(); } while (0)
+constexpr int kScMax = 4;       // 16-byte scale pieces per lane: NT * K/32 <= 64 * kScMax
 
 // Reference-exact slow path: one K step at a time, integer-exact
-// dequantisation.  Taken by a wavefront only after its fast pass met an
-// inf/NaN code or a scale byte outside [3, 252].
+// dequantisation.  Taken by a wavefront only after its fast pass over a unit
+// met an inf/NaN code or a scale byte outside [3, 252].
 template <int NT>
 __device__ __forceinline__ void resident_exact_pass(const uint8_t* const (&w_rows)[NT],
                                                     const uint8_t* const (&s_rows)[NT],
@@ -220,44 +223,29 @@ __device__ __forceinline__ void resident_exact_pass(const uint8_t* const (&w_row
   }
 }
 
-// S = number of wavefronts that share one unit, each taking 1/S of the K
-// steps; their partial sums meet in LDS.  With S > 1 a round of the unit
-// loop keeps all WAVES wavefronts busy on WAVES / S units, which evens out
-// the tail of a slice whose unit count is not a multiple of WAVES.
-template <int STAGE, int WAVES, int NT, int D, int S, int DBG = 0>
+template <int STAGE, int WAVES, int NT, int D>
 __global__ __launch_bounds__(64 * WAVES) void stream_resident_kernel(GemmArgs p) {
-  constexpr int kSlots = WAVES / S;  // units per round
-  extern __shared__ u32x4 a_lds[];   // [nsteps][4][64], then the partial sums
+  extern __shared__ u32x4 a_lds[];  // [nsteps][4][64] operand planes, then the scale regions
   __shared__ int run_block0[kMaxRuns];
   __shared__ int n_runs_sh;
-  __shared__ int row_flat[16];
-  __shared__ int bad_sh[WAVES];
-
   const int tid = threadIdx.x;
   const int lane = tid & 63;
-  const int wave = tid >> 6;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // uniform, and known to be
   const int ln = lane & 15;
   const int lq = lane >> 4;
-  const int part = wave / kSlots;  // which share of K
-  const int slot = wave % kSlots;
 
   const int K = p.K;
   const int groups = K / 32;
   const int nsteps = (groups + 3) / 4;  // K steps, the last one possibly partial
-  const int nfull = groups / 4;
   const int units = STAGE == 0 ? p.ncols / (8 * NT) : p.ncols / (16 * NT);
-  // full K steps of this wavefront's share; the last share also takes the
-  // partial step, if there is one
-  const int ks_begin = nfull * part / S;
-  const int ks_end = nfull * (part + 1) / S;
-  const int n_mine = ks_end - ks_begin;
-  const int last = n_mine > 0 ? ks_end - 1 : 0;
-  const int nmain = n_mine / D;
-  const bool takes_tail = part == S - 1 && nfull * 4 < groups;
-  f32x4* red = reinterpret_cast<f32x4*>(a_lds + (size_t)nsteps * 256);  // [S-1][kSlots][NT][64]
+  const int sc_tile_bytes = 16 * groups;  // scale bytes of one 16-row tile
+  uint8_t* sc_lds = reinterpret_cast<uint8_t*>(a_lds + (size_t)nsteps * 256) +
+                    (size_t)wave * NT * sc_tile_bytes;
+  // rows of W between the units a wavefront takes one after the other
+  const size_t unit_stride_rows = (size_t)WAVES * (STAGE == 0 ? 8 * NT : 16 * NT);
+  const size_t w_unit_stride = unit_stride_rows * (size_t)(K / 2);
+  const size_t s_unit_stride = unit_stride_rows * (size_t)groups;
 
-  int dbg_slot = 0;
-  VK_DBG_T(dbg_slot++);
   // ---- list the runs (first block of every run, in order) -----------------
   if (wave == 0) {
     int n = 0;
@@ -278,7 +266,6 @@ __global__ __launch_bounds__(64 * WAVES) void stream_resident_kernel(GemmArgs p)
     if (lane == 0) n_runs_sh = n < kMaxRuns ? n : kMaxRuns;
   }
   __syncthreads();
-  VK_DBG_T(dbg_slot++);
   const int n_runs = n_runs_sh;
   const long long total = (long long)n_runs * units;
   const long long per_wg = (total + gridDim.x - 1) / gridDim.x;
@@ -289,10 +276,6 @@ __global__ __launch_bounds__(64 * WAVES) void stream_resident_kernel(GemmArgs p)
   struct Stage {
     u32x4 w[NT];
   };
-  // scale bytes of this wavefront's current unit: [NT][16 rows][groups]
-  const int sc_tile_bytes = 16 * groups;
-  uint8_t* sc_lds = reinterpret_cast<uint8_t*>(a_lds + (size_t)nsteps * 256) +
-                    (size_t)(S - 1) * kSlots * NT * 1024 + (size_t)wave * NT * sc_tile_bytes;
 
   for (int r = (int)(s0 / units); r <= (int)((s1 - 1) / units); ++r) {
     const long long base_slot = (long long)r * units;
@@ -304,107 +287,149 @@ __global__ __launch_bounds__(64 * WAVES) void stream_resident_kernel(GemmArgs p)
     while (b0 + run_blocks < p.num_blocks && p.expert_ids[b0 + run_blocks] == e) ++run_blocks;
     const int run_row0 = b0 * p.block_size;
     const int run_tiles = run_blocks * (p.block_size / 16);
+    // units of this wavefront in the segment: first, first + WAVES, ...
+    const int first = u0 + wave;
+    const int n_my = first < u1 ? (u1 - first + WAVES - 1) / WAVES : 0;
 
-    for (int tile = 0; tile < run_tiles; ++tile) {
-      // ---- rows of this pass ------------------------------------------------
-      __syncthreads();  // previous pass is done with row_flat and a_lds
-      if (tid < 16) {
-        const int f = p.sorted_ids[run_row0 + tile * 16 + tid];
-        row_flat[tid] = (f >= 0 && f < p.n_flat) ? f : -1;
+    // Passes of 16 rows, four at a time: one load brings the ids of 64 rows,
+    // and a pass none of whose rows is routed is skipped.
+    for (int tile0 = 0; tile0 < run_tiles; tile0 += 4) {
+      int fl = -1;
+      if (tile0 * 16 + lane < run_tiles * 16) {
+        fl = p.sorted_ids[run_row0 + tile0 * 16 + lane];
+        if (fl < 0 || fl >= p.n_flat) fl = -1;
       }
-      __syncthreads();
-      bool any = false;
-#pragma unroll
-      for (int j = 0; j < 16; ++j) any |= row_flat[j] >= 0;
-      if (!any) continue;  // uniform
+      const unsigned long long routed = __ballot(fl >= 0);
+      for (int tt = 0; tt < 4; ++tt) {
+        if (((routed >> (16 * tt)) & 0xFFFFull) == 0ull) continue;  // same in every wavefront
+        const int tile = tile0 + tt;
+        const int my_flat = __shfl(fl, tt * 16 + ln);         // row of this lane's outputs
+        const int st_flat = __shfl(fl, tt * 16 + (lane >> 2));  // row this lane stages
+        const int srow = run_row0 + tile * 16 + ln;
 
-      // ---- stage the 16 rows, all of K, in operand order --------------------
-      // Lane (j, d) = (lane / 4, lane % 4) copies piece d of quad q of K step
-      // ks of row j; 4 lanes read 64 contiguous bytes.  Loads first, stores
-      // after, so that the copies of one wavefront are all in flight together.
-      {
-        constexpr int kBatch = 4;  // copies in flight per lane
-        const int d = lane & 3;
-        const int j = lane >> 2;
-        const int f = row_flat[j];
-        const uint16_t* src =
-            p.A + (size_t)(f >= 0 ? (STAGE == 0 ? f / p.top_k : run_row0 + tile * 16 + j) : 0) *
-                      (size_t)K;
-        for (int pq0 = wave; pq0 < nsteps * 4 && DBG < 3; pq0 += WAVES * kBatch) {
-          u32x4 v[kBatch];
-#pragma unroll
-          for (int it = 0; it < kBatch; ++it) {
-            const int pq = pq0 + it * WAVES;
-            const int k = (pq >> 2) * kKStep + (pq & 3) * 32 + d * 8;
-            v[it] = u32x4{0u, 0u, 0u, 0u};
-            if (pq < nsteps * 4 && k < K && f >= 0) v[it] = *reinterpret_cast<const u32x4*>(src + k);
-          }
-#pragma unroll
-          for (int it = 0; it < kBatch; ++it) {
-            const int pq = pq0 + it * WAVES;
-            if (pq < nsteps * 4)
-              a_lds[((pq >> 2) * 4 + d) * 64 + (((pq & 3) * 16 + j) ^ (4 * d))] = v[it];
-          }
-        }
-      }
-      VK_DBG_T(dbg_slot++);
-      __syncthreads();
-      VK_DBG_T(dbg_slot++);
-
-      const int my_flat = row_flat[ln];
-      const int srow = run_row0 + tile * 16 + ln;
-
-      // ---- rounds of kSlots units ---------------------------------------------
-      for (int ub = u0; ub < u1; ub += kSlots) {
-        const int unit = ub + slot;
-        const bool active = unit < u1;
-        const uint8_t* w_rows[NT];
-        const uint8_t* s_rows[NT];
+        // compute-side pointers of the current unit (start: the first one)
+        const uint8_t* cw[NT];
+        const uint8_t* cs[NT];
         int col0[NT];
-        unit_tiles<STAGE, NT>(p, e, active ? unit : u0, ln, w_rows, s_rows, col0);
+        unit_tiles<STAGE, NT>(p, e, n_my > 0 ? first : u0, ln, cw, cs, col0);
 
-        // The unit's scale bytes (16 rows x groups, contiguous per tile) come in
-        // with a few coalesced 16-byte loads instead of one load per K step.
-        if (active && DBG < 5) {
+        // ---- load cursor: runs D steps ahead and crosses unit boundaries -----
+        const uint8_t* lrow[NT];
 #pragma unroll
-          for (int t = 0; t < NT; ++t) {
-            const uint8_t* src = s_rows[t] - (size_t)ln * groups;
-            for (int off = lane * 16; off < sc_tile_bytes; off += 1024)
-              *reinterpret_cast<u32x4*>(sc_lds + t * sc_tile_bytes + off) =
-                  *reinterpret_cast<const u32x4*>(src + off);
-          }
-        }
-
-        auto load = [&](Stage& st, int ks) {
-          if (DBG == 2 && ks > 3) return;  // diagnosis: no weight traffic in steady state
-          const size_t g = (size_t)(ks * 4 + lq);
+        for (int t = 0; t < NT; ++t) lrow[t] = cw[t];
+        int ld_ks = 0;
+        int ld_units = n_my;  // units the cursor has not finished, the current one included
+        auto issue = [&](Stage& st) {
+          // lanes past the end of a partial last step re-read the last group: the
+          // operand planes there are zero, so what they load does not matter
+          const int g = min(ld_ks * 4 + lq, groups - 1);
 #pragma unroll
           for (int t = 0; t < NT; ++t)
-            st.w[t] = *reinterpret_cast<const u32x4*>(w_rows[t] + g * 16);
+            st.w[t] = *reinterpret_cast<const u32x4*>(lrow[t] + (size_t)g * 16);
+          if (++ld_ks == nsteps) {  // uniform, no memory operation inside
+            if (ld_units > 1) {
+              --ld_units;
+              ld_ks = 0;
+#pragma unroll
+              for (int t = 0; t < NT; ++t) lrow[t] += w_unit_stride;
+            } else {
+              ld_ks = nsteps - 1;  // past the last unit: stay on its last step
+            }
+          }
         };
+
+        // ---- scale block of a unit: coalesced loads into registers, parked in
+        // the wavefront's LDS region when the unit before it is complete --------
+        u32x4 scn[kScMax];
+        auto fetch_scales = [&](size_t ahead) {
+#pragma unroll
+          for (int j = 0; j < kScMax; ++j) {
+            const int piece = lane + 64 * j;
+            if (piece < NT * groups) {
+              const int t = piece / groups, off = (piece - t * groups) * 16;
+              const uint8_t* base = cs[0] - (size_t)ln * groups;
+#pragma unroll
+              for (int t2 = 1; t2 < NT; ++t2)
+                if (t == t2) base = cs[t2] - (size_t)ln * groups;
+              scn[j] = *reinterpret_cast<const u32x4*>(base + ahead + off);
+            }
+          }
+        };
+        auto park_scales = [&]() {
+#pragma unroll
+          for (int j = 0; j < kScMax; ++j) {
+            const int piece = lane + 64 * j;
+            if (piece < NT * groups) {
+              const int t = piece / groups, off = (piece - t * groups) * 16;
+              *reinterpret_cast<u32x4*>(sc_lds + t * sc_tile_bytes + off) = scn[j];
+            }
+          }
+        };
+
+        // The first loads of the stream go out before the rows are staged, so
+        // that they, the staging loads and the wait for the slowest wavefront
+        // of the previous pass all overlap.
+        Stage st[D];
+        if (n_my > 0) {
+          fetch_scales(0);
+#pragma unroll
+          for (int i = 0; i < D; ++i) issue(st[i]);
+        }
+
+        // ---- stage the 16 rows, all of K, in operand order ------------------
+        // Lane (j, d) = (lane / 4, lane % 4) copies piece d of quad q of K step
+        // ks of row j; 4 lanes read 64 contiguous bytes.  All the copies of a
+        // lane (up to kBatch) are in flight together.
+        {
+          constexpr int kBatch = 12;
+          const int d = lane & 3;
+          const int j = lane >> 2;
+          const uint16_t* src =
+              p.A + (size_t)(st_flat >= 0 ? (STAGE == 0 ? st_flat / p.top_k
+                                                        : run_row0 + tile * 16 + j)
+                                          : 0) * (size_t)K;
+          for (int pq0 = wave; pq0 < nsteps * 4; pq0 += WAVES * kBatch) {
+            u32x4 v[kBatch];
+#pragma unroll
+            for (int it = 0; it < kBatch; ++it) {
+              const int pq = pq0 + it * WAVES;
+              const int k = (pq >> 2) * kKStep + (pq & 3) * 32 + d * 8;
+              // branch-free: an invalid piece reads the row's first bytes instead
+              const bool valid = pq < nsteps * 4 && k < K && st_flat >= 0;
+              v[it] = *reinterpret_cast<const u32x4*>(src + (valid ? k : 0));
+            }
+            if (pq0 == wave) __syncthreads();  // the previous pass is done with a_lds
+#pragma unroll
+            for (int it = 0; it < kBatch; ++it) {
+              const int pq = pq0 + it * WAVES;
+              const int k = (pq >> 2) * kKStep + (pq & 3) * 32 + d * 8;
+              if (pq < nsteps * 4)
+                a_lds[((pq >> 2) * 4 + d) * 64 + (((pq & 3) * 16 + j) ^ (4 * d))] =
+                    (k < K && st_flat >= 0) ? v[it] : u32x4{0u, 0u, 0u, 0u};
+            }
+          }
+        }
+        if (n_my > 0) {
+          park_scales();
+          if (n_my > 1) fetch_scales(s_unit_stride);
+        }
+        __syncthreads();
+        if (n_my == 0) continue;  // no unit here; this wavefront still meets the barriers
 
         f32x4 acc[NT];
 #pragma unroll
         for (int t = 0; t < NT; ++t) acc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
         uint32_t bad = 0u;
 
-        auto compute = [&](const Stage& st, int ks, auto tail) {
-          if (DBG == 1 || DBG >= 3) {  // diagnosis: consume the data without dequant / LDS / MFMA
-#pragma unroll
-            for (int t = 0; t < NT; ++t)
-              acc[t][0] += __uint_as_float((st.w[t][0] ^ st.w[t][1] ^ st.w[t][2] ^ st.w[t][3]) & 0x3FFFFFFFu);
-            return;
-          }
+        auto compute = [&](const Stage& sg, int ks) {
           float sc[NT];
-          const int g = ks * 4 + lq;
+          const int g = min(ks * 4 + lq, groups - 1);
 #pragma unroll
           for (int t = 0; t < NT; ++t) {
-            const uint32_t sb = (!decltype(tail)::value || g < groups)
-                                    ? (uint32_t)sc_lds[t * sc_tile_bytes + ln * groups + g]
-                                    : 127u;
+            const uint32_t sb = sc_lds[t * sc_tile_bytes + ln * groups + g];
             bad |= (uint32_t)!scale_fast_ok(sb);
-            bad |= fp4x8_nonfinite(st.w[t][0]) | fp4x8_nonfinite(st.w[t][1]) |
-                   fp4x8_nonfinite(st.w[t][2]) | fp4x8_nonfinite(st.w[t][3]);
+            bad |= fp4x8_nonfinite(sg.w[t][0]) | fp4x8_nonfinite(sg.w[t][1]) |
+                   fp4x8_nonfinite(sg.w[t][2]) | fp4x8_nonfinite(sg.w[t][3]);
             sc[t] = scale_half_f32(sb);
           }
 #pragma unroll
@@ -413,77 +438,55 @@ __global__ __launch_bounds__(64 * WAVES) void stream_resident_kernel(GemmArgs p)
 #pragma unroll
             for (int t = 0; t < NT; ++t)
               acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
-                  as_bf16x8(dequant8_fast(st.w[t][d], sc[t])), af, acc[t], 0, 0, 0);
+                  as_bf16x8(dequant8_fast(sg.w[t][d], sc[t])), af, acc[t], 0, 0, 0);
           }
         };
 
-        if (active) {
-          if (n_mine > 0) {
-            Stage st[D];
+        const int total_steps = n_my * nsteps;
+        unsigned long long redo = 0ull;  // units (bit = index among this wavefront's) to redo
+        int cks = 0;    // K step of the unit being computed
+        int cunit = 0;  // its index among this wavefront's units
+        for (int f0 = 0; f0 < total_steps; f0 += D) {
 #pragma unroll
-            for (int i = 0; i < D; ++i) load(st[i], min(ks_begin + i, last));
-            for (int it = 0; it < nmain; ++it) {
+          for (int i = 0; i < D; ++i) {
+            if (f0 + i < total_steps) {  // uniform
+              compute(st[i], cks);
+              if (++cks == nsteps) {
+                // ---- the unit is complete -----------------------------------
+                // a unit that met a code or scale outside the fast path's domain
+                // is redone after the stream, so the hot loop stays small
+                if (__ballot(bad != 0u) != 0ull)
+                  redo |= 1ull << cunit;
+                else if (my_flat >= 0)
+                  epilogue_tile<STAGE, NT>(p, e, acc, col0, my_flat, srow, lq);
+                if (++cunit < n_my) {
+                  park_scales();
 #pragma unroll
-              for (int i = 0; i < D; ++i) {
-                compute(st[i], ks_begin + it * D + i, std::false_type{});
-                load(st[i], min(ks_begin + (it + 1) * D + i, last));
-                // keep the scheduler from pulling the next step's conversions
-                // up here: that only lengthens live ranges until they spill
-                __builtin_amdgcn_sched_barrier(0);
+                  for (int t = 0; t < NT; ++t) {
+                    cw[t] += w_unit_stride;
+                    cs[t] += s_unit_stride;
+                    col0[t] += WAVES * (STAGE == 0 ? 8 * NT : 16 * NT);
+                  }
+                  if (cunit + 1 < n_my) fetch_scales(s_unit_stride);
+                }
+                cks = 0;
+                bad = 0u;
+#pragma unroll
+                for (int t = 0; t < NT; ++t) acc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
               }
             }
-            const int rem = n_mine - nmain * D;
-#pragma unroll
-            for (int i = 0; i < D - 1; ++i)
-              if (i < rem) compute(st[i], ks_begin + nmain * D + i, std::false_type{});
-          }
-          if (takes_tail && DBG < 6) {
-            // last, partial K step: quads past the end contribute zeros
-            Stage st;
-            const int g = nfull * 4 + lq;
-            const bool ok = g < groups;
-#pragma unroll
-            for (int t = 0; t < NT; ++t) {
-              st.w[t] = u32x4{0u, 0u, 0u, 0u};
-              if (ok) st.w[t] = *reinterpret_cast<const u32x4*>(w_rows[t] + (size_t)g * 16);
-            }
-            compute(st, nfull, std::true_type{});
+            issue(st[i]);
           }
         }
-        bool wave_bad = __ballot(bad != 0u) != 0ull;
 
-        if (S > 1) {
-          // partial sums of the other shares meet in LDS
-          __syncthreads();  // the previous round's sums have been read
-          if (part > 0 && active) {
-#pragma unroll
-            for (int t = 0; t < NT; ++t)
-              red[(((part - 1) * kSlots + slot) * NT + t) * 64 + lane] = acc[t];
-          }
-          if (lane == 0) bad_sh[wave] = wave_bad ? 1 : 0;
-          __syncthreads();
-          if (part == 0 && active) {
-#pragma unroll
-            for (int o = 1; o < S; ++o) {
-#pragma unroll
-              for (int t = 0; t < NT; ++t) {
-                const f32x4 v = red[(((o - 1) * kSlots + slot) * NT + t) * 64 + lane];
-                acc[t][0] += v[0];
-                acc[t][1] += v[1];
-                acc[t][2] += v[2];
-                acc[t][3] += v[3];
-              }
-              wave_bad |= bad_sh[o * kSlots + slot] != 0;
-            }
-          }
+        // ---- reference-exact pass over the units the fast path could not take
+        while (redo != 0ull) {
+          const int idx = __builtin_ctzll(redo);
+          redo &= redo - 1ull;
+          unit_tiles<STAGE, NT>(p, e, first + idx * WAVES, ln, cw, cs, col0);
+          resident_exact_pass<NT>(cw, cs, a_lds, groups, lane, acc);
+          if (my_flat >= 0) epilogue_tile<STAGE, NT>(p, e, acc, col0, my_flat, srow, lq);
         }
-        VK_DBG_T(dbg_slot++);
-        if (part == 0 && active) {
-          if (wave_bad) resident_exact_pass<NT>(w_rows, s_rows, a_lds, groups, lane, acc);
-          if (DBG >= 4) { if (my_flat == 12345678) { float sum = 0.f; for (int t = 0; t < NT; ++t) sum += acc[t][0]; p.act[lane] = (uint16_t)sum; } }
-          else if (my_flat >= 0) epilogue_tile<STAGE, NT>(p, e, acc, col0, my_flat, srow, lq);
-        }
-        VK_DBG_T(dbg_slot++);
       }
     }
   }
@@ -768,9 +771,9 @@ int num_compute_units() {
 
 constexpr size_t kResidentLdsLimit = 152 * 1024;  // dynamic LDS the resident kernel may ask for
 
-template <int STAGE, int WAVES, int NT, int D, int S, int DBG = 0>
+template <int STAGE, int WAVES, int NT, int D>
 void launch_resident(const GemmArgs& g, size_t lds, hipStream_t stream) {
-  auto* kern = stream_resident_kernel<STAGE, WAVES, NT, D, S, DBG>;
+  auto* kern = stream_resident_kernel<STAGE, WAVES, NT, D>;
   static const bool configured = [kern] {
     (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                               hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -789,32 +792,22 @@ void launch_stage(const GemmArgs& g, hipStream_t stream) {
   const int nt = env_int("VK_MOE_NT", tile.nt);
   const int depth = env_int("VK_MOE_DEPTH", tile.depth);
   const int waves = env_int("VK_MOE_WAVES", tile.waves);
-  const int split = env_int("VK_MOE_SPLIT", tile.split);
-  const int nsteps = (g.K / 32 + 3) / 4;
-  // operand planes + partial sums of the K-split
-  const size_t resident_lds = (size_t)nsteps * 4096 +
-                              (size_t)(split - 1) * (waves / split) * nt * 1024 +
-                              (size_t)waves * nt * 16 * (g.K / 32);
-  if (resident_lds > kResidentLdsLimit || g.num_blocks > kMaxRuns || nsteps * 4 > 128)
+  const int groups = g.K / 32;
+  const int nsteps = (groups + 3) / 4;
+  // operand planes + one scale region per wavefront
+  const size_t resident_lds = (size_t)nsteps * 4096 + (size_t)waves * nt * 16 * groups;
+  const int res_units = STAGE == 0 ? g.ncols / (8 * nt) : g.ncols / (16 * nt);
+  if (resident_lds > kResidentLdsLimit || g.num_blocks > kMaxRuns || nt * groups > 64 * kScMax ||
+      (res_units + waves - 1) / waves > 64)  // one bit per unit of a wavefront in the redo mask
     variant = kMoeVariantLds;
   if (variant == kMoeVariantResident) {
-    const int dbg = env_int("VK_MOE_DBG", 0);
-    if (dbg == 1) return launch_resident<STAGE, 16, 2, 3, 1, 1>(g, resident_lds, stream);
-    if (dbg == 2) return launch_resident<STAGE, 16, 2, 3, 1, 2>(g, resident_lds, stream);
-    if (dbg == 3) return launch_resident<STAGE, 16, 2, 3, 1, 3>(g, resident_lds, stream);
-    if (dbg == 4) return launch_resident<STAGE, 16, 2, 3, 1, 4>(g, resident_lds, stream);
-    if (dbg == 5) return launch_resident<STAGE, 16, 2, 3, 1, 5>(g, resident_lds, stream);
-    if (dbg == 6) return launch_resident<STAGE, 16, 2, 3, 1, 6>(g, resident_lds, stream);
-#define VK_RESIDENT(W_, NT_, D_, S_) \
-  if (waves == W_ && nt == NT_ && depth == D_ && split == S_) \
-    return launch_resident<STAGE, W_, NT_, D_, S_>(g, resident_lds, stream)
-    VK_RESIDENT(16, 2, 3, 1); VK_RESIDENT(16, 2, 2, 2); VK_RESIDENT(16, 2, 3, 2);
-    VK_RESIDENT(16, 2, 4, 2); VK_RESIDENT(16, 2, 2, 4); VK_RESIDENT(16, 2, 3, 4);
-    VK_RESIDENT(8, 2, 4, 1); VK_RESIDENT(8, 2, 4, 2); VK_RESIDENT(8, 2, 6, 2); VK_RESIDENT(8, 2, 3, 2);
-    VK_RESIDENT(8, 4, 3, 2); VK_RESIDENT(8, 4, 2, 2); VK_RESIDENT(16, 4, 2, 2);
-    VK_RESIDENT(8, 2, 3, 1); VK_RESIDENT(8, 2, 6, 1); VK_RESIDENT(8, 2, 8, 1);
-    VK_RESIDENT(8, 4, 2, 1); VK_RESIDENT(8, 4, 3, 1); VK_RESIDENT(8, 4, 4, 1);
-    VK_RESIDENT(12, 2, 3, 1); VK_RESIDENT(12, 2, 4, 1); VK_RESIDENT(12, 2, 6, 1);
+#define VK_RESIDENT(W_, NT_, D_) \
+  if (waves == W_ && nt == NT_ && depth == D_) \
+    return launch_resident<STAGE, W_, NT_, D_>(g, resident_lds, stream)
+    VK_RESIDENT(16, 2, 2); VK_RESIDENT(16, 2, 3); VK_RESIDENT(16, 2, 4);
+    VK_RESIDENT(12, 2, 3); VK_RESIDENT(12, 2, 4); VK_RESIDENT(12, 2, 6);
+    VK_RESIDENT(8, 2, 3); VK_RESIDENT(8, 2, 4); VK_RESIDENT(8, 2, 6); VK_RESIDENT(8, 2, 8);
+    VK_RESIDENT(8, 4, 2); VK_RESIDENT(8, 4, 3); VK_RESIDENT(8, 4, 4);
 #undef VK_RESIDENT
     variant = kMoeVariantLds;
   }
@@ -844,10 +837,6 @@ GemmArgs common_args(const FusedMoeArgs& a) {
 }
 
 }  // namespace
-
-extern "C" void vk_hip_debug_read_times(unsigned long long* host) {
-  (void)hipMemcpyFromSymbol(host, HIP_SYMBOL(g_dbg_times), sizeof(unsigned long long) * 16 * 32);
-}
 
 void launch_moe_gateup(const FusedMoeArgs& a, hipStream_t stream) {
   if (a.M <= 0 || a.EM <= 0 || a.block_size <= 0) return;

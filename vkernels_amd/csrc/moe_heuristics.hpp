@@ -17,7 +17,6 @@ struct MoeTile {
   int waves;    // wavefronts per workgroup
   int nt;       // 16-row weight tiles per wavefront
   int depth;    // K steps in flight per wavefront (resident variant)
-  int split;    // wavefronts sharing the K steps of one unit (resident variant)
 };
 
 // n_flat = tokens * top_k routed rows in the call, K / ncols the GEMM's
@@ -27,8 +26,8 @@ struct MoeTile {
 inline MoeTile pick_moe_tile(int n_flat, int K, int ncols) {
   (void)K;
   (void)ncols;
-  if (n_flat <= 512) return MoeTile{kMoeVariantResident, 16, 2, 3, 1};
-  return MoeTile{kMoeVariantLds, 4, 4, 0, 1};
+  if (n_flat <= 512) return MoeTile{kMoeVariantResident, 8, 2, 4};
+  return MoeTile{kMoeVariantLds, 4, 4, 0};
 }
 
 }  // namespace vk
