@@ -35,6 +35,13 @@ sys.path.insert(0, str(ROOT))
 HBM_PEAK_GBS = 8000.0
 FP4_PEAK_TFLOPS = 10100.0
 
+# HBM bytes per launch of the gate/up kernel from rocprofv3 FETCH_SIZE and
+# WRITE_SIZE counters (two runs of this script under --pmc, scaled by what the
+# same counters read for the 512 MiB copy of --copy-calibration: x2.0 and x1.0).
+# Counters cannot be read from inside this process, so the figure of the last
+# profiled build is recorded here per workload; null for the others.
+MEASURED_TRAFFIC = {"c1:64": 308.3e6}
+
 
 def parse_args():
     ap = argparse.ArgumentParser()
@@ -191,9 +198,9 @@ def main():
             "block_size": bs, "active_experts": active, "weight_sets": n_sets,
         },
         "roofline": {
-            "bound": "hbm", "kernel": "stream_gemm_kernel<0> (gate/up + SwiGLU)",
+            "bound": "hbm", "kernel": "stream_resident_kernel<0, ...> (gate/up grouped GEMM + SwiGLU)",
             "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-            "frac": achieved / HBM_PEAK_GBS, "traffic": None,
+            "frac": achieved / HBM_PEAK_GBS, "traffic": MEASURED_TRAFFIC.get(args.workload),
             "bytes_per_launch": gate_bytes, "avg_launch_us": gate_avg * 1e3,
             "median_launch_us": gate_ms[len(gate_ms) // 2] * 1e3,
         },

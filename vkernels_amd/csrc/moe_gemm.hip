@@ -164,42 +164,110 @@ __device__ __forceinline__ void unit_tiles(const GemmArgs& p, int e, int unit, i
 // ---------------------------------------------------------------------------
 // Decode kernel ("resident"): one workgroup per compute unit, the activation
 // rows of a run resident in LDS for the whole K dimension, no barrier inside
-// the K loop, and every wavefront's weight loads one uninterrupted stream.
+// the K loop, every wavefront's weight loads one uninterrupted stream, and
+// the FP4 codes fed to the matrix cores as they are.
 //
-// The launch has as many workgroups as the device has compute units.  Every
-// workgroup lists the runs (consecutive blocks of one expert), flattens
-// (run, weight unit) into one index space and takes an equal contiguous
-// slice of it, so the weight bytes are spread evenly over the compute units
-// whatever the number of active experts.  For each run its slice touches,
-// and each 16-row pass of that run, the workgroup stages the 16 activation
-// rows, all of K, into LDS in MFMA-operand order (read coalesced; at most
-// nsteps x 4 KiB, 92 KiB for K = 2880).  Wavefront w then takes units
-// w, w + WAVES, ... of the slice and walks their K steps as ONE sequence:
-// a D-deep register pipeline of 16-byte-per-lane weight loads whose cursor
-// runs ahead of the arithmetic and crosses from one unit into the next, so
-// that neither the epilogue of a unit nor the start of the next one leaves
-// the memory pipe empty.  The scale bytes of a unit (16 rows x K/32,
-// contiguous per tile) are fetched with a few coalesced loads while the
-// previous unit streams and parked in a per-wavefront LDS region.
+// Arithmetic.  v_mfma_scale_f32_16x16x128_f8f6f4 multiplies an FP4 (E2M1)
+// operand by an FP8 (E4M3) operand, each with one E8M0 scale per lane that
+// covers the lane's block of 32 along K.  The weight side is the packed codes
+// moved onto the OCP code points (mxfp4.hpp: +2 on codes with a non-zero
+// exponent field, scale byte - 1), 16 bytes = one scale group = one lane.
+// The bf16 activations are split, per block of 32, as
+//     a = (hi + lo / 16) * 2^(sb - 127),   hi, lo in E4M3,
+// with sb = (largest exponent field of the block) - 7: hi takes the leading
+// four significant bits of a / 2^(sb-127), lo the other four, so the split is
+// exact for every element within 2^-13 of the block's largest and the two
+// MFMAs (hi, then lo with scale byte sb - 4) sum the same products the
+// reference forms, in fp32.
+// A unit whose weights hold an inf/NaN code or a scale byte outside
+// [kScaleLo, kScaleHi], and a pass whose activations hold an inf/NaN or a
+// block exponent outside that range, are computed by exact_unit_global
+// instead: integer-exact dequantisation, bf16 MFMAs, activations from global
+// memory.
 //
-// LDS layout of the operand of K step ks, MFMA d (one 1 KiB plane): lane L
-// reads its 16 bytes at slot L ^ (4 d).  The XOR makes the staging stores of
-// 16 consecutive lanes (4 rows x 4 consecutive pieces of 64 bytes) fall into
-// 16 different bank groups.  Planes past K are zero, which is what makes the
-// last, partial K step need no masking of the weight side.
+// Work split.  The launch has as many workgroups as the device has compute
+// units.  Every workgroup lists the runs (consecutive blocks of one expert),
+// flattens (run, weight unit) into one index space and takes a contiguous
+// slice of it (workgroup_slice), so the weight bytes are spread evenly over
+// the compute units whatever the number of active experts.  For each run its
+// slice touches, and each 16-row pass of that run, the workgroup stages the
+// 16 activation rows, all of K, into LDS as MFMA operands (split as above).
+// Wavefront w takes units w, w + WAVES, ... of the slice and walks their K
+// steps as ONE sequence: a D-deep register pipeline of 16-byte-per-lane
+// weight loads whose cursor runs ahead of the arithmetic and crosses from one
+// unit into the next.  The scale bytes of a unit (16 rows x K/32, contiguous
+// per tile) are fetched with a few coalesced loads while the previous unit
+// streams and parked in a per-wavefront LDS region.
+//
+// Order within a pass.  The memory pipe of a compute unit returns data in the
+// order of issue, and a pass starts with a burst of loads, so: (1) the first
+// D steps of the weight stream, which depend on the run alone, (2) the row
+// ids, (3) the rows, then the barrier with the previous pass.  The rows are
+// split and written in K order, a few K steps ahead of the first unit's
+// arithmetic with a barrier after each portion, so the stream starts after
+// the first portion and the rest of the splitting overlaps it.
+//
+// LDS operand planes of K step ks: [term hi/lo][half h][64 lanes] x 16 bytes;
+// lane (n, q') of half h holds the 16 values k = 128 ks + 64 h + 16 q' + 0..15
+// of row n, which is where the MFMA takes them from (operand bytes 16 h ..
+// 16 h + 15).  Planes past K are zero, so the last, partial K step needs no
+// masking of the weight side.
 // ---------------------------------------------------------------------------
-constexpr int kMaxRuns = 1024;  // runs the resident kernel can list in LDS
+constexpr int kMaxRuns = 512;   // runs the resident kernel can list in LDS
 constexpr int kScMax = 4;       // 16-byte scale pieces per lane: NT * K/32 <= 64 * kScMax
+constexpr uint32_t kScaleLo = 64u, kScaleHi = 190u;  // scale bytes the scaled MFMA path takes
 
-// Reference-exact slow path: one K step at a time, integer-exact
-// dequantisation.  Taken by a wavefront only after its fast pass over a unit
-// met an inf/NaN code or a scale byte outside [3, 252].
+typedef __attribute__((ext_vector_type(8))) int i32x8;
+
+// First item of part `i` when `total` items are cut into `parts` contiguous
+// slices whose sizes differ by at most one.
+__device__ __forceinline__ int slice_begin(int total, int i, int parts) {
+  const int q = total / parts, rem = total - q * parts;
+  return i * q + min(i, rem);
+}
+
+// A workgroup's slice [s0, s1) of the flat (run, unit) space.  Staging the rows
+// of a run costs about as much as streaming kStagingUnits units, so when every
+// run can have workgroups of its own the slices stop at run boundaries (runs
+// get floor or ceil of grid / n_runs workgroups each) unless that unbalances
+// the workgroups by more than a second staging would cost; otherwise the space
+// is cut evenly and a slice may span runs.
+constexpr int kStagingUnits = 4;
+__device__ __forceinline__ void workgroup_slice(int n_runs, int units, int wg, int grid, int& s0,
+                                                int& s1) {
+  const int total = n_runs * units;
+  if (n_runs <= grid) {
+    const int q = grid / n_runs, rem = grid - q * n_runs;
+    if ((units + q - 1) / q <= (total + grid - 1) / grid + kStagingUnits) {
+      int r, j, g;
+      if (wg < rem * (q + 1)) {
+        g = q + 1;
+        r = wg / g;
+        j = wg - r * g;
+      } else {
+        g = q;
+        r = rem + (wg - rem * (q + 1)) / q;
+        j = (wg - rem * (q + 1)) - (r - rem) * q;
+      }
+      s0 = r * units + slice_begin(units, j, g);
+      s1 = r * units + slice_begin(units, j + 1, g);
+      return;
+    }
+  }
+  s0 = slice_begin(total, wg, grid);
+  s1 = slice_begin(total, wg + 1, grid);
+}
+
+// Reference-exact slow path for one unit: one K step at a time, integer-exact
+// dequantisation, the activation row of this lane's column read from global
+// memory (a_row null = padding row).
 template <int NT>
-__device__ __forceinline__ void resident_exact_pass(const uint8_t* const (&w_rows)[NT],
-                                                    const uint8_t* const (&s_rows)[NT],
-                                                    const u32x4* a_lds, int groups, int lane,
-                                                    f32x4 (&acc)[NT]) {
+__device__ __forceinline__ void exact_unit_global(const uint8_t* const (&w_rows)[NT],
+                                                  const uint8_t* const (&s_rows)[NT],
+                                                  const uint16_t* a_row, int K, int lane,
+                                                  f32x4 (&acc)[NT]) {
   const int lq = lane >> 4;
+  const int groups = K / 32;
 #pragma unroll
   for (int t = 0; t < NT; ++t) acc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll 1
@@ -208,7 +276,8 @@ __device__ __forceinline__ void resident_exact_pass(const uint8_t* const (&w_row
     const bool ok = g < groups;
 #pragma unroll 1
     for (int d = 0; d < 4; ++d) {
-      const u32x4 av = a_lds[(ks * 4 + d) * 64 + (lane ^ (4 * d))];
+      u32x4 av = {0u, 0u, 0u, 0u};
+      if (ok && a_row != nullptr) av = *reinterpret_cast<const u32x4*>(a_row + g * 32 + d * 8);
 #pragma unroll
       for (int t = 0; t < NT; ++t) {
         uint32_t x = 0u, sc = 127u;
@@ -223,11 +292,60 @@ __device__ __forceinline__ void resident_exact_pass(const uint8_t* const (&w_row
   }
 }
 
+// Largest bf16 exponent field among the 8 values of v: the exponent of the
+// largest magnitude, found with packed 16-bit maxima.
+__device__ __forceinline__ uint32_t bf16x8_max_exponent(u32x4 v) {
+  typedef __attribute__((ext_vector_type(2))) unsigned short u16x2;
+  union { uint32_t u; u16x2 h; } a, b, c, d;
+  a.u = v[0] & 0x7FFF7FFFu;
+  b.u = v[1] & 0x7FFF7FFFu;
+  c.u = v[2] & 0x7FFF7FFFu;
+  d.u = v[3] & 0x7FFF7FFFu;
+  a.h = __builtin_elementwise_max(a.h, b.h);
+  c.h = __builtin_elementwise_max(c.h, d.h);
+  a.h = __builtin_elementwise_max(a.h, c.h);
+  const uint32_t m = max(a.u & 0xFFFFu, a.u >> 16);
+  return m >> 7;
+}
+
+// 8 bf16 values -> the 8 E4M3 leading parts of v / 2^(sb-127) and the 8 E4M3
+// remainders times 16.  gfx950's scaled conversions divide by the scale on the
+// way down to FP8 and multiply by it on the way up.
+__device__ __forceinline__ void split_bf16x8(u32x4 v, uint32_t sb, uint2& hi, uint2& lo) {
+  typedef __attribute__((ext_vector_type(2))) short i16x2;
+  typedef __attribute__((ext_vector_type(2))) float f32x2;
+  const float scale = __uint_as_float(sb << 23);
+  const float scale16 = __uint_as_float((sb - 4u) << 23);
+  union Pack { i16x2 h; uint32_t u; };
+  Pack h[2], l[2];
+  h[0].u = h[1].u = l[0].u = l[1].u = 0u;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    union { uint32_t u; bf16x2 b; } x;
+    x.u = v[i];
+    if (i & 1) h[i >> 1].h = __builtin_amdgcn_cvt_scalef32_pk_fp8_bf16(h[i >> 1].h, x.b, scale, true);
+    else h[i >> 1].h = __builtin_amdgcn_cvt_scalef32_pk_fp8_bf16(h[i >> 1].h, x.b, scale, false);
+    f32x2 back;
+    if (i & 1) back = __builtin_amdgcn_cvt_scalef32_pk_f32_fp8(h[i >> 1].u, scale, true);
+    else back = __builtin_amdgcn_cvt_scalef32_pk_f32_fp8(h[i >> 1].u, scale, false);
+    const float r0 = __uint_as_float(v[i] << 16) - back[0];
+    const float r1 = __uint_as_float(v[i] & 0xFFFF0000u) - back[1];
+    if (i & 1) l[i >> 1].h = __builtin_amdgcn_cvt_scalef32_pk_fp8_f32(l[i >> 1].h, r0, r1, scale16, true);
+    else l[i >> 1].h = __builtin_amdgcn_cvt_scalef32_pk_fp8_f32(l[i >> 1].h, r0, r1, scale16, false);
+  }
+  hi = make_uint2(h[0].u, h[1].u);
+  lo = make_uint2(l[0].u, l[1].u);
+}
+
 template <int STAGE, int WAVES, int NT, int D>
 __global__ __launch_bounds__(64 * WAVES) void stream_resident_kernel(GemmArgs p) {
-  extern __shared__ u32x4 a_lds[];  // [nsteps][4][64] operand planes, then the scale regions
+  extern __shared__ u32x4 b_lds[];  // [nsteps][2][2][64] operand planes, block scales, weight scales
   __shared__ int run_block0[kMaxRuns];
+  __shared__ int run_block1[kMaxRuns];  // one past the last block of the run
+  __shared__ int run_expert[kMaxRuns];
+  __shared__ int first_ids[64];         // sorted ids of the first 64 rows of this workgroup's first run
   __shared__ int n_runs_sh;
+  __shared__ int pass_slow[2];          // set while staging: this pass takes the exact path
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // uniform, and known to be
@@ -239,66 +357,168 @@ __global__ __launch_bounds__(64 * WAVES) void stream_resident_kernel(GemmArgs p)
   const int nsteps = (groups + 3) / 4;  // K steps, the last one possibly partial
   const int units = STAGE == 0 ? p.ncols / (8 * NT) : p.ncols / (16 * NT);
   const int sc_tile_bytes = 16 * groups;  // scale bytes of one 16-row tile
-  uint8_t* sc_lds = reinterpret_cast<uint8_t*>(a_lds + (size_t)nsteps * 256) +
-                    (size_t)wave * NT * sc_tile_bytes;
+  uint8_t* bsc_lds = reinterpret_cast<uint8_t*>(b_lds + (size_t)nsteps * 256);  // [nsteps][64]
+  uint8_t* sc_lds = bsc_lds + (size_t)nsteps * 64 + (size_t)wave * NT * sc_tile_bytes;
   // rows of W between the units a wavefront takes one after the other
   const size_t unit_stride_rows = (size_t)WAVES * (STAGE == 0 ? 8 * NT : 16 * NT);
   const size_t w_unit_stride = unit_stride_rows * (size_t)(K / 2);
   const size_t s_unit_stride = unit_stride_rows * (size_t)groups;
 
-  // ---- list the runs (first block of every run, in order) -----------------
+  // ---- list the runs (first and last block of every run, in order) ---------
   if (wave == 0) {
-    int n = 0;
+    int n = 0, n_last = 0;
     for (int base = 0; base < p.num_blocks; base += 64) {
       const int b = base + lane;
-      bool leader = false;
+      bool first = false, last = false;
+      int e = -1;
       if (b < p.num_blocks) {
-        const int e = p.expert_ids[b];
-        leader = e >= 0 && (b == 0 || p.expert_ids[b - 1] != e);
+        e = p.expert_ids[b];
+        first = e >= 0 && (b == 0 || p.expert_ids[b - 1] != e);
+        last = e >= 0 && (b == p.num_blocks - 1 || p.expert_ids[b + 1] != e);
       }
-      const unsigned long long m = __ballot(leader);
-      if (leader) {
-        const int idx = n + (int)__popcll(m & ((1ull << lane) - 1ull));
-        if (idx < kMaxRuns) run_block0[idx] = b;
+      const unsigned long long mf = __ballot(first), ml = __ballot(last);
+      const unsigned long long below = (1ull << lane) - 1ull;
+      if (first) {
+        const int idx = n + (int)__popcll(mf & below);
+        if (idx < kMaxRuns) {
+          run_block0[idx] = b;
+          run_expert[idx] = e;
+        }
       }
-      n += (int)__popcll(m);
+      if (last) {  // a run's last block is its first one or comes after it
+        const int idx = n_last + (int)__popcll(ml & below);
+        if (idx < kMaxRuns) run_block1[idx] = b + 1;
+      }
+      n += (int)__popcll(mf);
+      n_last += (int)__popcll(ml);
     }
-    if (lane == 0) n_runs_sh = n < kMaxRuns ? n : kMaxRuns;
+    n = n < kMaxRuns ? n : kMaxRuns;
+    if (lane == 0) {
+      n_runs_sh = n;
+      pass_slow[0] = 0;
+      pass_slow[1] = 0;
+    }
+    // The ids of the first rows this workgroup will stage, fetched once here
+    // rather than by every wavefront after the barrier.
+    int t0 = 0, t1 = 0;
+    if (n > 0) workgroup_slice(n, units, blockIdx.x, gridDim.x, t0, t1);
+    if (t0 < t1) {
+      const int r0 = t0 / units;
+      const int b0 = run_block0[r0];  // written by this wavefront, LDS operations stay in order
+      const int rows = (run_block1[r0] - b0) * p.block_size;
+      first_ids[lane] = lane < rows ? p.sorted_ids[b0 * p.block_size + lane] : -1;
+    }
   }
   __syncthreads();
   const int n_runs = n_runs_sh;
-  const long long total = (long long)n_runs * units;
-  const long long per_wg = (total + gridDim.x - 1) / gridDim.x;
-  const long long s0 = (long long)blockIdx.x * per_wg;
-  const long long s1 = s0 + per_wg < total ? s0 + per_wg : total;
+  int s0 = 0, s1 = 0;  // n_runs * units is far below 2^31: at most kMaxRuns runs
+  if (n_runs > 0) workgroup_slice(n_runs, units, blockIdx.x, gridDim.x, s0, s1);
   if (s0 >= s1) return;  // uniform over the workgroup
+  const int r_first = s0 / units;
 
   struct Stage {
     u32x4 w[NT];
   };
+  int pass_no = 0;
 
-  for (int r = (int)(s0 / units); r <= (int)((s1 - 1) / units); ++r) {
-    const long long base_slot = (long long)r * units;
-    const int u0 = (int)((s0 > base_slot ? s0 : base_slot) - base_slot);
-    const int u1 = (int)((s1 < base_slot + units ? s1 : base_slot + units) - base_slot);
+  for (int r = r_first; r <= (s1 - 1) / units; ++r) {
+    const int base_slot = r * units;
+    const int u0 = max(s0, base_slot) - base_slot;
+    const int u1 = min(s1, base_slot + units) - base_slot;
     const int b0 = run_block0[r];
-    const int e = p.expert_ids[b0];
-    int run_blocks = 1;
-    while (b0 + run_blocks < p.num_blocks && p.expert_ids[b0 + run_blocks] == e) ++run_blocks;
+    const int run_blocks = run_block1[r] - b0;
+    const int e = run_expert[r];
     const int run_row0 = b0 * p.block_size;
     const int run_tiles = run_blocks * (p.block_size / 16);
     // units of this wavefront in the segment: first, first + WAVES, ...
     const int first = u0 + wave;
     const int n_my = first < u1 ? (u1 - first + WAVES - 1) / WAVES : 0;
 
+    // compute-side pointers of the current unit (start: the first one)
+    const uint8_t* cw[NT];
+    const uint8_t* cs[NT];
+    int col0[NT];
+
+    // ---- load cursor: runs D steps ahead and crosses unit boundaries -----
+    const uint8_t* lrow[NT];
+#pragma unroll
+    for (int t = 0; t < NT; ++t) lrow[t] = nullptr;
+    int ld_ks = 0;
+    int ld_units = 0;  // units the cursor has not finished, the current one included
+    auto issue = [&](Stage& st) {
+      // lanes past the end of a partial last step re-read the last group: the
+      // operand planes there are zero, so what they load does not matter
+      const int g = min(ld_ks * 4 + lq, groups - 1);
+#pragma unroll
+      for (int t = 0; t < NT; ++t)
+        st.w[t] = *reinterpret_cast<const u32x4*>(lrow[t] + (size_t)g * 16);
+      if (++ld_ks == nsteps) {  // uniform, no memory operation inside
+        if (ld_units > 1) {
+          --ld_units;
+          ld_ks = 0;
+#pragma unroll
+          for (int t = 0; t < NT; ++t) lrow[t] += w_unit_stride;
+        } else {
+          ld_ks = nsteps - 1;  // past the last unit: stay on its last step
+        }
+      }
+    };
+
+    // ---- scale block of a unit: coalesced loads into registers, parked in
+    // the wavefront's LDS region when the unit before it is complete --------
+    u32x4 scn[kScMax];
+    auto fetch_scales = [&](size_t ahead) {
+#pragma unroll
+      for (int j = 0; j < kScMax; ++j) {
+        // branch-free: lanes past the end re-read the last piece
+        const int piece = min(lane + 64 * j, NT * groups - 1);
+        const int t = piece / groups, off = (piece - t * groups) * 16;
+        const uint8_t* base = cs[0] - (size_t)ln * groups;
+#pragma unroll
+        for (int t2 = 1; t2 < NT; ++t2)
+          if (t == t2) base = cs[t2] - (size_t)ln * groups;
+        scn[j] = *reinterpret_cast<const u32x4*>(base + ahead + off);
+      }
+    };
+    auto park_scales = [&]() {
+#pragma unroll
+      for (int j = 0; j < kScMax; ++j) {
+        const int piece = lane + 64 * j;
+        if (piece < NT * groups) {
+          const int t = piece / groups, off = (piece - t * groups) * 16;
+          *reinterpret_cast<u32x4*>(sc_lds + t * sc_tile_bytes + off) = scn[j];
+        }
+      }
+    };
+
+
+    // Start of a pass's weight stream: pointers of the wavefront's first unit,
+    // its scale block and the first D steps.  Issued before anything else of
+    // the pass (it depends on the run alone, not on the rows), so the loads
+    // are under way while the rows are fetched, split and written; a
+    // wavefront without units loads the slice's first unit and drops it.
+    Stage st[D];
+    bool primed = false;
+    auto prime = [&]() {
+      unit_tiles<STAGE, NT>(p, e, n_my > 0 ? first : u0, ln, cw, cs, col0);
+#pragma unroll
+      for (int t = 0; t < NT; ++t) lrow[t] = cw[t];
+      ld_ks = 0;
+      ld_units = max(n_my, 1);
+      fetch_scales(0);
+#pragma unroll
+      for (int i = 0; i < D; ++i) issue(st[i]);
+      primed = true;
+    };
+
     // Passes of 16 rows, four at a time: one load brings the ids of 64 rows,
     // and a pass none of whose rows is routed is skipped.
     for (int tile0 = 0; tile0 < run_tiles; tile0 += 4) {
+      if (!primed) prime();
       int fl = -1;
-      if (tile0 * 16 + lane < run_tiles * 16) {
-        fl = p.sorted_ids[run_row0 + tile0 * 16 + lane];
-        if (fl < 0 || fl >= p.n_flat) fl = -1;
-      }
+      if (r == r_first && tile0 == 0) fl = first_ids[lane];
+      else if (tile0 * 16 + lane < run_tiles * 16) fl = p.sorted_ids[run_row0 + tile0 * 16 + lane];
+      if (fl < 0 || fl >= p.n_flat) fl = -1;
       const unsigned long long routed = __ballot(fl >= 0);
       for (int tt = 0; tt < 4; ++tt) {
         if (((routed >> (16 * tt)) & 0xFFFFull) == 0ull) continue;  // same in every wavefront
@@ -306,186 +526,197 @@ __global__ __launch_bounds__(64 * WAVES) void stream_resident_kernel(GemmArgs p)
         const int my_flat = __shfl(fl, tt * 16 + ln);         // row of this lane's outputs
         const int st_flat = __shfl(fl, tt * 16 + (lane >> 2));  // row this lane stages
         const int srow = run_row0 + tile * 16 + ln;
+        const int flag = pass_no & 1;
+        ++pass_no;
+        if (!primed) prime();
+        primed = false;  // this pass consumes the stream
 
-        // compute-side pointers of the current unit (start: the first one)
-        const uint8_t* cw[NT];
-        const uint8_t* cs[NT];
-        int col0[NT];
-        unit_tiles<STAGE, NT>(p, e, n_my > 0 ? first : u0, ln, cw, cs, col0);
-
-        // ---- load cursor: runs D steps ahead and crosses unit boundaries -----
-        const uint8_t* lrow[NT];
+        // ---- stage the 16 rows, all of K, as MFMA operands --------------------
+        // Lane (j, d) = (lane / 4, lane % 4) takes the 8 values k = 32 g + 8 d ..
+        // of row j for group g = pq; the four lanes of a group share the block
+        // scale.  All the loads of a lane (up to kBatch) are in flight together.
+        // Order of issue: the row loads, then the first D steps of the weight
+        // stream (every wavefront, with or without units: no branch between
+        // the loads, so that the wait below counts only the row loads), then
+        // the wait for the slowest wavefront of the previous pass.  The weight
+        // loads so stay in flight while the rows are split and written.
+        constexpr int kBatch = 96 / WAVES;  // pieces per lane: K <= 3072 in one batch
+        const int n_pieces = (nsteps * 4 + WAVES - 1) / WAVES;  // the launcher keeps it <= kBatch
+        const int sd = lane & 3;
+        const int sj = lane >> 2;
+        const uint16_t* src =
+            p.A + (size_t)(st_flat >= 0 ? (STAGE == 0 ? st_flat / p.top_k
+                                                      : run_row0 + tile * 16 + sj)
+                                        : 0) * (size_t)K;
+        u32x4 v[kBatch];
 #pragma unroll
-        for (int t = 0; t < NT; ++t) lrow[t] = cw[t];
-        int ld_ks = 0;
-        int ld_units = n_my;  // units the cursor has not finished, the current one included
-        auto issue = [&](Stage& st) {
-          // lanes past the end of a partial last step re-read the last group: the
-          // operand planes there are zero, so what they load does not matter
-          const int g = min(ld_ks * 4 + lq, groups - 1);
-#pragma unroll
-          for (int t = 0; t < NT; ++t)
-            st.w[t] = *reinterpret_cast<const u32x4*>(lrow[t] + (size_t)g * 16);
-          if (++ld_ks == nsteps) {  // uniform, no memory operation inside
-            if (ld_units > 1) {
-              --ld_units;
-              ld_ks = 0;
-#pragma unroll
-              for (int t = 0; t < NT; ++t) lrow[t] += w_unit_stride;
-            } else {
-              ld_ks = nsteps - 1;  // past the last unit: stay on its last step
-            }
-          }
-        };
-
-        // ---- scale block of a unit: coalesced loads into registers, parked in
-        // the wavefront's LDS region when the unit before it is complete --------
-        u32x4 scn[kScMax];
-        auto fetch_scales = [&](size_t ahead) {
-#pragma unroll
-          for (int j = 0; j < kScMax; ++j) {
-            const int piece = lane + 64 * j;
-            if (piece < NT * groups) {
-              const int t = piece / groups, off = (piece - t * groups) * 16;
-              const uint8_t* base = cs[0] - (size_t)ln * groups;
-#pragma unroll
-              for (int t2 = 1; t2 < NT; ++t2)
-                if (t == t2) base = cs[t2] - (size_t)ln * groups;
-              scn[j] = *reinterpret_cast<const u32x4*>(base + ahead + off);
-            }
-          }
-        };
-        auto park_scales = [&]() {
-#pragma unroll
-          for (int j = 0; j < kScMax; ++j) {
-            const int piece = lane + 64 * j;
-            if (piece < NT * groups) {
-              const int t = piece / groups, off = (piece - t * groups) * 16;
-              *reinterpret_cast<u32x4*>(sc_lds + t * sc_tile_bytes + off) = scn[j];
-            }
-          }
-        };
-
-        // The first loads of the stream go out before the rows are staged, so
-        // that they, the staging loads and the wait for the slowest wavefront
-        // of the previous pass all overlap.
-        Stage st[D];
-        if (n_my > 0) {
-          fetch_scales(0);
-#pragma unroll
-          for (int i = 0; i < D; ++i) issue(st[i]);
+        for (int it = 0; it < kBatch; ++it) {
+          const int pq = wave + it * WAVES;
+          // branch-free: an invalid piece reads the row's first bytes instead
+          const bool valid = pq < groups && st_flat >= 0;
+          v[it] = *reinterpret_cast<const u32x4*>(src + (valid ? pq * 32 + sd * 8 : 0));
         }
+        // Block scale byte of piece `it` (0 = outside the fast path's range).
+        auto block_scale = [&](int it) -> uint32_t {
+          uint32_t emax = bf16x8_max_exponent(v[it]);
+          emax = max(emax, (uint32_t)__builtin_amdgcn_mov_dpp((int)emax, 0xB1, 0xF, 0xF, true));
+          emax = max(emax, (uint32_t)__builtin_amdgcn_mov_dpp((int)emax, 0x4E, 0xF, 0xF, true));
+          if (emax == 0u) return 127u;  // a block of zeros (or bf16 subnormals, taken as zero)
+          const uint32_t sb = emax - 7u;
+          return (sb < kScaleLo || sb > kScaleHi) ? 0u : sb;
+        };
+        // Split and write the pieces [staged, upto) of this lane.  Piece `it` of
+        // wavefront w is group w + it * WAVES, so once every wavefront has
+        // written `n` pieces the K steps below n * WAVES / 4 are complete.
+        int staged = 0;
+        auto write_rows = [&](int upto) {
+#pragma unroll
+          for (int it = 0; it < kBatch; ++it) {
+            const int pq = wave + it * WAVES;
+            if (it >= staged && it < upto && pq < nsteps * 4) {
+              uint32_t sb = block_scale(it);
+              if (sb == 0u) sb = 127u;  // the pass takes the exact path; keep the bytes defined
+              uint2 hi, lo;
+              split_bf16x8(v[it], sb, hi, lo);
+              const int ks = pq >> 2, qq = pq & 3;
+              const int slot = ((qq & 1) * 2 + (sd >> 1)) * 16 + sj;
+              uint8_t* plane = reinterpret_cast<uint8_t*>(b_lds) +
+                               (size_t)(((ks * 2) * 2 + (qq >> 1)) * 64 + slot) * 16 + (sd & 1) * 8;
+              *reinterpret_cast<uint2*>(plane) = hi;
+              *reinterpret_cast<uint2*>(plane + 2 * 64 * 16) = lo;
+              if (sd == 0) bsc_lds[ks * 64 + qq * 16 + sj] = (uint8_t)sb;
+            }
+          }
+          staged = upto;
+        };
+        // pieces every wavefront must have written before K steps [0, steps) can run
+        auto pieces_for = [&](int steps) { return min(n_pieces, (steps * 4 + WAVES - 1) / WAVES); };
 
-        // ---- stage the 16 rows, all of K, in operand order ------------------
-        // Lane (j, d) = (lane / 4, lane % 4) copies piece d of quad q of K step
-        // ks of row j; 4 lanes read 64 contiguous bytes.  All the copies of a
-        // lane (up to kBatch) are in flight together.
         {
-          constexpr int kBatch = 12;
-          const int d = lane & 3;
-          const int j = lane >> 2;
-          const uint16_t* src =
-              p.A + (size_t)(st_flat >= 0 ? (STAGE == 0 ? st_flat / p.top_k
-                                                        : run_row0 + tile * 16 + j)
-                                          : 0) * (size_t)K;
-          for (int pq0 = wave; pq0 < nsteps * 4; pq0 += WAVES * kBatch) {
-            u32x4 v[kBatch];
+          bool slow = false;
 #pragma unroll
-            for (int it = 0; it < kBatch; ++it) {
-              const int pq = pq0 + it * WAVES;
-              const int k = (pq >> 2) * kKStep + (pq & 3) * 32 + d * 8;
-              // branch-free: an invalid piece reads the row's first bytes instead
-              const bool valid = pq < nsteps * 4 && k < K && st_flat >= 0;
-              v[it] = *reinterpret_cast<const u32x4*>(src + (valid ? k : 0));
-            }
-            if (pq0 == wave) __syncthreads();  // the previous pass is done with a_lds
-#pragma unroll
-            for (int it = 0; it < kBatch; ++it) {
-              const int pq = pq0 + it * WAVES;
-              const int k = (pq >> 2) * kKStep + (pq & 3) * 32 + d * 8;
-              if (pq < nsteps * 4)
-                a_lds[((pq >> 2) * 4 + d) * 64 + (((pq & 3) * 16 + j) ^ (4 * d))] =
-                    (k < K && st_flat >= 0) ? v[it] : u32x4{0u, 0u, 0u, 0u};
-            }
+          for (int it = 0; it < kBatch; ++it) {
+            const int pq = wave + it * WAVES;
+            if (!(pq < groups && st_flat >= 0)) v[it] = u32x4{0u, 0u, 0u, 0u};
+            if (pq < nsteps * 4) slow |= block_scale(it) == 0u;
           }
+          __syncthreads();  // the previous pass is done with the planes and with its flag
+          if (slow) pass_slow[flag] = 1;
         }
+        // The rows are staged in K order, a few K steps ahead of the first unit's
+        // arithmetic, with a barrier after each portion: the weight stream starts
+        // after the first portion and the rest of the splitting overlaps it.
+        write_rows(pieces_for(min(nsteps, D)));
         if (n_my > 0) {
           park_scales();
           if (n_my > 1) fetch_scales(s_unit_stride);
         }
         __syncthreads();
-        if (n_my == 0) continue;  // no unit here; this wavefront still meets the barriers
+        if (tid == 0) pass_slow[flag ^ 1] = 0;  // for the next pass; its last reader is behind us
+        const bool slow_pass = pass_slow[flag] != 0;
+        if (n_my == 0 || slow_pass) {
+          // no fast stream here: finish the staging in step with the other wavefronts
+          for (int f0 = D; staged < n_pieces; f0 += D) {
+            write_rows(pieces_for(min(nsteps, f0 + D)));
+            __syncthreads();
+          }
+          if (n_my == 0) continue;
+        }
 
         f32x4 acc[NT];
-#pragma unroll
-        for (int t = 0; t < NT; ++t) acc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
-        uint32_t bad = 0u;
-
-        auto compute = [&](const Stage& sg, int ks) {
-          float sc[NT];
-          const int g = min(ks * 4 + lq, groups - 1);
-#pragma unroll
-          for (int t = 0; t < NT; ++t) {
-            const uint32_t sb = sc_lds[t * sc_tile_bytes + ln * groups + g];
-            bad |= (uint32_t)!scale_fast_ok(sb);
-            bad |= fp4x8_nonfinite(sg.w[t][0]) | fp4x8_nonfinite(sg.w[t][1]) |
-                   fp4x8_nonfinite(sg.w[t][2]) | fp4x8_nonfinite(sg.w[t][3]);
-            sc[t] = scale_half_f32(sb);
-          }
-#pragma unroll
-          for (int d = 0; d < 4; ++d) {
-            const bf16x8 af = as_bf16x8(a_lds[(ks * 4 + d) * 64 + (lane ^ (4 * d))]);
-#pragma unroll
-            for (int t = 0; t < NT; ++t)
-              acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
-                  as_bf16x8(dequant8_fast(sg.w[t][d], sc[t])), af, acc[t], 0, 0, 0);
-          }
-        };
-
-        const int total_steps = n_my * nsteps;
         unsigned long long redo = 0ull;  // units (bit = index among this wavefront's) to redo
-        int cks = 0;    // K step of the unit being computed
-        int cunit = 0;  // its index among this wavefront's units
-        for (int f0 = 0; f0 < total_steps; f0 += D) {
+        if (slow_pass) {
+          redo = n_my >= 64 ? ~0ull : (1ull << n_my) - 1ull;
+        } else {
 #pragma unroll
-          for (int i = 0; i < D; ++i) {
-            if (f0 + i < total_steps) {  // uniform
-              compute(st[i], cks);
-              if (++cks == nsteps) {
-                // ---- the unit is complete -----------------------------------
-                // a unit that met a code or scale outside the fast path's domain
-                // is redone after the stream, so the hot loop stays small
-                if (__ballot(bad != 0u) != 0ull)
-                  redo |= 1ull << cunit;
-                else if (my_flat >= 0)
-                  epilogue_tile<STAGE, NT>(p, e, acc, col0, my_flat, srow, lq);
-                if (++cunit < n_my) {
-                  park_scales();
+          for (int t = 0; t < NT; ++t) acc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+          uint32_t bad = 0u;
+
+          auto compute = [&](const Stage& sg, int ks) {
+            const int g = min(ks * 4 + lq, groups - 1);
+            int sa[NT];
 #pragma unroll
-                  for (int t = 0; t < NT; ++t) {
-                    cw[t] += w_unit_stride;
-                    cs[t] += s_unit_stride;
-                    col0[t] += WAVES * (STAGE == 0 ? 8 * NT : 16 * NT);
-                  }
-                  if (cunit + 1 < n_my) fetch_scales(s_unit_stride);
-                }
-                cks = 0;
-                bad = 0u;
-#pragma unroll
-                for (int t = 0; t < NT; ++t) acc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
-              }
+            for (int t = 0; t < NT; ++t) {
+              const uint32_t sb = sc_lds[t * sc_tile_bytes + ln * groups + g];
+              bad |= (uint32_t)((sb - kScaleLo) > (kScaleHi - kScaleLo));
+              bad |= fp4x8_nonfinite(sg.w[t][0]) | fp4x8_nonfinite(sg.w[t][1]) |
+                     fp4x8_nonfinite(sg.w[t][2]) | fp4x8_nonfinite(sg.w[t][3]);
+              sa[t] = (int)sb - 1;
             }
-            issue(st[i]);
+            const int sbh = bsc_lds[ks * 64 + lane];
+            const int sbl = sbh - 4;
+            const u32x4 h0 = b_lds[(ks * 4 + 0) * 64 + lane], h1 = b_lds[(ks * 4 + 1) * 64 + lane];
+            const u32x4 l0 = b_lds[(ks * 4 + 2) * 64 + lane], l1 = b_lds[(ks * 4 + 3) * 64 + lane];
+            const i32x8 bh = {(int)h0[0], (int)h0[1], (int)h0[2], (int)h0[3],
+                              (int)h1[0], (int)h1[1], (int)h1[2], (int)h1[3]};
+            const i32x8 bl = {(int)l0[0], (int)l0[1], (int)l0[2], (int)l0[3],
+                              (int)l1[0], (int)l1[1], (int)l1[2], (int)l1[3]};
+#pragma unroll
+            for (int t = 0; t < NT; ++t) {
+              const i32x8 wa = {(int)fp4x8_to_ocp_doubled(sg.w[t][0]),
+                                (int)fp4x8_to_ocp_doubled(sg.w[t][1]),
+                                (int)fp4x8_to_ocp_doubled(sg.w[t][2]),
+                                (int)fp4x8_to_ocp_doubled(sg.w[t][3]), 0, 0, 0, 0};
+              acc[t] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wa, bh, acc[t], 4, 0, 0,
+                                                                        sa[t], 0, sbh);
+              acc[t] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wa, bl, acc[t], 4, 0, 0,
+                                                                        sa[t], 0, sbl);
+            }
+          };
+
+          const int total_steps = n_my * nsteps;
+          int cks = 0;    // K step of the unit being computed
+          int cunit = 0;  // its index among this wavefront's units
+          for (int f0 = 0; f0 < total_steps; f0 += D) {
+            if (f0 > 0 && staged < n_pieces) {  // uniform, and the same in every wavefront
+              write_rows(pieces_for(min(nsteps, f0 + D)));
+              __syncthreads();
+            }
+#pragma unroll
+            for (int i = 0; i < D; ++i) {
+              if (f0 + i < total_steps) {  // uniform
+                compute(st[i], cks);
+                if (++cks == nsteps) {
+                  // ---- the unit is complete ---------------------------------
+                  // a unit that met a code or scale outside the fast path's
+                  // domain is redone after the stream, so the hot loop stays small
+                  if (__ballot(bad != 0u) != 0ull)
+                    redo |= 1ull << cunit;
+                  else if (my_flat >= 0)
+                    epilogue_tile<STAGE, NT>(p, e, acc, col0, my_flat, srow, lq);
+                  if (++cunit < n_my) {
+                    park_scales();
+#pragma unroll
+                    for (int t = 0; t < NT; ++t) {
+                      cw[t] += w_unit_stride;
+                      cs[t] += s_unit_stride;
+                      col0[t] += WAVES * (STAGE == 0 ? 8 * NT : 16 * NT);
+                    }
+                    if (cunit + 1 < n_my) fetch_scales(s_unit_stride);
+                  }
+                  cks = 0;
+                  bad = 0u;
+#pragma unroll
+                  for (int t = 0; t < NT; ++t) acc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+                }
+              }
+              issue(st[i]);
+            }
           }
         }
 
         // ---- reference-exact pass over the units the fast path could not take
-        while (redo != 0ull) {
-          const int idx = __builtin_ctzll(redo);
-          redo &= redo - 1ull;
-          unit_tiles<STAGE, NT>(p, e, first + idx * WAVES, ln, cw, cs, col0);
-          resident_exact_pass<NT>(cw, cs, a_lds, groups, lane, acc);
-          if (my_flat >= 0) epilogue_tile<STAGE, NT>(p, e, acc, col0, my_flat, srow, lq);
+        if (redo != 0ull) {
+          const uint16_t* a_row = nullptr;
+          if (my_flat >= 0)
+            a_row = p.A + (size_t)(STAGE == 0 ? my_flat / p.top_k : srow) * (size_t)K;
+          while (redo != 0ull) {
+            const int idx = __builtin_ctzll(redo);
+            redo &= redo - 1ull;
+            unit_tiles<STAGE, NT>(p, e, first + idx * WAVES, ln, cw, cs, col0);
+            exact_unit_global<NT>(cw, cs, a_row, K, lane, acc);
+            if (my_flat >= 0) epilogue_tile<STAGE, NT>(p, e, acc, col0, my_flat, srow, lq);
+          }
         }
       }
     }
@@ -769,20 +1000,24 @@ int num_compute_units() {
   return cus;
 }
 
-constexpr size_t kResidentLdsLimit = 152 * 1024;  // dynamic LDS the resident kernel may ask for
+constexpr size_t kResidentLdsLimit = 150 * 1024;  // dynamic LDS the resident kernel may ask for
 
+// False when the device refuses the kernel its dynamic LDS (the caller then
+// takes the other variant).
 template <int STAGE, int WAVES, int NT, int D>
-void launch_resident(const GemmArgs& g, size_t lds, hipStream_t stream) {
+bool launch_resident(const GemmArgs& g, size_t lds, hipStream_t stream) {
   auto* kern = stream_resident_kernel<STAGE, WAVES, NT, D>;
   static const bool configured = [kern] {
-    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                              hipFuncAttributeMaxDynamicSharedMemorySize,
-                              (int)kResidentLdsLimit);
-    return true;
+    const hipError_t err = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                               hipFuncAttributeMaxDynamicSharedMemorySize,
+                                               (int)kResidentLdsLimit);
+    if (err != hipSuccess) (void)hipGetLastError();  // not left for the next caller to find
+    return err == hipSuccess;
   }();
-  (void)configured;
+  if (!configured) return false;
   const int wgs = env_int("VK_MOE_WGS", num_compute_units());
   hipLaunchKernelGGL(kern, dim3(wgs), dim3(64 * WAVES), lds, stream, g);
+  return true;
 }
 
 template <int STAGE>
@@ -795,19 +1030,20 @@ void launch_stage(const GemmArgs& g, hipStream_t stream) {
   const int groups = g.K / 32;
   const int nsteps = (groups + 3) / 4;
   // operand planes + one scale region per wavefront
-  const size_t resident_lds = (size_t)nsteps * 4096 + (size_t)waves * nt * 16 * groups;
+  const size_t resident_lds = (size_t)nsteps * (4096 + 64) + (size_t)waves * nt * 16 * groups;
   const int res_units = STAGE == 0 ? g.ncols / (8 * nt) : g.ncols / (16 * nt);
   if (resident_lds > kResidentLdsLimit || g.num_blocks > kMaxRuns || nt * groups > 64 * kScMax ||
-      (res_units + waves - 1) / waves > 64)  // one bit per unit of a wavefront in the redo mask
+      (res_units + waves - 1) / waves > 64 ||  // one bit per unit of a wavefront in the redo mask
+      nsteps * 4 > 96)                         // the rows are staged in one batch of 96 / waves pieces
     variant = kMoeVariantLds;
   if (variant == kMoeVariantResident) {
 #define VK_RESIDENT(W_, NT_, D_) \
-  if (waves == W_ && nt == NT_ && depth == D_) \
-    return launch_resident<STAGE, W_, NT_, D_>(g, resident_lds, stream)
-    VK_RESIDENT(16, 2, 2); VK_RESIDENT(16, 2, 3); VK_RESIDENT(16, 2, 4);
-    VK_RESIDENT(12, 2, 3); VK_RESIDENT(12, 2, 4); VK_RESIDENT(12, 2, 6);
-    VK_RESIDENT(8, 2, 3); VK_RESIDENT(8, 2, 4); VK_RESIDENT(8, 2, 6); VK_RESIDENT(8, 2, 8);
-    VK_RESIDENT(8, 4, 2); VK_RESIDENT(8, 4, 3); VK_RESIDENT(8, 4, 4);
+  if (waves == W_ && nt == NT_ && depth == D_ && \
+      launch_resident<STAGE, W_, NT_, D_>(g, resident_lds, stream)) \
+    return
+    VK_RESIDENT(8, 2, 2); VK_RESIDENT(8, 2, 4); VK_RESIDENT(8, 2, 6);
+    VK_RESIDENT(6, 2, 4); VK_RESIDENT(6, 2, 6); VK_RESIDENT(6, 2, 8);
+    VK_RESIDENT(4, 2, 4); VK_RESIDENT(4, 2, 6); VK_RESIDENT(4, 2, 8); VK_RESIDENT(4, 2, 12);
 #undef VK_RESIDENT
     variant = kMoeVariantLds;
   }
