@@ -1,0 +1,261 @@
+"""GPU parity of the fused MXFP4 MoE layer on the larger configurations.
+
+Where the CPU oracle would need minutes (prefill sizes), the layer runs at
+full size on the GPU and the oracle computes a seeded sample of the tokens:
+a token's output row depends on that token's activations, its routing and
+the weights only, so `oracle(A[sample], ids[sample], w[sample])` must equal
+`gpu_out[sample]`.  The router and the alignment are always compared in full,
+bit for bit.  Full-size runs are also checked through batch-size independence:
+the inputs of a shorter batch are a prefix of the longer one's (the generator
+is counter based), so the shared rows must agree.
+"""
+from __future__ import annotations
+
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from vkernels_amd import synth
+from vkernels_amd import vllm_experts as ve
+
+from gpu_util import (MAX_ABS_TOL, REL_L2_TOL, cpu_layer, dev, error_metrics, to_dev)
+
+pytestmark = pytest.mark.gpu
+
+_WEIGHTS = {}
+
+
+def _weights(cfg, seed=None, **kw):
+    """Device weights of a config (one seed for all its batch sizes), cached."""
+    seed = int(cfg.name[1:]) * 1000 if seed is None else seed
+    key = (cfg.name, seed, tuple(sorted(kw.items())))
+    if key not in _WEIGHTS:
+        _WEIGHTS.clear()  # one config's weights at a time: the largest set is 5.6 GB
+        _WEIGHTS[key] = synth.make_weights(cfg.E, cfg.H, cfg.I, seed, device=dev(), **kw)
+    return _WEIGHTS[key]
+
+
+def _run_gpu(cfg, w, A_bits, logits, block_size=None, **kw):
+    fe = ve.FusedExperts(w.w13, w.w13_scale, w.w2, w.w2_scale, scratch=ve.CaptureSafeScratch(), **kw)
+    A = to_dev(A_bits, torch.bfloat16)
+    ids, tw = fe.route(to_dev(logits), cfg.top_k, True)
+    T = A.shape[0]
+    bs = ve.default_block_size(T) if block_size is None else block_size
+    sids, eids, out_em, max_em = fe.align(ids, bs)
+    out = fe.apply(A, ids, tw, block_size=bs)
+    torch.cuda.synchronize()
+    return dict(out=out.cpu().numpy(), ids=ids.cpu().numpy(), tw=tw.cpu().numpy(),
+                sids=sids.cpu().numpy(), eids=eids.cpu().numpy(), EM=int(out_em.item()),
+                max_EM=max_em, bs=bs)
+
+
+def _check(cfg, T, w, A_bits, logits, sample=None, block_size=None, weights_np=None,
+           gpu_kw=None, cpu_kw=None, seed=0):
+    g = _run_gpu(cfg, w, A_bits, logits, block_size, **(gpu_kw or {}))
+    # router and alignment: bit for bit, full size
+    ids, tw = oracle.route_topk(logits, cfg.top_k, True)
+    assert np.array_equal(g["ids"], ids), "top-k indices differ from the oracle"
+    assert np.array_equal(g["tw"].view(np.uint32), tw.view(np.uint32)), "router weights differ"
+    s_ref, e_ref, em_ref = oracle.moe_align_block_size_with_map(
+        ids.ravel(), cfg.E, g["bs"], None, max_EM=g["max_EM"])
+    assert g["EM"] == em_ref
+    assert np.array_equal(g["sids"], s_ref) and np.array_equal(g["eids"], e_ref)
+    # the layer: all tokens, or a seeded sample of them
+    rows = np.arange(T)
+    if sample is not None and sample < T:
+        rows = np.sort(np.random.default_rng(seed).choice(T, sample, replace=False))
+    wn = w.numpy() if weights_np is None else weights_np
+    c = cpu_layer(A_bits[rows], wn, ids[rows], tw[rows], threads=16, **(cpu_kw or {}))
+    max_rel, rel_l2, nf = error_metrics(g["out"][rows], c["out"])
+    print(f"{cfg.name} T={T} bs={g['bs']} rows checked {rows.size}: "
+          f"max_abs/rms={max_rel:.3e} rel_l2={rel_l2:.3e}")
+    assert nf and max_rel <= MAX_ABS_TOL and rel_l2 <= REL_L2_TOL
+    return g, wn
+
+
+def _inputs(cfg, T, seed):
+    A = synth.make_activations(T, cfg.H, seed)
+    lg = synth.make_logits(cfg.logits, T, cfg.E, seed, A, cfg.H)
+    return A, lg
+
+
+# ---- config 2: 128 experts, Zipf popularity -----------------------------------
+
+def test_config2_zipf_all_sizes():
+    cfg = synth.CONFIGS["c2"]
+    w = _weights(cfg)
+    wn = None
+    prev = None
+    for T, sample in ((4096, 24), (512, 24), (64, None)):
+        A, lg = _inputs(cfg, T, 2000)
+        g, wn = _check(cfg, T, w, A, lg, sample=sample, weights_np=wn)
+        counts = np.bincount(g["ids"].ravel(), minlength=cfg.E)
+        if T == 4096:
+            assert counts.max() > 8 * np.median(counts), "the Zipf routing should be imbalanced"
+        if prev is not None:  # same first rows as the longer batch
+            m, l2, nf = error_metrics(g["out"], prev[:T])
+            assert nf and m <= MAX_ABS_TOL and l2 <= REL_L2_TOL
+        prev = g["out"]
+
+
+# ---- config 3: wide hidden, 256 small experts, prefill ------------------------
+
+@pytest.mark.parametrize("T", [4096, 16384])
+def test_config3_prefill(T):
+    cfg = synth.CONFIGS["c3"]
+    w = _weights(cfg)
+    A, lg = _inputs(cfg, T, 3000)
+    g, _ = _check(cfg, T, w, A, lg, sample=12)
+    assert np.all(np.isfinite(g["out"]))
+    # weighted-combine sanity at full size: the routing weights of a token sum to 1,
+    # so scaling them by 2 through a second call must double the output
+    if T == 4096:
+        fe = ve.FusedExperts(w.w13, w.w13_scale, w.w2, w.w2_scale, scratch=ve.CaptureSafeScratch())
+        ids = to_dev(g["ids"])
+        out2 = fe.apply(to_dev(A, torch.bfloat16), ids, to_dev(2.0 * g["tw"])).cpu().numpy()
+        m, l2, nf = error_metrics(out2, 2.0 * g["out"])
+        assert nf and l2 <= 1e-5, (m, l2)
+
+
+# ---- config 4: robustness sweep ------------------------------------------------
+
+def _extreme_weights(cfg, seed):
+    """Block scales with exponents +-20 and all-zero blocks sprinkled in."""
+    w = synth.make_weights(cfg.E, cfg.H, cfg.I, seed, device=dev())
+    for t_codes, t_scale, stream in ((w.w13, w.w13_scale, 11), (w.w2, w.w2_scale, 12)):
+        n = t_scale.numel()
+        r = synth.rand_u63(n, seed, stream, dev()).reshape(t_scale.shape)
+        sel = (r >> 20) % 100
+        t_scale[sel == 0] = 107   # 2^-20
+        t_scale[sel == 1] = 147   # 2^+20
+        zero = (sel == 2)
+        blocks = t_codes.reshape(*t_scale.shape, 16)
+        blocks[zero] = 0          # all-zero block
+    return w
+
+
+@pytest.mark.parametrize("T", [1, 7, 33, 255, 1000, 8191])
+def test_config4_ragged(T):
+    cfg = synth.CONFIGS["c4"]
+    seed = 4000
+    key = ("c4x", seed)
+    if key not in _WEIGHTS:
+        _WEIGHTS.clear()
+        _WEIGHTS[key] = _extreme_weights(cfg, seed)
+    w = _WEIGHTS[key]
+    A, lg = _inputs(cfg, T, seed)
+    if T == 7:
+        lg[:] = lg[0]                      # every token on the same six experts
+    if T == 33:
+        lg[:, cfg.E // 2:] = -30.0         # half of the experts receive nothing
+    if T == 255:
+        lg[:, 5] += 12.0                   # one expert in every token's top-k
+    g, _ = _check(cfg, T, w, A, lg, sample=None if T <= 255 else 16)
+    counts = np.bincount(g["ids"].ravel(), minlength=cfg.E)
+    if T == 7:
+        assert np.count_nonzero(counts) == cfg.top_k
+    if T == 33:
+        assert counts[cfg.E // 2:].sum() == 0
+    if T == 255:
+        assert counts[5] == T
+
+
+# ---- epilogue variants, block sizes ---------------------------------------------
+
+@pytest.mark.parametrize("variant", ["bias", "limit", "situ", "situ_bias"])
+def test_epilogue_variants(variant):
+    cfg = synth.CONFIGS["c1"]
+    T, seed = 8, 1500
+    w = _weights(cfg, seed)
+    A, lg = _inputs(cfg, T, seed)
+    b13 = (synth.rand_normal((cfg.E, 2 * cfg.I), seed, 21) * 0.5).astype(np.float32)
+    b2 = (synth.rand_normal((cfg.E, cfg.H), seed, 22) * 0.5).astype(np.float32)
+    gpu_kw, cpu_kw = {}, {}
+    if "bias" in variant:
+        gpu_kw.update(b13=to_dev(b13), b2=to_dev(b2))
+        cpu_kw.update(b13=b13, b2=b2)
+    if variant == "limit":
+        gpu_kw.update(swiglu_limit=1.5)
+        cpu_kw.update(swiglu_limit=1.5)
+    if "situ" in variant:
+        gpu_kw.update(activation="situ", beta=3.0, linear_beta=20.0)
+        cpu_kw.update(activation=1, beta=3.0, linear_beta=20.0)
+    _check(cfg, T, w, A, lg, gpu_kw=gpu_kw, cpu_kw=cpu_kw)
+
+
+@pytest.mark.parametrize("bs", [16, 32, 64, 128])
+def test_block_sizes(bs):
+    cfg = synth.CONFIGS["c1"]
+    T, seed = 40, 1600
+    w = _weights(cfg, 1500)
+    A, lg = _inputs(cfg, T, seed)
+    _check(cfg, T, w, A, lg, block_size=bs)
+
+
+# ---- values outside the fast path's domain ---------------------------------------
+
+def _tiny_case(seed):
+    cfg = synth.CONFIGS["c0"]
+    w = synth.make_weights(cfg.E, cfg.H, cfg.I, seed, device=dev())
+    A = synth.make_activations(16, cfg.H, seed)
+    lg = synth.make_logits("uniform", 16, cfg.E, seed)
+    return cfg, w, A, lg
+
+
+def _check_columns(g_out, c_out):
+    """Column by column: the columns of these cases differ by many orders of magnitude."""
+    checked = 0
+    for h in range(c_out.shape[1]):
+        max_rel, rel_l2, nf = error_metrics(g_out[:, h], c_out[:, h])
+        assert nf and max_rel <= MAX_ABS_TOL and rel_l2 <= REL_L2_TOL, (h, max_rel, rel_l2)
+        checked += int(np.isfinite(c_out[:, h]).sum())
+    return checked
+
+
+def test_weight_scales_outside_fast_range():
+    """Scale bytes outside [64, 190] (and 0xFF, a zero block) take the exact path.  The large
+    ones go into the down weights only: through the gate/up product they would overflow."""
+    cfg, w, A, lg = _tiny_case(71)
+    for t, values in ((w.w13_scale, [0, 1, 2, 63, 255]), (w.w2_scale, [0, 1, 63, 191, 200, 255])):
+        special = torch.tensor(values, dtype=torch.uint8, device=dev())
+        r = synth.rand_u63(t.numel(), 71, 31, dev()).reshape(t.shape)
+        pick = (r >> 12) % 64
+        mask = pick < len(values)
+        t[mask] = special[pick[mask]]
+    g = _run_gpu(cfg, w, A, lg)
+    ids, tw = oracle.route_topk(lg, cfg.top_k, True)
+    c = cpu_layer(A, w.numpy(), ids, tw)
+    assert _check_columns(g["out"], c["out"]) == c["out"].size  # all finite, all compared
+
+
+def test_nonfinite_codes():
+    """inf and NaN codes in two experts: the tokens routed there get the oracle's non-finite
+    outputs position by position, the others stay finite and within tolerance."""
+    cfg, w, A, lg = _tiny_case(72)
+    r = synth.rand_u63(w.w13[0].numel(), 72, 32, dev()).reshape(w.w13[0].shape)
+    w.w13[0][(r >> 10) % 4096 == 0] = 0x6E   # +inf and -inf codes
+    r = synth.rand_u63(w.w2[1].numel(), 72, 33, dev()).reshape(w.w2[1].shape)
+    w.w2[1][(r >> 10) % 8192 == 0] = 0x7F    # NaN codes
+    g, _ = _check(cfg, 16, w, A, lg)
+    finite_rows = np.all(np.isfinite(g["out"]), axis=1)
+    assert 0 < finite_rows.sum() < 16
+
+
+def test_activations_outside_fast_range():
+    """Huge, tiny and non-finite activations: the pass falls back to the exact path."""
+    cfg, w, A, lg = _tiny_case(73)
+    A = A.copy()
+    A[0, 5] = 0x7F80      # +inf
+    A[1, 7] = 0x7FC0      # NaN
+    A[2, :] = synth.f32_to_bf16_bits(synth.bf16_bits_to_f32(A[2, :]) * np.float32(2.0 ** 80))
+    A[3, :] = synth.f32_to_bf16_bits(synth.bf16_bits_to_f32(A[3, :]) * np.float32(2.0 ** -90))
+    A[4, :] = 0
+    A[5, :] = synth.f32_to_bf16_bits(synth.bf16_bits_to_f32(A[5, :]) * np.float32(2.0 ** 30))
+    g = _run_gpu(cfg, w, A, lg)
+    ids, tw = oracle.route_topk(lg, cfg.top_k, True)
+    c = cpu_layer(A, w.numpy(), ids, tw)
+    for t in range(16):  # row by row: the rows differ by 50 orders of magnitude
+        max_rel, rel_l2, nf = error_metrics(g["out"][t], c["out"][t])
+        assert nf and max_rel <= MAX_ABS_TOL and rel_l2 <= REL_L2_TOL, (t, max_rel, rel_l2)
+    assert np.all(np.isfinite(g["out"][5])) and not np.all(np.isfinite(g["out"][:3]))
