@@ -111,6 +111,32 @@ void vk_hip_fused_moe_mxfp4(
     const float* b13, const float* b2, int block_size, void* stream);
 
 /*
+ * Additive: vk_hip_fused_moe_mxfp4 with a caller-owned device workspace, for
+ * callers that can provide one (the library itself allocates nothing).  With
+ * at least vk_hip_fused_moe_mxfp4_workspace_bytes(M, hidden, ispp, EM) bytes,
+ * 16-byte aligned, the prefill-sized path splits the bf16 rows into their FP8
+ * terms once per call instead of once per workgroup; results are the same.
+ * A null or short workspace is vk_hip_fused_moe_mxfp4 exactly.  The contents
+ * of the workspace are unspecified after the call; calls that share one
+ * must be ordered on a stream.  No counterpart in the reference, whose Python
+ * binding owns the scratch of its fused call the same way
+ * (src/python/vkernels/vllm_experts.py:160-214).
+ */
+size_t vk_hip_fused_moe_mxfp4_workspace_bytes(int M, int hidden, int ispp, int EM);
+
+void vk_hip_fused_moe_mxfp4_ws(
+    const uint16_t* A, const uint8_t* w13, const uint8_t* w13_scale,
+    const uint8_t* w2, const uint8_t* w2_scale,
+    const int32_t* topk_ids, const float* topk_w,
+    uint16_t* act_scratch, float* out,
+    int M, int hidden, int ispp, int top_k,
+    const int32_t* sorted_ids, const int32_t* expert_ids,
+    int EM, float swiglu_limit,
+    int activation, float beta, float linear_beta,
+    const float* b13, const float* b2, int block_size,
+    void* workspace, size_t workspace_bytes, void* stream);
+
+/*
  * Additive: the two stages of vk_hip_fused_moe_mxfp4 as separate launches,
  * for callers that place work between them (a tensor-parallel all-reduce, a
  * profiler's events).  Device counterparts of the reference's stage split,

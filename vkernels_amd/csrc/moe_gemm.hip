@@ -58,6 +58,14 @@ struct GemmArgs {
   const float* bias;        // b13 [E, 2I] or b2 [E, H], may be null
   uint16_t* act;            // stage 0 output [EM, I]
   float* out;               // stage 1 output [M, H]
+  // Optional "split rows" (tile kernel): the bf16 rows of A already split into
+  // the two E4M3 terms.  Row r, values 8p..8p+7: 16 bytes at Aq + r*2K + 16p,
+  // the 8 leading parts then the 8 remainders; As[r*K/32 + g] the scale byte of
+  // block g, 0 = block outside the fast path's range.  Null = split in-kernel.
+  const uint8_t* Aq;
+  const uint8_t* As;
+  uint8_t* actq;            // stage 0: act written in that form as well (or null)
+  uint8_t* actqs;
   int n_flat;               // M * top_k
   int top_k;
   int K;                    // hidden (stage 0) or ispp (stage 1)
@@ -218,6 +226,16 @@ constexpr int kScMax = 4;       // 16-byte scale pieces per lane: NT * K/32 <= 6
 constexpr uint32_t kScaleLo = 64u, kScaleHi = 190u;  // scale bytes the scaled MFMA path takes
 
 typedef __attribute__((ext_vector_type(8))) int i32x8;
+typedef __attribute__((ext_vector_type(4))) int i32x4;
+
+// The 32 codes of one lane as the FP4 operand of the scaled MFMA: moved onto the
+// OCP code points, in the low four of the operand's eight registers (the
+// instruction does not read the other four for FP4, so they are left undefined).
+__device__ __forceinline__ i32x8 fp4_operand(u32x4 w) {
+  const i32x4 y = {(int)fp4x8_to_ocp_doubled(w[0]), (int)fp4x8_to_ocp_doubled(w[1]),
+                   (int)fp4x8_to_ocp_doubled(w[2]), (int)fp4x8_to_ocp_doubled(w[3])};
+  return __builtin_shufflevector(y, y, 0, 1, 2, 3, -1, -1, -1, -1);
+}
 
 // First item of part `i` when `total` items are cut into `parts` contiguous
 // slices whose sizes differ by at most one.
@@ -653,10 +671,7 @@ __global__ __launch_bounds__(64 * WAVES) void stream_resident_kernel(GemmArgs p)
                               (int)l1[0], (int)l1[1], (int)l1[2], (int)l1[3]};
 #pragma unroll
             for (int t = 0; t < NT; ++t) {
-              const i32x8 wa = {(int)fp4x8_to_ocp_doubled(sg.w[t][0]),
-                                (int)fp4x8_to_ocp_doubled(sg.w[t][1]),
-                                (int)fp4x8_to_ocp_doubled(sg.w[t][2]),
-                                (int)fp4x8_to_ocp_doubled(sg.w[t][3]), 0, 0, 0, 0};
+              const i32x8 wa = fp4_operand(sg.w[t]);
               acc[t] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wa, bh, acc[t], 4, 0, 0,
                                                                         sa[t], 0, sbh);
               acc[t] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wa, bl, acc[t], 4, 0, 0,
@@ -723,265 +738,292 @@ __global__ __launch_bounds__(64 * WAVES) void stream_resident_kernel(GemmArgs p)
   }
 }
 
-// WAVES wavefronts per workgroup, NT weight tiles per wavefront, MT row tiles
-// per pass.  STAGE 0 = gate/up + activation, 1 = down + combine.
-template <int STAGE, int WAVES, int NT, int MT>
-__global__ __launch_bounds__(64 * WAVES) void stream_gemm_kernel(GemmArgs p) {
-  constexpr int kThreads = 64 * WAVES;
-  constexpr int kItemsPerChunk = MT * 16 * (kKChunk / 8);  // 16-byte pieces of A
-  constexpr int kItems = (kItemsPerChunk + kThreads - 1) / kThreads;
+// ---------------------------------------------------------------------------
+// Tile kernel: the general path (prefill, large K, many rows per expert).
+//
+// A workgroup of 4 wavefronts computes up to 64 sorted rows of one expert
+// (4 row tiles of 16) against 16 weight tiles (4 per wavefront: stage 0, two
+// gate tiles and the two up tiles of the same columns; stage 1, four
+// consecutive tiles), K in chunks of 512.  Per chunk: every lane loads its
+// wavefront's weights for the chunk straight into MFMA operand registers
+// (16 x 16 bytes) and the 16 scale bytes of its row, the workgroup splits the
+// 64 x 512 activations into the two E4M3 terms and writes them to LDS as MFMA
+// operands (64 KiB), and each wavefront then issues 4 steps x 4 row tiles x 4
+// weight tiles x 2 terms scaled MFMAs, every LDS operand read serving four of
+// them.  Two workgroups fit a compute unit (LDS and registers), so one
+// workgroup's splitting and barriers overlap the other's MFMAs.
+//
+// grid.x = chunks of 4 wavefront units along the output columns, grid.y =
+// groups of min(block_size, 64) sorted rows; a group lies inside one block,
+// hence one expert.  Arithmetic, operand layouts and the exact fallback are
+// those of the resident kernel above.
+// ---------------------------------------------------------------------------
+constexpr int kTileWaves = 4, kTileNT = 4, kTileMT = 4, kTileSteps = 4;
 
-  // A operand fragments of one chunk: [MT][steps][4 d][64 lanes] x 16 bytes.
-  __shared__ u32x4 a_lds[MT * kStepsPerChunk * 4 * 64];
-  __shared__ int row_src[MT * 16];   // A row to read for each tile row, -1 = none
-  __shared__ int row_flat[MT * 16];  // flat index of each tile row, -1 = padding
+template <int STAGE, bool PRESPLIT>
+__global__ __launch_bounds__(64 * kTileWaves, 2) void tile_gemm_kernel(GemmArgs p) {
+  constexpr int NT = kTileNT, MT = kTileMT, S = kTileSteps;
+  __shared__ u32x4 planes[S * MT * 4 * 64];  // [step][row tile][term][half][lane]
+  __shared__ uint8_t bsc[S * MT * 64];       // block scale bytes, [step][row tile][lane]
+  __shared__ int row_flat[MT * 16];
+  __shared__ int group_slow;
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
-  const int wave = tid >> 6;
-  const int ln = lane & 15;  // weight row within a tile / token within a row tile
-  const int lq = lane >> 4;  // quad
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int ln = lane & 15;
+  const int lq = lane >> 4;
 
-  // ---- run of blocks owned by this workgroup -----------------------------
-  const int b0 = blockIdx.y;
-  const int e = p.expert_ids[b0];
-  if (e < 0) return;
-  if (b0 > 0 && p.expert_ids[b0 - 1] == e) return;
-  int run_blocks = 1;
-  while (b0 + run_blocks < p.num_blocks && p.expert_ids[b0 + run_blocks] == e) ++run_blocks;
-  const int run_row0 = b0 * p.block_size;
-  const int run_tiles = run_blocks * (p.block_size / 16);
-
-  // ---- weight tiles owned by this wavefront --------------------------------
   const int K = p.K;
   const int groups = K / 32;
-  const int row_bytes = K / 2;
+  const int n_chunks = (groups + 4 * S - 1) / (4 * S);
   const int units = STAGE == 0 ? p.ncols / (8 * NT) : p.ncols / (16 * NT);
-  const int unit = blockIdx.x * WAVES + wave;
-  const bool wave_active = unit < units;
-  const int rows_w = STAGE == 0 ? 2 * p.ncols : p.ncols;
+
+  // ---- the rows of this group ------------------------------------------------
+  const int group_rows = min(p.block_size, 16 * MT);
+  const int row0 = blockIdx.y * group_rows;
+  const int e = p.expert_ids[row0 / p.block_size];
+  if (e < 0) return;
+  if (tid < MT * 16) {
+    int f = -1;
+    if (tid < group_rows) {
+      f = p.sorted_ids[row0 + tid];
+      if (f < 0 || f >= p.n_flat) f = -1;
+    }
+    row_flat[tid] = f;
+  }
+  if (tid == 0) group_slow = 0;
+  __syncthreads();
+  uint32_t live = 0u;  // bit m: row tile m has a routed row
+#pragma unroll
+  for (int m = 0; m < MT; ++m) {
+    bool any = false;
+#pragma unroll
+    for (int j = 0; j < 16; ++j) any |= row_flat[m * 16 + j] >= 0;
+    live |= (uint32_t)any << m;
+  }
+  if (live == 0u) return;  // uniform
+
+  // ---- this wavefront's weight tiles --------------------------------------------
+  const int unit = blockIdx.x * kTileWaves + wave;
+  const bool has_unit = unit < units;
   const uint8_t* w_rows[NT];
   const uint8_t* s_rows[NT];
-  int col0[NT];  // first output column of each tile (stage 0: gate column)
+  int col0[NT];
+  unit_tiles<STAGE, NT>(p, e, has_unit ? unit : 0, ln, w_rows, s_rows, col0);
+
+  // ---- staging role: lane (row, d) = (tid / 4, tid % 4) ---------------------------
+  const int sr = tid >> 2, sd = tid & 3;
+  const int sflat = row_flat[sr];
+  const size_t srow_in = sflat >= 0 ? (size_t)(STAGE == 0 ? sflat / p.top_k : row0 + sr) : 0;
+  // bf16 row, or the split row: the same 2 bytes per value either way
+  const uint16_t* src = (PRESPLIT ? reinterpret_cast<const uint16_t*>(p.Aq) : p.A) + srow_in * (size_t)K;
+  const uint8_t* src_scale = PRESPLIT ? p.As + srow_in * (size_t)groups : nullptr;
+  const int sm = sr >> 4, sn = sr & 15;
+
+  f32x4 acc[MT][NT];
 #pragma unroll
-  for (int t = 0; t < NT; ++t) {
-    int row;
-    if (STAGE == 0) {
-      const int half = t / (NT / 2), tt = t % (NT / 2);
-      col0[t] = unit * (8 * NT) + tt * 16;
-      row = half * p.ncols + col0[t] + ln;
-    } else {
-      col0[t] = unit * (16 * NT) + t * 16;
-      row = col0[t] + ln;
+  for (int m = 0; m < MT; ++m)
+#pragma unroll
+    for (int t = 0; t < NT; ++t) acc[m][t] = f32x4{0.f, 0.f, 0.f, 0.f};
+  uint32_t bad = 0u;
+  bool slow = false;
+
+#pragma unroll 1
+  for (int c = 0; c < n_chunks; ++c) {
+    // ---- weights of the chunk: operand registers and the rows' scale bytes -------
+    u32x4 wq[S][NT];
+    u32x4 scq[NT];
+    const int g0 = c * 4 * S;
+#pragma unroll
+    for (int s = 0; s < S; ++s) {
+      // groups past K re-read the last one; the operand planes there are zero
+      const int g = min(g0 + 4 * s + lq, groups - 1);
+#pragma unroll
+      for (int t = 0; t < NT; ++t)
+        wq[s][t] = *reinterpret_cast<const u32x4*>(w_rows[t] + (size_t)g * 16);
     }
-    if (!wave_active) row = 0;
-    const size_t r = (size_t)e * (size_t)rows_w + (size_t)row;
-    w_rows[t] = p.W + r * (size_t)row_bytes;
-    s_rows[t] = p.Ws + r * (size_t)groups;
-  }
-
-  const int n_chunks = (K + kKChunk - 1) / kKChunk;
-
-  for (int tile0 = 0; tile0 < run_tiles; tile0 += MT) {
-    // ---- rows of this pass ------------------------------------------------
-    __syncthreads();  // previous pass done with row_src / a_lds
-    for (int i = tid; i < MT * 16; i += kThreads) {
-      const int tile = tile0 + i / 16;
-      int flat = -1, src = -1;
-      if (tile < run_tiles) {
-        const int r = run_row0 + tile * 16 + (i & 15);
-        const int f = p.sorted_ids[r];
-        if (f >= 0 && f < p.n_flat) {
-          flat = f;
-          src = STAGE == 0 ? f / p.top_k : r;
+    if (g0 + 4 * S <= groups) {  // uniform
+#pragma unroll
+      for (int t = 0; t < NT; ++t) scq[t] = *reinterpret_cast<const u32x4*>(s_rows[t] + g0);
+    } else {  // last, partial chunk: byte by byte
+#pragma unroll
+      for (int t = 0; t < NT; ++t) {
+#pragma unroll
+        for (int s = 0; s < S; ++s) {
+          uint32_t v = 0u;
+#pragma unroll
+          for (int q = 0; q < 4; ++q)
+            v |= (uint32_t)s_rows[t][min(g0 + 4 * s + q, groups - 1)] << (8 * q);
+          scq[t][s] = v;
         }
       }
-      row_flat[i] = flat;
-      row_src[i] = src;
+    }
+
+    // ---- split the 64 x 512 activations of the chunk into LDS operands -----------
+    __syncthreads();  // the previous chunk's arithmetic is done with the planes
+    u32x4 row_scales = {0u, 0u, 0u, 0u};  // PRESPLIT: the 16 scale bytes of this lane's row
+    if (PRESPLIT) {
+      // (the workspace pads the scale array, so the last row's partial chunk may over-read)
+      const u32x4* ps = reinterpret_cast<const u32x4*>(src_scale + g0);
+      row_scales = *ps;
+    }
+#pragma unroll
+    for (int half = 0; half < 2; ++half) {
+      u32x4 v[8];
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        const int g = g0 + half * 8 + i;
+        const bool valid = g < groups && sflat >= 0;
+        v[i] = *reinterpret_cast<const u32x4*>(src + (valid ? g * 32 + sd * 8 : 0));
+      }
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        const int b = half * 8 + i;  // block of 32 within the chunk
+        const int g = g0 + b;
+        if (!(g < groups && sflat >= 0)) v[i] = u32x4{0u, 0u, 0u, 0u};
+        uint32_t sb;
+        uint2 hi, lo;
+        if (PRESPLIT) {
+          sb = (row_scales[b >> 2] >> (8 * (b & 3))) & 0xFFu;
+          if (!(g < groups && sflat >= 0)) sb = 127u;
+          if (sb == 0u) { slow = true; sb = 127u; }
+          hi = make_uint2(v[i][0], v[i][1]);
+          lo = make_uint2(v[i][2], v[i][3]);
+        } else {
+          uint32_t emax = bf16x8_max_exponent(v[i]);
+          emax = max(emax, (uint32_t)__builtin_amdgcn_mov_dpp((int)emax, 0xB1, 0xF, 0xF, true));
+          emax = max(emax, (uint32_t)__builtin_amdgcn_mov_dpp((int)emax, 0x4E, 0xF, 0xF, true));
+          sb = emax - 7u;
+          if (emax == 0u) sb = 127u;  // a block of zeros (or bf16 subnormals, taken as zero)
+          else if (sb < kScaleLo || sb > kScaleHi) { slow = true; sb = 127u; }
+          split_bf16x8(v[i], sb, hi, lo);
+        }
+        const int s = b >> 2, qq = b & 3;
+        const int slot = ((qq & 1) * 2 + (sd >> 1)) * 16 + sn;
+        uint8_t* plane = reinterpret_cast<uint8_t*>(planes) +
+                         (size_t)((((s * MT + sm) * 2) * 2 + (qq >> 1)) * 64 + slot) * 16 +
+                         (sd & 1) * 8;
+        *reinterpret_cast<uint2*>(plane) = hi;
+        *reinterpret_cast<uint2*>(plane + 2 * 64 * 16) = lo;
+        if (sd == 0) bsc[(s * MT + sm) * 64 + qq * 16 + sn] = (uint8_t)sb;
+      }
     }
     __syncthreads();
-    bool tile_live[MT];
-    bool any_live = false;
-#pragma unroll
-    for (int mt = 0; mt < MT; ++mt) {
-      tile_live[mt] = __ballot(lane < 16 && row_flat[mt * 16 + (lane & 15)] >= 0) != 0ull;
-      any_live |= tile_live[mt];
-    }
-    if (!any_live) continue;  // uniform over the workgroup
 
-    // ---- A staging bookkeeping: item -> (tile, row, 8-wide k piece) -------
-    // item = (mt * 32 + piece) * 16 + row; piece = step*16 + q*4 + d.
-    const uint16_t* a_src[kItems];
-    int a_dst[kItems];
-    int a_k[kItems];
+    // ---- arithmetic ---------------------------------------------------------------
+    if (has_unit) {
 #pragma unroll
-    for (int it = 0; it < kItems; ++it) {
-      const int item = tid + it * kThreads;
-      a_src[it] = nullptr;
-      a_dst[it] = 0;
-      a_k[it] = 0;
-      if (item < kItemsPerChunk) {
-        const int row = item & 15;
-        const int piece = (item >> 4) & 31;
-        const int mt = item >> 9;
-        const int step = piece >> 4, q = (piece >> 2) & 3, d = piece & 3;
-        const int src = row_src[mt * 16 + row];
-        a_dst[it] = ((mt * kStepsPerChunk + step) * 4 + d) * 64 + q * 16 + row;
-        a_k[it] = step * kKStep + q * 32 + d * 8;
-        if (src >= 0) a_src[it] = p.A + (size_t)src * (size_t)K;
-      }
-    }
-
-    u32x4 a_reg[kItems];
-    auto load_a = [&](int chunk) {
-#pragma unroll
-      for (int it = 0; it < kItems; ++it) {
-        const int k = chunk * kKChunk + a_k[it];
-        u32x4 v = {0u, 0u, 0u, 0u};
-        if (a_src[it] != nullptr && k < K)
-          v = *reinterpret_cast<const u32x4*>(a_src[it] + k);
-        a_reg[it] = v;
-      }
-    };
-    auto store_a = [&]() {
-#pragma unroll
-      for (int it = 0; it < kItems; ++it)
-        if (tid + it * kThreads < kItemsPerChunk) a_lds[a_dst[it]] = a_reg[it];
-    };
-
-    // ---- weight registers of one chunk ------------------------------------
-    u32x4 w_reg[kStepsPerChunk][NT];
-    uint32_t s_reg[kStepsPerChunk][NT];
-    auto load_w = [&](int chunk, u32x4 (&w)[kStepsPerChunk][NT],
-                      uint32_t (&s)[kStepsPerChunk][NT]) {
-#pragma unroll
-      for (int st = 0; st < kStepsPerChunk; ++st) {
-        const int g = (chunk * kStepsPerChunk + st) * 4 + lq;
-        const bool ok = wave_active && g < groups;
+      for (int s = 0; s < S; ++s) {
+        i32x8 wa[NT];
+        int sa[NT];
 #pragma unroll
         for (int t = 0; t < NT; ++t) {
-          u32x4 v = {0u, 0u, 0u, 0u};
-          uint32_t sc = 127u;
-          if (ok) {
-            v = *reinterpret_cast<const u32x4*>(w_rows[t] + (size_t)g * 16);
-            sc = s_rows[t][g];
-          }
-          w[st][t] = v;
-          s[st][t] = sc;
+          const uint32_t sbw = (scq[t][s] >> (8 * lq)) & 0xFFu;
+          bad |= (uint32_t)((sbw - kScaleLo) > (kScaleHi - kScaleLo));
+          bad |= fp4x8_nonfinite(wq[s][t][0]) | fp4x8_nonfinite(wq[s][t][1]) |
+                 fp4x8_nonfinite(wq[s][t][2]) | fp4x8_nonfinite(wq[s][t][3]);
+          sa[t] = (int)sbw - 1;
+          wa[t] = fp4_operand(wq[s][t]);
         }
-      }
-    };
-
-    f32x4 acc[NT][MT];
 #pragma unroll
-    for (int t = 0; t < NT; ++t)
+        for (int m = 0; m < MT; ++m) {
+          if (!((live >> m) & 1u)) continue;  // uniform
+          const u32x4* pl = planes + (size_t)((s * MT + m) * 4) * 64 + lane;
+          const u32x4 h0 = pl[0], h1 = pl[64], l0 = pl[128], l1 = pl[192];
+          const int sbh = bsc[(s * MT + m) * 64 + lane];
+          const int sbl = sbh - 4;
+          const i32x8 bh = {(int)h0[0], (int)h0[1], (int)h0[2], (int)h0[3],
+                            (int)h1[0], (int)h1[1], (int)h1[2], (int)h1[3]};
+          const i32x8 bl = {(int)l0[0], (int)l0[1], (int)l0[2], (int)l0[3],
+                            (int)l1[0], (int)l1[1], (int)l1[2], (int)l1[3]};
 #pragma unroll
-      for (int mt = 0; mt < MT; ++mt) acc[t][mt] = f32x4{0.f, 0.f, 0.f, 0.f};
-
-    load_a(0);
-    load_w(0, w_reg, s_reg);
-
-    for (int chunk = 0; chunk < n_chunks; ++chunk) {
-      __syncthreads();  // everyone is done reading the previous chunk
-      store_a();
-      __syncthreads();
-      if (chunk + 1 < n_chunks) load_a(chunk + 1);
-
-      // Move this chunk's weights out of the prefetch registers and start
-      // the next chunk's loads before the arithmetic.
-      u32x4 w_cur[kStepsPerChunk][NT];
-      uint32_t s_cur[kStepsPerChunk][NT];
-#pragma unroll
-      for (int st = 0; st < kStepsPerChunk; ++st)
-#pragma unroll
-        for (int t = 0; t < NT; ++t) {
-          w_cur[st][t] = w_reg[st][t];
-          s_cur[st][t] = s_reg[st][t];
-        }
-      if (chunk + 1 < n_chunks) load_w(chunk + 1, w_reg, s_reg);
-
-#pragma unroll
-      for (int st = 0; st < kStepsPerChunk; ++st) {
-        // Fast conversion is valid only for finite codes and mid-range scales.
-        bool slow = false;
-#pragma unroll
-        for (int t = 0; t < NT; ++t) {
-          slow |= !scale_fast_ok(s_cur[st][t]);
-          slow |= (fp4x8_nonfinite(w_cur[st][t][0]) | fp4x8_nonfinite(w_cur[st][t][1]) |
-                   fp4x8_nonfinite(w_cur[st][t][2]) | fp4x8_nonfinite(w_cur[st][t][3])) != 0u;
-        }
-        const bool wave_slow = __ballot(slow) != 0ull;
-#pragma unroll
-        for (int d = 0; d < 4; ++d) {
-          bf16x8 wf[NT];
-          if (!wave_slow) {
-#pragma unroll
-            for (int t = 0; t < NT; ++t)
-              wf[t] = as_bf16x8(dequant8_fast(w_cur[st][t][d], scale_half_f32(s_cur[st][t])));
-          } else {
-#pragma unroll
-            for (int t = 0; t < NT; ++t)
-              wf[t] = as_bf16x8(dequant8_exact(w_cur[st][t][d], s_cur[st][t]));
-          }
-#pragma unroll
-          for (int mt = 0; mt < MT; ++mt) {
-            if (!tile_live[mt]) continue;
-            const bf16x8 af = as_bf16x8(a_lds[((mt * kStepsPerChunk + st) * 4 + d) * 64 + lane]);
-#pragma unroll
-            for (int t = 0; t < NT; ++t)
-              acc[t][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[t], af, acc[t][mt], 0, 0, 0);
-          }
-        }
-      }
-    }
-
-    // ---- epilogue -----------------------------------------------------------
-    // acc[t][mt][r] = C[weight row 4*lq + r of tile t][row ln of row tile mt]
-    if (!wave_active) continue;
-#pragma unroll
-    for (int mt = 0; mt < MT; ++mt) {
-      if (!tile_live[mt]) continue;
-      const int flat = row_flat[mt * 16 + ln];
-      if (flat < 0) continue;
-      const int srow = run_row0 + (tile0 + mt) * 16 + ln;
-      if (STAGE == 0) {
-#pragma unroll
-        for (int t = 0; t < NT / 2; ++t) {
-          const int c = col0[t] + 4 * lq;
-          uint32_t packed[2];
-#pragma unroll
-          for (int r = 0; r < 4; ++r) {
-            float g = acc[t][mt][r];
-            float u = acc[t + NT / 2][mt][r];
-            if (p.bias != nullptr) {
-              const float* b = p.bias + (size_t)e * (size_t)(2 * p.ncols);
-              g += b[c + r];
-              u += b[p.ncols + c + r];
-            }
-            const uint32_t v = f32_to_bf16_bits(
-                act_value(p.activation, g, u, p.swiglu_limit, p.beta, p.linear_beta));
-            if (r & 1) packed[r >> 1] |= v << 16;
-            else packed[r >> 1] = v;
-          }
-          uint2 st2 = make_uint2(packed[0], packed[1]);
-          *reinterpret_cast<uint2*>(p.act + (size_t)srow * (size_t)p.ncols + c) = st2;
-        }
-      } else {
-        const float w = p.topk_w[flat];
-        float* orow = p.out + (size_t)(flat / p.top_k) * (size_t)p.ncols;
-#pragma unroll
-        for (int t = 0; t < NT; ++t) {
-          const int c = col0[t] + 4 * lq;
-#pragma unroll
-          for (int r = 0; r < 4; ++r) {
-            float v = acc[t][mt][r];
-            if (p.bias != nullptr) v += p.bias[(size_t)e * (size_t)p.ncols + c + r];
-            unsafeAtomicAdd(orow + c + r, v * w);
+          for (int t = 0; t < NT; ++t) {
+            acc[m][t] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wa[t], bh, acc[m][t], 4, 0,
+                                                                         0, sa[t], 0, sbh);
+            acc[m][t] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wa[t], bl, acc[m][t], 4, 0,
+                                                                         0, sa[t], 0, sbl);
           }
         }
       }
     }
   }
+
+  // ---- fall back to the exact path where the fast one was outside its domain ----
+  if (slow) group_slow = 1;
+  __syncthreads();
+  if (!has_unit) return;
+  const bool redo = group_slow != 0 || __ballot(bad != 0u) != 0ull;
+
+  // ---- epilogue -----------------------------------------------------------------------
+#pragma unroll
+  for (int m = 0; m < MT; ++m) {
+    if (!((live >> m) & 1u)) continue;
+    const int flat = row_flat[m * 16 + ln];
+    const int srow = row0 + m * 16 + ln;
+    if (redo) {
+      const uint16_t* a_row = nullptr;
+      if (flat >= 0) a_row = p.A + (size_t)(STAGE == 0 ? flat / p.top_k : srow) * (size_t)K;
+      exact_unit_global<NT>(w_rows, s_rows, a_row, K, lane, acc[m]);
+    }
+    if (flat >= 0) epilogue_tile<STAGE, NT>(p, e, acc[m], col0, flat, srow, lq);
+    if (STAGE == 0 && p.actq != nullptr) {
+      // The 32 act columns of this unit, as the next stage's split rows.  The
+      // lane re-reads the 8 bf16 values it has just stored; the four lanes
+      // (n, q = 0..3) of a row share the block.
+      u32x4 v = {0u, 0u, 0u, 0u};
+      if (flat >= 0) {
+        const uint16_t* arow = p.act + (size_t)srow * (size_t)p.ncols;
+        const uint2 a0 = *reinterpret_cast<const uint2*>(arow + col0[0] + 4 * lq);
+        const uint2 a1 = *reinterpret_cast<const uint2*>(arow + col0[1] + 4 * lq);
+        v = u32x4{a0.x, a0.y, a1.x, a1.y};
+      }
+      uint32_t emax = bf16x8_max_exponent(v);
+      emax = max(emax, (uint32_t)__shfl_xor((int)emax, 16));
+      emax = max(emax, (uint32_t)__shfl_xor((int)emax, 32));
+      uint32_t sb = emax - 7u, stored;
+      if (emax == 0u) sb = 127u;
+      stored = sb;
+      if (emax != 0u && (sb < kScaleLo || sb > kScaleHi)) { stored = 0u; sb = 127u; }
+      uint2 hi, lo;
+      split_bf16x8(v, sb, hi, lo);
+      if (flat >= 0) {
+        uint8_t* qrow = p.actq + (size_t)srow * (size_t)p.ncols * 2;
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+          const int c = col0[t] + 4 * lq;  // 4 values: half of the piece c / 8
+          uint8_t* piece = qrow + (size_t)(c >> 3) * 16 + (c & 4);
+          *reinterpret_cast<uint32_t*>(piece) = t == 0 ? hi.x : hi.y;
+          *reinterpret_cast<uint32_t*>(piece + 8) = t == 0 ? lo.x : lo.y;
+        }
+        if (lq == 0) p.actqs[(size_t)srow * (size_t)(p.ncols / 32) + (col0[0] >> 5)] = (uint8_t)stored;
+      }
+    }
+  }
+}
+
+// bf16 rows [R, K] -> split rows (see GemmArgs::Aq).  One lane per 8 values.
+__global__ __launch_bounds__(256) void split_rows_kernel(const uint16_t* __restrict__ x,
+                                                         uint8_t* __restrict__ xq,
+                                                         uint8_t* __restrict__ xs, long long pieces,
+                                                         int K) {
+  const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;  // piece index, 8 values
+  u32x4 v = {0u, 0u, 0u, 0u};
+  if (i < pieces) v = *reinterpret_cast<const u32x4*>(x + i * 8);
+  uint32_t emax = bf16x8_max_exponent(v);
+  emax = max(emax, (uint32_t)__builtin_amdgcn_mov_dpp((int)emax, 0xB1, 0xF, 0xF, true));
+  emax = max(emax, (uint32_t)__builtin_amdgcn_mov_dpp((int)emax, 0x4E, 0xF, 0xF, true));
+  uint32_t sb = emax - 7u, stored;
+  if (emax == 0u) sb = 127u;
+  stored = sb;
+  if (emax != 0u && (sb < kScaleLo || sb > kScaleHi)) { stored = 0u; sb = 127u; }
+  uint2 hi, lo;
+  split_bf16x8(v, sb, hi, lo);
+  if (i < pieces) {
+    *reinterpret_cast<u32x4*>(xq + i * 16) = u32x4{hi.x, hi.y, lo.x, lo.y};
+    if ((i & 3) == 0) xs[i >> 2] = (uint8_t)stored;  // K is a multiple of 32: blocks do not straddle rows
+  }
+  (void)K;
 }
 
 int env_int(const char* name, int fallback) {
@@ -1020,38 +1062,78 @@ bool launch_resident(const GemmArgs& g, size_t lds, hipStream_t stream) {
   return true;
 }
 
+// Launch shape of one stage.  variant kMoeVariantLds = the tile kernel.
+struct StagePlan {
+  int variant, waves, nt, depth;
+  size_t resident_lds;
+};
+
 template <int STAGE>
-void launch_stage(const GemmArgs& g, hipStream_t stream) {
+StagePlan plan_stage(const GemmArgs& g) {
   const MoeTile tile = pick_moe_tile(g.n_flat, g.K, g.ncols);
-  int variant = env_int("VK_MOE_VARIANT", tile.variant);
-  const int nt = env_int("VK_MOE_NT", tile.nt);
-  const int depth = env_int("VK_MOE_DEPTH", tile.depth);
-  const int waves = env_int("VK_MOE_WAVES", tile.waves);
+  StagePlan pl;
+  pl.variant = env_int("VK_MOE_VARIANT", tile.variant);
+  pl.nt = env_int("VK_MOE_NT", tile.nt);
+  pl.depth = env_int("VK_MOE_DEPTH", tile.depth);
+  pl.waves = env_int("VK_MOE_WAVES", tile.waves);
   const int groups = g.K / 32;
   const int nsteps = (groups + 3) / 4;
-  // operand planes + one scale region per wavefront
-  const size_t resident_lds = (size_t)nsteps * (4096 + 64) + (size_t)waves * nt * 16 * groups;
-  const int res_units = STAGE == 0 ? g.ncols / (8 * nt) : g.ncols / (16 * nt);
-  if (resident_lds > kResidentLdsLimit || g.num_blocks > kMaxRuns || nt * groups > 64 * kScMax ||
-      (res_units + waves - 1) / waves > 64 ||  // one bit per unit of a wavefront in the redo mask
-      nsteps * 4 > 96)                         // the rows are staged in one batch of 96 / waves pieces
-    variant = kMoeVariantLds;
-  if (variant == kMoeVariantResident) {
+  // operand planes + block scales + one weight-scale region per wavefront
+  pl.resident_lds = (size_t)nsteps * (4096 + 64) + (size_t)pl.waves * pl.nt * 16 * groups;
+  const int res_units = STAGE == 0 ? g.ncols / (8 * pl.nt) : g.ncols / (16 * pl.nt);
+  if (pl.resident_lds > kResidentLdsLimit || g.num_blocks > kMaxRuns ||
+      pl.nt * groups > 64 * kScMax ||
+      (res_units + pl.waves - 1) / pl.waves > 64 ||  // one bit per unit in a wavefront's redo mask
+      nsteps * 4 > 96)  // the rows are staged in one batch of 96 / waves pieces
+    pl.variant = kMoeVariantLds;
+  return pl;
+}
+
+template <int STAGE>
+void launch_stage(const GemmArgs& g, const StagePlan& pl, hipStream_t stream) {
+  if (pl.variant == kMoeVariantResident) {
 #define VK_RESIDENT(W_, NT_, D_) \
-  if (waves == W_ && nt == NT_ && depth == D_ && \
-      launch_resident<STAGE, W_, NT_, D_>(g, resident_lds, stream)) \
+  if (pl.waves == W_ && pl.nt == NT_ && pl.depth == D_ && \
+      launch_resident<STAGE, W_, NT_, D_>(g, pl.resident_lds, stream)) \
     return
     VK_RESIDENT(8, 2, 2); VK_RESIDENT(8, 2, 4); VK_RESIDENT(8, 2, 6);
-    VK_RESIDENT(6, 2, 4); VK_RESIDENT(6, 2, 6); VK_RESIDENT(6, 2, 8);
-    VK_RESIDENT(4, 2, 4); VK_RESIDENT(4, 2, 6); VK_RESIDENT(4, 2, 8); VK_RESIDENT(4, 2, 12);
+    VK_RESIDENT(4, 2, 4); VK_RESIDENT(4, 2, 8);
 #undef VK_RESIDENT
-    variant = kMoeVariantLds;
   }
-  constexpr int WAVES = 4, NT = 4, MT = 4;
-  const int units = STAGE == 0 ? g.ncols / (8 * NT) : g.ncols / (16 * NT);
-  const dim3 grid((units + WAVES - 1) / WAVES, g.num_blocks);
-  hipLaunchKernelGGL((stream_gemm_kernel<STAGE, WAVES, NT, MT>), grid, dim3(64 * WAVES), 0,
-                     stream, g);
+  const int units = STAGE == 0 ? g.ncols / (8 * kTileNT) : g.ncols / (16 * kTileNT);
+  const int group_rows = g.block_size < 16 * kTileMT ? g.block_size : 16 * kTileMT;
+  const dim3 grid((units + kTileWaves - 1) / kTileWaves, g.num_blocks * (g.block_size / group_rows));
+  if (g.Aq != nullptr && pl.variant != kMoeVariantResident)
+    hipLaunchKernelGGL((tile_gemm_kernel<STAGE, true>), grid, dim3(64 * kTileWaves), 0, stream, g);
+  else
+    hipLaunchKernelGGL((tile_gemm_kernel<STAGE, false>), grid, dim3(64 * kTileWaves), 0, stream, g);
+}
+
+// Workspace of the fused call: split rows of A, then of act, each followed by
+// its scale bytes (padded: the tile kernel reads 16 scale bytes at a time).
+struct Workspace {
+  uint8_t* a_q;
+  uint8_t* a_s;
+  uint8_t* act_q;
+  uint8_t* act_s;
+};
+
+size_t align256(size_t n) { return (n + 255) & ~(size_t)255; }
+
+bool carve_workspace(const FusedMoeArgs& a, Workspace& w) {
+  if (a.workspace == nullptr) return false;
+  const size_t aq = align256((size_t)a.M * a.hidden * 2);
+  const size_t as = align256((size_t)a.M * (a.hidden / 32) + 16);
+  const size_t cq = align256((size_t)a.EM * a.ispp * 2);
+  const size_t cs = align256((size_t)a.EM * (a.ispp / 32) + 16);
+  if (a.workspace_bytes < aq + as + cq + cs) return false;
+  uint8_t* base = static_cast<uint8_t*>(a.workspace);
+  if ((reinterpret_cast<uintptr_t>(base) & 15) != 0) return false;
+  w.a_q = base;
+  w.a_s = base + aq;
+  w.act_q = base + aq + as;
+  w.act_s = base + aq + as + cq;
+  return true;
 }
 
 GemmArgs common_args(const FusedMoeArgs& a) {
@@ -1072,10 +1154,7 @@ GemmArgs common_args(const FusedMoeArgs& a) {
   return g;
 }
 
-}  // namespace
-
-void launch_moe_gateup(const FusedMoeArgs& a, hipStream_t stream) {
-  if (a.M <= 0 || a.EM <= 0 || a.block_size <= 0) return;
+GemmArgs gateup_args(const FusedMoeArgs& a) {
   GemmArgs g = common_args(a);
   g.A = a.A;
   g.W = a.w13;
@@ -1083,11 +1162,10 @@ void launch_moe_gateup(const FusedMoeArgs& a, hipStream_t stream) {
   g.bias = a.b13;
   g.K = a.hidden;
   g.ncols = a.ispp;
-  launch_stage<0>(g, stream);
+  return g;
 }
 
-void launch_moe_down(const FusedMoeArgs& a, hipStream_t stream) {
-  if (a.M <= 0 || a.EM <= 0 || a.block_size <= 0) return;
+GemmArgs down_args(const FusedMoeArgs& a) {
   GemmArgs g = common_args(a);
   g.A = a.act;
   g.W = a.w2;
@@ -1095,12 +1173,56 @@ void launch_moe_down(const FusedMoeArgs& a, hipStream_t stream) {
   g.bias = a.b2;
   g.K = a.ispp;
   g.ncols = a.hidden;
-  launch_stage<1>(g, stream);
+  return g;
 }
 
+}  // namespace
+
+size_t fused_moe_workspace_bytes(int M, int hidden, int ispp, int EM) {
+  if (M <= 0 || EM <= 0 || hidden <= 0 || ispp <= 0) return 0;
+  return align256((size_t)M * hidden * 2) + align256((size_t)M * (hidden / 32) + 16) +
+         align256((size_t)EM * ispp * 2) + align256((size_t)EM * (ispp / 32) + 16);
+}
+
+void launch_moe_gateup(const FusedMoeArgs& a, hipStream_t stream) {
+  if (a.M <= 0 || a.EM <= 0 || a.block_size <= 0) return;
+  const GemmArgs g = gateup_args(a);
+  launch_stage<0>(g, plan_stage<0>(g), stream);
+}
+
+void launch_moe_down(const FusedMoeArgs& a, hipStream_t stream) {
+  if (a.M <= 0 || a.EM <= 0 || a.block_size <= 0) return;
+  const GemmArgs g = down_args(a);
+  launch_stage<1>(g, plan_stage<1>(g), stream);
+}
+
+// Both stages.  With a workspace, a stage that runs as the tile kernel takes
+// its rows already split: A by a pass of its own, act by the first stage's
+// epilogue (which writes the bf16 act as well; the exact fallback reads it).
 void launch_fused_moe(const FusedMoeArgs& a, hipStream_t stream) {
-  launch_moe_gateup(a, stream);
-  launch_moe_down(a, stream);
+  if (a.M <= 0 || a.EM <= 0 || a.block_size <= 0) return;
+  GemmArgs g0 = gateup_args(a);
+  GemmArgs g1 = down_args(a);
+  const StagePlan p0 = plan_stage<0>(g0), p1 = plan_stage<1>(g1);
+  Workspace w;
+  if (carve_workspace(a, w) && env_int("VK_MOE_PRESPLIT", 1) != 0) {
+    const bool tile0 = p0.variant != kMoeVariantResident, tile1 = p1.variant != kMoeVariantResident;
+    if (tile0) {
+      const long long pieces = (long long)a.M * a.hidden / 8;
+      hipLaunchKernelGGL(split_rows_kernel, dim3((unsigned)((pieces + 255) / 256)), dim3(256), 0,
+                         stream, a.A, w.a_q, w.a_s, pieces, a.hidden);
+      g0.Aq = w.a_q;
+      g0.As = w.a_s;
+    }
+    if (tile0 && tile1) {
+      g0.actq = w.act_q;
+      g0.actqs = w.act_s;
+      g1.Aq = w.act_q;
+      g1.As = w.act_s;
+    }
+  }
+  launch_stage<0>(g0, p0, stream);
+  launch_stage<1>(g1, p1, stream);
 }
 
 }  // namespace vk

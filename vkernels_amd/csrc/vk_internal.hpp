@@ -37,7 +37,12 @@ struct FusedMoeArgs {
   int M, hidden, ispp, top_k, EM, block_size;
   float swiglu_limit, beta, linear_beta;
   int activation;
+  void* workspace;         // optional, see fused_moe_workspace_bytes
+  size_t workspace_bytes;
 };
+
+// Bytes of workspace with which launch_fused_moe runs its fastest path.
+size_t fused_moe_workspace_bytes(int M, int hidden, int ispp, int EM);
 
 void launch_fused_moe(const FusedMoeArgs& a, hipStream_t stream);
 void launch_moe_gateup(const FusedMoeArgs& a, hipStream_t stream);

@@ -231,6 +231,20 @@ def resolve_moe_fn(lib):
     return fn
 
 
+def resolve_moe_ws_fn(lib):
+    """(``vk_hip_fused_moe_mxfp4_ws``, ``vk_hip_fused_moe_mxfp4_workspace_bytes``), the fused
+    call with a caller-owned workspace, or (None, None) when the library predates it."""
+    fn = getattr(lib, "vk_hip_fused_moe_mxfp4_ws", None)
+    size_fn = getattr(lib, "vk_hip_fused_moe_mxfp4_workspace_bytes", None)
+    if fn is None or size_fn is None:
+        return None, None
+    fn.restype = None
+    fn.argtypes = _MOE_ARGTYPES[:-1] + [_P, ctypes.c_size_t, _P]
+    size_fn.restype = ctypes.c_size_t
+    size_fn.argtypes = [_I, _I, _I, _I]
+    return fn, size_fn
+
+
 def resolve_align_fn(lib):
     """``vk_hip_moe_align_block_size`` or None when the symbol is absent."""
     fn = getattr(lib, "vk_hip_moe_align_block_size", None)
@@ -302,6 +316,7 @@ class FusedExperts:
         self.torch = torch
         self.lib = load_libvkernels_hip()
         self.moe_fn = resolve_moe_fn(self.lib)
+        self.moe_ws_fn, self.ws_bytes_fn = resolve_moe_ws_fn(self.lib)
         self.align_fn = resolve_align_fn(self.lib)
         if self.align_fn is None:
             raise RuntimeError("vk_hip_moe_align_block_size not found in libvkernels_hip.so")
@@ -320,6 +335,9 @@ class FusedExperts:
             raise ValueError("hidden and ispp must be multiples of 64")
         self.w13, self.w13_scale, self.w2, self.w2_scale = w13, w13_scale, w2, w2_scale
         self.b13, self.b2 = b13, b2
+        # routed rows (tokens * top_k) above which apply() hands the library a workspace;
+        # below it the decode kernel runs, which has no use for one
+        self.workspace_min_rows = 512
         self.activation = {"swiglu": 0, "situ": 1}[activation] if isinstance(activation, str) \
             else int(activation)
         self.swiglu_limit, self.beta, self.linear_beta = swiglu_limit, beta, linear_beta
@@ -389,12 +407,21 @@ class FusedExperts:
         cap = _align_em_bound(max(M, max_tokens or 0), top_k, self.local_n, block_size)
         act = self.scratch.get(("act", self.ispp), max_em * self.ispp, dtype=torch.bfloat16,
                                device=dev, capacity=cap * self.ispp, name="act_scratch")
-        self.moe_fn(_ptr(hidden_states), _ptr(self.w13), _ptr(self.w13_scale), _ptr(self.w2),
-                    _ptr(self.w2_scale), _ptr(topk_ids), _ptr(topk_weights), _ptr(act),
-                    _ptr(out_fp32), M, K, self.ispp, top_k, _ptr(sids), _ptr(eids), max_em,
-                    float(self.swiglu_limit), self.activation, float(self.beta),
-                    float(self.linear_beta), _ptr(self.b13), _ptr(self.b2), block_size,
-                    _stream(torch))
+        args = (_ptr(hidden_states), _ptr(self.w13), _ptr(self.w13_scale), _ptr(self.w2),
+                _ptr(self.w2_scale), _ptr(topk_ids), _ptr(topk_weights), _ptr(act),
+                _ptr(out_fp32), M, K, self.ispp, top_k, _ptr(sids), _ptr(eids), max_em,
+                float(self.swiglu_limit), self.activation, float(self.beta),
+                float(self.linear_beta), _ptr(self.b13), _ptr(self.b2), block_size)
+        if self.moe_ws_fn is not None and M * top_k > self.workspace_min_rows:
+            # prefill-sized call: the library splits the rows once, into a workspace
+            # held like the other scratch (sized once at the token budget)
+            need = int(self.ws_bytes_fn(M, K, self.ispp, max_em))
+            cap_bytes = int(self.ws_bytes_fn(max(M, max_tokens or 0), K, self.ispp, cap))
+            ws = self.scratch.get(("ws", K, self.ispp), need, dtype=torch.uint8, device=dev,
+                                  capacity=cap_bytes, name="workspace")
+            self.moe_ws_fn(*args, _ptr(ws), need, _stream(torch))
+        else:
+            self.moe_fn(*args, _stream(torch))
         return out_fp32
 
     def forward(self, hidden_states, router_logits, top_k: int, **kw):
