@@ -58,10 +58,10 @@ struct GemmArgs {
   const float* bias;        // b13 [E, 2I] or b2 [E, H], may be null
   uint16_t* act;            // stage 0 output [EM, I]
   float* out;               // stage 1 output [M, H]
-  // Optional "split rows" (tile kernel): the bf16 rows of A already split into
-  // the two E4M3 terms.  Row r, values 8p..8p+7: 16 bytes at Aq + r*2K + 16p,
-  // the 8 leading parts then the 8 remainders; As[r*K/32 + g] the scale byte of
-  // block g, 0 = block outside the fast path's range.  Null = split in-kernel.
+  // Optional "split rows" (workspace tile kernel): the bf16 rows of A already
+  // split into the two E4M3 terms.  Row r: 2K bytes at Aq + r*2K, the K leading
+  // parts then the K remainders (times 16); As[r*split_scale_stride(K) + g] the
+  // scale byte of block g, 0 = block outside the fast path's range.
   const uint8_t* Aq;
   const uint8_t* As;
   uint8_t* actq;            // stage 0: act written in that form as well (or null)
@@ -75,6 +75,9 @@ struct GemmArgs {
   float swiglu_limit, beta, linear_beta;
   int activation;
 };
+
+// Bytes between the scale rows of split rows: K/32 rounded up to 16.
+__host__ __device__ inline int split_scale_stride(int K) { return (K / 32 + 15) & ~15; }
 
 __device__ __forceinline__ float act_value(int activation, float g, float u,
                                            float limit, float beta,
@@ -669,14 +672,18 @@ __global__ __launch_bounds__(64 * WAVES) void stream_resident_kernel(GemmArgs p)
                               (int)h1[0], (int)h1[1], (int)h1[2], (int)h1[3]};
             const i32x8 bl = {(int)l0[0], (int)l0[1], (int)l0[2], (int)l0[3],
                               (int)l1[0], (int)l1[1], (int)l1[2], (int)l1[3]};
+            i32x8 wa[NT];
 #pragma unroll
-            for (int t = 0; t < NT; ++t) {
-              const i32x8 wa = fp4_operand(sg.w[t]);
-              acc[t] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wa, bh, acc[t], 4, 0, 0,
+            for (int t = 0; t < NT; ++t) wa[t] = fp4_operand(sg.w[t]);
+            // the two MFMAs of an accumulator are kept NT instructions apart
+#pragma unroll
+            for (int t = 0; t < NT; ++t)
+              acc[t] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wa[t], bh, acc[t], 4, 0, 0,
                                                                         sa[t], 0, sbh);
-              acc[t] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wa, bl, acc[t], 4, 0, 0,
+#pragma unroll
+            for (int t = 0; t < NT; ++t)
+              acc[t] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wa[t], bl, acc[t], 4, 0, 0,
                                                                         sa[t], 0, sbl);
-            }
           };
 
           const int total_steps = n_my * nsteps;
@@ -738,6 +745,41 @@ __global__ __launch_bounds__(64 * WAVES) void stream_resident_kernel(GemmArgs p)
   }
 }
 
+// Stage 0 with a workspace: 32 consecutive act columns (two 16-column tiles, first
+// columns c0 and c1 = c0 + 16) of one 16-row tile as the next stage's split rows.
+// The lane re-reads the 8 bf16 values it has just stored; the four lanes
+// (n, q = 0..3) of a row share the block.  Called by whole wavefronts
+// (flat < 0 = padding row: takes part in the shuffles, stores nothing).
+__device__ __forceinline__ void store_split_act(const GemmArgs& p, int c0, int c1, int flat, int srow,
+                                                int lane) {
+  const int lq = lane >> 4;
+  u32x4 v = {0u, 0u, 0u, 0u};
+  if (flat >= 0) {
+    const uint16_t* arow = p.act + (size_t)srow * (size_t)p.ncols;
+    const uint2 a0 = *reinterpret_cast<const uint2*>(arow + c0 + 4 * lq);
+    const uint2 a1 = *reinterpret_cast<const uint2*>(arow + c1 + 4 * lq);
+    v = u32x4{a0.x, a0.y, a1.x, a1.y};
+  }
+  uint32_t emax = bf16x8_max_exponent(v);
+  emax = max(emax, (uint32_t)__shfl_xor((int)emax, 16));
+  emax = max(emax, (uint32_t)__shfl_xor((int)emax, 32));
+  uint32_t sb = emax - 7u, stored;
+  if (emax == 0u) sb = 127u;
+  stored = sb;
+  if (emax != 0u && (sb < kScaleLo || sb > kScaleHi)) { stored = 0u; sb = 127u; }
+  uint2 hi, lo;
+  split_bf16x8(v, sb, hi, lo);
+  if (flat >= 0) {
+    uint8_t* qrow = p.actq + (size_t)srow * (size_t)p.ncols * 2;
+    *reinterpret_cast<uint32_t*>(qrow + c0 + 4 * lq) = hi.x;
+    *reinterpret_cast<uint32_t*>(qrow + c1 + 4 * lq) = hi.y;
+    *reinterpret_cast<uint32_t*>(qrow + p.ncols + c0 + 4 * lq) = lo.x;
+    *reinterpret_cast<uint32_t*>(qrow + p.ncols + c1 + 4 * lq) = lo.y;
+    if (lq == 0)
+      p.actqs[(size_t)srow * (size_t)split_scale_stride(p.ncols) + (c0 >> 5)] = (uint8_t)stored;
+  }
+}
+
 // ---------------------------------------------------------------------------
 // Tile kernel: the general path (prefill, large K, many rows per expert).
 //
@@ -760,7 +802,7 @@ __global__ __launch_bounds__(64 * WAVES) void stream_resident_kernel(GemmArgs p)
 // ---------------------------------------------------------------------------
 constexpr int kTileWaves = 4, kTileNT = 4, kTileMT = 4, kTileSteps = 4;
 
-template <int STAGE, bool PRESPLIT>
+template <int STAGE>
 __global__ __launch_bounds__(64 * kTileWaves, 2) void tile_gemm_kernel(GemmArgs p) {
   constexpr int NT = kTileNT, MT = kTileMT, S = kTileSteps;
   __shared__ u32x4 planes[S * MT * 4 * 64];  // [step][row tile][term][half][lane]
@@ -815,10 +857,8 @@ __global__ __launch_bounds__(64 * kTileWaves, 2) void tile_gemm_kernel(GemmArgs 
   // ---- staging role: lane (row, d) = (tid / 4, tid % 4) ---------------------------
   const int sr = tid >> 2, sd = tid & 3;
   const int sflat = row_flat[sr];
-  const size_t srow_in = sflat >= 0 ? (size_t)(STAGE == 0 ? sflat / p.top_k : row0 + sr) : 0;
-  // bf16 row, or the split row: the same 2 bytes per value either way
-  const uint16_t* src = (PRESPLIT ? reinterpret_cast<const uint16_t*>(p.Aq) : p.A) + srow_in * (size_t)K;
-  const uint8_t* src_scale = PRESPLIT ? p.As + srow_in * (size_t)groups : nullptr;
+  const uint16_t* src =
+      p.A + (size_t)(sflat >= 0 ? (STAGE == 0 ? sflat / p.top_k : row0 + sr) : 0) * (size_t)K;
   const int sm = sr >> 4, sn = sr & 15;
 
   f32x4 acc[MT][NT];
@@ -862,12 +902,6 @@ __global__ __launch_bounds__(64 * kTileWaves, 2) void tile_gemm_kernel(GemmArgs 
 
     // ---- split the 64 x 512 activations of the chunk into LDS operands -----------
     __syncthreads();  // the previous chunk's arithmetic is done with the planes
-    u32x4 row_scales = {0u, 0u, 0u, 0u};  // PRESPLIT: the 16 scale bytes of this lane's row
-    if (PRESPLIT) {
-      // (the workspace pads the scale array, so the last row's partial chunk may over-read)
-      const u32x4* ps = reinterpret_cast<const u32x4*>(src_scale + g0);
-      row_scales = *ps;
-    }
 #pragma unroll
     for (int half = 0; half < 2; ++half) {
       u32x4 v[8];
@@ -882,23 +916,14 @@ __global__ __launch_bounds__(64 * kTileWaves, 2) void tile_gemm_kernel(GemmArgs 
         const int b = half * 8 + i;  // block of 32 within the chunk
         const int g = g0 + b;
         if (!(g < groups && sflat >= 0)) v[i] = u32x4{0u, 0u, 0u, 0u};
-        uint32_t sb;
+        uint32_t emax = bf16x8_max_exponent(v[i]);
+        emax = max(emax, (uint32_t)__builtin_amdgcn_mov_dpp((int)emax, 0xB1, 0xF, 0xF, true));
+        emax = max(emax, (uint32_t)__builtin_amdgcn_mov_dpp((int)emax, 0x4E, 0xF, 0xF, true));
+        uint32_t sb = emax - 7u;
+        if (emax == 0u) sb = 127u;  // a block of zeros (or bf16 subnormals, taken as zero)
+        else if (sb < kScaleLo || sb > kScaleHi) { slow = true; sb = 127u; }
         uint2 hi, lo;
-        if (PRESPLIT) {
-          sb = (row_scales[b >> 2] >> (8 * (b & 3))) & 0xFFu;
-          if (!(g < groups && sflat >= 0)) sb = 127u;
-          if (sb == 0u) { slow = true; sb = 127u; }
-          hi = make_uint2(v[i][0], v[i][1]);
-          lo = make_uint2(v[i][2], v[i][3]);
-        } else {
-          uint32_t emax = bf16x8_max_exponent(v[i]);
-          emax = max(emax, (uint32_t)__builtin_amdgcn_mov_dpp((int)emax, 0xB1, 0xF, 0xF, true));
-          emax = max(emax, (uint32_t)__builtin_amdgcn_mov_dpp((int)emax, 0x4E, 0xF, 0xF, true));
-          sb = emax - 7u;
-          if (emax == 0u) sb = 127u;  // a block of zeros (or bf16 subnormals, taken as zero)
-          else if (sb < kScaleLo || sb > kScaleHi) { slow = true; sb = 127u; }
-          split_bf16x8(v[i], sb, hi, lo);
-        }
+        split_bf16x8(v[i], sb, hi, lo);
         const int s = b >> 2, qq = b & 3;
         const int slot = ((qq & 1) * 2 + (sd >> 1)) * 16 + sn;
         uint8_t* plane = reinterpret_cast<uint8_t*>(planes) +
@@ -937,13 +962,15 @@ __global__ __launch_bounds__(64 * kTileWaves, 2) void tile_gemm_kernel(GemmArgs 
                             (int)h1[0], (int)h1[1], (int)h1[2], (int)h1[3]};
           const i32x8 bl = {(int)l0[0], (int)l0[1], (int)l0[2], (int)l0[3],
                             (int)l1[0], (int)l1[1], (int)l1[2], (int)l1[3]};
+          // the two MFMAs of an accumulator are kept NT instructions apart
 #pragma unroll
-          for (int t = 0; t < NT; ++t) {
+          for (int t = 0; t < NT; ++t)
             acc[m][t] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wa[t], bh, acc[m][t], 4, 0,
                                                                          0, sa[t], 0, sbh);
+#pragma unroll
+          for (int t = 0; t < NT; ++t)
             acc[m][t] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wa[t], bl, acc[m][t], 4, 0,
                                                                          0, sa[t], 0, sbl);
-          }
         }
       }
     }
@@ -967,42 +994,12 @@ __global__ __launch_bounds__(64 * kTileWaves, 2) void tile_gemm_kernel(GemmArgs 
       exact_unit_global<NT>(w_rows, s_rows, a_row, K, lane, acc[m]);
     }
     if (flat >= 0) epilogue_tile<STAGE, NT>(p, e, acc[m], col0, flat, srow, lq);
-    if (STAGE == 0 && p.actq != nullptr) {
-      // The 32 act columns of this unit, as the next stage's split rows.  The
-      // lane re-reads the 8 bf16 values it has just stored; the four lanes
-      // (n, q = 0..3) of a row share the block.
-      u32x4 v = {0u, 0u, 0u, 0u};
-      if (flat >= 0) {
-        const uint16_t* arow = p.act + (size_t)srow * (size_t)p.ncols;
-        const uint2 a0 = *reinterpret_cast<const uint2*>(arow + col0[0] + 4 * lq);
-        const uint2 a1 = *reinterpret_cast<const uint2*>(arow + col0[1] + 4 * lq);
-        v = u32x4{a0.x, a0.y, a1.x, a1.y};
-      }
-      uint32_t emax = bf16x8_max_exponent(v);
-      emax = max(emax, (uint32_t)__shfl_xor((int)emax, 16));
-      emax = max(emax, (uint32_t)__shfl_xor((int)emax, 32));
-      uint32_t sb = emax - 7u, stored;
-      if (emax == 0u) sb = 127u;
-      stored = sb;
-      if (emax != 0u && (sb < kScaleLo || sb > kScaleHi)) { stored = 0u; sb = 127u; }
-      uint2 hi, lo;
-      split_bf16x8(v, sb, hi, lo);
-      if (flat >= 0) {
-        uint8_t* qrow = p.actq + (size_t)srow * (size_t)p.ncols * 2;
-#pragma unroll
-        for (int t = 0; t < 2; ++t) {
-          const int c = col0[t] + 4 * lq;  // 4 values: half of the piece c / 8
-          uint8_t* piece = qrow + (size_t)(c >> 3) * 16 + (c & 4);
-          *reinterpret_cast<uint32_t*>(piece) = t == 0 ? hi.x : hi.y;
-          *reinterpret_cast<uint32_t*>(piece + 8) = t == 0 ? lo.x : lo.y;
-        }
-        if (lq == 0) p.actqs[(size_t)srow * (size_t)(p.ncols / 32) + (col0[0] >> 5)] = (uint8_t)stored;
-      }
-    }
+    if (STAGE == 0 && p.actq != nullptr) store_split_act(p, col0[0], col0[1], flat, srow, lane);
   }
 }
 
-// bf16 rows [R, K] -> split rows (see GemmArgs::Aq).  One lane per 8 values.
+// bf16 rows [R, K] -> split rows (see GemmArgs::Aq).  One lane per 8 values; the four lanes
+// of a block of 32 are a quad (K is a multiple of 32, so no block straddles two rows).
 __global__ __launch_bounds__(256) void split_rows_kernel(const uint16_t* __restrict__ x,
                                                          uint8_t* __restrict__ xq,
                                                          uint8_t* __restrict__ xs, long long pieces,
@@ -1020,10 +1017,13 @@ __global__ __launch_bounds__(256) void split_rows_kernel(const uint16_t* __restr
   uint2 hi, lo;
   split_bf16x8(v, sb, hi, lo);
   if (i < pieces) {
-    *reinterpret_cast<u32x4*>(xq + i * 16) = u32x4{hi.x, hi.y, lo.x, lo.y};
-    if ((i & 3) == 0) xs[i >> 2] = (uint8_t)stored;  // K is a multiple of 32: blocks do not straddle rows
+    const long long row = i / (K / 8);
+    const int k = (int)(i - row * (K / 8)) * 8;
+    uint8_t* qrow = xq + row * 2 * K;
+    *reinterpret_cast<uint2*>(qrow + k) = hi;
+    *reinterpret_cast<uint2*>(qrow + K + k) = lo;
+    if ((k & 31) == 0) xs[row * split_scale_stride(K) + (k >> 5)] = (uint8_t)stored;
   }
-  (void)K;
 }
 
 int env_int(const char* name, int fallback) {
@@ -1103,14 +1103,11 @@ void launch_stage(const GemmArgs& g, const StagePlan& pl, hipStream_t stream) {
   const int units = STAGE == 0 ? g.ncols / (8 * kTileNT) : g.ncols / (16 * kTileNT);
   const int group_rows = g.block_size < 16 * kTileMT ? g.block_size : 16 * kTileMT;
   const dim3 grid((units + kTileWaves - 1) / kTileWaves, g.num_blocks * (g.block_size / group_rows));
-  if (g.Aq != nullptr && pl.variant != kMoeVariantResident)
-    hipLaunchKernelGGL((tile_gemm_kernel<STAGE, true>), grid, dim3(64 * kTileWaves), 0, stream, g);
-  else
-    hipLaunchKernelGGL((tile_gemm_kernel<STAGE, false>), grid, dim3(64 * kTileWaves), 0, stream, g);
+  hipLaunchKernelGGL((tile_gemm_kernel<STAGE>), grid, dim3(64 * kTileWaves), 0, stream, g);
 }
 
 // Workspace of the fused call: split rows of A, then of act, each followed by
-// its scale bytes (padded: the tile kernel reads 16 scale bytes at a time).
+// its scale bytes.
 struct Workspace {
   uint8_t* a_q;
   uint8_t* a_s;
@@ -1123,9 +1120,9 @@ size_t align256(size_t n) { return (n + 255) & ~(size_t)255; }
 bool carve_workspace(const FusedMoeArgs& a, Workspace& w) {
   if (a.workspace == nullptr) return false;
   const size_t aq = align256((size_t)a.M * a.hidden * 2);
-  const size_t as = align256((size_t)a.M * (a.hidden / 32) + 16);
+  const size_t as = align256((size_t)a.M * split_scale_stride(a.hidden));
   const size_t cq = align256((size_t)a.EM * a.ispp * 2);
-  const size_t cs = align256((size_t)a.EM * (a.ispp / 32) + 16);
+  const size_t cs = align256((size_t)a.EM * split_scale_stride(a.ispp));
   if (a.workspace_bytes < aq + as + cq + cs) return false;
   uint8_t* base = static_cast<uint8_t*>(a.workspace);
   if ((reinterpret_cast<uintptr_t>(base) & 15) != 0) return false;
@@ -1180,8 +1177,8 @@ GemmArgs down_args(const FusedMoeArgs& a) {
 
 size_t fused_moe_workspace_bytes(int M, int hidden, int ispp, int EM) {
   if (M <= 0 || EM <= 0 || hidden <= 0 || ispp <= 0) return 0;
-  return align256((size_t)M * hidden * 2) + align256((size_t)M * (hidden / 32) + 16) +
-         align256((size_t)EM * ispp * 2) + align256((size_t)EM * (ispp / 32) + 16);
+  return align256((size_t)M * hidden * 2) + align256((size_t)M * split_scale_stride(hidden)) +
+         align256((size_t)EM * ispp * 2) + align256((size_t)EM * split_scale_stride(ispp));
 }
 
 void launch_moe_gateup(const FusedMoeArgs& a, hipStream_t stream) {
