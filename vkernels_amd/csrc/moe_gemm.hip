@@ -1139,6 +1139,8 @@ __global__ __launch_bounds__(64 * kWsWaves) void tile_ws_kernel(GemmArgs p) {
 
 #pragma unroll 1
   for (int c = 0; c < n_chunks; ++c) {
+    // the copies of the next chunk go out first: the S load_steps below are younger
+    if (c + 1 < n_chunks) copy_chunk(c + 1);
     const u32x4* planes = ws_lds + (size_t)(c & 1) * (kWsBufferBytes / 16);
     const uint8_t* bsc = reinterpret_cast<const uint8_t*>(planes) + S * MT * 4096;
 #pragma unroll
@@ -1187,14 +1189,11 @@ __global__ __launch_bounds__(64 * kWsWaves) void tile_ws_kernel(GemmArgs p) {
         }
       }
       load_step(st[s2], step + S);  // branch-free: past the end it re-reads the last groups
-      // the copies of the next chunk go out after the first step's loads, so that at
-      // the end of the chunk exactly (S - 1) load_steps are younger than they are
-      if (s2 == 0 && c + 1 < n_chunks) copy_chunk(c + 1);
     }
-    // This wavefront's copies have landed once at most (S - 1) * kStepOps memory
+    // This wavefront's copies have landed once at most S * kStepOps memory
     // instructions are outstanding (they complete in order); a smaller count
     // only waits longer.  vmcnt is a 6-bit field split over bits 3:0 and 15:14.
-    constexpr int kKeep = (S - 1) * kStepOps - 4;
+    constexpr int kKeep = S * kStepOps - 4;
     __builtin_amdgcn_s_waitcnt((kKeep & 15) | ((kKeep >> 4) << 14) | 0x0F70);
     __builtin_amdgcn_s_barrier();  // everyone's copies of chunk c + 1 are in; chunk c's buffer is free
     __asm__ volatile("" ::: "memory");
