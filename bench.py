@@ -118,6 +118,7 @@ def main():
     logits = torch.from_numpy(logits_np).to(dev)
     out = torch.empty((T, cfg.H), dtype=torch.float32, device=dev)
     bs = args.block_size or ve.default_block_size(T)
+    prefill = T * cfg.top_k > 512  # the library's own split between its decode and tile kernels
 
     def step(i, events=None):
         fe = experts[i % n_sets]
@@ -125,9 +126,16 @@ def main():
         if events is None:
             fe.apply(A, ids, w, block_size=bs, out_fp32=out)
             return
-        # same launches, with events around the two GEMM stages
+        # same launches, with events around the two GEMM stages (decode) or around
+        # the fused call (prefill-sized batches, which run with a workspace)
         out.zero_()
         sids, eids, _, max_em = fe.align(ids, bs)
+        if prefill:
+            events[0].record()
+            events[1].record()
+            fe.fused_call(A, ids, w, sids, eids, max_em, bs, out)
+            events[2].record()
+            return
         act = fe.scratch.get(("act", fe.ispp), max_em * fe.ispp, dtype=torch.bfloat16, device=dev)
         st = ve._P(torch.cuda.current_stream().cuda_stream)
         e0, e1, e2 = events
@@ -177,7 +185,26 @@ def main():
     down_bytes = active * (H * I // 2 + H * I // 32) + 2 * T * k * I + 4 * T * H
     layer_bytes = synth.algorithmic_bytes(H, I, cfg.E, k, T, active)
     flops = synth.algorithmic_flops(H, I, k, T)
-    achieved = gate_bytes / (gate_avg * 1e-3) / 1e9
+    if prefill:
+        # events[1]..[2] bracket the whole fused call (split pass + both grouped GEMMs)
+        fused_tflops = flops / (down_avg * 1e-3) / 1e12
+        roofline = {
+            "bound": "mfma", "kernel": "vk_hip_fused_moe_mxfp4_ws (split_rows_kernel + tile_ws_kernel<0> "
+                                       "+ tile_ws_kernel<1>)",
+            "achieved": fused_tflops, "peak": FP4_PEAK_TFLOPS, "unit": "TFLOP/s",
+            "frac": fused_tflops / FP4_PEAK_TFLOPS, "traffic": None,
+            "flops_per_launch": flops, "avg_launch_us": down_avg * 1e3,
+            "median_launch_us": down_ms[len(down_ms) // 2] * 1e3,
+        }
+    else:
+        achieved = gate_bytes / (gate_avg * 1e-3) / 1e9
+        roofline = {
+            "bound": "hbm", "kernel": "stream_resident_kernel<0, ...> (gate/up grouped GEMM + SwiGLU)",
+            "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+            "frac": achieved / HBM_PEAK_GBS, "traffic": MEASURED_TRAFFIC.get(args.workload),
+            "bytes_per_launch": gate_bytes, "avg_launch_us": gate_avg * 1e3,
+            "median_launch_us": gate_ms[len(gate_ms) // 2] * 1e3,
+        }
 
     line = {
         "metric": "MoE layer tokens/s; % HBM BW roofline (decode), % FP4 MFMA peak (prefill)",
@@ -197,19 +224,13 @@ def main():
                         f"top-{k}, MXFP4 weights, bf16 activations, {cfg.logits} routing",
             "block_size": bs, "active_experts": active, "weight_sets": n_sets,
         },
-        "roofline": {
-            "bound": "hbm", "kernel": "stream_resident_kernel<0, ...> (gate/up grouped GEMM + SwiGLU)",
-            "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-            "frac": achieved / HBM_PEAK_GBS, "traffic": MEASURED_TRAFFIC.get(args.workload),
-            "bytes_per_launch": gate_bytes, "avg_launch_us": gate_avg * 1e3,
-            "median_launch_us": gate_ms[len(gate_ms) // 2] * 1e3,
-        },
+        "roofline": roofline,
         "layer": {
             "algorithmic_bytes": layer_bytes, "algorithmic_flops": flops,
             "hbm_frac_whole_step": layer_bytes / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS,
             "fp4_mfma_frac_whole_step": flops / (ms_per_step * 1e-3) / 1e12 / FP4_PEAK_TFLOPS,
-            "down_kernel_avg_us": down_avg * 1e3,
-            "down_kernel_gbs": down_bytes / (down_avg * 1e-3) / 1e9,
+            "down_kernel_avg_us": None if prefill else down_avg * 1e3,
+            "down_kernel_gbs": None if prefill else down_bytes / (down_avg * 1e-3) / 1e9,
         },
     }
     if args.copy_calibration:

@@ -7,30 +7,30 @@
 // for every sorted row r of every block whose expert_ids entry e is >= 0
 // (reference semantics: src/c/vkernels/kernels/moe_fused.cpp:235-564).
 //
-// Weight-streaming design.  The weights dominate the bytes (4.25 bits per
-// weight against a handful of activation rows per expert), so the kernels
-// are organised around reading every weight byte of an active expert once,
-// in 16-byte pieces, straight into the register layout of the MFMA operand:
+// Three kernels share the arithmetic (scaled FP4 x FP8 MFMA, see the decode
+// kernel's comment) and the work decomposition:
 //
-//   * a run = the consecutive blocks of one expert; the workgroup of the
-//     run's first block does the whole run, later blocks exit at once, so
-//     an expert's weights are streamed once however many rows it has;
+//   * a run = the consecutive blocks of one expert; padding rows (sorted id
+//     >= M*top_k) and blocks with expert id < 0 are skipped;
 //   * a wavefront owns NT weight tiles of 16 rows each (stage 0: NT/2 gate
 //     tiles and the NT/2 up tiles of the same columns, so the activation is
 //     fused; stage 1: NT consecutive tiles) and walks the whole K dimension;
-//   * weights sit on the A side of v_mfma_f32_16x16x32_bf16: lane (n, q) =
-//     (lane % 16, lane / 16) holds row n, so one global_load_dwordx4 of that
-//     lane brings the 32 codes of one scale group, enough for four MFMAs;
-//     quad q of a K step of 128 takes group 4*step + q, so a wavefront reads
-//     64 contiguous bytes of each of its 16 rows per step;
-//   * dequantisation is exact: the codes are turned into the bf16 value the
-//     reference computes (see mxfp4.hpp) and multiplied by bf16 activations
-//     with fp32 accumulation, as the reference does;
-//   * the activation rows (up to MT tiles of 16 rows per pass) are staged by
-//     the whole workgroup through LDS in MFMA-operand order, one 256-wide K
-//     chunk at a time, prefetched through registers;
+//   * weights sit on the A side of the MFMA: lane (n, q) = (lane % 16,
+//     lane / 16) holds row n, so one global_load_dwordx4 of that lane brings
+//     the 32 codes of one scale group -- the lane's whole operand for a K step
+//     of 128; quad q takes group 4*step + q, so a wavefront reads 64
+//     contiguous bytes of each of its 16 rows per step.  Weights never pass
+//     through LDS;
+//   * the activation rows are split into two E4M3 terms per block of 32 and
+//     held in LDS as MFMA operands, shared by the workgroup's wavefronts;
 //   * stage 1 adds into `out` with hardware fp32 atomics, as the ABI
 //     requires `out` to be accumulated into.
+//
+// stream_resident_kernel: decode (few rows per expert, K up to 3072): HBM
+//   bound, one workgroup per compute unit, all of K of 16 rows resident.
+// tile_ws_kernel / tile_gemm_kernel: everything else: 64 rows x 32 (16) weight
+//   tiles per workgroup, K in chunks of 512, rows pre-split in a caller-owned
+//   workspace / split in-kernel.
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 #include <stdlib.h>
@@ -44,9 +44,7 @@
 namespace vk {
 namespace {
 
-constexpr int kKStep = 128;    // K per MFMA group of four (one scale group per quad)
-constexpr int kKChunk = 256;   // K staged through LDS per barrier pair
-constexpr int kStepsPerChunk = kKChunk / kKStep;
+constexpr int kKStep = 128;    // K per MFMA step (one scale group per quad of lanes)
 
 struct GemmArgs {
   const uint16_t* A;        // stage 0: activations [M, K]; stage 1: act [EM, K]

@@ -404,6 +404,18 @@ class FusedExperts:
         if M == 0:
             return out_fp32
         sids, eids, _, max_em = self.align(topk_ids, block_size, max_tokens=max_tokens)
+        self.fused_call(hidden_states, topk_ids, topk_weights, sids, eids, max_em, block_size,
+                        out_fp32, max_tokens=max_tokens)
+        return out_fp32
+
+    def fused_call(self, hidden_states, topk_ids, topk_weights, sids, eids, max_em: int,
+                   block_size: int, out_fp32, *, max_tokens: int | None = None):
+        """The C call of apply() alone: accumulates the layer into out_fp32 for rows already
+        aligned (sids, eids, max_em from align()).  Scratch comes from self.scratch."""
+        torch = self.torch
+        M, K = hidden_states.shape
+        top_k = topk_ids.shape[1]
+        dev = hidden_states.device
         cap = _align_em_bound(max(M, max_tokens or 0), top_k, self.local_n, block_size)
         act = self.scratch.get(("act", self.ispp), max_em * self.ispp, dtype=torch.bfloat16,
                                device=dev, capacity=cap * self.ispp, name="act_scratch")
@@ -422,7 +434,6 @@ class FusedExperts:
             self.moe_ws_fn(*args, _ptr(ws), need, _stream(torch))
         else:
             self.moe_fn(*args, _stream(torch))
-        return out_fp32
 
     def forward(self, hidden_states, router_logits, top_k: int, **kw):
         """Router + layer: returns (out fp32 [M, H], topk_ids, topk_w)."""
