@@ -1,0 +1,280 @@
+"""CPU tests of the host side: the Python helpers that mirror the reference's
+`vllm_experts` module for this path (cases modelled on the reference's
+tests/python/test_vllm_experts.py), the loader rules, and the C ABI library
+itself -- that it loads without a GPU, exports every symbol the header
+declares and rejects contract violations before touching a device."""
+from __future__ import annotations
+
+import ctypes
+import os
+import re
+import tempfile
+from pathlib import Path
+
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from vkernels_amd import native_runtime
+from vkernels_amd import synth
+from vkernels_amd import vllm_experts as ve
+
+ROOT = Path(__file__).resolve().parent.parent
+
+
+# ---- pure helpers -------------------------------------------------------------
+
+def test_max_em_count_pads_to_64():
+    # reference: tests/python/test_vllm_experts.py:54-59
+    assert ve.max_em_count(1, 16, 896) == ((16 + 896 + 63) // 64) * 64
+    assert ve.max_em_count(8192, 16, 896) % 64 == 0
+    assert ve.max_em_count(0, 1, 0) == 0
+
+
+def test_max_num_tokens_hint_env(monkeypatch):
+    # reference: tests/python/test_vllm_experts.py:61-96
+    for k in ("MAX_NUM_BATCHED_TOKENS", "VLLM_MAX_NUM_BATCHED_TOKENS"):
+        monkeypatch.delenv(k, raising=False)
+    assert ve.max_num_tokens_hint() == 8192
+    monkeypatch.setenv("MAX_NUM_BATCHED_TOKENS", "12345")
+    assert ve.max_num_tokens_hint() == 12345
+    monkeypatch.setenv("MAX_NUM_BATCHED_TOKENS", "not-a-number")
+    assert ve.max_num_tokens_hint() == 8192
+
+
+def test_default_block_size():
+    assert ve.default_block_size(1) == 16 and ve.default_block_size(32) == 16
+    assert ve.default_block_size(33) == 64 and ve.default_block_size(8192) == 64
+
+
+@pytest.mark.parametrize("M,top_k,E,bs", [(1, 1, 8, 16), (4, 2, 8, 16), (64, 4, 32, 64),
+                                          (100, 8, 256, 64), (7, 6, 64, 32)])
+def test_align_with_map_matches_oracle(M, top_k, E, bs):
+    """No map, identity map and a skipping map against the oracle's alignment
+    (reference: tests/python/test_vllm_experts.py:104-175)."""
+    rng = np.random.default_rng(M * 131 + E)
+    ids = rng.integers(0, E, size=M * top_k).astype(np.int32)
+    ident = np.arange(E, dtype=np.int32)
+    skip = np.full(E, -1, dtype=np.int32)
+    owned = rng.permutation(E)[:max(1, E // 4)]
+    skip[owned] = np.arange(owned.size, dtype=np.int32)
+    for emap, local_n in ((None, E), (ident, E), (skip, owned.size)):
+        s, e, em = ve.moe_align_block_size_with_map(ids, E, bs, emap)
+        rs, re_, rem = oracle.moe_align_block_size_with_map(ids, E, bs, emap, local_n=local_n)
+        assert int(em) == rem
+        assert np.array_equal(np.asarray(s)[:rem], rs[:rem])
+        assert np.array_equal(np.asarray(e)[:rem // bs], re_[:rem // bs])
+
+
+def test_align_with_map_empty_routing_keeps_one_block():
+    # reference: tests/python/test_vllm_experts.py:159-175
+    ids = np.zeros(4, dtype=np.int32)
+    emap = np.array([-1, -1], dtype=np.int32)
+    s, e, em = ve.moe_align_block_size_with_map(ids, 2, 16, emap)
+    assert int(em) >= 16 and np.all(np.asarray(e)[:int(em) // 16] < 0)
+
+
+@pytest.mark.parametrize("kind", ["uniform", "hot", "skewed", "tp_shard", "empty"])
+def test_align_em_bound_covers_actual(kind):
+    """_align_em_bound is an upper bound of the EM the alignment produces
+    (reference: tests/python/test_vllm_experts.py:230-275)."""
+    rng = np.random.default_rng(5)
+    E, top_k, bs, M = 64, 6, 64, 300
+    ids = rng.integers(0, E, size=M * top_k).astype(np.int32)
+    emap, local_n = None, E
+    if kind == "hot":
+        ids[:] = 3
+    if kind == "skewed":
+        ids = np.minimum((rng.pareto(1.1, M * top_k) * 2).astype(np.int32), E - 1)
+    if kind == "tp_shard":
+        local_n = 16
+        emap = np.full(E, -1, dtype=np.int32)
+        emap[16:32] = np.arange(16, dtype=np.int32)
+    if kind == "empty":
+        local_n = 1
+        emap = np.full(E, -1, dtype=np.int32)
+    _, _, em = oracle.moe_align_block_size_with_map(ids, E, bs, emap, local_n=local_n)
+    bound = ve._align_em_bound(M, top_k, local_n, bs)
+    assert em <= bound and bound % bs == 0 and bound >= bs
+    assert bound == oracle.align_em_bound(M, top_k, local_n, bs)
+
+
+# ---- CaptureSafeScratch (reference: tests/python/test_vllm_experts.py:318-405) --
+
+def _cpu():
+    return torch.device("cpu")
+
+
+def test_scratch_allocates_once_at_capacity():
+    s = ve.CaptureSafeScratch()
+    a = s.get("out", 10, dtype=torch.float32, device=_cpu(), capacity=100)
+    assert a.numel() == 10
+    b = s.get("out", 60, dtype=torch.float32, device=_cpu())
+    assert b.numel() == 60 and a.data_ptr() == b.data_ptr()
+    c = s.get("other", 5, dtype=torch.float32, device=_cpu())
+    assert c.data_ptr() != a.data_ptr()
+    assert len(s.keys()) == 2
+    s.reset()
+    assert s.keys() == []
+
+
+def test_scratch_growth_refused_during_capture_only():
+    capturing = {"on": True}
+    s = ve.CaptureSafeScratch(capture_probe=lambda: capturing["on"])
+    capturing["on"] = False
+    s.get("act", 8, dtype=torch.float32, device=_cpu(), capacity=16)
+    capturing["on"] = True
+    assert s.get("act", 16, dtype=torch.float32, device=_cpu()).numel() == 16  # within capacity
+    with pytest.raises(RuntimeError):
+        s.get("act", 17, dtype=torch.float32, device=_cpu(), name="act_scratch")
+    capturing["on"] = False
+    assert s.get("act", 17, dtype=torch.float32, device=_cpu()).numel() == 17
+
+
+def test_scratch_negative_count():
+    with pytest.raises(ValueError):
+        ve.CaptureSafeScratch().get("x", -1, dtype=torch.float32, device=_cpu())
+
+
+# ---- loader (reference: native_runtime.py:10-26, tests/python/test_vllm_experts.py:281-310)
+
+def test_loader_prefers_vkernels_lib(monkeypatch):
+    with tempfile.TemporaryDirectory() as d:
+        lib = os.path.join(d, "libvkernels_hip.so")
+        Path(lib).write_bytes(b"\x7fELF")
+        monkeypatch.setenv("VKERNELS_LIB", lib)
+        assert native_runtime.find_library(("libvkernels_hip.so",)) == str(Path(lib).resolve())
+        assert ve.find_libvkernels_hip() == str(Path(lib).resolve())
+
+
+def test_loader_missing_override_is_an_error(monkeypatch):
+    # as in the reference: an override that does not exist is not silently skipped
+    monkeypatch.setenv("VKERNELS_LIB", "/definitely/not/here/libvkernels_hip.so")
+    with pytest.raises(FileNotFoundError):
+        ve.find_libvkernels_hip()
+
+
+def test_loader_search_order(monkeypatch):
+    for k in ("VKERNELS_LIB", "VKERNELS_BUILD_DIR", "K3"):
+        monkeypatch.delenv(k, raising=False)
+    assert native_runtime.find_library(("libvkernels_nope.so",)) is None
+    with tempfile.TemporaryDirectory() as d:
+        (Path(d) / "src" / "c").mkdir(parents=True)
+        (Path(d) / "home" / "pylib").mkdir(parents=True)
+        (Path(d) / "home" / "pylib" / "libvkernels_nope.so").write_bytes(b"\x7fELF")
+        monkeypatch.setenv("K3", d)
+        assert native_runtime.find_library(("libvkernels_nope.so",)).endswith("home/pylib/libvkernels_nope.so")
+        (Path(d) / "src" / "c" / "libvkernels_nope.so").write_bytes(b"\x7fELF")
+        monkeypatch.setenv("VKERNELS_BUILD_DIR", d)
+        assert native_runtime.find_library(("libvkernels_nope.so",)).endswith("src/c/libvkernels_nope.so")
+    built = ROOT / "vkernels_amd" / "libvkernels_hip.so"
+    if built.exists():  # the package directory comes first
+        assert ve.find_libvkernels_hip() == str(built.resolve())
+
+
+# ---- the C ABI library ------------------------------------------------------------
+
+@pytest.fixture(scope="module")
+def lib():
+    path = ROOT / "vkernels_amd" / "libvkernels_hip.so"
+    if not path.exists():
+        pytest.skip("libvkernels_hip.so is not built (python -m vkernels_amd.build)")
+    return ctypes.CDLL(str(path))
+
+
+def _declared_symbols():
+    text = (ROOT / "include" / "vkernels_hip.h").read_text()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(vk_\w+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol(lib):
+    names = _declared_symbols()
+    assert len(names) >= 14 and "vk_hip_fused_moe_mxfp4" in names
+    missing = [n for n in names if not hasattr(lib, n)]
+    assert not missing, f"declared in include/vkernels_hip.h but not exported: {missing}"
+
+
+def test_version_and_error_plumbing(lib):
+    lib.vk_version.restype = ctypes.c_char_p
+    lib.vk_last_error.restype = ctypes.c_char_p
+    assert lib.vk_version()
+    assert lib.vk_has_cuda() == 0
+    lib.vk_set_last_error(0, b"")
+    assert lib.vk_last_error_code() == 0 and lib.vk_last_error() == b""
+    lib.vk_set_last_error(3, b"boom")
+    assert lib.vk_last_error_code() == 3 and lib.vk_last_error() == b"boom"
+    lib.vk_set_last_error(0, b"")
+
+
+def test_max_em_matches_oracle(lib):
+    lib.vk_moe_align_block_size_max_em.restype = ctypes.c_size_t
+    lib.vk_moe_align_block_size_max_em.argtypes = [ctypes.c_int] * 4
+    for M, k, bs, E in [(1, 1, 16, 8), (64, 4, 64, 32), (8192, 8, 64, 256), (0, 2, 16, 4),
+                        (33, 6, 32, 64)]:
+        assert lib.vk_moe_align_block_size_max_em(M, k, bs, E) == oracle.align_max_em(M, k, bs, E)
+
+
+def test_workspace_bytes(lib):
+    f = lib.vk_hip_fused_moe_mxfp4_workspace_bytes
+    f.restype = ctypes.c_size_t
+    f.argtypes = [ctypes.c_int] * 4
+    assert f(0, 2880, 2880, 64) == 0 and f(64, 2880, 2880, 0) == 0
+    M, H, I, EM = 4096, 7168, 2048, 49152
+    need = f(M, H, I, EM)
+    # both split copies (2 bytes per value) and their scale rows, with alignment slack
+    floor = 2 * M * H + M * H // 32 + 2 * EM * I + EM * I // 32
+    assert floor <= need <= floor + M * 16 + EM * 16 + 4 * 256
+    assert f(M + 1, H, I, EM) > need and f(M, H, I, EM + 64) > need
+
+
+def test_entry_points_reject_contract_violations_without_a_device(lib):
+    """Argument checks run before any launch, so they can be exercised on a machine
+    without a GPU: the int-returning calls report the code, the void ones leave it in
+    vk_last_error."""
+    lib.vk_last_error.restype = ctypes.c_char_p
+    P = ctypes.c_void_p
+    align = lib.vk_hip_moe_align_block_size
+    align.restype = ctypes.c_int
+    align.argtypes = [P, P] + [ctypes.c_int] * 6 + [P] * 4
+    buf = ctypes.create_string_buffer(4096)
+    p = ctypes.cast(buf, P)
+    assert align(None, None, 4, 2, 16, 8, 8, 64, p, p, p, None) != 0          # null topk_ids
+    assert align(p, None, 4, 2, 24, 8, 8, 64, p, p, p, None) != 0             # block size not /16
+    assert align(p, None, 4, 2, 16, 8, 8, 8, p, p, p, None) != 0              # max_EM too small
+    assert lib.vk_last_error_code() != 0 and lib.vk_last_error() != b""
+    route = lib.vk_hip_moe_route_topk
+    route.restype = ctypes.c_int
+    route.argtypes = [P, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, P, P, P]
+    assert route(p, 4, 8, 9, 1, p, p, None) != 0                              # top_k > experts
+    assert route(None, 4, 8, 2, 1, p, p, None) != 0
+    moe = lib.vk_hip_fused_moe_mxfp4
+    moe.restype = None
+    moe.argtypes = ve._MOE_ARGTYPES
+    lib.vk_set_last_error(0, b"")
+    F = ctypes.c_float
+    moe(p, p, p, p, p, p, p, p, p, 4, 100, 128, 2, p, p, 64, F(0), 0, F(4), F(25), None, None,
+        16, None)                                                             # hidden not /64
+    assert lib.vk_last_error_code() != 0 and b"vk_hip_fused_moe_mxfp4" in lib.vk_last_error()
+    lib.vk_set_last_error(0, b"")
+    moe(p, p, p, p, p, p, p, p, p, 0, 128, 128, 2, p, p, 64, F(0), 0, F(4), F(25), None, None,
+        16, None)                                                             # nothing routed: no-op
+    assert lib.vk_last_error_code() == 0
+
+
+# ---- synthetic inputs ------------------------------------------------------------------
+
+def test_synth_is_deterministic_and_prefix_stable():
+    a = synth.make_activations(8, 64, 11)
+    b = synth.make_activations(16, 64, 11)
+    assert np.array_equal(a, b[:8])  # a shorter batch is a prefix of a longer one
+    w1 = synth.make_weights(2, 64, 64, 5)
+    w2 = synth.make_weights(2, 64, 64, 5)
+    assert torch.equal(w1.w13, w2.w13) and torch.equal(w1.w2_scale, w2.w2_scale)
+    codes = torch.cat([w1.w13.flatten() & 15, w1.w13.flatten() >> 4])
+    assert set(codes.tolist()) <= set(synth.FINITE_CODES)
+    assert int(w1.w13_scale.min()) >= 123 and int(w1.w13_scale.max()) <= 129
+    lg = synth.make_logits("zipf", 512, 128, 3)
+    top = np.bincount(np.argsort(-lg, axis=1)[:, :4].ravel(), minlength=128)
+    assert top.max() > 6 * np.median(top)

@@ -44,7 +44,6 @@
 namespace vk {
 namespace {
 
-constexpr int kKStep = 128;    // K per MFMA step (one scale group per quad of lanes)
 
 struct GemmArgs {
   const uint16_t* A;        // stage 0: activations [M, K]; stage 1: act [EM, K]
