@@ -228,6 +228,13 @@ constexpr uint32_t kScaleLo = 64u, kScaleHi = 190u;  // scale bytes the scaled M
 typedef __attribute__((ext_vector_type(8))) int i32x8;
 typedef __attribute__((ext_vector_type(4))) int i32x4;
 
+// Two 16-byte LDS reads as the 32-byte FP8 operand of the scaled MFMA.
+__device__ __forceinline__ i32x8 fp8_operand(u32x4 lo16, u32x4 hi16) {
+  typedef __attribute__((ext_vector_type(8))) uint32_t u32x8;
+  const u32x8 v = __builtin_shufflevector(lo16, hi16, 0, 1, 2, 3, 4, 5, 6, 7);
+  return (i32x8)v;
+}
+
 // The 32 codes of one lane as the FP4 operand of the scaled MFMA: moved onto the
 // OCP code points, in the low four of the operand's eight registers (the
 // instruction does not read the other four for FP4, so they are left undefined).
@@ -665,10 +672,8 @@ __global__ __launch_bounds__(64 * WAVES) void stream_resident_kernel(GemmArgs p)
             const int sbl = sbh - 4;
             const u32x4 h0 = b_lds[(ks * 4 + 0) * 64 + lane], h1 = b_lds[(ks * 4 + 1) * 64 + lane];
             const u32x4 l0 = b_lds[(ks * 4 + 2) * 64 + lane], l1 = b_lds[(ks * 4 + 3) * 64 + lane];
-            const i32x8 bh = {(int)h0[0], (int)h0[1], (int)h0[2], (int)h0[3],
-                              (int)h1[0], (int)h1[1], (int)h1[2], (int)h1[3]};
-            const i32x8 bl = {(int)l0[0], (int)l0[1], (int)l0[2], (int)l0[3],
-                              (int)l1[0], (int)l1[1], (int)l1[2], (int)l1[3]};
+            const i32x8 bh = fp8_operand(h0, h1);
+            const i32x8 bl = fp8_operand(l0, l1);
             i32x8 wa[NT];
 #pragma unroll
             for (int t = 0; t < NT; ++t) wa[t] = fp4_operand(sg.w[t]);
@@ -955,10 +960,8 @@ __global__ __launch_bounds__(64 * kTileWaves, 2) void tile_gemm_kernel(GemmArgs 
           const u32x4 h0 = pl[0], h1 = pl[64], l0 = pl[128], l1 = pl[192];
           const int sbh = bsc[(s * MT + m) * 64 + lane];
           const int sbl = sbh - 4;
-          const i32x8 bh = {(int)h0[0], (int)h0[1], (int)h0[2], (int)h0[3],
-                            (int)h1[0], (int)h1[1], (int)h1[2], (int)h1[3]};
-          const i32x8 bl = {(int)l0[0], (int)l0[1], (int)l0[2], (int)l0[3],
-                            (int)l1[0], (int)l1[1], (int)l1[2], (int)l1[3]};
+          const i32x8 bh = fp8_operand(h0, h1);
+          const i32x8 bl = fp8_operand(l0, l1);
           // the two MFMAs of an accumulator are kept NT instructions apart
 #pragma unroll
           for (int t = 0; t < NT; ++t)
@@ -1170,10 +1173,8 @@ __global__ __launch_bounds__(64 * kWsWaves) void tile_ws_kernel(GemmArgs p) {
           if (!in_k) sbh = 127;
           bad |= (uint32_t)(sbh == 0);
           const int sbl = sbh - 4;
-          const i32x8 bh = {(int)h0[0], (int)h0[1], (int)h0[2], (int)h0[3],
-                            (int)h1[0], (int)h1[1], (int)h1[2], (int)h1[3]};
-          const i32x8 bl = {(int)l0[0], (int)l0[1], (int)l0[2], (int)l0[3],
-                            (int)l1[0], (int)l1[1], (int)l1[2], (int)l1[3]};
+          const i32x8 bh = fp8_operand(h0, h1);
+          const i32x8 bl = fp8_operand(l0, l1);
           // the two MFMAs of an accumulator are kept NT instructions apart
 #pragma unroll
           for (int t = 0; t < NT; ++t)
