@@ -117,7 +117,7 @@ def main():
     A = torch.from_numpy(A_bits.view(np.int16)).view(torch.bfloat16).to(dev)
     logits = torch.from_numpy(logits_np).to(dev)
     out = torch.empty((T, cfg.H), dtype=torch.float32, device=dev)
-    bs = args.block_size or ve.default_block_size(T)
+    bs = args.block_size or ve.default_block_size(T, cfg.top_k)
     prefill = T * cfg.top_k > 512  # the library's own split between its decode and tile kernels
 
     def step(i, events=None):

@@ -251,34 +251,34 @@ __device__ __forceinline__ int slice_begin(int total, int i, int parts) {
   return i * q + min(i, rem);
 }
 
-// A workgroup's slice [s0, s1) of the flat (run, unit) space.  Staging the rows
-// of a run costs about as much as streaming kStagingUnits units, so when every
-// run can have workgroups of its own the slices stop at run boundaries (runs
-// get floor or ceil of grid / n_runs workgroups each) unless that unbalances
-// the workgroups by more than a second staging would cost; otherwise the space
-// is cut evenly and a slice may span runs.
+// A workgroup's slice [s0, s1) of the flat (run, unit) space.
+//
+// Streaming a run's units costs (units) x (its 16-row passes), and staging the
+// rows of a run costs about as much as streaming kStagingUnits units.  So when
+// every run can have workgroups of its own, run r gets a share of the grid
+// proportional to its passes (taken as its 16-row tiles, an upper bound that
+// is exact for block size 16) and the slices stop at run boundaries; `aligned` says whether that gives every run
+// a workgroup and does not unbalance the workgroups by more than a second
+// staging would cost.  Otherwise the space is cut evenly and a slice may span
+// runs.
 constexpr int kStagingUnits = 4;
-__device__ __forceinline__ void workgroup_slice(int n_runs, int units, int wg, int grid, int& s0,
+__device__ __forceinline__ void workgroup_slice(int n_runs, int units, int wg, int grid,
+                                                const int* run_end, bool aligned, int& s0,
                                                 int& s1) {
-  const int total = n_runs * units;
-  if (n_runs <= grid) {
-    const int q = grid / n_runs, rem = grid - q * n_runs;
-    if ((units + q - 1) / q <= (total + grid - 1) / grid + kStagingUnits) {
-      int r, j, g;
-      if (wg < rem * (q + 1)) {
-        g = q + 1;
-        r = wg / g;
-        j = wg - r * g;
-      } else {
-        g = q;
-        r = rem + (wg - rem * (q + 1)) / q;
-        j = (wg - rem * (q + 1)) - (r - rem) * q;
-      }
-      s0 = r * units + slice_begin(units, j, g);
-      s1 = r * units + slice_begin(units, j + 1, g);
-      return;
+  if (aligned) {  // run_end[r] = workgroups of the runs up to r
+    int lo = 0, hi = n_runs - 1;  // smallest r with run_end[r] > wg
+    while (lo < hi) {
+      const int mid = (lo + hi) >> 1;
+      if (run_end[mid] > wg) hi = mid;
+      else lo = mid + 1;
     }
+    const int first = lo == 0 ? 0 : run_end[lo - 1];
+    const int g = run_end[lo] - first;
+    s0 = lo * units + slice_begin(units, wg - first, g);
+    s1 = lo * units + slice_begin(units, wg - first + 1, g);
+    return;
   }
+  const int total = n_runs * units;
   s0 = slice_begin(total, wg, grid);
   s1 = slice_begin(total, wg + 1, grid);
 }
@@ -368,8 +368,9 @@ __global__ __launch_bounds__(64 * WAVES) void stream_resident_kernel(GemmArgs p)
   __shared__ int run_block0[kMaxRuns];
   __shared__ int run_block1[kMaxRuns];  // one past the last block of the run
   __shared__ int run_expert[kMaxRuns];
+  __shared__ int run_end[kMaxRuns];     // aligned slicing: workgroups of the runs up to this one
+  __shared__ int slice_sh[2];           // this workgroup's slice of the (run, unit) space
   __shared__ int first_ids[64];         // sorted ids of the first 64 rows of this workgroup's first run
-  __shared__ int n_runs_sh;
   __shared__ int pass_slow[2];          // set while staging: this pass takes the exact path
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -419,14 +420,57 @@ __global__ __launch_bounds__(64 * WAVES) void stream_resident_kernel(GemmArgs p)
     }
     n = n < kMaxRuns ? n : kMaxRuns;
     if (lane == 0) {
-      n_runs_sh = n;
       pass_slow[0] = 0;
       pass_slow[1] = 0;
     }
+    // ---- weights of the runs and this workgroup's slice ------------------------
+    // weight of a run = its 16-row tiles; run_end[r] = floor(grid * (weights up to
+    // r) / (all weights)).  Two sweeps over the runs, 64 at a time.
+    const int tiles_per_block = p.block_size / 16;
+    int total_weight = 0;
+    for (int base = 0; base < n; base += 64) {
+      const int r = base + lane;
+      int w = r < n ? (run_block1[r] - run_block0[r]) * tiles_per_block : 0;
+#pragma unroll
+      for (int d = 32; d >= 1; d >>= 1) w += __shfl_xor(w, d);
+      total_weight += w;
+    }
+    bool ok = n > 0 && n <= (int)gridDim.x;
+    if (ok) {
+      int carry = 0, worst = 0;  // worst = largest (units per workgroup) x (passes) over the runs
+      for (int base = 0; base < n; base += 64) {
+        const int r = base + lane;
+        const int w = r < n ? (run_block1[r] - run_block0[r]) * tiles_per_block : 0;
+        int x = w;
+#pragma unroll
+        for (int d = 1; d < 64; d <<= 1) {
+          const int y = __shfl_up(x, d);
+          if (lane >= d) x += y;
+        }
+        const int cum = carry + x;
+        const int end = (int)((unsigned)(gridDim.x * cum) / (unsigned)total_weight);
+        const int begin = (int)((unsigned)(gridDim.x * (cum - w)) / (unsigned)total_weight);
+        int cost = 0;
+        if (r < n) {
+          run_end[r] = end;
+          if (end > begin) cost = (units + end - begin - 1) / (end - begin) * w;
+        }
+        ok = ok && __ballot(r < n && end <= begin) == 0ull;
+#pragma unroll
+        for (int d = 32; d >= 1; d >>= 1) cost = max(cost, __shfl_xor(cost, d));
+        worst = max(worst, cost);
+        carry += __shfl(x, 63);
+      }
+      ok = ok && worst <= (units * total_weight + (int)gridDim.x - 1) / (int)gridDim.x + kStagingUnits;
+    }
+    int t0 = 0, t1 = 0;
+    if (n > 0) workgroup_slice(n, units, blockIdx.x, gridDim.x, run_end, ok, t0, t1);
+    if (lane == 0) {
+      slice_sh[0] = t0;
+      slice_sh[1] = t1;
+    }
     // The ids of the first rows this workgroup will stage, fetched once here
     // rather than by every wavefront after the barrier.
-    int t0 = 0, t1 = 0;
-    if (n > 0) workgroup_slice(n, units, blockIdx.x, gridDim.x, t0, t1);
     if (t0 < t1) {
       const int r0 = t0 / units;
       const int b0 = run_block0[r0];  // written by this wavefront, LDS operations stay in order
@@ -435,9 +479,7 @@ __global__ __launch_bounds__(64 * WAVES) void stream_resident_kernel(GemmArgs p)
     }
   }
   __syncthreads();
-  const int n_runs = n_runs_sh;
-  int s0 = 0, s1 = 0;  // n_runs * units is far below 2^31: at most kMaxRuns runs
-  if (n_runs > 0) workgroup_slice(n_runs, units, blockIdx.x, gridDim.x, s0, s1);
+  const int s0 = slice_sh[0], s1 = slice_sh[1];  // n_runs * units is far below 2^31
   if (s0 >= s1) return;  // uniform over the workgroup
   const int r_first = s0 / units;
 

@@ -294,9 +294,13 @@ def _stream(torch):
 _scratch = CaptureSafeScratch()
 
 
-def default_block_size(M: int) -> int:
+def default_block_size(M: int, top_k: int | None = None) -> int:
     """The reference's policy: 16-row alignment for decode batches, 64 above
-    (vllm_experts.py:846)."""
+    (vllm_experts.py:846).  With top_k given the split follows the library's own
+    (M * top_k <= 512 routed rows run the decode kernel, which makes a pass per 16
+    rows: blocks of 16 tell it the passes of every expert exactly and pad least)."""
+    if top_k is not None:
+        return 16 if M * top_k <= 512 else 64
     return 16 if M <= 32 else 64
 
 
@@ -390,7 +394,7 @@ class FusedExperts:
             raise ValueError(f"hidden size {K} does not match the weights ({self.hidden})")
         top_k = topk_ids.shape[1]
         dev = hidden_states.device
-        block_size = default_block_size(M) if block_size is None else block_size
+        block_size = default_block_size(M, top_k) if block_size is None else block_size
         hidden_states = hidden_states.contiguous()
         topk_ids = topk_ids.to(torch.int32).contiguous()
         if topk_weights is None:
