@@ -36,8 +36,10 @@ def _weights(cfg, seed=None, **kw):
     return _WEIGHTS[key]
 
 
-def _run_gpu(cfg, w, A_bits, logits, block_size=None, **kw):
+def _run_gpu(cfg, w, A_bits, logits, block_size=None, use_workspace=None, **kw):
     fe = ve.FusedExperts(w.w13, w.w13_scale, w.w2, w.w2_scale, scratch=ve.CaptureSafeScratch(), **kw)
+    if use_workspace is not None:
+        fe.use_workspace = use_workspace
     A = to_dev(A_bits, torch.bfloat16)
     ids, tw = fe.route(to_dev(logits), cfg.top_k, True)
     T = A.shape[0]
@@ -97,8 +99,8 @@ def _check_stagewise(cfg, T, g, A_bits, wn, tw):
 
 
 def _check(cfg, T, w, A_bits, logits, sample=None, block_size=None, weights_np=None,
-           gpu_kw=None, cpu_kw=None, seed=0, stagewise=False):
-    g = _run_gpu(cfg, w, A_bits, logits, block_size, **(gpu_kw or {}))
+           gpu_kw=None, cpu_kw=None, seed=0, stagewise=False, use_workspace=None):
+    g = _run_gpu(cfg, w, A_bits, logits, block_size, use_workspace, **(gpu_kw or {}))
     # router and alignment: bit for bit, full size
     ids, tw = oracle.route_topk(logits, cfg.top_k, True)
     assert np.array_equal(g["ids"], ids), "top-k indices differ from the oracle"
@@ -241,6 +243,31 @@ def test_block_sizes(bs):
     w = _weights(cfg, 1500)
     A, lg = _inputs(cfg, T, seed)
     _check(cfg, T, w, A, lg, block_size=bs)
+
+
+@pytest.mark.parametrize("use_workspace", [True, False])
+@pytest.mark.parametrize("bs", [16, 48, 80, 128])
+def test_tile_kernels_block_sizes(bs, use_workspace):
+    """The tile kernels (more than 512 routed rows) with and without the caller's workspace,
+    for block sizes below, above and not dividing their 64-row groups."""
+    cfg = synth.CONFIGS["c1"]
+    T, seed = 160, 1700
+    w = _weights(cfg, 1500)
+    A, lg = _inputs(cfg, T, seed)
+    _check(cfg, T, w, A, lg, sample=32, block_size=bs, use_workspace=use_workspace)
+
+
+def test_workspace_and_plain_entry_points_agree():
+    """Large K (the decode kernel does not apply) at a decode-sized batch: the workspace path
+    and the plain entry point compute the same layer."""
+    cfg = synth.CONFIGS["c4"]
+    T, seed = 24, 4100
+    w = _weights(cfg, 4100)
+    A, lg = _inputs(cfg, T, seed)
+    g1, wn = _check(cfg, T, w, A, lg, use_workspace=True)
+    g0, _ = _check(cfg, T, w, A, lg, use_workspace=False, weights_np=wn)
+    m, l2, nf = error_metrics(g1["out"], g0["out"])
+    assert nf and l2 <= 1e-4, (m, l2)
 
 
 # ---- values outside the fast path's domain ---------------------------------------

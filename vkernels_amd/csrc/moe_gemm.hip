@@ -73,6 +73,15 @@ struct GemmArgs {
   int activation;
 };
 
+// Rows a tile-kernel workgroup takes at a time: the largest multiple of 16 that
+// divides the block size and does not exceed `max_rows` (a group never spans
+// two blocks, hence never two experts).
+__host__ __device__ inline int tile_group_rows(int block_size, int max_rows) {
+  for (int rows = max_rows; rows > 16; rows -= 16)
+    if (block_size % rows == 0) return rows;
+  return 16;
+}
+
 // Bytes between the scale rows of split rows: K/32 rounded up to 16.
 __host__ __device__ inline int split_scale_stride(int K) { return (K / 32 + 15) & ~15; }
 
@@ -866,7 +875,7 @@ __global__ __launch_bounds__(64 * kTileWaves, 2) void tile_gemm_kernel(GemmArgs 
   const int units = STAGE == 0 ? p.ncols / (8 * NT) : p.ncols / (16 * NT);
 
   // ---- the rows of this group ------------------------------------------------
-  const int group_rows = min(p.block_size, 16 * MT);
+  const int group_rows = tile_group_rows(p.block_size, 16 * MT);
   const int row0 = blockIdx.y * group_rows;
   const int e = p.expert_ids[row0 / p.block_size];
   if (e < 0) return;
@@ -1080,7 +1089,7 @@ __global__ __launch_bounds__(64 * kWsWaves) void tile_ws_kernel(GemmArgs p) {
   const int sstride = split_scale_stride(K);
 
   // ---- the rows of this group ------------------------------------------------
-  const int group_rows = min(p.block_size, 16 * MT);
+  const int group_rows = tile_group_rows(p.block_size, 16 * MT);
   const int row0 = blockIdx.y * group_rows;
   const int e = p.expert_ids[row0 / p.block_size];
   if (e < 0) return;
@@ -1382,7 +1391,7 @@ void launch_stage(const GemmArgs& g, const StagePlan& pl, hipStream_t stream) {
 #undef VK_RESIDENT
   }
   const int units = STAGE == 0 ? g.ncols / (8 * kTileNT) : g.ncols / (16 * kTileNT);
-  const int group_rows = g.block_size < 16 * kTileMT ? g.block_size : 16 * kTileMT;
+  const int group_rows = tile_group_rows(g.block_size, 16 * kTileMT);
   const dim3 grid((units + kTileWaves - 1) / kTileWaves, g.num_blocks * (g.block_size / group_rows));
   if (g.Aq != nullptr && g.K >= 128) {  // the kernel reads weight scale bytes four at a time
     auto* kern = tile_ws_kernel<STAGE>;

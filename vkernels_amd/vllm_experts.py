@@ -339,9 +339,8 @@ class FusedExperts:
             raise ValueError("hidden and ispp must be multiples of 64")
         self.w13, self.w13_scale, self.w2, self.w2_scale = w13, w13_scale, w2, w2_scale
         self.b13, self.b2 = b13, b2
-        # routed rows (tokens * top_k) above which apply() hands the library a workspace;
-        # below it the decode kernel runs, which has no use for one
-        self.workspace_min_rows = 512
+        # hand the library a workspace (VKERNELS_MOE_WORKSPACE=0: the plain entry point)
+        self.use_workspace = os.environ.get("VKERNELS_MOE_WORKSPACE", "1") != "0"
         self.activation = {"swiglu": 0, "situ": 1}[activation] if isinstance(activation, str) \
             else int(activation)
         self.swiglu_limit, self.beta, self.linear_beta = swiglu_limit, beta, linear_beta
@@ -428,9 +427,10 @@ class FusedExperts:
                 _ptr(out_fp32), M, K, self.ispp, top_k, _ptr(sids), _ptr(eids), max_em,
                 float(self.swiglu_limit), self.activation, float(self.beta),
                 float(self.linear_beta), _ptr(self.b13), _ptr(self.b2), block_size)
-        if self.moe_ws_fn is not None and M * top_k > self.workspace_min_rows:
-            # prefill-sized call: the library splits the rows once, into a workspace
-            # held like the other scratch (sized once at the token budget)
+        if self.moe_ws_fn is not None and self.use_workspace:
+            # the library splits the rows once per call into this workspace where its
+            # tile kernels run (large batches, large K); held like the other scratch
+            # (sized once at the token budget)
             need = int(self.ws_bytes_fn(M, K, self.ispp, max_em))
             cap_bytes = int(self.ws_bytes_fn(max(M, max_tokens or 0), K, self.ispp, cap))
             ws = self.scratch.get(("ws", K, self.ispp), need, dtype=torch.uint8, device=dev,
