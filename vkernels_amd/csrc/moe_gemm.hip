@@ -1360,7 +1360,7 @@ struct StagePlan {
 
 template <int STAGE>
 StagePlan plan_stage(const GemmArgs& g) {
-  const MoeTile tile = pick_moe_tile(g.n_flat, g.K, g.ncols);
+  const MoeTile tile = pick_moe_tile(g.n_flat, g.K, g.ncols, STAGE);
   StagePlan pl;
   pl.variant = env_int("VK_MOE_VARIANT", tile.variant);
   pl.nt = env_int("VK_MOE_NT", tile.nt);
@@ -1386,8 +1386,13 @@ void launch_stage(const GemmArgs& g, const StagePlan& pl, hipStream_t stream) {
   if (pl.waves == W_ && pl.nt == NT_ && pl.depth == D_ && \
       launch_resident<STAGE, W_, NT_, D_>(g, pl.resident_lds, stream)) \
     return
-    VK_RESIDENT(8, 2, 2); VK_RESIDENT(8, 2, 4); VK_RESIDENT(8, 2, 6);
-    VK_RESIDENT(4, 2, 4); VK_RESIDENT(4, 2, 8);
+    if constexpr (STAGE == 0) {
+      VK_RESIDENT(8, 2, 2); VK_RESIDENT(8, 2, 4); VK_RESIDENT(8, 2, 6);
+      VK_RESIDENT(4, 2, 4); VK_RESIDENT(4, 2, 8);
+    } else {
+      VK_RESIDENT(8, 2, 4); VK_RESIDENT(8, 1, 4); VK_RESIDENT(8, 1, 6); VK_RESIDENT(8, 1, 8);
+      VK_RESIDENT(8, 1, 12);
+    }
 #undef VK_RESIDENT
   }
   const int units = STAGE == 0 ? g.ncols / (8 * kTileNT) : g.ncols / (16 * kTileNT);
