@@ -128,14 +128,14 @@ def main():
             return
         # same launches, with events around the two GEMM stages (decode) or around
         # the fused call (prefill-sized batches, which run with a workspace)
-        out.zero_()
         sids, eids, _, max_em = fe.align(ids, bs)
         if prefill:
             events[0].record()
             events[1].record()
-            fe.fused_call(A, ids, w, sids, eids, max_em, bs, out)
+            fe.fused_call(A, ids, w, sids, eids, max_em, bs, out, overwrite=True)
             events[2].record()
             return
+        out.zero_()
         act = fe.scratch.get(("act", fe.ispp), max_em * fe.ispp, dtype=torch.bfloat16, device=dev)
         st = ve._P(torch.cuda.current_stream().cuda_stream)
         e0, e1, e2 = events

@@ -137,6 +137,29 @@ void vk_hip_fused_moe_mxfp4_ws(
     void* workspace, size_t workspace_bytes, void* stream);
 
 /*
+ * Additive: vk_hip_fused_moe_mxfp4_ws with flags.  VK_HIP_MOE_OVERWRITE_OUT:
+ * `out` need not be initialised; the call clears it while its first stage runs
+ * and the result is the layer alone (saves the caller's clearing launch, which
+ * costs as much as 4 % of a decode-sized call).  Whenever M and EM are
+ * positive and the arguments valid, that is: a call that returns early leaves
+ * `out` as it is.  flags = 0 is vk_hip_fused_moe_mxfp4_ws exactly.  No
+ * counterpart in the reference.
+ */
+#define VK_HIP_MOE_OVERWRITE_OUT 1u
+
+void vk_hip_fused_moe_mxfp4_ex(
+    const uint16_t* A, const uint8_t* w13, const uint8_t* w13_scale,
+    const uint8_t* w2, const uint8_t* w2_scale,
+    const int32_t* topk_ids, const float* topk_w,
+    uint16_t* act_scratch, float* out,
+    int M, int hidden, int ispp, int top_k,
+    const int32_t* sorted_ids, const int32_t* expert_ids,
+    int EM, float swiglu_limit,
+    int activation, float beta, float linear_beta,
+    const float* b13, const float* b2, int block_size,
+    void* workspace, size_t workspace_bytes, unsigned flags, void* stream);
+
+/*
  * Additive: the two stages of vk_hip_fused_moe_mxfp4 as separate launches,
  * for callers that place work between them (a tensor-parallel all-reduce, a
  * profiler's events).  Device counterparts of the reference's stage split,

@@ -270,6 +270,31 @@ def test_workspace_and_plain_entry_points_agree():
     assert nf and l2 <= 1e-4, (m, l2)
 
 
+@pytest.mark.parametrize("T", [8, 200])
+def test_accumulate_and_overwrite(T):
+    """The ABI accumulates into `out`; VK_HIP_MOE_OVERWRITE_OUT writes it whatever it held."""
+    cfg = synth.CONFIGS["c1"]
+    w = _weights(cfg, 1500)
+    A_bits, lg = _inputs(cfg, T, 1800)
+    fe = ve.FusedExperts(w.w13, w.w13_scale, w.w2, w.w2_scale, scratch=ve.CaptureSafeScratch())
+    A = to_dev(A_bits, torch.bfloat16)
+    ids, tw = fe.route(to_dev(lg), cfg.top_k, True)
+    bs = ve.default_block_size(T, cfg.top_k)
+    sids, eids, _, max_em = fe.align(ids, bs)
+    base = torch.zeros((T, cfg.H), dtype=torch.float32, device=dev())
+    fe.fused_call(A, ids, tw, sids, eids, max_em, bs, base)
+    acc = torch.full((T, cfg.H), 3.0, dtype=torch.float32, device=dev())
+    fe.fused_call(A, ids, tw, sids, eids, max_em, bs, acc)
+    over = torch.full((T, cfg.H), float("nan"), dtype=torch.float32, device=dev())
+    fe.fused_call(A, ids, tw, sids, eids, max_em, bs, over, overwrite=True)
+    torch.cuda.synchronize()
+    b = base.cpu().numpy()
+    m, l2, nf = error_metrics(acc.cpu().numpy() - 3.0, b)
+    assert nf and l2 <= 1e-4, (m, l2)
+    m, l2, nf = error_metrics(over.cpu().numpy(), b)
+    assert nf and l2 <= 1e-4, (m, l2)
+
+
 # ---- values outside the fast path's domain ---------------------------------------
 
 def _tiny_case(seed):

@@ -104,10 +104,27 @@ void vk_hip_fused_moe_mxfp4_ws(
     int activation, float beta, float linear_beta,
     const float* b13, const float* b2, int block_size,
     void* workspace, size_t workspace_bytes, void* stream) {
+  vk_hip_fused_moe_mxfp4_ex(A, w13, w13_scale, w2, w2_scale, topk_ids, topk_w, act_scratch, out,
+                            M, hidden, ispp, top_k, sorted_ids, expert_ids, EM, swiglu_limit,
+                            activation, beta, linear_beta, b13, b2, block_size, workspace,
+                            workspace_bytes, 0u, stream);
+}
+
+void vk_hip_fused_moe_mxfp4_ex(
+    const uint16_t* A, const uint8_t* w13, const uint8_t* w13_scale,
+    const uint8_t* w2, const uint8_t* w2_scale,
+    const int32_t* topk_ids, const float* topk_w,
+    uint16_t* act_scratch, float* out,
+    int M, int hidden, int ispp, int top_k,
+    const int32_t* sorted_ids, const int32_t* expert_ids,
+    int EM, float swiglu_limit,
+    int activation, float beta, float linear_beta,
+    const float* b13, const float* b2, int block_size,
+    void* workspace, size_t workspace_bytes, unsigned flags, void* stream) {
   (void)topk_ids;
   if (M <= 0 || EM <= 0) return;  // nothing routed: out is left as it is
   vk::FusedMoeArgs a{};
-  a.workspace = workspace; a.workspace_bytes = workspace_bytes;
+  a.workspace = workspace; a.workspace_bytes = workspace_bytes; a.flags = flags;
   a.A = A; a.w13 = w13; a.w13_scale = w13_scale; a.w2 = w2; a.w2_scale = w2_scale;
   a.topk_w = topk_w; a.act = act_scratch; a.out = out;
   a.sorted_ids = sorted_ids; a.expert_ids = expert_ids; a.b13 = b13; a.b2 = b2;

@@ -62,6 +62,8 @@ struct GemmArgs {
   const uint8_t* Aq;
   const uint8_t* As;
   uint8_t* actq;            // stage 0: act written in that form as well (or null)
+  float* zero_out;          // stage 0: buffer to clear while the stage runs (or null)
+  long long zero_count;     // its floats (a multiple of 4)
   uint8_t* actqs;
   int n_flat;               // M * top_k
   int top_k;
@@ -109,6 +111,18 @@ __device__ __forceinline__ bf16x8 as_bf16x8(u32x4 v) {
   return c.b;
 }
 
+
+// Stage 0 of a call that was asked to overwrite `out`: every workgroup clears
+// its share (the stage does not use `out`; the next stage starts after this one).
+__device__ __forceinline__ void clear_out_share(const GemmArgs& p) {
+  if (p.zero_out == nullptr) return;
+  const long long n4 = p.zero_count / 4;
+  const long long wg = (long long)blockIdx.y * gridDim.x + blockIdx.x;
+  const long long wgs = (long long)gridDim.x * gridDim.y;
+  f32x4* out4 = reinterpret_cast<f32x4*>(p.zero_out);
+  for (long long i = wg * blockDim.x + threadIdx.x; i < n4; i += wgs * blockDim.x)
+    out4[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+}
 
 // Epilogue of one 16-row activation tile: acc[t][r] = C[weight row 4*lq + r of
 // tile t][activation row ln].  Stage 0 applies bias + activation to the
@@ -381,6 +395,7 @@ __global__ __launch_bounds__(64 * WAVES) void stream_resident_kernel(GemmArgs p)
   __shared__ int slice_sh[2];           // this workgroup's slice of the (run, unit) space
   __shared__ int first_ids[64];         // sorted ids of the first 64 rows of this workgroup's first run
   __shared__ int pass_slow[2];          // set while staging: this pass takes the exact path
+  if (STAGE == 0) clear_out_share(p);
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // uniform, and known to be
@@ -863,6 +878,7 @@ __global__ __launch_bounds__(64 * kTileWaves, 2) void tile_gemm_kernel(GemmArgs 
   __shared__ int row_flat[MT * 16];
   __shared__ int group_slow;
 
+  if (STAGE == 0) clear_out_share(p);
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -1075,6 +1091,7 @@ __global__ __launch_bounds__(64 * kWsWaves) void tile_ws_kernel(GemmArgs p) {
   extern __shared__ u32x4 ws_lds[];  // 2 x { planes [step][row tile][term][half][lane], scales }
   __shared__ int row_flat[MT * 16];
 
+  if (STAGE == 0) clear_out_share(p);
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -1528,6 +1545,10 @@ void launch_fused_moe(const FusedMoeArgs& a, hipStream_t stream) {
       g1.Aq = w.act_q;
       g1.As = w.act_s;
     }
+  }
+  if ((a.flags & 1u) != 0u) {  // VK_HIP_MOE_OVERWRITE_OUT
+    g0.zero_out = a.out;
+    g0.zero_count = (long long)a.M * a.hidden;
   }
   launch_stage<0>(g0, p0, stream);
   launch_stage<1>(g1, p1, stream);

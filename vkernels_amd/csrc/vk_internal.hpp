@@ -39,6 +39,7 @@ struct FusedMoeArgs {
   int activation;
   void* workspace;         // optional, see fused_moe_workspace_bytes
   size_t workspace_bytes;
+  unsigned flags;          // VK_HIP_MOE_* of vkernels_hip.h
 };
 
 // Bytes of workspace with which launch_fused_moe runs its fastest path.

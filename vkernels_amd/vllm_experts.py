@@ -245,6 +245,19 @@ def resolve_moe_ws_fn(lib):
     return fn, size_fn
 
 
+MOE_OVERWRITE_OUT = 1  # VK_HIP_MOE_OVERWRITE_OUT
+
+
+def resolve_moe_ex_fn(lib):
+    """``vk_hip_fused_moe_mxfp4_ex`` (workspace and flags) or None."""
+    fn = getattr(lib, "vk_hip_fused_moe_mxfp4_ex", None)
+    if fn is None:
+        return None
+    fn.restype = None
+    fn.argtypes = _MOE_ARGTYPES[:-1] + [_P, ctypes.c_size_t, ctypes.c_uint, _P]
+    return fn
+
+
 def resolve_align_fn(lib):
     """``vk_hip_moe_align_block_size`` or None when the symbol is absent."""
     fn = getattr(lib, "vk_hip_moe_align_block_size", None)
@@ -321,6 +334,7 @@ class FusedExperts:
         self.lib = load_libvkernels_hip()
         self.moe_fn = resolve_moe_fn(self.lib)
         self.moe_ws_fn, self.ws_bytes_fn = resolve_moe_ws_fn(self.lib)
+        self.moe_ex_fn = resolve_moe_ex_fn(self.lib)
         self.align_fn = resolve_align_fn(self.lib)
         if self.align_fn is None:
             raise RuntimeError("vk_hip_moe_align_block_size not found in libvkernels_hip.so")
@@ -403,18 +417,23 @@ class FusedExperts:
         topk_weights = topk_weights.to(torch.float32).contiguous()
         if out_fp32 is None:
             out_fp32 = torch.empty((M, K), dtype=torch.float32, device=dev)
-        out_fp32.zero_()
+        # with the flags entry point the library clears `out` inside its first stage
+        overwrite = self.moe_ex_fn is not None and self.use_workspace and M > 0
+        if not overwrite:
+            out_fp32.zero_()
         if M == 0:
             return out_fp32
         sids, eids, _, max_em = self.align(topk_ids, block_size, max_tokens=max_tokens)
         self.fused_call(hidden_states, topk_ids, topk_weights, sids, eids, max_em, block_size,
-                        out_fp32, max_tokens=max_tokens)
+                        out_fp32, max_tokens=max_tokens, overwrite=overwrite)
         return out_fp32
 
     def fused_call(self, hidden_states, topk_ids, topk_weights, sids, eids, max_em: int,
-                   block_size: int, out_fp32, *, max_tokens: int | None = None):
-        """The C call of apply() alone: accumulates the layer into out_fp32 for rows already
-        aligned (sids, eids, max_em from align()).  Scratch comes from self.scratch."""
+                   block_size: int, out_fp32, *, max_tokens: int | None = None,
+                   overwrite: bool = False):
+        """The C call of apply() alone: accumulates the layer into out_fp32 (overwrite=True:
+        writes it, whatever it held) for rows already aligned (sids, eids, max_em from
+        align()).  Scratch comes from self.scratch."""
         torch = self.torch
         M, K = hidden_states.shape
         top_k = topk_ids.shape[1]
@@ -435,7 +454,15 @@ class FusedExperts:
             cap_bytes = int(self.ws_bytes_fn(max(M, max_tokens or 0), K, self.ispp, cap))
             ws = self.scratch.get(("ws", K, self.ispp), need, dtype=torch.uint8, device=dev,
                                   capacity=cap_bytes, name="workspace")
-            self.moe_ws_fn(*args, _ptr(ws), need, _stream(torch))
+            if self.moe_ex_fn is not None:
+                self.moe_ex_fn(*args, _ptr(ws), need, MOE_OVERWRITE_OUT if overwrite else 0,
+                               _stream(torch))
+            elif overwrite:
+                raise RuntimeError("overwrite=True needs vk_hip_fused_moe_mxfp4_ex")
+            else:
+                self.moe_ws_fn(*args, _ptr(ws), need, _stream(torch))
+        elif overwrite:
+            raise RuntimeError("overwrite=True needs the workspace entry points")
         else:
             self.moe_fn(*args, _stream(torch))
 
