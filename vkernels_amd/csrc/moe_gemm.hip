@@ -56,9 +56,11 @@ struct GemmArgs {
   uint16_t* act;            // stage 0 output [EM, I]
   float* out;               // stage 1 output [M, H]
   // Optional "split rows" (workspace tile kernel): the bf16 rows of A already
-  // split into the two E4M3 terms.  Row r: 2K bytes at Aq + r*2K, the K leading
-  // parts then the K remainders (times 16); As[r*split_scale_stride(K) + g] the
-  // scale byte of block g, 0 = block outside the fast path's range.
+  // split into the two E4M3 terms.  With Kp = split_row_k(K) (K rounded up to a
+  // whole K step of 128), row r is 2 Kp bytes at Aq + r * 2 Kp: the leading parts
+  // (K of them, then zeros up to Kp), then the remainders (times 16) likewise.
+  // As[r * split_scale_stride(K) + g] is the scale byte of block g, 0 = block
+  // outside the fast path's range, 127 for the blocks between K and Kp.
   const uint8_t* Aq;
   const uint8_t* As;
   uint8_t* actq;            // stage 0: act written in that form as well (or null)
@@ -86,6 +88,9 @@ __host__ __device__ inline int tile_group_rows(int block_size, int max_rows) {
 
 // Bytes between the scale rows of split rows: K/32 rounded up to 16.
 __host__ __device__ inline int split_scale_stride(int K) { return (K / 32 + 15) & ~15; }
+
+// Values per term of a split row: K rounded up to a whole K step.
+__host__ __device__ inline int split_row_k(int K) { return (K + 127) & ~127; }
 
 __device__ __forceinline__ float act_value(int activation, float g, float u,
                                            float limit, float beta,
@@ -838,11 +843,12 @@ __device__ __forceinline__ void store_split_act(const GemmArgs& p, int c0, int c
   uint2 hi, lo;
   split_bf16x8(v, sb, hi, lo);
   if (flat >= 0) {
-    uint8_t* qrow = p.actq + (size_t)srow * (size_t)p.ncols * 2;
+    const int kp = split_row_k(p.ncols);
+    uint8_t* qrow = p.actq + (size_t)srow * (size_t)kp * 2;
     *reinterpret_cast<uint32_t*>(qrow + c0 + 4 * lq) = hi.x;
     *reinterpret_cast<uint32_t*>(qrow + c1 + 4 * lq) = hi.y;
-    *reinterpret_cast<uint32_t*>(qrow + p.ncols + c0 + 4 * lq) = lo.x;
-    *reinterpret_cast<uint32_t*>(qrow + p.ncols + c1 + 4 * lq) = lo.y;
+    *reinterpret_cast<uint32_t*>(qrow + kp + c0 + 4 * lq) = lo.x;
+    *reinterpret_cast<uint32_t*>(qrow + kp + c1 + 4 * lq) = lo.y;
     if (lq == 0)
       p.actqs[(size_t)srow * (size_t)split_scale_stride(p.ncols) + (c0 >> 5)] = (uint8_t)stored;
   }
@@ -1149,7 +1155,7 @@ __global__ __launch_bounds__(64 * kWsWaves) void tile_ws_kernel(GemmArgs p) {
     const int m = (wave & 1) * 2 + i;
     const int f = row_flat[m * 16 + ln];
     const size_t r = f >= 0 ? (size_t)(STAGE == 0 ? f / p.top_k : row0 + m * 16 + ln) : 0;
-    cp_row[i] = p.Aq + r * (size_t)(2 * K);
+    cp_row[i] = p.Aq + r * (size_t)(2 * split_row_k(K));
   }
   // scale bytes: wavefronts 0..3 copy step = wave, lane (row tile, n) = (lane / 16, lane % 16)
   const uint8_t* cp_scale;
@@ -1166,7 +1172,7 @@ __global__ __launch_bounds__(64 * kWsWaves) void tile_ws_kernel(GemmArgs p) {
       const int i = j >> 2, term = (j >> 1) & 1, h = j & 1;
       const int k = min(k0 + 64 * h + 16 * lq, K - 16);  // past K: the last piece again
       const int plane = ((cp_step * MT + (wave & 1) * 2 + i) * 2 + term) * 2 + h;
-      __builtin_amdgcn_global_load_lds(cp_row[i] + (size_t)term * K + k,
+      __builtin_amdgcn_global_load_lds(cp_row[i] + (size_t)term * split_row_k(K) + k,
                                        (lds_ptr)(buf + (size_t)plane * 1024), 16, 0, 0);
     }
     if (wave < S) {  // 4 scale bytes per (row tile, row): groups 4 step .. 4 step + 3
@@ -1305,15 +1311,382 @@ __global__ __launch_bounds__(64 * kWsWaves) void tile_ws_kernel(GemmArgs p) {
   }
 }
 
-// bf16 rows [R, K] -> split rows (see GemmArgs::Aq).  One lane per 8 values; the four lanes
-// of a block of 32 are a quad (K is a multiple of 32, so no block straddles two rows).
+// ---------------------------------------------------------------------------
+// Wide tile kernel (workspace path): up to 128 sorted rows of one expert per
+// workgroup, so that the preparation of a weight tile (code points, inf/NaN and
+// scale-range checks) is shared by 16 MFMAs and every LDS operand read by 8.
+//
+// 4 wavefronts, one per SIMD, each with the full register file: 8 row tiles x
+// 4 weight tiles of accumulators, the weights of the next 4 K steps in flight
+// in registers, and the LDS operands of the next (K step, row tile) read while
+// the MFMAs of the current one issue.
+//
+// Rows.  A workgroup takes a window of 128 sorted rows (block sizes that divide
+// 128; otherwise one group of tile_group_rows rows) and cuts it into segments
+// of consecutive blocks of one expert; each segment is one pass of the K loop.
+//
+// LDS: a ring of 4 K steps.  Per step the 8 row tiles' operand planes
+// [row tile][term][half][lane] x 16 bytes and the rows' 4 scale bytes
+// [row][group], copied from the split rows (whose zero blocks between K and the
+// next multiple of 128 make the last, partial step an ordinary one) by the DMA
+// form of the global load, 9 instructions per wavefront and step, three steps
+// ahead.  One barrier per K step: before it every wavefront waits for its own
+// copies of the NEXT step, so after it (a) that step may be read ahead and (b)
+// the slot of the previous step may be overwritten.
+// ---------------------------------------------------------------------------
+constexpr int kWideWaves = 4, kWideNT = 4, kWideMT = 8, kWideRing = 4;
+constexpr int kWideRows = 16 * kWideMT;
+constexpr int kWideStepBytes = kWideMT * 4 * 1024 + kWideRows * 4;
+constexpr int kWideLdsBytes = kWideRing * kWideStepBytes;
+
+// Sorted rows one workgroup of the wide kernel covers.
+__host__ __device__ inline int wide_window_rows(int block_size) {
+  return kWideRows % block_size == 0 ? kWideRows : tile_group_rows(block_size, kWideRows);
+}
+
+// s_waitcnt immediate that waits until at most n vector-memory operations are
+// outstanding and for nothing else (vmcnt is split over bits 3:0 and 15:14).
+constexpr int vmcnt_only(int n) { return (n & 15) | ((n >> 4) << 14) | 0x0F70; }
+
+template <int N>
+struct IntC {
+  static constexpr int value = N;
+};
+
+// The DMA form of the global load: every lane's 16 (4) bytes at `src` go to LDS
+// at byte address lds_base + 16 (4) * lane.  Written as assembly because the
+// compiler makes every later LDS read wait for all DMA loads it has emitted
+// itself, and for every register load issued along with them: a ring that is
+// filled several steps ahead needs the counted waits of the kernel instead.
+__device__ __forceinline__ void dma_load_16(const void* src, uint32_t lds_base) {
+  __asm__ volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off"
+                   :
+                   : "s"(lds_base), "v"(src)
+                   : "memory");
+}
+__device__ __forceinline__ void dma_load_4(const void* src, uint32_t lds_base) {
+  __asm__ volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, off"
+                   :
+                   : "s"(lds_base), "v"(src)
+                   : "memory");
+}
+
+// Register loads the compiler does not know to be pending (its own wait counts
+// would leave the DMA loads above out and wait for far more than needed): the
+// value must pass through wait_loaded() before its first use.
+__device__ __forceinline__ u32x4 untracked_load_16(const void* src) {
+  u32x4 v;
+  __asm__ volatile("global_load_dwordx4 %0, %1, off" : "=v"(v) : "v"(src) : "memory");
+  return v;
+}
+__device__ __forceinline__ uint32_t untracked_load_4(const void* src) {
+  uint32_t v;
+  __asm__ volatile("global_load_dword %0, %1, off" : "=v"(v) : "v"(src) : "memory");
+  return v;
+}
+
+template <int STAGE>
+__global__ __launch_bounds__(64 * kWideWaves) void tile_wide_kernel(GemmArgs p) {
+  constexpr int NT = kWideNT, MT = kWideMT, R = kWideRing;
+  typedef __attribute__((address_space(3))) void* lds_ptr;
+  extern __shared__ u32x4 wide_lds[];
+  __shared__ int row_flat[kWideRows];
+  __shared__ int wave_valid[2];
+
+  if (STAGE == 0) clear_out_share(p);
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int ln = lane & 15;
+  const int lq = lane >> 4;
+
+  const int K = p.K;
+  const int Kp = split_row_k(K);
+  const int groups = K / 32;
+  const int nsteps = Kp / 128;
+  const int units = STAGE == 0 ? p.ncols / (8 * NT) : p.ncols / (16 * NT);
+  const int sstride = split_scale_stride(K);
+  const int unit = blockIdx.x * kWideWaves + wave;
+  const bool has_unit = unit < units;
+
+  struct Stage {
+    u32x4 w[NT];
+    uint32_t sc[NT];  // the 4 scale bytes of the row for the step's 4 groups
+  };
+  struct Rows {
+    u32x4 h0, h1, l0, l1;
+    int sb;
+  };
+  constexpr int kCopyOps = 9, kLoadOps = 2 * NT;  // memory operations of copy_step, load_step
+
+  auto segment = [&](const int row0, const int n_rows, const int e) {
+    __syncthreads();  // the previous segment is done with row_flat and the ring
+    if (tid < kWideRows) {
+      int f = -1;
+      if (tid < n_rows) {
+        f = p.sorted_ids[row0 + tid];
+        if (f < 0 || f >= p.n_flat) f = -1;
+      }
+      row_flat[tid] = f;
+      const int cnt = (int)__popcll(__ballot(f >= 0));
+      if (lane == 0) wave_valid[wave] = cnt;
+    }
+    __syncthreads();
+    // routed rows are a prefix of an expert's rows (padding follows them)
+    const int n_live = (wave_valid[0] + wave_valid[1] + 15) >> 4;
+    if (n_live == 0) return;  // uniform
+
+    const uint8_t* w_rows[NT];
+    const uint8_t* s_rows[NT];
+    int col0[NT];
+    unit_tiles<STAGE, NT>(p, e, has_unit ? unit : 0, ln, w_rows, s_rows, col0);
+
+    // ---- copies: row tiles 2 wave and 2 wave + 1; the 4 scale bytes of rows 64 (wave % 2)
+    // .. + 63 (twice over, so that every wavefront issues the same number of copies) ----
+    const uint8_t* cp_row[2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      const int m = wave * 2 + i;
+      const int f = row_flat[m * 16 + ln];
+      const size_t r = f >= 0 ? (size_t)(STAGE == 0 ? f / p.top_k : row0 + m * 16 + ln) : 0;
+      cp_row[i] = p.Aq + r * (size_t)(2 * Kp) + 16 * lq;
+    }
+    const uint8_t* cp_scale;
+    {
+      const int rl = (wave & 1) * 64 + lane;
+      const int f = row_flat[rl];
+      const size_t r = f >= 0 ? (size_t)(STAGE == 0 ? f / p.top_k : row0 + rl) : 0;
+      cp_scale = p.As + r * (size_t)sstride;
+    }
+    const uint32_t ring_base = (uint32_t)(uintptr_t)(lds_ptr)wide_lds;
+    auto copy_step = [&](int step, int slot) {
+      const uint32_t buf = ring_base + (uint32_t)(slot * kWideStepBytes);
+      const int k0 = min(step, nsteps - 1) * 128;  // past the end: the last step again
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const int i = j >> 2, term = (j >> 1) & 1, h = j & 1;
+        const int plane = ((wave * 2 + i) * 2 + term) * 2 + h;
+        dma_load_16(cp_row[i] + (size_t)term * Kp + k0 + 64 * h, buf + (uint32_t)(plane * 1024));
+      }
+      dma_load_4(cp_scale + (k0 >> 5), buf + (uint32_t)(MT * 4096 + (wave & 1) * 256));
+    };
+    auto load_step = [&](Stage& st, int step) {  // branch-free: past the end, the last groups
+      const int g4 = min(step * 4, groups - 4);  // K >= 128: at least 4 groups
+      const int g = min(step * 4 + lq, groups - 1);
+#pragma unroll
+      for (int t = 0; t < NT; ++t) {
+        st.w[t] = untracked_load_16(w_rows[t] + (size_t)g * 16);
+        st.sc[t] = untracked_load_4(s_rows[t] + g4);
+      }
+    };
+    auto read_rows = [&](int slot, int m) {
+      const u32x4* planes = wide_lds + (size_t)slot * (kWideStepBytes / 16);
+      const u32x4* pl = planes + (size_t)(m * 4) * 64 + lane;
+      const uint8_t* bsc = reinterpret_cast<const uint8_t*>(planes) + MT * 4096;
+      Rows b;
+      b.h0 = pl[0];
+      b.h1 = pl[64];
+      b.l0 = pl[128];
+      b.l1 = pl[192];
+      b.sb = bsc[(m * 16 + ln) * 4 + lq];
+      return b;
+    };
+
+    f32x4 acc[MT][NT];
+#pragma unroll
+    for (int m = 0; m < MT; ++m)
+#pragma unroll
+      for (int t = 0; t < NT; ++t) acc[m][t] = f32x4{0.f, 0.f, 0.f, 0.f};
+    uint32_t bad = 0u;
+
+    // The K loop, compiled once per number of row tiles it multiplies (LIVE >= n_live:
+    // straight-line code, so that the order reads of the next tile -> MFMAs of this
+    // one survives; the tiles between n_live and LIVE are padding rows).
+    auto k_loop = [&](auto live_c) {
+      constexpr int LIVE = decltype(live_c)::value;
+      // Memory operations in program order, per K step c: the 9 copies of step c + 4,
+      // then the 8 weight loads of step c + 4.  The prologue issues steps 0 .. 3 in
+      // that order, so the counts below hold from the first step on.
+      constexpr int kStepOps = kCopyOps + kLoadOps;
+      Stage st[R];
+#pragma unroll
+      for (int j = 0; j < R; ++j) {
+        copy_step(j, j);
+        load_step(st[j], j);
+      }
+      // copies of step 0: everything issued after them may still be outstanding
+      __asm__ volatile("s_waitcnt vmcnt(%0)" ::"n"(kLoadOps + 3 * kStepOps) : "memory");
+      __builtin_amdgcn_s_barrier();
+      __asm__ volatile("" ::: "memory");
+      Rows cur = read_rows(0, 0);
+
+      auto tile_mfmas = [&](int m, const i32x8 (&wa)[NT], const int (&sa)[NT]) {
+        // (opaque, so that no use of the byte moves up into the previous tile's
+        // region and makes the MFMAs there wait for the read)
+        int sbh = cur.sb;
+        __asm__ volatile("" : "+v"(sbh));
+        bad |= (uint32_t)(sbh == 0);
+        const int sbl = sbh - 4;
+        const i32x8 bh = fp8_operand(cur.h0, cur.h1);
+        const i32x8 bl = fp8_operand(cur.l0, cur.l1);
+        // the two MFMAs of an accumulator are kept NT instructions apart
+#pragma unroll
+        for (int t = 0; t < NT; ++t)
+          acc[m][t] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wa[t], bh, acc[m][t], 4, 0, 0,
+                                                                       sa[t], 0, sbh);
+#pragma unroll
+        for (int t = 0; t < NT; ++t)
+          acc[m][t] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wa[t], bl, acc[m][t], 4, 0, 0,
+                                                                       sa[t], 0, sbl);
+      };
+
+#pragma unroll 1
+      for (int c0 = 0; c0 < nsteps; c0 += R) {
+#pragma unroll
+        for (int j = 0; j < R; ++j) {
+          // Steps past the last one (nsteps is rounded up to the ring here) only keep
+          // the sequence of memory operations, hence the counted waits, the same.
+          const int c = c0 + j;
+          const bool work = has_unit && c < nsteps;  // uniform
+          i32x8 wa[NT];
+          int sa[NT];
+          if (work) {
+            // the weights of step c: issued four steps ago, 3 steps of operations since
+#pragma unroll
+            for (int t = 0; t < NT; ++t)
+              __asm__ volatile("s_waitcnt vmcnt(%2)"
+                               : "+v"(st[j].w[t]), "+v"(st[j].sc[t])
+                               : "n"(3 * kStepOps));
+            const int g4 = min(c * 4, groups - 4);
+            const int g = min(c * 4 + lq, groups - 1);
+#pragma unroll
+            for (int t = 0; t < NT; ++t) {
+              const uint32_t sbw = (st[j].sc[t] >> (8 * (g - g4))) & 0xFFu;
+              bad |= (uint32_t)((sbw - kScaleLo) > (kScaleHi - kScaleLo));
+              const u32x4 w = st[j].w[t];
+              bad |= fp4x8_nonfinite(w[0]) | fp4x8_nonfinite(w[1]) | fp4x8_nonfinite(w[2]) |
+                     fp4x8_nonfinite(w[3]);
+              sa[t] = (int)sbw - 1;
+              wa[t] = fp4_operand(w);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int m = 0; m + 1 < LIVE; ++m) {
+              const Rows nxt = read_rows(j, m + 1);
+              __builtin_amdgcn_sched_barrier(0);
+              tile_mfmas(m, wa, sa);
+              __builtin_amdgcn_sched_barrier(0);
+              cur = nxt;
+            }
+          }
+          // Before the last tile: this wavefront's copies of step c + 1 have landed
+          // (outstanding after them: its weights, then 2 whole steps) and its reads of
+          // step c are complete; after the barrier that holds for every wavefront, so
+          // slot j takes the copies of step c + 4 and step c + 1 can be read.
+          __asm__ volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(kLoadOps + 2 * kStepOps) : "memory");
+          __builtin_amdgcn_s_barrier();
+          __asm__ volatile("" ::: "memory");
+          copy_step(c + R, j);
+          if (work) {
+            const Rows nxt = read_rows((j + 1) % R, 0);
+            __builtin_amdgcn_sched_barrier(0);
+            tile_mfmas(LIVE - 1, wa, sa);
+            __builtin_amdgcn_sched_barrier(0);
+            cur = nxt;
+          }
+          load_step(st[j], c + R);
+        }
+      }
+    };
+    if (n_live > 6) k_loop(IntC<8>{});
+    else if (n_live > 4) k_loop(IntC<6>{});
+    else if (n_live > 2) k_loop(IntC<4>{});
+    else if (n_live == 2) k_loop(IntC<2>{});
+    else k_loop(IntC<1>{});
+    // the copies past the last step land in the ring, which the epilogue reuses
+    __builtin_amdgcn_s_waitcnt(vmcnt_only(0));
+    __syncthreads();
+
+    // Stage 0: the zero blocks and scale bytes between ncols and the next multiple of
+    // 128 of the act split rows, written by the workgroups of the first columns.
+    if (STAGE == 0 && p.actq != nullptr && blockIdx.x == 0 && tid < n_rows && row_flat[tid] >= 0) {
+      const int ip = split_row_k(p.ncols);
+      uint8_t* qrow = p.actq + (size_t)(row0 + tid) * (size_t)ip * 2;
+      for (int k = p.ncols; k < ip; k += 16) {
+        *reinterpret_cast<u32x4*>(qrow + k) = u32x4{0u, 0u, 0u, 0u};
+        *reinterpret_cast<u32x4*>(qrow + ip + k) = u32x4{0u, 0u, 0u, 0u};
+      }
+      uint8_t* srow_s = p.actqs + (size_t)(row0 + tid) * (size_t)split_scale_stride(p.ncols);
+      for (int g = p.ncols / 32; g < ip / 32; ++g) srow_s[g] = 127u;
+    }
+    if (!has_unit) return;
+
+    // ---- epilogue; the exact path where the fast one was outside its domain -------
+    // (a scale byte 0 among a column's blocks marks rows outside the range: the
+    // whole unit is redone, from the bf16 rows)
+    const bool redo = __ballot(bad != 0u) != 0ull;
+#pragma unroll
+    for (int m = 0; m < MT; ++m) {
+      if (m >= n_live) break;
+      const int flat = row_flat[m * 16 + ln];
+      const int srow = row0 + m * 16 + ln;
+      if (redo) {
+        const uint16_t* a_row = nullptr;
+        if (flat >= 0) a_row = p.A + (size_t)(STAGE == 0 ? flat / p.top_k : srow) * (size_t)K;
+        exact_unit_global<NT>(w_rows, s_rows, a_row, K, lane, acc[m]);
+      }
+      if (STAGE == 0) {
+        if (flat >= 0) epilogue_tile<STAGE, NT>(p, e, acc[m], col0, flat, srow, lq);
+        if (p.actq != nullptr) store_split_act(p, col0[0], col0[1], flat, srow, lane);
+      } else {
+        // Transposed through this wavefront's part of the (now idle) ring, so
+        // that one atomic instruction adds 64 consecutive columns of one token
+        // instead of 4 x 4 scattered columns of 16 tokens.
+        constexpr int kRowStride = 16 * NT + 4;  // floats; the pad spreads the rows over the banks
+        float* tr = reinterpret_cast<float*>(wide_lds) + (size_t)wave * 16 * kRowStride;
+#pragma unroll
+        for (int t = 0; t < NT; ++t)
+          *reinterpret_cast<f32x4*>(tr + ln * kRowStride + t * 16 + 4 * lq) = acc[m][t];
+        const int c = col0[0] + lane;  // the unit's 16 NT columns are consecutive
+        const float b = p.bias != nullptr ? p.bias[(size_t)e * (size_t)p.ncols + c] : 0.0f;
+#pragma unroll 4
+        for (int i = 0; i < 16; ++i) {
+          const int fi = row_flat[m * 16 + i];  // uniform
+          if (fi < 0) continue;
+          const float v = tr[i * kRowStride + lane];
+          unsafeAtomicAdd(p.out + (size_t)(fi / p.top_k) * (size_t)p.ncols + c, (v + b) * p.topk_w[fi]);
+        }
+      }
+    }
+  };
+
+  const int total_rows = p.num_blocks * p.block_size;
+  const int win = wide_window_rows(p.block_size);
+  int row = blockIdx.y * win;
+  const int win_end = min(row + win, total_rows);
+  while (row < win_end) {  // uniform
+    const int e = p.expert_ids[row / p.block_size];
+    int seg_end = min(win_end, (row / p.block_size + 1) * p.block_size);
+    while (seg_end < win_end && p.expert_ids[seg_end / p.block_size] == e)
+      seg_end = min(win_end, seg_end + p.block_size);
+    if (e >= 0) segment(row, seg_end - row, e);
+    row = seg_end;
+  }
+}
+
+// bf16 rows [R, K] -> split rows (see GemmArgs::Aq), zero blocks between K and
+// split_row_k(K) included.  One lane per 8 values; the four lanes of a block of 32
+// are a quad (K is a multiple of 32, so no block straddles two rows or the end of K).
 __global__ __launch_bounds__(256) void split_rows_kernel(const uint16_t* __restrict__ x,
                                                          uint8_t* __restrict__ xq,
                                                          uint8_t* __restrict__ xs, long long pieces,
                                                          int K) {
+  const int kp = split_row_k(K);
   const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;  // piece index, 8 values
+  const long long row = i / (kp / 8);
+  const int k = (int)(i - row * (kp / 8)) * 8;
   u32x4 v = {0u, 0u, 0u, 0u};
-  if (i < pieces) v = *reinterpret_cast<const u32x4*>(x + i * 8);
+  if (i < pieces && k < K) v = *reinterpret_cast<const u32x4*>(x + row * K + k);
   uint32_t emax = bf16x8_max_exponent(v);
   emax = max(emax, (uint32_t)__builtin_amdgcn_mov_dpp((int)emax, 0xB1, 0xF, 0xF, true));
   emax = max(emax, (uint32_t)__builtin_amdgcn_mov_dpp((int)emax, 0x4E, 0xF, 0xF, true));
@@ -1324,11 +1697,9 @@ __global__ __launch_bounds__(256) void split_rows_kernel(const uint16_t* __restr
   uint2 hi, lo;
   split_bf16x8(v, sb, hi, lo);
   if (i < pieces) {
-    const long long row = i / (K / 8);
-    const int k = (int)(i - row * (K / 8)) * 8;
-    uint8_t* qrow = xq + row * 2 * K;
+    uint8_t* qrow = xq + row * 2 * kp;
     *reinterpret_cast<uint2*>(qrow + k) = hi;
-    *reinterpret_cast<uint2*>(qrow + K + k) = lo;
+    *reinterpret_cast<uint2*>(qrow + kp + k) = lo;
     if ((k & 31) == 0) xs[row * split_scale_stride(K) + (k >> 5)] = (uint8_t)stored;
   }
 }
@@ -1415,6 +1786,24 @@ void launch_stage(const GemmArgs& g, const StagePlan& pl, hipStream_t stream) {
   const int units = STAGE == 0 ? g.ncols / (8 * kTileNT) : g.ncols / (16 * kTileNT);
   const int group_rows = tile_group_rows(g.block_size, 16 * kTileMT);
   const dim3 grid((units + kTileWaves - 1) / kTileWaves, g.num_blocks * (g.block_size / group_rows));
+  if (g.Aq != nullptr && g.K >= 128 && env_int("VK_MOE_WIDE", 1) != 0) {
+    auto* kern = tile_wide_kernel<STAGE>;
+    static const bool configured = [kern] {
+      const hipError_t err = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                                 hipFuncAttributeMaxDynamicSharedMemorySize,
+                                                 kWideLdsBytes);
+      if (err != hipSuccess) (void)hipGetLastError();
+      return err == hipSuccess;
+    }();
+    if (configured) {
+      const int wide_units = STAGE == 0 ? g.ncols / (8 * kWideNT) : g.ncols / (16 * kWideNT);
+      const int win = wide_window_rows(g.block_size);
+      const dim3 grid_wide((wide_units + kWideWaves - 1) / kWideWaves,
+                           (g.num_blocks * g.block_size + win - 1) / win);
+      hipLaunchKernelGGL(kern, grid_wide, dim3(64 * kWideWaves), kWideLdsBytes, stream, g);
+      return;
+    }
+  }
   if (g.Aq != nullptr && g.K >= 128) {  // the kernel reads weight scale bytes four at a time
     auto* kern = tile_ws_kernel<STAGE>;
     static const bool configured = [kern] {
@@ -1447,9 +1836,9 @@ size_t align256(size_t n) { return (n + 255) & ~(size_t)255; }
 
 bool carve_workspace(const FusedMoeArgs& a, Workspace& w) {
   if (a.workspace == nullptr) return false;
-  const size_t aq = align256((size_t)a.M * a.hidden * 2);
+  const size_t aq = align256((size_t)a.M * split_row_k(a.hidden) * 2);
   const size_t as = align256((size_t)a.M * split_scale_stride(a.hidden));
-  const size_t cq = align256((size_t)a.EM * a.ispp * 2);
+  const size_t cq = align256((size_t)a.EM * split_row_k(a.ispp) * 2);
   const size_t cs = align256((size_t)a.EM * split_scale_stride(a.ispp));
   if (a.workspace_bytes < aq + as + cq + cs) return false;
   uint8_t* base = static_cast<uint8_t*>(a.workspace);
@@ -1505,8 +1894,10 @@ GemmArgs down_args(const FusedMoeArgs& a) {
 
 size_t fused_moe_workspace_bytes(int M, int hidden, int ispp, int EM) {
   if (M <= 0 || EM <= 0 || hidden <= 0 || ispp <= 0) return 0;
-  return align256((size_t)M * hidden * 2) + align256((size_t)M * split_scale_stride(hidden)) +
-         align256((size_t)EM * ispp * 2) + align256((size_t)EM * split_scale_stride(ispp));
+  return align256((size_t)M * split_row_k(hidden) * 2) +
+         align256((size_t)M * split_scale_stride(hidden)) +
+         align256((size_t)EM * split_row_k(ispp) * 2) +
+         align256((size_t)EM * split_scale_stride(ispp));
 }
 
 void launch_moe_gateup(const FusedMoeArgs& a, hipStream_t stream) {
@@ -1533,7 +1924,7 @@ void launch_fused_moe(const FusedMoeArgs& a, hipStream_t stream) {
   if (carve_workspace(a, w) && env_int("VK_MOE_PRESPLIT", 1) != 0) {
     const bool tile0 = p0.variant != kMoeVariantResident, tile1 = p1.variant != kMoeVariantResident;
     if (tile0) {
-      const long long pieces = (long long)a.M * a.hidden / 8;
+      const long long pieces = (long long)a.M * split_row_k(a.hidden) / 8;
       hipLaunchKernelGGL(split_rows_kernel, dim3((unsigned)((pieces + 255) / 256)), dim3(256), 0,
                          stream, a.A, w.a_q, w.a_s, pieces, a.hidden);
       g0.Aq = w.a_q;
