@@ -113,16 +113,19 @@ void vk_hip_fused_moe_mxfp4(
 /*
  * Additive: vk_hip_fused_moe_mxfp4 with a caller-owned device workspace, for
  * callers that can provide one (the library itself allocates nothing).  With
- * at least vk_hip_fused_moe_mxfp4_workspace_bytes(M, hidden, ispp, EM) bytes,
- * 16-byte aligned, the prefill-sized path splits the bf16 rows into their FP8
- * terms once per call instead of once per workgroup; results are the same.
+ * at least vk_hip_fused_moe_mxfp4_workspace_bytes(M, hidden, ispp, top_k, EM)
+ * bytes, 16-byte aligned, the prefill-sized path splits the bf16 rows into their
+ * FP8 terms once per call instead of once per workgroup, and its second stage
+ * stores its rows (fp32, [EM, hidden], the bulk of the workspace) for a last pass
+ * that sums each token's rows in selection order, instead of one atomic add per
+ * row and column; results agree to fp32 rounding.
  * A null or short workspace is vk_hip_fused_moe_mxfp4 exactly.  The contents
  * of the workspace are unspecified after the call; calls that share one
  * must be ordered on a stream.  No counterpart in the reference, whose Python
  * binding owns the scratch of its fused call the same way
  * (src/python/vkernels/vllm_experts.py:160-214).
  */
-size_t vk_hip_fused_moe_mxfp4_workspace_bytes(int M, int hidden, int ispp, int EM);
+size_t vk_hip_fused_moe_mxfp4_workspace_bytes(int M, int hidden, int ispp, int top_k, int EM);
 
 void vk_hip_fused_moe_mxfp4_ws(
     const uint16_t* A, const uint8_t* w13, const uint8_t* w13_scale,

@@ -89,8 +89,8 @@ void vk_hip_fused_moe_mxfp4(
                             activation, beta, linear_beta, b13, b2, block_size, nullptr, 0, stream);
 }
 
-size_t vk_hip_fused_moe_mxfp4_workspace_bytes(int M, int hidden, int ispp, int EM) {
-  return vk::fused_moe_workspace_bytes(M, hidden, ispp, EM);
+size_t vk_hip_fused_moe_mxfp4_workspace_bytes(int M, int hidden, int ispp, int top_k, int EM) {
+  return vk::fused_moe_workspace_bytes(M, hidden, ispp, top_k, EM);
 }
 
 void vk_hip_fused_moe_mxfp4_ws(

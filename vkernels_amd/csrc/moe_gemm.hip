@@ -67,6 +67,11 @@ struct GemmArgs {
   float* zero_out;          // stage 0: buffer to clear while the stage runs (or null)
   long long zero_count;     // its floats (a multiple of 4)
   uint8_t* actqs;
+  // Stage 1, optional: instead of adding into `out`, row `srow` of the sorted rows goes
+  // to y[srow, :] (bias and routing weight applied) and pos[flat] = srow; combine_kernel
+  // then sums each token's rows.
+  float* y;
+  int32_t* pos;
   int n_flat;               // M * top_k
   int top_k;
   int K;                    // hidden (stage 0) or ispp (stage 1)
@@ -133,9 +138,11 @@ __device__ __forceinline__ void clear_out_share(const GemmArgs& p) {
 // tile t][activation row ln].  Stage 0 applies bias + activation to the
 // (gate, up) pairs and stores bf16; stage 1 applies bias and the routing
 // weight and adds into `out`.
+// Stage 0 also returns what it stored: packed[t] = the 4 bf16 act values of tile pair t.
 template <int STAGE, int NT>
 __device__ __forceinline__ void epilogue_tile(const GemmArgs& p, int e, const f32x4 (&acc)[NT],
-                                              const int (&col0)[NT], int flat, int srow, int lq) {
+                                              const int (&col0)[NT], int flat, int srow, int lq,
+                                              uint2* packed_out = nullptr) {
   if (STAGE == 0) {
 #pragma unroll
     for (int t = 0; t < NT / 2; ++t) {
@@ -157,6 +164,7 @@ __device__ __forceinline__ void epilogue_tile(const GemmArgs& p, int e, const f3
       }
       *reinterpret_cast<uint2*>(p.act + (size_t)srow * (size_t)p.ncols + c) =
           make_uint2(packed[0], packed[1]);
+      if (packed_out != nullptr) packed_out[t] = make_uint2(packed[0], packed[1]);
     }
   } else {
     const float w = p.topk_w[flat];
@@ -820,19 +828,15 @@ __global__ __launch_bounds__(64 * WAVES) void stream_resident_kernel(GemmArgs p)
 
 // Stage 0 with a workspace: 32 consecutive act columns (two 16-column tiles, first
 // columns c0 and c1 = c0 + 16) of one 16-row tile as the next stage's split rows.
-// The lane re-reads the 8 bf16 values it has just stored; the four lanes
-// (n, q = 0..3) of a row share the block.  Called by whole wavefronts
-// (flat < 0 = padding row: takes part in the shuffles, stores nothing).
+// a0, a1: the lane's 4 + 4 bf16 values of the two tiles (columns c0 + 4 lq .. and
+// c1 + 4 lq ..), as epilogue_tile stored them; the four lanes (n, q = 0..3) of a row
+// share the block.  Called by whole wavefronts (flat < 0 = padding row: takes
+// part in the shuffles, stores nothing).
 __device__ __forceinline__ void store_split_act(const GemmArgs& p, int c0, int c1, int flat, int srow,
-                                                int lane) {
+                                                int lane, uint2 a0, uint2 a1) {
   const int lq = lane >> 4;
   u32x4 v = {0u, 0u, 0u, 0u};
-  if (flat >= 0) {
-    const uint16_t* arow = p.act + (size_t)srow * (size_t)p.ncols;
-    const uint2 a0 = *reinterpret_cast<const uint2*>(arow + c0 + 4 * lq);
-    const uint2 a1 = *reinterpret_cast<const uint2*>(arow + c1 + 4 * lq);
-    v = u32x4{a0.x, a0.y, a1.x, a1.y};
-  }
+  if (flat >= 0) v = u32x4{a0.x, a0.y, a1.x, a1.y};
   uint32_t emax = bf16x8_max_exponent(v);
   emax = max(emax, (uint32_t)__shfl_xor((int)emax, 16));
   emax = max(emax, (uint32_t)__shfl_xor((int)emax, 32));
@@ -1066,8 +1070,10 @@ __global__ __launch_bounds__(64 * kTileWaves, 2) void tile_gemm_kernel(GemmArgs 
       if (flat >= 0) a_row = p.A + (size_t)(STAGE == 0 ? flat / p.top_k : srow) * (size_t)K;
       exact_unit_global<NT>(w_rows, s_rows, a_row, K, lane, acc[m]);
     }
-    if (flat >= 0) epilogue_tile<STAGE, NT>(p, e, acc[m], col0, flat, srow, lq);
-    if (STAGE == 0 && p.actq != nullptr) store_split_act(p, col0[0], col0[1], flat, srow, lane);
+    uint2 packed[NT / 2] = {};
+    if (flat >= 0) epilogue_tile<STAGE, NT>(p, e, acc[m], col0, flat, srow, lq, packed);
+    if (STAGE == 0 && p.actq != nullptr)
+      store_split_act(p, col0[0], col0[1], flat, srow, lane, packed[0], packed[1]);
   }
 }
 
@@ -1287,8 +1293,10 @@ __global__ __launch_bounds__(64 * kWsWaves) void tile_ws_kernel(GemmArgs p) {
       exact_unit_global<NT>(w_rows, s_rows, a_row, K, lane, acc[m]);
     }
     if (STAGE == 0) {
-      if (flat >= 0) epilogue_tile<STAGE, NT>(p, e, acc[m], col0, flat, srow, lq);
-      if (p.actq != nullptr) store_split_act(p, col0[0], col0[1], flat, srow, lane);
+      uint2 packed[NT / 2] = {};
+      if (flat >= 0) epilogue_tile<STAGE, NT>(p, e, acc[m], col0, flat, srow, lq, packed);
+      if (p.actq != nullptr)
+        store_split_act(p, col0[0], col0[1], flat, srow, lane, packed[0], packed[1]);
     } else {
       // Transposed through this wavefront's part of the (now idle) operand
       // buffers, so that one atomic instruction adds 64 consecutive columns of
@@ -1619,6 +1627,8 @@ __global__ __launch_bounds__(64 * kWideWaves) void tile_wide_kernel(GemmArgs p) 
       uint8_t* srow_s = p.actqs + (size_t)(row0 + tid) * (size_t)split_scale_stride(p.ncols);
       for (int g = p.ncols / 32; g < ip / 32; ++g) srow_s[g] = 127u;
     }
+    if (STAGE == 1 && p.pos != nullptr && blockIdx.x == 0 && tid < n_rows && row_flat[tid] >= 0)
+      p.pos[row_flat[tid]] = row0 + tid;
     if (!has_unit) return;
 
     // ---- epilogue; the exact path where the fast one was outside its domain -------
@@ -1636,8 +1646,24 @@ __global__ __launch_bounds__(64 * kWideWaves) void tile_wide_kernel(GemmArgs p) 
         exact_unit_global<NT>(w_rows, s_rows, a_row, K, lane, acc[m]);
       }
       if (STAGE == 0) {
-        if (flat >= 0) epilogue_tile<STAGE, NT>(p, e, acc[m], col0, flat, srow, lq);
-        if (p.actq != nullptr) store_split_act(p, col0[0], col0[1], flat, srow, lane);
+        uint2 packed[NT / 2] = {};
+        if (flat >= 0) epilogue_tile<STAGE, NT>(p, e, acc[m], col0, flat, srow, lq, packed);
+        if (p.actq != nullptr)
+          store_split_act(p, col0[0], col0[1], flat, srow, lane, packed[0], packed[1]);
+      } else if (p.y != nullptr) {
+        // plain stores of the row's 4 x 4 columns; combine_kernel sums the tokens' rows
+        if (flat >= 0) {
+          const float w = p.topk_w[flat];
+          float* yrow = p.y + (size_t)srow * (size_t)p.ncols;
+#pragma unroll
+          for (int t = 0; t < NT; ++t) {
+            const int c = col0[t] + 4 * lq;
+            f32x4 v = acc[m][t];
+            if (p.bias != nullptr)
+              v += *reinterpret_cast<const f32x4*>(p.bias + (size_t)e * (size_t)p.ncols + c);
+            *reinterpret_cast<f32x4*>(yrow + c) = v * w;
+          }
+        }
       } else {
         // Transposed through this wavefront's part of the (now idle) ring, so
         // that one atomic instruction adds 64 consecutive columns of one token
@@ -1672,6 +1698,29 @@ __global__ __launch_bounds__(64 * kWideWaves) void tile_wide_kernel(GemmArgs p) 
     if (e >= 0) segment(row, seg_end - row, e);
     row = seg_end;
   }
+}
+
+__global__ __launch_bounds__(256) void fill_i32_kernel(int32_t* dst, int32_t value, int n) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) dst[i] = value;
+}
+
+// out[t, :] (+)= the sum over the token's selections s, in order, of y[pos[t * top_k + s], :]
+// (selections whose expert is not local have pos < 0).  One thread per 4 columns.
+__global__ __launch_bounds__(256) void combine_kernel(const float* __restrict__ y,
+                                                      const int32_t* __restrict__ pos,
+                                                      float* __restrict__ out, int top_k, int ncols,
+                                                      int overwrite) {
+  const int t = blockIdx.y;
+  const int c = (blockIdx.x * blockDim.x + threadIdx.x) * 4;
+  if (c >= ncols) return;
+  f32x4 sum = {0.f, 0.f, 0.f, 0.f};
+  for (int s = 0; s < top_k; ++s) {
+    const int r = pos[t * top_k + s];  // uniform
+    if (r >= 0) sum += *reinterpret_cast<const f32x4*>(y + (size_t)r * (size_t)ncols + c);
+  }
+  f32x4* o = reinterpret_cast<f32x4*>(out + (size_t)t * (size_t)ncols + c);
+  *o = overwrite ? sum : *o + sum;
 }
 
 // bf16 rows [R, K] -> split rows (see GemmArgs::Aq), zero blocks between K and
@@ -1767,6 +1816,11 @@ StagePlan plan_stage(const GemmArgs& g) {
   return pl;
 }
 
+// The wide kernel takes split rows and reads weight scale bytes four at a time.
+bool wide_kernel_applies(const GemmArgs& g) {
+  return g.Aq != nullptr && g.K >= 128 && env_int("VK_MOE_WIDE", 1) != 0;
+}
+
 template <int STAGE>
 void launch_stage(const GemmArgs& g, const StagePlan& pl, hipStream_t stream) {
   if (pl.variant == kMoeVariantResident) {
@@ -1786,7 +1840,7 @@ void launch_stage(const GemmArgs& g, const StagePlan& pl, hipStream_t stream) {
   const int units = STAGE == 0 ? g.ncols / (8 * kTileNT) : g.ncols / (16 * kTileNT);
   const int group_rows = tile_group_rows(g.block_size, 16 * kTileMT);
   const dim3 grid((units + kTileWaves - 1) / kTileWaves, g.num_blocks * (g.block_size / group_rows));
-  if (g.Aq != nullptr && g.K >= 128 && env_int("VK_MOE_WIDE", 1) != 0) {
+  if (wide_kernel_applies(g)) {
     auto* kern = tile_wide_kernel<STAGE>;
     static const bool configured = [kern] {
       const hipError_t err = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
@@ -1824,29 +1878,47 @@ void launch_stage(const GemmArgs& g, const StagePlan& pl, hipStream_t stream) {
 }
 
 // Workspace of the fused call: split rows of A, then of act, each followed by
-// its scale bytes.
+// its scale bytes; then the second stage's rows before the combine (fp32,
+// [EM, hidden]) and the sorted position of every flat index.
 struct Workspace {
   uint8_t* a_q;
   uint8_t* a_s;
   uint8_t* act_q;
   uint8_t* act_s;
+  float* y;
+  int32_t* pos;
+};
+
+struct WorkspaceLayout {
+  size_t aq, as, cq, cs, y, pos;
+  size_t total() const { return aq + as + cq + cs + y + pos; }
 };
 
 size_t align256(size_t n) { return (n + 255) & ~(size_t)255; }
 
+WorkspaceLayout workspace_layout(int M, int hidden, int ispp, int top_k, int EM) {
+  WorkspaceLayout l;
+  l.aq = align256((size_t)M * split_row_k(hidden) * 2);
+  l.as = align256((size_t)M * split_scale_stride(hidden));
+  l.cq = align256((size_t)EM * split_row_k(ispp) * 2);
+  l.cs = align256((size_t)EM * split_scale_stride(ispp));
+  l.y = align256((size_t)EM * hidden * sizeof(float));
+  l.pos = align256((size_t)M * top_k * sizeof(int32_t));
+  return l;
+}
+
 bool carve_workspace(const FusedMoeArgs& a, Workspace& w) {
   if (a.workspace == nullptr) return false;
-  const size_t aq = align256((size_t)a.M * split_row_k(a.hidden) * 2);
-  const size_t as = align256((size_t)a.M * split_scale_stride(a.hidden));
-  const size_t cq = align256((size_t)a.EM * split_row_k(a.ispp) * 2);
-  const size_t cs = align256((size_t)a.EM * split_scale_stride(a.ispp));
-  if (a.workspace_bytes < aq + as + cq + cs) return false;
+  const WorkspaceLayout l = workspace_layout(a.M, a.hidden, a.ispp, a.top_k, a.EM);
+  if (a.workspace_bytes < l.total()) return false;
   uint8_t* base = static_cast<uint8_t*>(a.workspace);
   if ((reinterpret_cast<uintptr_t>(base) & 15) != 0) return false;
   w.a_q = base;
-  w.a_s = base + aq;
-  w.act_q = base + aq + as;
-  w.act_s = base + aq + as + cq;
+  w.a_s = w.a_q + l.aq;
+  w.act_q = w.a_s + l.as;
+  w.act_s = w.act_q + l.cq;
+  w.y = reinterpret_cast<float*>(w.act_s + l.cs);
+  w.pos = reinterpret_cast<int32_t*>(w.act_s + l.cs + l.y);
   return true;
 }
 
@@ -1892,12 +1964,9 @@ GemmArgs down_args(const FusedMoeArgs& a) {
 
 }  // namespace
 
-size_t fused_moe_workspace_bytes(int M, int hidden, int ispp, int EM) {
-  if (M <= 0 || EM <= 0 || hidden <= 0 || ispp <= 0) return 0;
-  return align256((size_t)M * split_row_k(hidden) * 2) +
-         align256((size_t)M * split_scale_stride(hidden)) +
-         align256((size_t)EM * split_row_k(ispp) * 2) +
-         align256((size_t)EM * split_scale_stride(ispp));
+size_t fused_moe_workspace_bytes(int M, int hidden, int ispp, int top_k, int EM) {
+  if (M <= 0 || EM <= 0 || hidden <= 0 || ispp <= 0 || top_k <= 0) return 0;
+  return workspace_layout(M, hidden, ispp, top_k, EM).total();
 }
 
 void launch_moe_gateup(const FusedMoeArgs& a, hipStream_t stream) {
@@ -1921,6 +1990,7 @@ void launch_fused_moe(const FusedMoeArgs& a, hipStream_t stream) {
   GemmArgs g1 = down_args(a);
   const StagePlan p0 = plan_stage<0>(g0), p1 = plan_stage<1>(g1);
   Workspace w;
+  bool combine = false;
   if (carve_workspace(a, w) && env_int("VK_MOE_PRESPLIT", 1) != 0) {
     const bool tile0 = p0.variant != kMoeVariantResident, tile1 = p1.variant != kMoeVariantResident;
     if (tile0) {
@@ -1935,14 +2005,30 @@ void launch_fused_moe(const FusedMoeArgs& a, hipStream_t stream) {
       g0.actqs = w.act_s;
       g1.Aq = w.act_q;
       g1.As = w.act_s;
+      // The second stage stores its rows and a last pass sums them per token (the
+      // wide kernel only; far cheaper than one atomic per row and column).
+      if (wide_kernel_applies(g1) && env_int("VK_MOE_COMBINE", 1) != 0) {
+        combine = true;
+        g1.y = w.y;
+        g1.pos = w.pos;
+        const int n = a.M * a.top_k;
+        hipLaunchKernelGGL(fill_i32_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream,
+                           w.pos, -1, n);
+      }
     }
   }
-  if ((a.flags & 1u) != 0u) {  // VK_HIP_MOE_OVERWRITE_OUT
+  const bool overwrite = (a.flags & 1u) != 0u;  // VK_HIP_MOE_OVERWRITE_OUT
+  if (overwrite && !combine) {
     g0.zero_out = a.out;
     g0.zero_count = (long long)a.M * a.hidden;
   }
   launch_stage<0>(g0, p0, stream);
   launch_stage<1>(g1, p1, stream);
+  if (combine) {
+    const dim3 grid((unsigned)((a.hidden / 4 + 255) / 256), (unsigned)a.M);
+    hipLaunchKernelGGL(combine_kernel, grid, dim3(256), 0, stream, w.y, w.pos, a.out, a.top_k,
+                       a.hidden, overwrite ? 1 : 0);
+  }
 }
 
 }  // namespace vk

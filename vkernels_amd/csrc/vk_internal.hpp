@@ -43,7 +43,7 @@ struct FusedMoeArgs {
 };
 
 // Bytes of workspace with which launch_fused_moe runs its fastest path.
-size_t fused_moe_workspace_bytes(int M, int hidden, int ispp, int EM);
+size_t fused_moe_workspace_bytes(int M, int hidden, int ispp, int top_k, int EM);
 
 void launch_fused_moe(const FusedMoeArgs& a, hipStream_t stream);
 void launch_moe_gateup(const FusedMoeArgs& a, hipStream_t stream);

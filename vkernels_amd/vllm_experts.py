@@ -241,7 +241,7 @@ def resolve_moe_ws_fn(lib):
     fn.restype = None
     fn.argtypes = _MOE_ARGTYPES[:-1] + [_P, ctypes.c_size_t, _P]
     size_fn.restype = ctypes.c_size_t
-    size_fn.argtypes = [_I, _I, _I, _I]
+    size_fn.argtypes = [_I, _I, _I, _I, _I]
     return fn, size_fn
 
 
@@ -450,8 +450,8 @@ class FusedExperts:
             # the library splits the rows once per call into this workspace where its
             # tile kernels run (large batches, large K); held like the other scratch
             # (sized once at the token budget)
-            need = int(self.ws_bytes_fn(M, K, self.ispp, max_em))
-            cap_bytes = int(self.ws_bytes_fn(max(M, max_tokens or 0), K, self.ispp, cap))
+            need = int(self.ws_bytes_fn(M, K, self.ispp, top_k, max_em))
+            cap_bytes = int(self.ws_bytes_fn(max(M, max_tokens or 0), K, self.ispp, top_k, cap))
             ws = self.scratch.get(("ws", K, self.ispp), need, dtype=torch.uint8, device=dev,
                                   capacity=cap_bytes, name="workspace")
             if self.moe_ex_fn is not None:
