@@ -1344,8 +1344,8 @@ __global__ __launch_bounds__(64 * kWsWaves) void tile_ws_kernel(GemmArgs p) {
 // ---------------------------------------------------------------------------
 constexpr int kWideWaves = 4, kWideNT = 4, kWideMT = 8, kWideRing = 4;
 constexpr int kWideRows = 16 * kWideMT;
-constexpr int kWideStepBytes = kWideMT * 4 * 1024 + kWideRows * 4;
-constexpr int kWideLdsBytes = kWideRing * kWideStepBytes;
+constexpr int kWideStepBytes = kWideMT * 4 * 1024;
+constexpr int kWideLdsBytes = kWideRing * kWideStepBytes + 2 * kWideRows * 16;  // + two scale slots
 
 // Sorted rows one workgroup of the wide kernel covers.
 __host__ __device__ inline int wide_window_rows(int block_size) {
@@ -1379,20 +1379,6 @@ __device__ __forceinline__ void dma_load_4(const void* src, uint32_t lds_base) {
                    : "memory");
 }
 
-// Register loads the compiler does not know to be pending (its own wait counts
-// would leave the DMA loads above out and wait for far more than needed): the
-// value must pass through wait_loaded() before its first use.
-__device__ __forceinline__ u32x4 untracked_load_16(const void* src) {
-  u32x4 v;
-  __asm__ volatile("global_load_dwordx4 %0, %1, off" : "=v"(v) : "v"(src) : "memory");
-  return v;
-}
-__device__ __forceinline__ uint32_t untracked_load_4(const void* src) {
-  uint32_t v;
-  __asm__ volatile("global_load_dword %0, %1, off" : "=v"(v) : "v"(src) : "memory");
-  return v;
-}
-
 template <int STAGE>
 __global__ __launch_bounds__(64 * kWideWaves) void tile_wide_kernel(GemmArgs p) {
   constexpr int NT = kWideNT, MT = kWideMT, R = kWideRing;
@@ -1417,15 +1403,16 @@ __global__ __launch_bounds__(64 * kWideWaves) void tile_wide_kernel(GemmArgs p) 
   const int unit = blockIdx.x * kWideWaves + wave;
   const bool has_unit = unit < units;
 
-  struct Stage {
-    u32x4 w[NT];
-    uint32_t sc[NT];  // the 4 scale bytes of the row for the step's 4 groups
-  };
   struct Rows {
     u32x4 h0, h1, l0, l1;
     int sb;
   };
-  constexpr int kCopyOps = 9, kLoadOps = 2 * NT;  // memory operations of copy_step, load_step
+  // Memory operations per K step, in program order: the 8 row copies, the copy of
+  // the rows' scale bytes (every 4th step, for the next 4), the 4 weight loads,
+  // the 4 loads of the weights' scale bytes (every 4th step, for the next 4).
+  constexpr int kCopyOps = 8, kLoadOps = NT;
+  constexpr int kOpsStep0 = kCopyOps + 1 + 2 * kLoadOps, kOpsStep = kCopyOps + kLoadOps;
+  constexpr int kOpsCycle = kOpsStep0 + 3 * kOpsStep;
 
   auto segment = [&](const int row0, const int n_rows, const int e) {
     __syncthreads();  // the previous segment is done with row_flat and the ring
@@ -1449,16 +1436,25 @@ __global__ __launch_bounds__(64 * kWideWaves) void tile_wide_kernel(GemmArgs p) 
     int col0[NT];
     unit_tiles<STAGE, NT>(p, e, has_unit ? unit : 0, ln, w_rows, s_rows, col0);
 
-    // ---- copies: row tiles 2 wave and 2 wave + 1; the 4 scale bytes of rows 64 (wave % 2)
-    // .. + 63 (twice over, so that every wavefront issues the same number of copies) ----
-    const uint8_t* cp_row[2];
+    // ---- copies.  One copy instruction moves 8 rows x 128 bytes (one K step of one
+    // term): whole cache lines, which the memory pipe serves three times as fast as
+    // 64-byte pieces of 16 rows.  Lane (r, j) = (lane / 8, lane % 8) copies piece
+    // j ^ r of row r, so that the 16-byte pieces of a row sit in LDS rotated by the
+    // row and the MFMA operand reads (16 rows, one piece each) spread over the banks.
+    // Wavefront w copies row tiles 2 w and 2 w + 1.
+    const int cr = lane >> 3, cj = lane & 7;
+    const uint8_t* cp_row[2][2];
 #pragma unroll
-    for (int i = 0; i < 2; ++i) {
-      const int m = wave * 2 + i;
-      const int f = row_flat[m * 16 + ln];
-      const size_t r = f >= 0 ? (size_t)(STAGE == 0 ? f / p.top_k : row0 + m * 16 + ln) : 0;
-      cp_row[i] = p.Aq + r * (size_t)(2 * Kp) + 16 * lq;
-    }
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+      for (int rh = 0; rh < 2; ++rh) {
+        const int rl = (wave * 2 + i) * 16 + rh * 8 + cr;
+        const int f = row_flat[rl];
+        const size_t r = f >= 0 ? (size_t)(STAGE == 0 ? f / p.top_k : row0 + rl) : 0;
+        cp_row[i][rh] = p.Aq + r * (size_t)(2 * Kp) + 16 * (cj ^ cr);
+      }
+    // scale bytes: 16 per row = 4 K steps; rows 64 (wave % 2) .. + 63 (twice over, so
+    // that every wavefront issues the same number of copies)
     const uint8_t* cp_scale;
     {
       const int rl = (wave & 1) * 64 + lane;
@@ -1472,31 +1468,41 @@ __global__ __launch_bounds__(64 * kWideWaves) void tile_wide_kernel(GemmArgs p) 
       const int k0 = min(step, nsteps - 1) * 128;  // past the end: the last step again
 #pragma unroll
       for (int j = 0; j < 8; ++j) {
-        const int i = j >> 2, term = (j >> 1) & 1, h = j & 1;
-        const int plane = ((wave * 2 + i) * 2 + term) * 2 + h;
-        dma_load_16(cp_row[i] + (size_t)term * Kp + k0 + 64 * h, buf + (uint32_t)(plane * 1024));
+        const int i = j >> 2, term = (j >> 1) & 1, rh = j & 1;
+        const int plane = ((wave * 2 + i) * 2 + term) * 2 + rh;
+        dma_load_16(cp_row[i][rh] + (size_t)term * Kp + k0, buf + (uint32_t)(plane * 1024));
       }
-      dma_load_4(cp_scale + (k0 >> 5), buf + (uint32_t)(MT * 4096 + (wave & 1) * 256));
     };
-    auto load_step = [&](Stage& st, int step) {  // branch-free: past the end, the last groups
-      const int g4 = min(step * 4, groups - 4);  // K >= 128: at least 4 groups
+    auto copy_scales = [&](int group) {  // the rows' scale bytes of K steps 4 group .. + 3
+      const int g = min(group * 16, sstride - 16);
+      dma_load_16(cp_scale + g, ring_base + (uint32_t)(R * kWideStepBytes + (group & 1) * 2048 +
+                                                      (wave & 1) * 1024));
+    };
+    auto load_step = [&](u32x4 (&w)[NT], int step) {  // branch-free: past the end, the last group
       const int g = min(step * 4 + lq, groups - 1);
 #pragma unroll
-      for (int t = 0; t < NT; ++t) {
-        st.w[t] = untracked_load_16(w_rows[t] + (size_t)g * 16);
-        st.sc[t] = untracked_load_4(s_rows[t] + g4);
-      }
+      for (int t = 0; t < NT; ++t) w[t] = *reinterpret_cast<const u32x4*>(w_rows[t] + (size_t)g * 16);
     };
-    auto read_rows = [&](int slot, int m) {
-      const u32x4* planes = wide_lds + (size_t)slot * (kWideStepBytes / 16);
-      const u32x4* pl = planes + (size_t)(m * 4) * 64 + lane;
-      const uint8_t* bsc = reinterpret_cast<const uint8_t*>(planes) + MT * 4096;
+    // the 16 scale bytes of the lane's weight rows for K steps 4 group .. + 3; the last
+    // group of a K that is no multiple of 512 starts early (see weight_scale)
+    auto load_scales = [&](u32x4 (&sc)[NT], int group) {
+      const int g = min(group * 16, groups - 16);
+#pragma unroll
+      for (int t = 0; t < NT; ++t) sc[t] = *reinterpret_cast<const u32x4*>(s_rows[t] + g);
+    };
+    // operand reads of row tile m of a slot: lane (n, q) takes piece q (q + 4) of row n
+    const int rd0 = (ln >> 3) * 1024 + (ln & 7) * 128 + ((lq ^ (ln & 7)) * 16);
+    const int rd1 = rd0 ^ 64;
+    const uint8_t* ring_bytes = reinterpret_cast<const uint8_t*>(wide_lds);
+    auto read_rows = [&](int slot, int m, int step) {
+      const uint8_t* tile = ring_bytes + slot * kWideStepBytes + m * 4096;
       Rows b;
-      b.h0 = pl[0];
-      b.h1 = pl[64];
-      b.l0 = pl[128];
-      b.l1 = pl[192];
-      b.sb = bsc[(m * 16 + ln) * 4 + lq];
+      b.h0 = *reinterpret_cast<const u32x4*>(tile + rd0);
+      b.h1 = *reinterpret_cast<const u32x4*>(tile + rd1);
+      b.l0 = *reinterpret_cast<const u32x4*>(tile + 2048 + rd0);
+      b.l1 = *reinterpret_cast<const u32x4*>(tile + 2048 + rd1);
+      b.sb = ring_bytes[R * kWideStepBytes + ((step >> 2) & 1) * 2048 + (m * 16 + ln) * 16 +
+                        (step & 3) * 4 + lq];
       return b;
     };
 
@@ -1512,21 +1518,23 @@ __global__ __launch_bounds__(64 * kWideWaves) void tile_wide_kernel(GemmArgs p) 
     // one survives; the tiles between n_live and LIVE are padding rows).
     auto k_loop = [&](auto live_c) {
       constexpr int LIVE = decltype(live_c)::value;
-      // Memory operations in program order, per K step c: the 9 copies of step c + 4,
-      // then the 8 weight loads of step c + 4.  The prologue issues steps 0 .. 3 in
-      // that order, so the counts below hold from the first step on.
-      constexpr int kStepOps = kCopyOps + kLoadOps;
-      Stage st[R];
+      u32x4 st[R][NT];
+      u32x4 sc_cur[NT], sc_nxt[NT];
+      // The prologue issues steps 0 .. 3 in the order of the loop, so the counts
+      // below hold from the first step on.
 #pragma unroll
       for (int j = 0; j < R; ++j) {
         copy_step(j, j);
+        if (j == 0) copy_scales(0);
         load_step(st[j], j);
+        if (j == 0) load_scales(sc_nxt, 0);
       }
-      // copies of step 0: everything issued after them may still be outstanding
-      __asm__ volatile("s_waitcnt vmcnt(%0)" ::"n"(kLoadOps + 3 * kStepOps) : "memory");
+      // copies of step 0 and of the first scale bytes: all that was issued after them
+      // may still be outstanding
+      __asm__ volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * kLoadOps + 3 * kOpsStep) : "memory");
       __builtin_amdgcn_s_barrier();
       __asm__ volatile("" ::: "memory");
-      Rows cur = read_rows(0, 0);
+      Rows cur = read_rows(0, 0, 0);
 
       auto tile_mfmas = [&](int m, const i32x8 (&wa)[NT], const int (&sa)[NT]) {
         // (opaque, so that no use of the byte moves up into the previous tile's
@@ -1550,28 +1558,37 @@ __global__ __launch_bounds__(64 * kWideWaves) void tile_wide_kernel(GemmArgs p) 
 
 #pragma unroll 1
       for (int c0 = 0; c0 < nsteps; c0 += R) {
-#pragma unroll
-        for (int j = 0; j < R; ++j) {
+        // only the last group of 4 steps can start early (K no multiple of 512)
+        const int sc_shift = c0 * 4 - min(c0 * 4, groups - 16);  // uniform
+        auto step = [&](auto j_c) {
+          constexpr int j = decltype(j_c)::value;
           // Steps past the last one (nsteps is rounded up to the ring here) only keep
           // the sequence of memory operations, hence the counted waits, the same.
           const int c = c0 + j;
           const bool work = has_unit && c < nsteps;  // uniform
+          // The weights of step c (and, first step of four, their scale bytes) were
+          // issued four steps ago.  The compiler waits for them itself; its count
+          // leaves the copies out, so it also waits for the copies of two steps ago.
+          if (j == 0) {
+#pragma unroll
+            for (int t = 0; t < NT; ++t) sc_cur[t] = sc_nxt[t];
+          }
           i32x8 wa[NT];
           int sa[NT];
           if (work) {
-            // the weights of step c: issued four steps ago, 3 steps of operations since
-#pragma unroll
-            for (int t = 0; t < NT; ++t)
-              __asm__ volatile("s_waitcnt vmcnt(%2)"
-                               : "+v"(st[j].w[t]), "+v"(st[j].sc[t])
-                               : "n"(3 * kStepOps));
-            const int g4 = min(c * 4, groups - 4);
-            const int g = min(c * 4 + lq, groups - 1);
+            const int gi = min(c * 4 + lq, groups - 1) - c0 * 4 + sc_shift;  // byte of the 16
 #pragma unroll
             for (int t = 0; t < NT; ++t) {
-              const uint32_t sbw = (st[j].sc[t] >> (8 * (g - g4))) & 0xFFu;
+              uint32_t sbw;
+              if (sc_shift == 0) {  // uniform; the byte is in dword j
+                sbw = (sc_cur[t][j] >> (8 * lq)) & 0xFFu;
+              } else {
+                const uint32_t lo = (gi & 4) ? sc_cur[t][1] : sc_cur[t][0];
+                const uint32_t hi = (gi & 4) ? sc_cur[t][3] : sc_cur[t][2];
+                sbw = (((gi & 8) ? hi : lo) >> (8 * (gi & 3))) & 0xFFu;
+              }
               bad |= (uint32_t)((sbw - kScaleLo) > (kScaleHi - kScaleLo));
-              const u32x4 w = st[j].w[t];
+              const u32x4 w = st[j][t];
               bad |= fp4x8_nonfinite(w[0]) | fp4x8_nonfinite(w[1]) | fp4x8_nonfinite(w[2]) |
                      fp4x8_nonfinite(w[3]);
               sa[t] = (int)sbw - 1;
@@ -1580,30 +1597,39 @@ __global__ __launch_bounds__(64 * kWideWaves) void tile_wide_kernel(GemmArgs p) 
             __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
             for (int m = 0; m + 1 < LIVE; ++m) {
-              const Rows nxt = read_rows(j, m + 1);
+              const Rows nxt = read_rows(j, m + 1, c);
               __builtin_amdgcn_sched_barrier(0);
               tile_mfmas(m, wa, sa);
               __builtin_amdgcn_sched_barrier(0);
               cur = nxt;
             }
           }
-          // Before the last tile: this wavefront's copies of step c + 1 have landed
-          // (outstanding after them: its weights, then 2 whole steps) and its reads of
-          // step c are complete; after the barrier that holds for every wavefront, so
-          // slot j takes the copies of step c + 4 and step c + 1 can be read.
-          __asm__ volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(kLoadOps + 2 * kStepOps) : "memory");
+          // Before the last tile: this wavefront's copies of step c + 1 (issued three
+          // steps ago, with the scale bytes if that was a first step of four) have
+          // landed and its reads of step c are complete; after the barrier that holds
+          // for every wavefront, so slot j takes the copies of step c + 4 and step
+          // c + 1 can be read.
+          constexpr int kCopyWait = (j == 3 ? 2 * kLoadOps : kLoadOps) +
+                                    (j == 0 || j == 3 ? 2 * kOpsStep : kOpsStep + kOpsStep0);
+          __asm__ volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(kCopyWait) : "memory");
           __builtin_amdgcn_s_barrier();
           __asm__ volatile("" ::: "memory");
           copy_step(c + R, j);
+          if (j == 0) copy_scales((c >> 2) + 1);
           if (work) {
-            const Rows nxt = read_rows((j + 1) % R, 0);
+            const Rows nxt = read_rows((j + 1) % R, 0, c + 1);
             __builtin_amdgcn_sched_barrier(0);
             tile_mfmas(LIVE - 1, wa, sa);
             __builtin_amdgcn_sched_barrier(0);
             cur = nxt;
           }
           load_step(st[j], c + R);
-        }
+          if (j == 0) load_scales(sc_nxt, (c >> 2) + 1);
+        };
+        step(IntC<0>{});
+        step(IntC<1>{});
+        step(IntC<2>{});
+        step(IntC<3>{});
       }
     };
     if (n_live > 6) k_loop(IntC<8>{});
@@ -1816,9 +1842,9 @@ StagePlan plan_stage(const GemmArgs& g) {
   return pl;
 }
 
-// The wide kernel takes split rows and reads weight scale bytes four at a time.
+// The wide kernel takes split rows and reads weight scale bytes sixteen at a time.
 bool wide_kernel_applies(const GemmArgs& g) {
-  return g.Aq != nullptr && g.K >= 128 && env_int("VK_MOE_WIDE", 1) != 0;
+  return g.Aq != nullptr && g.K >= 512 && env_int("VK_MOE_WIDE", 1) != 0;
 }
 
 template <int STAGE>
