@@ -1536,7 +1536,50 @@ __global__ __launch_bounds__(64 * kWideWaves) void tile_wide_kernel(GemmArgs p) 
       __asm__ volatile("" ::: "memory");
       Rows cur = read_rows(0, 0, 0);
 
-      auto tile_mfmas = [&](int m, const i32x8 (&wa)[NT], const int (&sa)[NT]) {
+      // Scale bytes of a group of 4 K steps: byte 4 j + q of the 16 is step j's for
+      // lane block q.  The last group of a K that is no multiple of 512 was loaded
+      // from `shift` bytes before its start: moved down here, once.
+      auto align_scales = [&](u32x4 (&sc)[NT], int shift) {
+        if (shift == 0) return;  // uniform
+        const int ds = shift >> 2, bs = shift & 3;
+#pragma unroll
+        for (int t = 0; t < NT; ++t) {
+          uint32_t v[8] = {sc[t][0], sc[t][1], sc[t][2], sc[t][3], 0u, 0u, 0u, 0u};
+          u32x4 r;
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            uint32_t lo = v[i], hi = v[i + 1];
+            if (ds == 1) { lo = v[i + 1]; hi = v[i + 2]; }
+            if (ds == 2) { lo = v[i + 2]; hi = v[i + 3]; }
+            if (ds == 3) { lo = v[i + 3]; hi = v[i + 4]; }
+            r[i] = (uint32_t)(((uint64_t)hi << 32 | lo) >> (8 * bs));
+          }
+          sc[t] = r;
+        }
+      };
+      auto scale_shift = [&](int first_step) {  // uniform
+        return first_step * 4 - min(first_step * 4, groups - 16);
+      };
+      // MFMA operand and scale of weight tile t for K step cc, whose scale bytes are
+      // dword jj of sc (lanes past K: the step's weights were loaded from the last
+      // group again and meet zero rows; their scale byte is made a neutral one).
+      auto prep_tile = [&](int cc, int jj, const u32x4& w, const u32x4& sc, i32x8& wa, int& sa) {
+        uint32_t sbw = (sc[jj] >> (8 * lq)) & 0xFFu;
+        if (cc * 4 + lq >= groups) sbw = 127u;
+        bad |= (uint32_t)((sbw - kScaleLo) > (kScaleHi - kScaleLo));
+        bad |= fp4x8_nonfinite(w[0]) | fp4x8_nonfinite(w[1]) | fp4x8_nonfinite(w[2]) |
+               fp4x8_nonfinite(w[3]);
+        sa = (int)sbw - 1;
+        wa = fp4_operand(w);
+      };
+      // operands of the current step in wa[j % 2], of the next in the other half
+      i32x8 wa[2][NT];
+      int sa[2][NT];
+      align_scales(sc_nxt, scale_shift(0));
+#pragma unroll
+      for (int t = 0; t < NT; ++t) prep_tile(0, 0, st[0][t], sc_nxt[t], wa[0][t], sa[0][t]);
+
+      auto tile_mfmas = [&](int m, const i32x8 (&wa_)[NT], const int (&sa_)[NT]) {
         // (opaque, so that no use of the byte moves up into the previous tile's
         // region and makes the MFMAs there wait for the read)
         int sbh = cur.sb;
@@ -1548,58 +1591,54 @@ __global__ __launch_bounds__(64 * kWideWaves) void tile_wide_kernel(GemmArgs p) 
         // the two MFMAs of an accumulator are kept NT instructions apart
 #pragma unroll
         for (int t = 0; t < NT; ++t)
-          acc[m][t] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wa[t], bh, acc[m][t], 4, 0, 0,
-                                                                       sa[t], 0, sbh);
+          acc[m][t] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wa_[t], bh, acc[m][t], 4, 0, 0,
+                                                                       sa_[t], 0, sbh);
 #pragma unroll
         for (int t = 0; t < NT; ++t)
-          acc[m][t] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wa[t], bl, acc[m][t], 4, 0, 0,
-                                                                       sa[t], 0, sbl);
+          acc[m][t] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wa_[t], bl, acc[m][t], 4, 0, 0,
+                                                                       sa_[t], 0, sbl);
+      };
+      // Order within a tile's region: the LDS reads of the next tile, then each MFMA
+      // followed by a few of the region's vector instructions (the preparation of one
+      // of the next step's weight tiles), which run while the matrix pipe is busy.
+      auto interleave = [&]() {
+        __builtin_amdgcn_sched_group_barrier(0x100, 5, 0);
+#pragma unroll
+        for (int i = 0; i < 2 * NT; ++i) {
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+          __builtin_amdgcn_sched_group_barrier(0x002, 5, 0);
+        }
       };
 
 #pragma unroll 1
       for (int c0 = 0; c0 < nsteps; c0 += R) {
-        // only the last group of 4 steps can start early (K no multiple of 512)
-        const int sc_shift = c0 * 4 - min(c0 * 4, groups - 16);  // uniform
+        const int shift_nxt = scale_shift(c0 + R);  // of the scale bytes in sc_nxt
         auto step = [&](auto j_c) {
           constexpr int j = decltype(j_c)::value;
+          constexpr int jn = (j + 1) % R, cb = j & 1, nb = cb ^ 1;
           // Steps past the last one (nsteps is rounded up to the ring here) only keep
           // the sequence of memory operations, hence the counted waits, the same.
           const int c = c0 + j;
           const bool work = has_unit && c < nsteps;  // uniform
-          // The weights of step c (and, first step of four, their scale bytes) were
-          // issued four steps ago.  The compiler waits for them itself; its count
-          // leaves the copies out, so it also waits for the copies of two steps ago.
           if (j == 0) {
 #pragma unroll
             for (int t = 0; t < NT; ++t) sc_cur[t] = sc_nxt[t];
           }
-          i32x8 wa[NT];
-          int sa[NT];
+          if (j == R - 1) align_scales(sc_nxt, shift_nxt);
+          // The weights of step c + 1 (issued three steps ago; the compiler waits for
+          // them itself, and as its count leaves the copies out, for the copies of two
+          // steps ago as well) are prepared one tile per row tile of this step.
+          auto prep_next = [&](int t) {
+            prep_tile(c + 1, jn, st[jn][t], j == R - 1 ? sc_nxt[t] : sc_cur[t], wa[nb][t], sa[nb][t]);
+          };
           if (work) {
-            const int gi = min(c * 4 + lq, groups - 1) - c0 * 4 + sc_shift;  // byte of the 16
-#pragma unroll
-            for (int t = 0; t < NT; ++t) {
-              uint32_t sbw;
-              if (sc_shift == 0) {  // uniform; the byte is in dword j
-                sbw = (sc_cur[t][j] >> (8 * lq)) & 0xFFu;
-              } else {
-                const uint32_t lo = (gi & 4) ? sc_cur[t][1] : sc_cur[t][0];
-                const uint32_t hi = (gi & 4) ? sc_cur[t][3] : sc_cur[t][2];
-                sbw = (((gi & 8) ? hi : lo) >> (8 * (gi & 3))) & 0xFFu;
-              }
-              bad |= (uint32_t)((sbw - kScaleLo) > (kScaleHi - kScaleLo));
-              const u32x4 w = st[j][t];
-              bad |= fp4x8_nonfinite(w[0]) | fp4x8_nonfinite(w[1]) | fp4x8_nonfinite(w[2]) |
-                     fp4x8_nonfinite(w[3]);
-              sa[t] = (int)sbw - 1;
-              wa[t] = fp4_operand(w);
-            }
             __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
             for (int m = 0; m + 1 < LIVE; ++m) {
               const Rows nxt = read_rows(j, m + 1, c);
-              __builtin_amdgcn_sched_barrier(0);
-              tile_mfmas(m, wa, sa);
+              if (m < NT) prep_next(m);
+              tile_mfmas(m, wa[cb], sa[cb]);
+              interleave();
               __builtin_amdgcn_sched_barrier(0);
               cur = nxt;
             }
@@ -1617,9 +1656,12 @@ __global__ __launch_bounds__(64 * kWideWaves) void tile_wide_kernel(GemmArgs p) 
           copy_step(c + R, j);
           if (j == 0) copy_scales((c >> 2) + 1);
           if (work) {
-            const Rows nxt = read_rows((j + 1) % R, 0, c + 1);
             __builtin_amdgcn_sched_barrier(0);
-            tile_mfmas(LIVE - 1, wa, sa);
+            const Rows nxt = read_rows(jn, 0, c + 1);
+#pragma unroll
+            for (int t = LIVE - 1; t < NT; ++t) prep_next(t);
+            tile_mfmas(LIVE - 1, wa[cb], sa[cb]);
+            interleave();
             __builtin_amdgcn_sched_barrier(0);
             cur = nxt;
           }
