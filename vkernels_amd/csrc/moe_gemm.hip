@@ -1325,27 +1325,39 @@ __global__ __launch_bounds__(64 * kWsWaves) void tile_ws_kernel(GemmArgs p) {
 // scale-range checks) is shared by 16 MFMAs and every LDS operand read by 8.
 //
 // 4 wavefronts, one per SIMD, each with the full register file: 8 row tiles x
-// 4 weight tiles of accumulators, the weights of the next 4 K steps in flight
-// in registers, and the LDS operands of the next (K step, row tile) read while
-// the MFMAs of the current one issue.
+// 4 weight tiles of accumulators.  Everything the K loop reads from global
+// memory arrives in LDS by the DMA form of the global load, three K steps
+// ahead, and no wavefront ever waits for a load it has just issued: the waits
+// are s_waitcnt instructions with counts derived from the fixed order in which
+// each wavefront issues its memory operations.
 //
 // Rows.  A workgroup takes a window of 128 sorted rows (block sizes that divide
 // 128; otherwise one group of tile_group_rows rows) and cuts it into segments
 // of consecutive blocks of one expert; each segment is one pass of the K loop.
 //
-// LDS: a ring of 4 K steps.  Per step the 8 row tiles' operand planes
-// [row tile][term][half][lane] x 16 bytes and the rows' 4 scale bytes
-// [row][group], copied from the split rows (whose zero blocks between K and the
-// next multiple of 128 make the last, partial step an ordinary one) by the DMA
-// form of the global load, 9 instructions per wavefront and step, three steps
-// ahead.  One barrier per K step: before it every wavefront waits for its own
-// copies of the NEXT step, so after it (a) that step may be read ahead and (b)
-// the slot of the previous step may be overwritten.
+// LDS (bytes):
+//   row ring     3 x 32 KiB   per K step, 8 row tiles x {hi, lo} x 16 rows x 128
+//                             bytes, copied from the split rows (whose zero blocks
+//                             between K and the next multiple of 128 make the last,
+//                             partial step an ordinary one) as whole cache lines;
+//   row scales   2 x 2 KiB    16 scale bytes per row, of which a group of 3 K steps
+//                             uses 12;
+//   weight ring  4 x 3 x 4 KiB  per wavefront and K step, its 4 weight tiles as MFMA
+//                             operands (lane order);
+//   weight scales 4 x 2 x 1 KiB per wavefront, 16 scale bytes per weight row.
+// One barrier per K step, before its last row tile: every wavefront first waits
+// for its own row copies of the NEXT step, so after the barrier (a) that step may
+// be read ahead and (b) the slot of the current step, whose last tile is already
+// in registers, takes the copies of step + 3.  The weight ring is private to a
+// wavefront and needs no barrier.
 // ---------------------------------------------------------------------------
-constexpr int kWideWaves = 4, kWideNT = 4, kWideMT = 8, kWideRing = 4;
+constexpr int kWideWaves = 4, kWideNT = 4, kWideMT = 8, kWideRing = 3;
 constexpr int kWideRows = 16 * kWideMT;
 constexpr int kWideStepBytes = kWideMT * 4 * 1024;
-constexpr int kWideLdsBytes = kWideRing * kWideStepBytes + 2 * kWideRows * 16;  // + two scale slots
+constexpr int kWideRowScales = kWideRing * kWideStepBytes;            // 2 slots x 128 rows x 16
+constexpr int kWideWeights = kWideRowScales + 2 * kWideRows * 16;     // per wavefront: 3 x 4 KiB
+constexpr int kWideWeightScales = kWideWeights + kWideWaves * kWideRing * 4096;  // per wavefront: 2 x 1 KiB
+constexpr int kWideLdsBytes = kWideWeightScales + kWideWaves * 2 * 1024;
 
 // Sorted rows one workgroup of the wide kernel covers.
 __host__ __device__ inline int wide_window_rows(int block_size) {
@@ -1369,13 +1381,13 @@ struct IntC {
 __device__ __forceinline__ void dma_load_16(const void* src, uint32_t lds_base) {
   __asm__ volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off"
                    :
-                   : "s"(lds_base), "v"(src)
+                   : "s"(__builtin_amdgcn_readfirstlane(lds_base)), "v"(src)
                    : "memory");
 }
 __device__ __forceinline__ void dma_load_4(const void* src, uint32_t lds_base) {
   __asm__ volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, off"
                    :
-                   : "s"(lds_base), "v"(src)
+                   : "s"(__builtin_amdgcn_readfirstlane(lds_base)), "v"(src)
                    : "memory");
 }
 
@@ -1407,15 +1419,22 @@ __global__ __launch_bounds__(64 * kWideWaves) void tile_wide_kernel(GemmArgs p) 
     u32x4 h0, h1, l0, l1;
     int sb;
   };
-  // Memory operations per K step, in program order: the 8 row copies, the copy of
-  // the rows' scale bytes (every 4th step, for the next 4), the 4 weight loads,
-  // the 4 loads of the weights' scale bytes (every 4th step, for the next 4).
-  constexpr int kCopyOps = 8, kLoadOps = NT;
-  constexpr int kOpsStep0 = kCopyOps + 1 + 2 * kLoadOps, kOpsStep = kCopyOps + kLoadOps;
-  constexpr int kOpsCycle = kOpsStep0 + 3 * kOpsStep;
+  // Memory operations of a wavefront in K step c, in program order (all DMA; j = c % 3):
+  //   0 .. 4    pieces 3 .. 7 of its row copies of step c + 2 (the slot was freed by the
+  //             barrier of step c - 1);
+  //   5 .. 8    its 4 weight tiles of step c + 3 (their slot was read during step c - 1);
+  //   9 .. 12   j = 0 only: the weight-scale copies of the next group of three steps;
+  //   -- the barrier of step c --
+  //   13 .. 15  pieces 0 .. 2 of its row copies of step c + 3, into the slot just freed;
+  //   16        j = 0 only: the row scales of the next group.
+  // The operations before the barrier are spread over the row tiles of the step, so that
+  // the memory pipe, which all four wavefronts share, is fed evenly while the MFMAs run.
+  constexpr int kRowsLate = 5, kRowsEarly = 3, kWeightOps = NT;
+  auto ops_before = [](int j) constexpr { return kRowsLate + kWeightOps + (j == 0 ? NT : 0); };
+  auto ops_after = [](int j) constexpr { return kRowsEarly + (j == 0 ? 1 : 0); };
 
   auto segment = [&](const int row0, const int n_rows, const int e) {
-    __syncthreads();  // the previous segment is done with row_flat and the ring
+    __syncthreads();  // the previous segment is done with row_flat and the rings
     if (tid < kWideRows) {
       int f = -1;
       if (tid < n_rows) {
@@ -1436,9 +1455,12 @@ __global__ __launch_bounds__(64 * kWideWaves) void tile_wide_kernel(GemmArgs p) 
     int col0[NT];
     unit_tiles<STAGE, NT>(p, e, has_unit ? unit : 0, ln, w_rows, s_rows, col0);
 
-    // ---- copies.  One copy instruction moves 8 rows x 128 bytes (one K step of one
-    // term): whole cache lines, which the memory pipe serves three times as fast as
-    // 64-byte pieces of 16 rows.  Lane (r, j) = (lane / 8, lane % 8) copies piece
+    const uint32_t lds_base = (uint32_t)(uintptr_t)(lds_ptr)wide_lds;
+    const uint8_t* lds_bytes = reinterpret_cast<const uint8_t*>(wide_lds);
+
+    // ---- row copies.  One copy instruction moves 8 rows x 128 bytes (one K step of
+    // one term): whole cache lines, which the memory pipe serves three times as fast
+    // as 64-byte pieces of 16 rows.  Lane (r, j) = (lane / 8, lane % 8) copies piece
     // j ^ r of row r, so that the 16-byte pieces of a row sit in LDS rotated by the
     // row and the MFMA operand reads (16 rows, one piece each) spread over the banks.
     // Wavefront w copies row tiles 2 w and 2 w + 1.
@@ -1453,8 +1475,8 @@ __global__ __launch_bounds__(64 * kWideWaves) void tile_wide_kernel(GemmArgs p) 
         const size_t r = f >= 0 ? (size_t)(STAGE == 0 ? f / p.top_k : row0 + rl) : 0;
         cp_row[i][rh] = p.Aq + r * (size_t)(2 * Kp) + 16 * (cj ^ cr);
       }
-    // scale bytes: 16 per row = 4 K steps; rows 64 (wave % 2) .. + 63 (twice over, so
-    // that every wavefront issues the same number of copies)
+    // row scale bytes: 16 per row from byte 12 g on (a group of 3 K steps uses 12);
+    // rows 64 (wave % 2) .. + 63, twice over, so that all wavefronts issue alike
     const uint8_t* cp_scale;
     {
       const int rl = (wave & 1) * 64 + lane;
@@ -1462,47 +1484,47 @@ __global__ __launch_bounds__(64 * kWideWaves) void tile_wide_kernel(GemmArgs p) 
       const size_t r = f >= 0 ? (size_t)(STAGE == 0 ? f / p.top_k : row0 + rl) : 0;
       cp_scale = p.As + r * (size_t)sstride;
     }
-    const uint32_t ring_base = (uint32_t)(uintptr_t)(lds_ptr)wide_lds;
-    auto copy_step = [&](int step, int slot) {
-      const uint32_t buf = ring_base + (uint32_t)(slot * kWideStepBytes);
+    // piece j (0 .. 7) of this wavefront's row copies of a K step
+    auto copy_row_piece = [&](int step, int slot, int j) {
+      const uint32_t buf = lds_base + (uint32_t)(slot * kWideStepBytes);
       const int k0 = min(step, nsteps - 1) * 128;  // past the end: the last step again
-#pragma unroll
-      for (int j = 0; j < 8; ++j) {
-        const int i = j >> 2, term = (j >> 1) & 1, rh = j & 1;
-        const int plane = ((wave * 2 + i) * 2 + term) * 2 + rh;
-        dma_load_16(cp_row[i][rh] + (size_t)term * Kp + k0, buf + (uint32_t)(plane * 1024));
-      }
+      const int i = j >> 2, term = (j >> 1) & 1, rh = j & 1;
+      const int plane = ((wave * 2 + i) * 2 + term) * 2 + rh;
+      dma_load_16(cp_row[i][rh] + (size_t)term * Kp + k0, buf + (uint32_t)(plane * 1024));
     };
-    auto copy_scales = [&](int group) {  // the rows' scale bytes of K steps 4 group .. + 3
-      const int g = min(group * 16, sstride - 16);
-      dma_load_16(cp_scale + g, ring_base + (uint32_t)(R * kWideStepBytes + (group & 1) * 2048 +
-                                                      (wave & 1) * 1024));
+    // first byte of the 16 that hold group g's 12 (the last group starts early rather
+    // than read past the row: see scale_index)
+    auto row_scale_start = [&](int g) { return min(g * 12, sstride - 16); };
+    auto weight_scale_start = [&](int g) { return min(g * 12, groups - 16); };
+    auto copy_row_scales = [&](int g) {
+      dma_load_16(cp_scale + row_scale_start(g),
+                  lds_base + (uint32_t)(kWideRowScales + (g & 1) * 2048 + (wave & 1) * 1024));
     };
-    auto load_step = [&](u32x4 (&w)[NT], int step) {  // branch-free: past the end, the last group
+    // ---- weight copies: a tile's 64 x 16 bytes in lane order, per wavefront
+    const uint32_t w_ring = lds_base + (uint32_t)(kWideWeights + wave * (R * 4096));
+    const uint32_t ws_ring = lds_base + (uint32_t)(kWideWeightScales + wave * 2048);
+    auto copy_weight_tile = [&](int step, int slot, int t) {  // past the end: the last group
       const int g = min(step * 4 + lq, groups - 1);
-#pragma unroll
-      for (int t = 0; t < NT; ++t) w[t] = *reinterpret_cast<const u32x4*>(w_rows[t] + (size_t)g * 16);
+      dma_load_16(w_rows[t] + (size_t)g * 16, w_ring + (uint32_t)(slot * 4096 + t * 1024));
     };
-    // the 16 scale bytes of the lane's weight rows for K steps 4 group .. + 3; the last
-    // group of a K that is no multiple of 512 starts early (see weight_scale)
-    auto load_scales = [&](u32x4 (&sc)[NT], int group) {
-      const int g = min(group * 16, groups - 16);
-#pragma unroll
-      for (int t = 0; t < NT; ++t) sc[t] = *reinterpret_cast<const u32x4*>(s_rows[t] + g);
+    // lane (n, q) copies dword q of weight row n's 16 scale bytes: LDS [q][n] dwords
+    auto copy_weight_scale_tile = [&](int g, int t) {
+      const int b0 = weight_scale_start(g) + 4 * lq;
+      dma_load_4(s_rows[t] + b0, ws_ring + (uint32_t)((g & 1) * 1024 + t * 256));
     };
     // operand reads of row tile m of a slot: lane (n, q) takes piece q (q + 4) of row n
     const int rd0 = (ln >> 3) * 1024 + (ln & 7) * 128 + ((lq ^ (ln & 7)) * 16);
     const int rd1 = rd0 ^ 64;
-    const uint8_t* ring_bytes = reinterpret_cast<const uint8_t*>(wide_lds);
     auto read_rows = [&](int slot, int m, int step) {
-      const uint8_t* tile = ring_bytes + slot * kWideStepBytes + m * 4096;
+      const uint8_t* tile = lds_bytes + slot * kWideStepBytes + m * 4096;
       Rows b;
       b.h0 = *reinterpret_cast<const u32x4*>(tile + rd0);
       b.h1 = *reinterpret_cast<const u32x4*>(tile + rd1);
       b.l0 = *reinterpret_cast<const u32x4*>(tile + 2048 + rd0);
       b.l1 = *reinterpret_cast<const u32x4*>(tile + 2048 + rd1);
-      b.sb = ring_bytes[R * kWideStepBytes + ((step >> 2) & 1) * 2048 + (m * 16 + ln) * 16 +
-                        (step & 3) * 4 + lq];
+      const int g = step / 3;  // uniform
+      const int idx = step * 4 + lq - row_scale_start(g);
+      b.sb = lds_bytes[kWideRowScales + (g & 1) * 2048 + (m * 16 + ln) * 16 + idx];
       return b;
     };
 
@@ -1518,53 +1540,39 @@ __global__ __launch_bounds__(64 * kWideWaves) void tile_wide_kernel(GemmArgs p) 
     // one survives; the tiles between n_live and LIVE are padding rows).
     auto k_loop = [&](auto live_c) {
       constexpr int LIVE = decltype(live_c)::value;
-      u32x4 st[R][NT];
-      u32x4 sc_cur[NT], sc_nxt[NT];
-      // The prologue issues steps 0 .. 3 in the order of the loop, so the counts
-      // below hold from the first step on.
+      // operation k (see above) of K step c, c % 3 = j
+      auto issue = [&](int c, int j, int k) {
+        if (k < 5) copy_row_piece(c + 2, (j + 2) % R, 3 + k);
+        else if (k < 9) copy_weight_tile(c + R, j, k - 5);
+        else if (k < 13) { if (j == 0) copy_weight_scale_tile(c / 3 + 1, k - 9); }
+        else if (k < 16) copy_row_piece(c + R, j, k - 13);
+        else if (j == 0) copy_row_scales(c / 3 + 1);
+      };
+      // The prologue issues what steps -3, -2, -1 would, less the row pieces of step -1.
 #pragma unroll
       for (int j = 0; j < R; ++j) {
-        copy_step(j, j);
-        if (j == 0) copy_scales(0);
-        load_step(st[j], j);
-        if (j == 0) load_scales(sc_nxt, 0);
+#pragma unroll
+        for (int k = (j == 0 ? 5 : 0); k < 17; ++k) issue(j - R, j, k);
       }
-      // copies of step 0 and of the first scale bytes: all that was issued after them
-      // may still be outstanding
-      __asm__ volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * kLoadOps + 3 * kOpsStep) : "memory");
+      // all of steps 0's rows, weights and scale bytes have landed once only what was
+      // issued after the late row pieces of step 0 is outstanding
+      __asm__ volatile("s_waitcnt vmcnt(%0)" ::"n"(kWeightOps + ops_after(1) + ops_before(2) + ops_after(2))
+                       : "memory");
       __builtin_amdgcn_s_barrier();
       __asm__ volatile("" ::: "memory");
       Rows cur = read_rows(0, 0, 0);
 
-      // Scale bytes of a group of 4 K steps: byte 4 j + q of the 16 is step j's for
-      // lane block q.  The last group of a K that is no multiple of 512 was loaded
-      // from `shift` bytes before its start: moved down here, once.
-      auto align_scales = [&](u32x4 (&sc)[NT], int shift) {
-        if (shift == 0) return;  // uniform
-        const int ds = shift >> 2, bs = shift & 3;
-#pragma unroll
-        for (int t = 0; t < NT; ++t) {
-          uint32_t v[8] = {sc[t][0], sc[t][1], sc[t][2], sc[t][3], 0u, 0u, 0u, 0u};
-          u32x4 r;
-#pragma unroll
-          for (int i = 0; i < 4; ++i) {
-            uint32_t lo = v[i], hi = v[i + 1];
-            if (ds == 1) { lo = v[i + 1]; hi = v[i + 2]; }
-            if (ds == 2) { lo = v[i + 2]; hi = v[i + 3]; }
-            if (ds == 3) { lo = v[i + 3]; hi = v[i + 4]; }
-            r[i] = (uint32_t)(((uint64_t)hi << 32 | lo) >> (8 * bs));
-          }
-          sc[t] = r;
-        }
-      };
-      auto scale_shift = [&](int first_step) {  // uniform
-        return first_step * 4 - min(first_step * 4, groups - 16);
-      };
-      // MFMA operand and scale of weight tile t for K step cc, whose scale bytes are
-      // dword jj of sc (lanes past K: the step's weights were loaded from the last
-      // group again and meet zero rows; their scale byte is made a neutral one).
-      auto prep_tile = [&](int cc, int jj, const u32x4& w, const u32x4& sc, i32x8& wa, int& sa) {
-        uint32_t sbw = (sc[jj] >> (8 * lq)) & 0xFFu;
+      // MFMA operand and scale of weight tile t for K step cc from the weight ring
+      // (lanes past K: the step's weights are the last group's again and meet zero
+      // rows; their scale byte is made a neutral one).
+      auto prep_tile = [&](int cc, int slot, int t, i32x8& wa, int& sa) {
+        cc = min(cc, nsteps - 1);  // past the end the slot holds the last step again
+        const uint8_t* wr = lds_bytes + kWideWeights + wave * (R * 4096) + slot * 4096 + t * 1024;
+        const u32x4 w = *reinterpret_cast<const u32x4*>(wr + lane * 16);
+        const int g = cc / 3;  // uniform
+        const int idx = min(cc * 4 + lq, groups - 1) - weight_scale_start(g);
+        uint32_t sbw = lds_bytes[kWideWeightScales + wave * 2048 + (g & 1) * 1024 + t * 256 +
+                                 (idx >> 2) * 64 + ln * 4 + (idx & 3)];
         if (cc * 4 + lq >= groups) sbw = 127u;
         bad |= (uint32_t)((sbw - kScaleLo) > (kScaleHi - kScaleLo));
         bad |= fp4x8_nonfinite(w[0]) | fp4x8_nonfinite(w[1]) | fp4x8_nonfinite(w[2]) |
@@ -1572,14 +1580,17 @@ __global__ __launch_bounds__(64 * kWideWaves) void tile_wide_kernel(GemmArgs p) 
         sa = (int)sbw - 1;
         wa = fp4_operand(w);
       };
-      // operands of the current step in wa[j % 2], of the next in the other half
+      // operands of the current step in wa[c % 2], of the next in the other half
       i32x8 wa[2][NT];
       int sa[2][NT];
-      align_scales(sc_nxt, scale_shift(0));
 #pragma unroll
-      for (int t = 0; t < NT; ++t) prep_tile(0, 0, st[0][t], sc_nxt[t], wa[0][t], sa[0][t]);
+      for (int t = 0; t < NT; ++t) prep_tile(0, 0, t, wa[0][t], sa[0][t]);
 
-      auto tile_mfmas = [&](int m, const i32x8 (&wa_)[NT], const int (&sa_)[NT]) {
+      // One row tile: its MFMAs in two halves (the leading terms, the remainders), a
+      // memory operation ahead of each half, the vector work of the region (among it
+      // the preparation of one of the next step's weight tiles) spread between the
+      // MFMAs, during which the matrix pipe is busy anyway.
+      auto tile = [&](int m, const i32x8 (&wa_)[NT], const int (&sa_)[NT], auto&& op_a, auto&& op_b) {
         // (opaque, so that no use of the byte moves up into the previous tile's
         // region and makes the MFMAs there wait for the read)
         int sbh = cur.sb;
@@ -1588,90 +1599,89 @@ __global__ __launch_bounds__(64 * kWideWaves) void tile_wide_kernel(GemmArgs p) 
         const int sbl = sbh - 4;
         const i32x8 bh = fp8_operand(cur.h0, cur.h1);
         const i32x8 bl = fp8_operand(cur.l0, cur.l1);
+        op_a();
         // the two MFMAs of an accumulator are kept NT instructions apart
 #pragma unroll
         for (int t = 0; t < NT; ++t)
           acc[m][t] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wa_[t], bh, acc[m][t], 4, 0, 0,
                                                                        sa_[t], 0, sbh);
+        __builtin_amdgcn_sched_barrier(0);
+        op_b();
 #pragma unroll
         for (int t = 0; t < NT; ++t)
           acc[m][t] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wa_[t], bl, acc[m][t], 4, 0, 0,
                                                                        sa_[t], 0, sbl);
-      };
-      // Order within a tile's region: the LDS reads of the next tile, then each MFMA
-      // followed by a few of the region's vector instructions (the preparation of one
-      // of the next step's weight tiles), which run while the matrix pipe is busy.
-      auto interleave = [&]() {
-        __builtin_amdgcn_sched_group_barrier(0x100, 5, 0);
-#pragma unroll
-        for (int i = 0; i < 2 * NT; ++i) {
-          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-          __builtin_amdgcn_sched_group_barrier(0x002, 5, 0);
-        }
+        __builtin_amdgcn_sched_barrier(0);
       };
 
+      // Two K steps per pass of the unrolled body would fix c % 2 but not c % 3; six do.
 #pragma unroll 1
-      for (int c0 = 0; c0 < nsteps; c0 += R) {
-        const int shift_nxt = scale_shift(c0 + R);  // of the scale bytes in sc_nxt
-        auto step = [&](auto j_c) {
-          constexpr int j = decltype(j_c)::value;
-          constexpr int jn = (j + 1) % R, cb = j & 1, nb = cb ^ 1;
-          // Steps past the last one (nsteps is rounded up to the ring here) only keep
-          // the sequence of memory operations, hence the counted waits, the same.
-          const int c = c0 + j;
+      for (int c0 = 0; c0 < nsteps; c0 += 2 * R) {
+        auto step = [&](auto i_c) {
+          constexpr int i = decltype(i_c)::value;
+          constexpr int j = i % R, jn = (j + 1) % R, jp = (j + 2) % R, cb = i & 1, nb = cb ^ 1;
+          // Steps past the last one (nsteps is rounded up here) only keep the sequence
+          // of memory operations, hence the counted waits, the same.
+          const int c = c0 + i;
           const bool work = has_unit && c < nsteps;  // uniform
-          if (j == 0) {
+          // The weights of step c + 1 (and, when that is a first step of three, their
+          // scale bytes) were issued in step c - 2; since then: the early row pieces of
+          // that step (and row scales) and all of step c - 1.
+          constexpr int kWeightWait = ops_after(jn) + ops_before(jp) + ops_after(jp);
+          __asm__ volatile("s_waitcnt vmcnt(%0)" ::"n"(kWeightWait) : "memory");
+          auto prep_next = [&](int t) { prep_tile(c + 1, jn, t, wa[nb][t], sa[nb][t]); };
+          // operations before the barrier: two per row tile but the last (all at once
+          // where the step has a single tile, or does no arithmetic)
+          constexpr int kBefore = 13;
+          constexpr int kPer = LIVE > 1 ? (kBefore + 2 * (LIVE - 1) - 1) / (2 * (LIVE - 1)) : kBefore;
+          auto before = [&](int first) {
 #pragma unroll
-            for (int t = 0; t < NT; ++t) sc_cur[t] = sc_nxt[t];
-          }
-          if (j == R - 1) align_scales(sc_nxt, shift_nxt);
-          // The weights of step c + 1 (issued three steps ago; the compiler waits for
-          // them itself, and as its count leaves the copies out, for the copies of two
-          // steps ago as well) are prepared one tile per row tile of this step.
-          auto prep_next = [&](int t) {
-            prep_tile(c + 1, jn, st[jn][t], j == R - 1 ? sc_nxt[t] : sc_cur[t], wa[nb][t], sa[nb][t]);
+            for (int k = first; k < first + kPer; ++k)
+              if (k < kBefore) issue(c, j, k);
           };
-          if (work) {
+          if (work && LIVE > 1) {
             __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
             for (int m = 0; m + 1 < LIVE; ++m) {
               const Rows nxt = read_rows(j, m + 1, c);
               if (m < NT) prep_next(m);
-              tile_mfmas(m, wa[cb], sa[cb]);
-              interleave();
-              __builtin_amdgcn_sched_barrier(0);
+              tile(m, wa[cb], sa[cb], [&]() { before(2 * m * kPer); }, [&]() { before((2 * m + 1) * kPer); });
               cur = nxt;
             }
+          } else {
+#pragma unroll
+            for (int k = 0; k < kBefore; ++k) issue(c, j, k);
           }
-          // Before the last tile: this wavefront's copies of step c + 1 (issued three
-          // steps ago, with the scale bytes if that was a first step of four) have
-          // landed and its reads of step c are complete; after the barrier that holds
-          // for every wavefront, so slot j takes the copies of step c + 4 and step
-          // c + 1 can be read.
-          constexpr int kCopyWait = (j == 3 ? 2 * kLoadOps : kLoadOps) +
-                                    (j == 0 || j == 3 ? 2 * kOpsStep : kOpsStep + kOpsStep0);
-          __asm__ volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(kCopyWait) : "memory");
+          // Before the last tile: this wavefront's row copies of step c + 1 (the early
+          // pieces, with the row scales if c + 1 is a first step of three, from after
+          // the barrier of step c - 2; the late ones from step c - 1) have landed and
+          // its reads of step c are complete; after the barrier that holds for every
+          // wavefront, so slot j takes the early pieces of step c + 3 and step c + 1
+          // can be read.  Outstanding may be what followed the late pieces in step
+          // c - 1 and what this step has issued so far.
+          constexpr int kRowWait = kWeightOps + (jp == 0 ? NT : 0) + ops_after(jp) + ops_before(j);
+          __asm__ volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(kRowWait) : "memory");
           __builtin_amdgcn_s_barrier();
           __asm__ volatile("" ::: "memory");
-          copy_step(c + R, j);
-          if (j == 0) copy_scales((c >> 2) + 1);
           if (work) {
             __builtin_amdgcn_sched_barrier(0);
             const Rows nxt = read_rows(jn, 0, c + 1);
 #pragma unroll
             for (int t = LIVE - 1; t < NT; ++t) prep_next(t);
-            tile_mfmas(LIVE - 1, wa[cb], sa[cb]);
-            interleave();
-            __builtin_amdgcn_sched_barrier(0);
+            tile(LIVE - 1, wa[cb], sa[cb], [&]() { issue(c, j, 13); issue(c, j, 14); },
+                 [&]() { issue(c, j, 15); issue(c, j, 16); });
             cur = nxt;
+          } else {
+#pragma unroll
+            for (int k = 13; k < 17; ++k) issue(c, j, k);
           }
-          load_step(st[j], c + R);
-          if (j == 0) load_scales(sc_nxt, (c >> 2) + 1);
         };
         step(IntC<0>{});
         step(IntC<1>{});
         step(IntC<2>{});
         step(IntC<3>{});
+        step(IntC<4>{});
+        step(IntC<5>{});
       }
     };
     if (n_live > 6) k_loop(IntC<8>{});
