@@ -43,7 +43,7 @@ def _run_gpu(cfg, w, A_bits, logits, block_size=None, use_workspace=None, **kw):
     A = to_dev(A_bits, torch.bfloat16)
     ids, tw = fe.route(to_dev(logits), cfg.top_k, True)
     T = A.shape[0]
-    bs = ve.default_block_size(T) if block_size is None else block_size
+    bs = ve.default_block_size(T, cfg.top_k) if block_size is None else block_size
     sids, eids, out_em, max_em = fe.align(ids, bs)
     out = fe.apply(A, ids, tw, block_size=bs)
     torch.cuda.synchronize()

@@ -1321,21 +1321,15 @@ __global__ __launch_bounds__(64 * kWsWaves) void tile_ws_kernel(GemmArgs p) {
 
 // ---------------------------------------------------------------------------
 // Wide tile kernel (workspace path): up to 128 sorted rows of one expert per
-// workgroup against 4 weight units (16 tiles), so that every LDS operand read
-// serves 8 MFMAs and every weight byte 128 rows.
+// workgroup, so that the preparation of a weight tile (code points, inf/NaN and
+// scale-range checks) is shared by 16 MFMAs and every LDS operand read by 8.
 //
-// 8 wavefronts, two per SIMD.  A wavefront issues at most one instruction every
-// four cycles, and the loop needs about six instructions besides each 32-cycle
-// MFMA (operand reads, code-point fixes, scale checks, copies): one wavefront per
-// SIMD cannot keep the matrix pipe busy, two can, one's bookkeeping under the
-// other's MFMAs.  Wavefronts 2 u and 2 u + 1 share weight unit u; the first takes
-// the even row tiles, the second the odd ones (4 x 4 accumulator tiles each).
-//
-// Everything the K loop reads from global memory arrives in LDS by the DMA form
-// of the global load, three K steps ahead, and no wavefront ever waits for a
-// load it has just issued: the waits are s_waitcnt instructions with counts
-// derived from the fixed order in which each wavefront issues its memory
-// operations.
+// 4 wavefronts, one per SIMD, each with the full register file: 8 row tiles x
+// 4 weight tiles of accumulators.  Everything the K loop reads from global
+// memory arrives in LDS by the DMA form of the global load, three K steps
+// ahead, and no wavefront ever waits for a load it has just issued: the waits
+// are s_waitcnt instructions with counts derived from the fixed order in which
+// each wavefront issues its memory operations.
 //
 // Rows.  A workgroup takes a window of 128 sorted rows (block sizes that divide
 // 128; otherwise one group of tile_group_rows rows) and cuts it into segments
@@ -1348,21 +1342,22 @@ __global__ __launch_bounds__(64 * kWsWaves) void tile_ws_kernel(GemmArgs p) {
 //                             partial step an ordinary one) as whole cache lines;
 //   row scales   2 x 2 KiB    16 scale bytes per row, of which a group of 3 K steps
 //                             uses 12;
-//   weight ring  4 x 3 x 4 KiB  per weight unit and K step, its 4 tiles as MFMA
+//   weight ring  4 x 3 x 4 KiB  per wavefront and K step, its 4 weight tiles as MFMA
 //                             operands (lane order);
-//   weight scales 4 x 2 x 1 KiB per weight unit, 16 scale bytes per weight row.
-// One barrier per K step, before a wavefront's last row tile: every wavefront
-// first waits for its own copies of the NEXT step, so after the barrier (a) that
-// step may be read and (b) the slots of the current step, whose last tile and
-// weights are already in registers, take the copies of step + 3.
+//   weight scales 4 x 2 x 1 KiB per wavefront, 16 scale bytes per weight row.
+// One barrier per K step, before its last row tile: every wavefront first waits
+// for its own row copies of the NEXT step, so after the barrier (a) that step may
+// be read ahead and (b) the slot of the current step, whose last tile is already
+// in registers, takes the copies of step + 3.  The weight ring is private to a
+// wavefront and needs no barrier.
 // ---------------------------------------------------------------------------
-constexpr int kWideWaves = 8, kWideUnits = 4, kWideNT = 4, kWideMT = 8, kWideRing = 3;
+constexpr int kWideWaves = 4, kWideNT = 4, kWideMT = 8, kWideRing = 3;
 constexpr int kWideRows = 16 * kWideMT;
 constexpr int kWideStepBytes = kWideMT * 4 * 1024;
 constexpr int kWideRowScales = kWideRing * kWideStepBytes;            // 2 slots x 128 rows x 16
-constexpr int kWideWeights = kWideRowScales + 2 * kWideRows * 16;     // per unit: 3 x 4 KiB
-constexpr int kWideWeightScales = kWideWeights + kWideUnits * kWideRing * 4096;  // per unit: 2 x 1 KiB
-constexpr int kWideLdsBytes = kWideWeightScales + kWideUnits * 2 * 1024;
+constexpr int kWideWeights = kWideRowScales + 2 * kWideRows * 16;     // per wavefront: 3 x 4 KiB
+constexpr int kWideWeightScales = kWideWeights + kWideWaves * kWideRing * 4096;  // per wavefront: 2 x 1 KiB
+constexpr int kWideLdsBytes = kWideWeightScales + kWideWaves * 2 * 1024;
 
 // Sorted rows one workgroup of the wide kernel covers.
 __host__ __device__ inline int wide_window_rows(int block_size) {
@@ -1378,35 +1373,27 @@ struct IntC {
   static constexpr int value = N;
 };
 
-// The DMA form of the global load: every lane's 16 (4) bytes at base + offset go to
-// LDS at byte address lds_base + 16 (4) * lane.  `base` is uniform (scalar
-// registers), the per-lane part is a 32-bit offset: one register per lane instead of
-// a pointer.  Written as assembly because the compiler makes every later LDS read
-// wait for all DMA loads it has emitted itself, and for every register load issued
-// along with them: a ring that is filled several steps ahead needs the counted
-// waits of the kernel instead.
-__device__ __forceinline__ uint64_t uniform_address(const void* p) {
-  const uint64_t a = reinterpret_cast<uint64_t>(p);
-  const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)a);
-  const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)(a >> 32));
-  return ((uint64_t)hi << 32) | lo;
-}
-__device__ __forceinline__ void dma_load_16(const void* base, uint32_t offset, uint32_t lds_base) {
-  __asm__ volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+// The DMA form of the global load: every lane's 16 (4) bytes at `src` go to LDS
+// at byte address lds_base + 16 (4) * lane.  Written as assembly because the
+// compiler makes every later LDS read wait for all DMA loads it has emitted
+// itself, and for every register load issued along with them: a ring that is
+// filled several steps ahead needs the counted waits of the kernel instead.
+__device__ __forceinline__ void dma_load_16(const void* src, uint32_t lds_base) {
+  __asm__ volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off"
                    :
-                   : "s"(__builtin_amdgcn_readfirstlane(lds_base)), "v"(offset), "s"(uniform_address(base))
+                   : "s"(__builtin_amdgcn_readfirstlane(lds_base)), "v"(src)
                    : "memory");
 }
-__device__ __forceinline__ void dma_load_4(const void* base, uint32_t offset, uint32_t lds_base) {
-  __asm__ volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, %2"
+__device__ __forceinline__ void dma_load_4(const void* src, uint32_t lds_base) {
+  __asm__ volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, off"
                    :
-                   : "s"(__builtin_amdgcn_readfirstlane(lds_base)), "v"(offset), "s"(uniform_address(base))
+                   : "s"(__builtin_amdgcn_readfirstlane(lds_base)), "v"(src)
                    : "memory");
 }
 
 template <int STAGE>
 __global__ __launch_bounds__(64 * kWideWaves) void tile_wide_kernel(GemmArgs p) {
-  constexpr int NT = kWideNT, MT = kWideMT, R = kWideRing, MW = MT / 2;  // MW: row tiles per wavefront
+  constexpr int NT = kWideNT, MT = kWideMT, R = kWideRing;
   typedef __attribute__((address_space(3))) void* lds_ptr;
   extern __shared__ u32x4 wide_lds[];
   __shared__ int row_flat[kWideRows];
@@ -1416,8 +1403,6 @@ __global__ __launch_bounds__(64 * kWideWaves) void tile_wide_kernel(GemmArgs p) 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int uw = wave >> 1;  // weight unit within the workgroup
-  const int hw = wave & 1;   // this wavefront takes row tiles hw, hw + 2, ...
   const int ln = lane & 15;
   const int lq = lane >> 4;
 
@@ -1427,7 +1412,7 @@ __global__ __launch_bounds__(64 * kWideWaves) void tile_wide_kernel(GemmArgs p) 
   const int nsteps = Kp / 128;
   const int units = STAGE == 0 ? p.ncols / (8 * NT) : p.ncols / (16 * NT);
   const int sstride = split_scale_stride(K);
-  const int unit = blockIdx.x * kWideUnits + uw;
+  const int unit = blockIdx.x * kWideWaves + wave;
   const bool has_unit = unit < units;
 
   struct Rows {
@@ -1435,14 +1420,18 @@ __global__ __launch_bounds__(64 * kWideWaves) void tile_wide_kernel(GemmArgs p) 
     int sb;
   };
   // Memory operations of a wavefront in K step c, in program order (all DMA; j = c % 3):
-  //   2 pieces of its row copies of step c + 2 (the slot was freed by the barrier of
-  //   step c - 1), spread over its row tiles;
+  //   0 .. 4    pieces 3 .. 7 of its row copies of step c + 2 (the slot was freed by the
+  //             barrier of step c - 1);
+  //   5 .. 8    its 4 weight tiles of step c + 3 (their slot was read during step c - 1);
+  //   9 .. 12   j = 0 only: the weight-scale copies of the next group of three steps;
   //   -- the barrier of step c --
-  //   the other 2 pieces of its row copies of step c + 3 and its 2 weight tiles of step
-  //   c + 3, into the slots just freed; j = 0 only: its 2 weight-scale copies and the
-  //   row-scale copy of the next group of three steps.
-  constexpr int kOpsBefore = 2;
-  auto ops_after = [](int j) constexpr { return 4 + (j == 0 ? 3 : 0); };
+  //   13 .. 15  pieces 0 .. 2 of its row copies of step c + 3, into the slot just freed;
+  //   16        j = 0 only: the row scales of the next group.
+  // The operations before the barrier are spread over the row tiles of the step, so that
+  // the memory pipe, which all four wavefronts share, is fed evenly while the MFMAs run.
+  constexpr int kRowsLate = 5, kRowsEarly = 3, kWeightOps = NT;
+  auto ops_before = [](int j) constexpr { return kRowsLate + kWeightOps + (j == 0 ? NT : 0); };
+  auto ops_after = [](int j) constexpr { return kRowsEarly + (j == 0 ? 1 : 0); };
 
   auto segment = [&](const int row0, const int n_rows, const int e) {
     __syncthreads();  // the previous segment is done with row_flat and the rings
@@ -1460,7 +1449,11 @@ __global__ __launch_bounds__(64 * kWideWaves) void tile_wide_kernel(GemmArgs p) 
     // routed rows are a prefix of an expert's rows (padding follows them)
     const int n_live = (wave_valid[0] + wave_valid[1] + 15) >> 4;
     if (n_live == 0) return;  // uniform
-    const int my_live = (n_live - hw + 1) >> 1;  // row tiles hw, hw + 2, ... below n_live
+
+    const uint8_t* w_rows[NT];
+    const uint8_t* s_rows[NT];
+    int col0[NT];
+    unit_tiles<STAGE, NT>(p, e, has_unit ? unit : 0, ln, w_rows, s_rows, col0);
 
     const uint32_t lds_base = (uint32_t)(uintptr_t)(lds_ptr)wide_lds;
     const uint8_t* lds_bytes = reinterpret_cast<const uint8_t*>(wide_lds);
@@ -1470,76 +1463,54 @@ __global__ __launch_bounds__(64 * kWideWaves) void tile_wide_kernel(GemmArgs p) 
     // as 64-byte pieces of 16 rows.  Lane (r, j) = (lane / 8, lane % 8) copies piece
     // j ^ r of row r, so that the 16-byte pieces of a row sit in LDS rotated by the
     // row and the MFMA operand reads (16 rows, one piece each) spread over the banks.
-    // Wavefront w copies row tile w: pieces (term, row half).
-    // (per-lane parts of the addresses are 32-bit offsets: the launcher keeps the split
-    // rows and one expert's weights below 4 GiB)
+    // Wavefront w copies row tiles 2 w and 2 w + 1.
     const int cr = lane >> 3, cj = lane & 7;
-    uint32_t cp_row[2];
+    const uint8_t* cp_row[2][2];
 #pragma unroll
-    for (int rh = 0; rh < 2; ++rh) {
-      const int rl = wave * 16 + rh * 8 + cr;
-      const int f = row_flat[rl];
-      const uint32_t r = f >= 0 ? (uint32_t)(STAGE == 0 ? f / p.top_k : row0 + rl) : 0u;
-      cp_row[rh] = r * (uint32_t)(2 * Kp) + 16u * (uint32_t)(cj ^ cr);
-    }
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+      for (int rh = 0; rh < 2; ++rh) {
+        const int rl = (wave * 2 + i) * 16 + rh * 8 + cr;
+        const int f = row_flat[rl];
+        const size_t r = f >= 0 ? (size_t)(STAGE == 0 ? f / p.top_k : row0 + rl) : 0;
+        cp_row[i][rh] = p.Aq + r * (size_t)(2 * Kp) + 16 * (cj ^ cr);
+      }
     // row scale bytes: 16 per row from byte 12 g on (a group of 3 K steps uses 12);
-    // rows 64 (wave % 2) .. + 63, four times over, so that all wavefronts issue alike
-    uint32_t cp_scale;
+    // rows 64 (wave % 2) .. + 63, twice over, so that all wavefronts issue alike
+    const uint8_t* cp_scale;
     {
       const int rl = (wave & 1) * 64 + lane;
       const int f = row_flat[rl];
-      const uint32_t r = f >= 0 ? (uint32_t)(STAGE == 0 ? f / p.top_k : row0 + rl) : 0u;
-      cp_scale = r * (uint32_t)sstride;
+      const size_t r = f >= 0 ? (size_t)(STAGE == 0 ? f / p.top_k : row0 + rl) : 0;
+      cp_scale = p.As + r * (size_t)sstride;
     }
-    // piece j (0 .. 3) of this wavefront's row copies of a K step
+    // piece j (0 .. 7) of this wavefront's row copies of a K step
     auto copy_row_piece = [&](int step, int slot, int j) {
+      const uint32_t buf = lds_base + (uint32_t)(slot * kWideStepBytes);
       const int k0 = min(step, nsteps - 1) * 128;  // past the end: the last step again
-      const int term = j >> 1, rh = j & 1;
-      const int plane = (wave * 2 + term) * 2 + rh;
-      dma_load_16(p.Aq + (size_t)term * Kp + k0, cp_row[rh],
-                  lds_base + (uint32_t)(slot * kWideStepBytes + plane * 1024));
+      const int i = j >> 2, term = (j >> 1) & 1, rh = j & 1;
+      const int plane = ((wave * 2 + i) * 2 + term) * 2 + rh;
+      dma_load_16(cp_row[i][rh] + (size_t)term * Kp + k0, buf + (uint32_t)(plane * 1024));
     };
     // first byte of the 16 that hold group g's 12 (the last group starts early rather
-    // than read past the row)
+    // than read past the row: see scale_index)
     auto row_scale_start = [&](int g) { return min(g * 12, sstride - 16); };
     auto weight_scale_start = [&](int g) { return min(g * 12, groups - 16); };
     auto copy_row_scales = [&](int g) {
-      dma_load_16(p.As + row_scale_start(g), cp_scale,
+      dma_load_16(cp_scale + row_scale_start(g),
                   lds_base + (uint32_t)(kWideRowScales + (g & 1) * 2048 + (wave & 1) * 1024));
     };
-    // ---- weight copies: a tile's 64 x 16 bytes in lane order; the two wavefronts of a
-    // unit copy tiles 2 hw and 2 hw + 1 each
-    const uint32_t w_ring = lds_base + (uint32_t)(kWideWeights + uw * (R * 4096));
-    const uint32_t ws_ring = lds_base + (uint32_t)(kWideWeightScales + uw * 2048);
-    // (the copies take tiles 2 hw and 2 hw + 1 only: offsets of those two)
-    const size_t rows_w = (size_t)(STAGE == 0 ? 2 * p.ncols : p.ncols);
-    const uint8_t* w_expert = p.W + (size_t)e * rows_w * (size_t)(K / 2);
-    const uint8_t* s_expert = p.Ws + (size_t)e * rows_w * (size_t)groups;
-    uint32_t w_off[2], s_off[2];
-    {
-      const uint8_t* w_rows[NT];
-      const uint8_t* s_rows[NT];
-      int col0[NT];
-      unit_tiles<STAGE, NT>(p, e, has_unit ? unit : 0, ln, w_rows, s_rows, col0);
-#pragma unroll
-      for (int i = 0; i < 2; ++i) {
-        w_off[i] = (uint32_t)(w_rows[2 * hw + i] - w_expert) + 16u * (uint32_t)lq;
-        s_off[i] = (uint32_t)(s_rows[2 * hw + i] - s_expert) + 4u * (uint32_t)lq;
-      }
-    }
-    auto copy_weight_tile = [&](int step, int slot, int i) {
-      // past the end of K: the last group again
-      const int step_c = min(step, nsteps - 1);
-      uint32_t off = w_off[i];
-      if (step_c * 4 + 3 >= groups)  // uniform: the last, partial step
-        off -= 16u * (uint32_t)max(step_c * 4 + lq - (groups - 1), 0);
-      dma_load_16(w_expert + (size_t)step_c * 64, off,
-                  w_ring + (uint32_t)(slot * 4096 + (2 * hw + i) * 1024));
+    // ---- weight copies: a tile's 64 x 16 bytes in lane order, per wavefront
+    const uint32_t w_ring = lds_base + (uint32_t)(kWideWeights + wave * (R * 4096));
+    const uint32_t ws_ring = lds_base + (uint32_t)(kWideWeightScales + wave * 2048);
+    auto copy_weight_tile = [&](int step, int slot, int t) {  // past the end: the last group
+      const int g = min(step * 4 + lq, groups - 1);
+      dma_load_16(w_rows[t] + (size_t)g * 16, w_ring + (uint32_t)(slot * 4096 + t * 1024));
     };
     // lane (n, q) copies dword q of weight row n's 16 scale bytes: LDS [q][n] dwords
-    auto copy_weight_scale_tile = [&](int g, int i) {
-      dma_load_4(s_expert + weight_scale_start(g), s_off[i],
-                 ws_ring + (uint32_t)((g & 1) * 1024 + (2 * hw + i) * 256));
+    auto copy_weight_scale_tile = [&](int g, int t) {
+      const int b0 = weight_scale_start(g) + 4 * lq;
+      dma_load_4(s_rows[t] + b0, ws_ring + (uint32_t)((g & 1) * 1024 + t * 256));
     };
     // operand reads of row tile m of a slot: lane (n, q) takes piece q (q + 4) of row n
     const int rd0 = (ln >> 3) * 1024 + (ln & 7) * 128 + ((lq ^ (ln & 7)) * 16);
@@ -1557,50 +1528,50 @@ __global__ __launch_bounds__(64 * kWideWaves) void tile_wide_kernel(GemmArgs p) 
       return b;
     };
 
-    f32x4 acc[MW][NT];
+    f32x4 acc[MT][NT];
 #pragma unroll
-    for (int m = 0; m < MW; ++m)
+    for (int m = 0; m < MT; ++m)
 #pragma unroll
       for (int t = 0; t < NT; ++t) acc[m][t] = f32x4{0.f, 0.f, 0.f, 0.f};
     uint32_t bad = 0u;
 
-    // The K loop, compiled once per number of row tiles the wavefront multiplies
-    // (LIVE >= my_live: straight-line code; the tiles past my_live are padding rows;
-    // LIVE = 0: a wavefront without a tile, which only copies).
+    // The K loop, compiled once per number of row tiles it multiplies (LIVE >= n_live:
+    // straight-line code, so that the order reads of the next tile -> MFMAs of this
+    // one survives; the tiles between n_live and LIVE are padding rows).
     auto k_loop = [&](auto live_c) {
       constexpr int LIVE = decltype(live_c)::value;
-      // operations of step c, c % 3 = j: k = 0, 1 before the barrier, 2 .. 8 after it
+      // operation k (see above) of K step c, c % 3 = j
       auto issue = [&](int c, int j, int k) {
-        if (k < 2) copy_row_piece(c + 2, (j + 2) % R, 2 + k);
-        else if (k < 4) copy_row_piece(c + R, j, k - 2);
-        else if (k < 6) copy_weight_tile(c + R, j, k - 4);
-        else if (k < 8) { if (j == 0) copy_weight_scale_tile(c / 3 + 1, k - 6); }
+        if (k < 5) copy_row_piece(c + 2, (j + 2) % R, 3 + k);
+        else if (k < 9) copy_weight_tile(c + R, j, k - 5);
+        else if (k < 13) { if (j == 0) copy_weight_scale_tile(c / 3 + 1, k - 9); }
+        else if (k < 16) copy_row_piece(c + R, j, k - 13);
         else if (j == 0) copy_row_scales(c / 3 + 1);
       };
-      // The prologue issues what steps -3, -2, -1 would, less the late row pieces of
-      // step -1.
+      // The prologue issues what steps -3, -2, -1 would, less the row pieces of step -1.
 #pragma unroll
       for (int j = 0; j < R; ++j) {
 #pragma unroll
-        for (int k = (j == 0 ? 2 : 0); k < 9; ++k) issue(j - R, j, k);
+        for (int k = (j == 0 ? 5 : 0); k < 17; ++k) issue(j - R, j, k);
       }
-      // all of step 0's rows, weights and scale bytes have landed once only what was
+      // all of steps 0's rows, weights and scale bytes have landed once only what was
       // issued after the late row pieces of step 0 is outstanding
-      __asm__ volatile("s_waitcnt vmcnt(%0)" ::"n"(ops_after(1) + kOpsBefore + ops_after(2)) : "memory");
+      __asm__ volatile("s_waitcnt vmcnt(%0)" ::"n"(kWeightOps + ops_after(1) + ops_before(2) + ops_after(2))
+                       : "memory");
       __builtin_amdgcn_s_barrier();
       __asm__ volatile("" ::: "memory");
-      Rows cur;
-      if (LIVE > 0) cur = read_rows(0, hw, 0);
+      Rows cur = read_rows(0, 0, 0);
 
       // MFMA operand and scale of weight tile t for K step cc from the weight ring
       // (lanes past K: the step's weights are the last group's again and meet zero
       // rows; their scale byte is made a neutral one).
       auto prep_tile = [&](int cc, int slot, int t, i32x8& wa, int& sa) {
-        const uint8_t* wr = lds_bytes + kWideWeights + uw * (R * 4096) + slot * 4096 + t * 1024;
+        cc = min(cc, nsteps - 1);  // past the end the slot holds the last step again
+        const uint8_t* wr = lds_bytes + kWideWeights + wave * (R * 4096) + slot * 4096 + t * 1024;
         const u32x4 w = *reinterpret_cast<const u32x4*>(wr + lane * 16);
         const int g = cc / 3;  // uniform
         const int idx = min(cc * 4 + lq, groups - 1) - weight_scale_start(g);
-        uint32_t sbw = lds_bytes[kWideWeightScales + uw * 2048 + (g & 1) * 1024 + t * 256 +
+        uint32_t sbw = lds_bytes[kWideWeightScales + wave * 2048 + (g & 1) * 1024 + t * 256 +
                                  (idx >> 2) * 64 + ln * 4 + (idx & 3)];
         if (cc * 4 + lq >= groups) sbw = 127u;
         bad |= (uint32_t)((sbw - kScaleLo) > (kScaleHi - kScaleLo));
@@ -1609,10 +1580,17 @@ __global__ __launch_bounds__(64 * kWideWaves) void tile_wide_kernel(GemmArgs p) 
         sa = (int)sbw - 1;
         wa = fp4_operand(w);
       };
+      // operands of the current step in wa[c % 2], of the next in the other half
+      i32x8 wa[2][NT];
+      int sa[2][NT];
+#pragma unroll
+      for (int t = 0; t < NT; ++t) prep_tile(0, 0, t, wa[0][t], sa[0][t]);
 
-      // One row tile: its MFMAs in two halves (the leading terms, the remainders), an
-      // optional memory operation ahead of each half.
-      auto tile = [&](int mi, const i32x8 (&wa)[NT], const int (&sa)[NT], auto&& op_a, auto&& op_b) {
+      // One row tile: its MFMAs in two halves (the leading terms, the remainders), a
+      // memory operation ahead of each half, the vector work of the region (among it
+      // the preparation of one of the next step's weight tiles) spread between the
+      // MFMAs, during which the matrix pipe is busy anyway.
+      auto tile = [&](int m, const i32x8 (&wa_)[NT], const int (&sa_)[NT], auto&& op_a, auto&& op_b) {
         // (opaque, so that no use of the byte moves up into the previous tile's
         // region and makes the MFMAs there wait for the read)
         int sbh = cur.sb;
@@ -1625,77 +1603,93 @@ __global__ __launch_bounds__(64 * kWideWaves) void tile_wide_kernel(GemmArgs p) 
         // the two MFMAs of an accumulator are kept NT instructions apart
 #pragma unroll
         for (int t = 0; t < NT; ++t)
-          acc[mi][t] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wa[t], bh, acc[mi][t], 4, 0, 0,
-                                                                        sa[t], 0, sbh);
+          acc[m][t] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wa_[t], bh, acc[m][t], 4, 0, 0,
+                                                                       sa_[t], 0, sbh);
         __builtin_amdgcn_sched_barrier(0);
         op_b();
 #pragma unroll
         for (int t = 0; t < NT; ++t)
-          acc[mi][t] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wa[t], bl, acc[mi][t], 4, 0, 0,
-                                                                        sa[t], 0, sbl);
+          acc[m][t] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wa_[t], bl, acc[m][t], 4, 0, 0,
+                                                                       sa_[t], 0, sbl);
         __builtin_amdgcn_sched_barrier(0);
       };
 
+      // Two K steps per pass of the unrolled body would fix c % 2 but not c % 3; six do.
 #pragma unroll 1
-      for (int c0 = 0; c0 < nsteps; c0 += R) {
-        auto step = [&](auto j_c) {
-          constexpr int j = decltype(j_c)::value;
-          constexpr int jn = (j + 1) % R, jp = (j + 2) % R;
+      for (int c0 = 0; c0 < nsteps; c0 += 2 * R) {
+        auto step = [&](auto i_c) {
+          constexpr int i = decltype(i_c)::value;
+          constexpr int j = i % R, jn = (j + 1) % R, jp = (j + 2) % R, cb = i & 1, nb = cb ^ 1;
           // Steps past the last one (nsteps is rounded up here) only keep the sequence
           // of memory operations, hence the counted waits, the same.
-          const int c = c0 + j;
-          const bool work = LIVE > 0 && has_unit && c < nsteps;  // uniform
-          i32x8 wa[NT];
-          int sa[NT];
-          if (work) {
-            // the weights of step c are in LDS since the barrier of step c - 1
+          const int c = c0 + i;
+          const bool work = has_unit && c < nsteps;  // uniform
+          // The weights of step c + 1 (and, when that is a first step of three, their
+          // scale bytes) were issued in step c - 2; since then: the early row pieces of
+          // that step (and row scales) and all of step c - 1.
+          constexpr int kWeightWait = ops_after(jn) + ops_before(jp) + ops_after(jp);
+          __asm__ volatile("s_waitcnt vmcnt(%0)" ::"n"(kWeightWait) : "memory");
+          auto prep_next = [&](int t) { prep_tile(c + 1, jn, t, wa[nb][t], sa[nb][t]); };
+          // operations before the barrier: two per row tile but the last (all at once
+          // where the step has a single tile, or does no arithmetic)
+          constexpr int kBefore = 13;
+          constexpr int kPer = LIVE > 1 ? (kBefore + 2 * (LIVE - 1) - 1) / (2 * (LIVE - 1)) : kBefore;
+          auto before = [&](int first) {
 #pragma unroll
-            for (int t = 0; t < NT; ++t) prep_tile(c, j, t, wa[t], sa[t]);
+            for (int k = first; k < first + kPer; ++k)
+              if (k < kBefore) issue(c, j, k);
+          };
+          if (work && LIVE > 1) {
             __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-            for (int mi = 0; mi + 1 < LIVE; ++mi) {
-              const Rows nxt = read_rows(j, 2 * (mi + 1) + hw, c);
-              __builtin_amdgcn_sched_barrier(0);
-              tile(mi, wa, sa, [&]() { if (mi == 0) issue(c, j, 0); }, [&]() { if (mi == 0) issue(c, j, 1); });
+            for (int m = 0; m + 1 < LIVE; ++m) {
+              const Rows nxt = read_rows(j, m + 1, c);
+              if (m < NT) prep_next(m);
+              tile(m, wa[cb], sa[cb], [&]() { before(2 * m * kPer); }, [&]() { before((2 * m + 1) * kPer); });
               cur = nxt;
             }
-            if (LIVE == 1) { issue(c, j, 0); issue(c, j, 1); }
           } else {
-            issue(c, j, 0);
-            issue(c, j, 1);
+#pragma unroll
+            for (int k = 0; k < kBefore; ++k) issue(c, j, k);
           }
-          // Before the last tile: this wavefront's copies of step c + 1 (the early row
-          // pieces, the weights and, if c + 1 is a first step of three, the scale bytes
-          // from after the barrier of step c - 2; the late row pieces from step c - 1)
-          // have landed and its reads of step c are complete; after the barrier that
-          // holds for every wavefront, so the slots of step c take the copies of step
-          // c + 3 and step c + 1 can be read.  Outstanding may be what followed the
-          // late pieces in step c - 1 and this step's two.
-          constexpr int kWait = ops_after(jp) + kOpsBefore;
-          __asm__ volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(kWait) : "memory");
+          // Before the last tile: this wavefront's row copies of step c + 1 (the early
+          // pieces, with the row scales if c + 1 is a first step of three, from after
+          // the barrier of step c - 2; the late ones from step c - 1) have landed and
+          // its reads of step c are complete; after the barrier that holds for every
+          // wavefront, so slot j takes the early pieces of step c + 3 and step c + 1
+          // can be read.  Outstanding may be what followed the late pieces in step
+          // c - 1 and what this step has issued so far.
+          constexpr int kRowWait = kWeightOps + (jp == 0 ? NT : 0) + ops_after(jp) + ops_before(j);
+          __asm__ volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(kRowWait) : "memory");
           __builtin_amdgcn_s_barrier();
           __asm__ volatile("" ::: "memory");
           if (work) {
-            const Rows nxt = read_rows(jn, hw, c + 1);
             __builtin_amdgcn_sched_barrier(0);
-            tile(LIVE - 1, wa, sa, [&]() { issue(c, j, 2); issue(c, j, 3); issue(c, j, 4); },
-                 [&]() { issue(c, j, 5); issue(c, j, 6); issue(c, j, 7); issue(c, j, 8); });
+            const Rows nxt = read_rows(jn, 0, c + 1);
+#pragma unroll
+            for (int t = LIVE - 1; t < NT; ++t) prep_next(t);
+            tile(LIVE - 1, wa[cb], sa[cb], [&]() { issue(c, j, 13); issue(c, j, 14); },
+                 [&]() { issue(c, j, 15); issue(c, j, 16); });
             cur = nxt;
           } else {
 #pragma unroll
-            for (int k = 2; k < 9; ++k) issue(c, j, k);
+            for (int k = 13; k < 17; ++k) issue(c, j, k);
           }
         };
         step(IntC<0>{});
         step(IntC<1>{});
         step(IntC<2>{});
+        step(IntC<3>{});
+        step(IntC<4>{});
+        step(IntC<5>{});
       }
     };
-    if (my_live > 2) k_loop(IntC<4>{});
-    else if (my_live == 2) k_loop(IntC<2>{});
-    else if (my_live == 1) k_loop(IntC<1>{});
-    else k_loop(IntC<0>{});
-    // the copies past the last step land in the rings, which the epilogue reuses
+    if (n_live > 6) k_loop(IntC<8>{});
+    else if (n_live > 4) k_loop(IntC<6>{});
+    else if (n_live > 2) k_loop(IntC<4>{});
+    else if (n_live == 2) k_loop(IntC<2>{});
+    else k_loop(IntC<1>{});
+    // the copies past the last step land in the ring, which the epilogue reuses
     __builtin_amdgcn_s_waitcnt(vmcnt_only(0));
     __syncthreads();
 
@@ -1714,29 +1708,24 @@ __global__ __launch_bounds__(64 * kWideWaves) void tile_wide_kernel(GemmArgs p) 
     if (STAGE == 1 && p.pos != nullptr && blockIdx.x == 0 && tid < n_rows && row_flat[tid] >= 0)
       p.pos[row_flat[tid]] = row0 + tid;
     if (!has_unit) return;
-    const uint8_t* w_rows[NT];
-    const uint8_t* s_rows[NT];
-    int col0[NT];
-    unit_tiles<STAGE, NT>(p, e, unit, ln, w_rows, s_rows, col0);
 
     // ---- epilogue; the exact path where the fast one was outside its domain -------
     // (a scale byte 0 among a column's blocks marks rows outside the range: the
     // whole unit is redone, from the bf16 rows)
     const bool redo = __ballot(bad != 0u) != 0ull;
 #pragma unroll
-    for (int mi = 0; mi < MW; ++mi) {
-      const int m = 2 * mi + hw;
+    for (int m = 0; m < MT; ++m) {
       if (m >= n_live) break;
       const int flat = row_flat[m * 16 + ln];
       const int srow = row0 + m * 16 + ln;
       if (redo) {
         const uint16_t* a_row = nullptr;
         if (flat >= 0) a_row = p.A + (size_t)(STAGE == 0 ? flat / p.top_k : srow) * (size_t)K;
-        exact_unit_global<NT>(w_rows, s_rows, a_row, K, lane, acc[mi]);
+        exact_unit_global<NT>(w_rows, s_rows, a_row, K, lane, acc[m]);
       }
       if (STAGE == 0) {
         uint2 packed[NT / 2] = {};
-        if (flat >= 0) epilogue_tile<STAGE, NT>(p, e, acc[mi], col0, flat, srow, lq, packed);
+        if (flat >= 0) epilogue_tile<STAGE, NT>(p, e, acc[m], col0, flat, srow, lq, packed);
         if (p.actq != nullptr)
           store_split_act(p, col0[0], col0[1], flat, srow, lane, packed[0], packed[1]);
       } else if (p.y != nullptr) {
@@ -1747,7 +1736,7 @@ __global__ __launch_bounds__(64 * kWideWaves) void tile_wide_kernel(GemmArgs p) 
 #pragma unroll
           for (int t = 0; t < NT; ++t) {
             const int c = col0[t] + 4 * lq;
-            f32x4 v = acc[mi][t];
+            f32x4 v = acc[m][t];
             if (p.bias != nullptr)
               v += *reinterpret_cast<const f32x4*>(p.bias + (size_t)e * (size_t)p.ncols + c);
             *reinterpret_cast<f32x4*>(yrow + c) = v * w;
@@ -1761,7 +1750,7 @@ __global__ __launch_bounds__(64 * kWideWaves) void tile_wide_kernel(GemmArgs p) 
         float* tr = reinterpret_cast<float*>(wide_lds) + (size_t)wave * 16 * kRowStride;
 #pragma unroll
         for (int t = 0; t < NT; ++t)
-          *reinterpret_cast<f32x4*>(tr + ln * kRowStride + t * 16 + 4 * lq) = acc[mi][t];
+          *reinterpret_cast<f32x4*>(tr + ln * kRowStride + t * 16 + 4 * lq) = acc[m][t];
         const int c = col0[0] + lane;  // the unit's 16 NT columns are consecutive
         const float b = p.bias != nullptr ? p.bias[(size_t)e * (size_t)p.ncols + c] : 0.0f;
 #pragma unroll 4
@@ -1941,7 +1930,7 @@ void launch_stage(const GemmArgs& g, const StagePlan& pl, hipStream_t stream) {
     if (configured) {
       const int wide_units = STAGE == 0 ? g.ncols / (8 * kWideNT) : g.ncols / (16 * kWideNT);
       const int win = wide_window_rows(g.block_size);
-      const dim3 grid_wide((wide_units + kWideUnits - 1) / kWideUnits,
+      const dim3 grid_wide((wide_units + kWideWaves - 1) / kWideWaves,
                            (g.num_blocks * g.block_size + win - 1) / win);
       hipLaunchKernelGGL(kern, grid_wide, dim3(64 * kWideWaves), kWideLdsBytes, stream, g);
       return;
