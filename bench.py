@@ -189,8 +189,8 @@ def main():
         # events[1]..[2] bracket the whole fused call (split pass + both grouped GEMMs)
         fused_tflops = flops / (down_avg * 1e-3) / 1e12
         roofline = {
-            "bound": "mfma", "kernel": "vk_hip_fused_moe_mxfp4_ws (split_rows_kernel + tile_ws_kernel<0> "
-                                       "+ tile_ws_kernel<1>)",
+            "bound": "mfma", "kernel": "vk_hip_fused_moe_mxfp4_ex (split_rows_kernel + tile_wide_kernel<0> "
+                                       "+ tile_wide_kernel<1> + combine_kernel)",
             "achieved": fused_tflops, "peak": FP4_PEAK_TFLOPS, "unit": "TFLOP/s",
             "frac": fused_tflops / FP4_PEAK_TFLOPS, "traffic": None,
             "flops_per_launch": flops, "avg_launch_us": down_avg * 1e3,

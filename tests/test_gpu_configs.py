@@ -257,6 +257,20 @@ def test_tile_kernels_block_sizes(bs, use_workspace):
     _check(cfg, T, w, A, lg, sample=32, block_size=bs, use_workspace=use_workspace)
 
 
+def test_second_stage_alone_on_the_workspace_path():
+    """Small hidden, large intermediate, decode-sized batch: the first stage runs as the
+    decode kernel, the second (K = 4096) as the workspace tile kernel, whose split rows
+    are then made from act between the stages."""
+    cfg = synth.MoEConfig("t", 1024, 4096, 8, 2, (32,), "uniform")
+    T, seed = 32, 4200
+    w = _weights(cfg, 4200)
+    A, lg = _inputs(cfg, T, seed)
+    g1, wn = _check(cfg, T, w, A, lg, use_workspace=True)
+    g0, _ = _check(cfg, T, w, A, lg, use_workspace=False, weights_np=wn)
+    m, l2, nf = error_metrics(g1["out"], g0["out"])
+    assert nf and l2 <= 1e-4, (m, l2)
+
+
 def test_workspace_and_plain_entry_points_agree():
     """Large K (the decode kernel does not apply) at a decode-sized batch: the workspace path
     and the plain entry point compute the same layer."""

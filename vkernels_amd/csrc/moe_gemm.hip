@@ -28,9 +28,12 @@
 //
 // stream_resident_kernel: decode (few rows per expert, K up to 3072): HBM
 //   bound, one workgroup per compute unit, all of K of 16 rows resident.
-// tile_ws_kernel / tile_gemm_kernel: everything else: 64 rows x 32 (16) weight
-//   tiles per workgroup, K in chunks of 512, rows pre-split in a caller-owned
-//   workspace / split in-kernel.
+// tile_wide_kernel: everything else when the caller lends a workspace (and K >=
+//   512): 128 rows x 16 weight tiles per workgroup, rows pre-split in the
+//   workspace, operands brought to LDS by DMA three K steps ahead; the second
+//   stage stores its rows and combine_kernel sums them per token.
+// tile_gemm_kernel: everything else without a workspace: 64 rows x 16 weight
+//   tiles per workgroup, K in chunks of 512, rows split in-kernel.
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 #include <stdlib.h>
@@ -1078,248 +1081,6 @@ __global__ __launch_bounds__(64 * kTileWaves, 2) void tile_gemm_kernel(GemmArgs 
 }
 
 // ---------------------------------------------------------------------------
-// Workspace tile kernel: the tile kernel for rows that arrive already split
-// (GemmArgs::Aq / As).  8 wavefronts, 64 sorted rows x 32 weight tiles per
-// workgroup (4 tiles per wavefront), K in chunks of 512.
-//
-// The operand planes of a chunk are copied from the split rows straight into
-// LDS by global_load_lds_dwordx4 (no registers, no LDS stores): one instruction
-// fills one 1 KiB plane, lane (q', n) fetching the 16 bytes k = 16 q' .. of
-// row n.  Two LDS buffers: the copies of chunk c + 1 are issued during the
-// arithmetic of chunk c; before the barrier that ends the chunk every
-// wavefront waits until its copies have landed (s_waitcnt vmcnt with the count
-// of the weight loads issued after them, which stay in flight).  Padding rows
-// copy row 0 (their columns
-// are never stored); K steps past K copy the row's last piece and zero the
-// weight operand instead.
-// ---------------------------------------------------------------------------
-constexpr int kWsWaves = 8, kWsNT = 4;
-constexpr int kWsBufferBytes = kTileSteps * kTileMT * 4 * 1024 + kTileSteps * kTileMT * 64;
-
-template <int STAGE>
-__global__ __launch_bounds__(64 * kWsWaves) void tile_ws_kernel(GemmArgs p) {
-  constexpr int NT = kWsNT, MT = kTileMT, S = kTileSteps;
-  typedef __attribute__((address_space(3))) void* lds_ptr;
-  extern __shared__ u32x4 ws_lds[];  // 2 x { planes [step][row tile][term][half][lane], scales }
-  __shared__ int row_flat[MT * 16];
-
-  if (STAGE == 0) clear_out_share(p);
-  const int tid = threadIdx.x;
-  const int lane = tid & 63;
-  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int ln = lane & 15;
-  const int lq = lane >> 4;
-
-  const int K = p.K;
-  const int groups = K / 32;
-  const int nsteps = (groups + 3) / 4;
-  const int n_chunks = (nsteps + S - 1) / S;
-  const int units = STAGE == 0 ? p.ncols / (8 * NT) : p.ncols / (16 * NT);
-  const int sstride = split_scale_stride(K);
-
-  // ---- the rows of this group ------------------------------------------------
-  const int group_rows = tile_group_rows(p.block_size, 16 * MT);
-  const int row0 = blockIdx.y * group_rows;
-  const int e = p.expert_ids[row0 / p.block_size];
-  if (e < 0) return;
-  if (tid < MT * 16) {
-    int f = -1;
-    if (tid < group_rows) {
-      f = p.sorted_ids[row0 + tid];
-      if (f < 0 || f >= p.n_flat) f = -1;
-    }
-    row_flat[tid] = f;
-  }
-  __syncthreads();
-  uint32_t live = 0u;  // bit m: row tile m has a routed row
-#pragma unroll
-  for (int m = 0; m < MT; ++m) {
-    bool any = false;
-#pragma unroll
-    for (int j = 0; j < 16; ++j) any |= row_flat[m * 16 + j] >= 0;
-    live |= (uint32_t)any << m;
-  }
-  if (live == 0u) return;  // uniform
-  // routed rows are a prefix of a group (padding follows them): tiles 0 .. n_live - 1
-  const int n_live = 32 - __builtin_clz(live);
-
-  // ---- this wavefront's weight tiles --------------------------------------------
-  const int unit = blockIdx.x * kWsWaves + wave;
-  const bool has_unit = unit < units;
-  const uint8_t* w_rows[NT];
-  const uint8_t* s_rows[NT];
-  int col0[NT];
-  unit_tiles<STAGE, NT>(p, e, has_unit ? unit : 0, ln, w_rows, s_rows, col0);
-
-  // ---- copies: this wavefront fills planes 8 wave .. 8 wave + 7 of a chunk -----
-  // plane index = ((step * MT + row tile) * 2 + term) * 2 + half: step = wave / 2,
-  // row tiles 2 (wave % 2) and + 1.  Lane (q', n) = (lane / 16, lane % 16).
-  const int cp_step = wave >> 1;
-  const uint8_t* cp_row[2];
-#pragma unroll
-  for (int i = 0; i < 2; ++i) {
-    const int m = (wave & 1) * 2 + i;
-    const int f = row_flat[m * 16 + ln];
-    const size_t r = f >= 0 ? (size_t)(STAGE == 0 ? f / p.top_k : row0 + m * 16 + ln) : 0;
-    cp_row[i] = p.Aq + r * (size_t)(2 * split_row_k(K));
-  }
-  // scale bytes: wavefronts 0..3 copy step = wave, lane (row tile, n) = (lane / 16, lane % 16)
-  const uint8_t* cp_scale;
-  {
-    const int f = row_flat[lane];
-    const size_t r = f >= 0 ? (size_t)(STAGE == 0 ? f / p.top_k : row0 + lane) : 0;
-    cp_scale = p.As + r * (size_t)sstride;
-  }
-  auto copy_chunk = [&](int c) {
-    uint8_t* buf = reinterpret_cast<uint8_t*>(ws_lds) + (size_t)(c & 1) * kWsBufferBytes;
-    const int k0 = (c * S + cp_step) * 128;
-#pragma unroll
-    for (int j = 0; j < 8; ++j) {
-      const int i = j >> 2, term = (j >> 1) & 1, h = j & 1;
-      const int k = min(k0 + 64 * h + 16 * lq, K - 16);  // past K: the last piece again
-      const int plane = ((cp_step * MT + (wave & 1) * 2 + i) * 2 + term) * 2 + h;
-      __builtin_amdgcn_global_load_lds(cp_row[i] + (size_t)term * split_row_k(K) + k,
-                                       (lds_ptr)(buf + (size_t)plane * 1024), 16, 0, 0);
-    }
-    if (wave < S) {  // 4 scale bytes per (row tile, row): groups 4 step .. 4 step + 3
-      const int g = min((c * S + wave) * 4, sstride - 4);
-      __builtin_amdgcn_global_load_lds(cp_scale + g,
-                                       (lds_ptr)(buf + S * MT * 4096 + (size_t)wave * MT * 64), 4, 0, 0);
-    }
-  };
-
-  // ---- weight pipeline: S steps in flight, independent of the chunks ------------
-  struct Stage {
-    u32x4 w[NT];
-    uint32_t sc[NT];  // the 4 scale bytes of the row for the step's 4 groups
-  };
-  auto load_step = [&](Stage& st, int step) {
-    const int g4 = min(step * 4, groups - 4);  // K >= 128: at least 4 groups
-    const int g = min(step * 4 + lq, groups - 1);
-#pragma unroll
-    for (int t = 0; t < NT; ++t) {
-      st.w[t] = *reinterpret_cast<const u32x4*>(w_rows[t] + (size_t)g * 16);
-      st.sc[t] = *reinterpret_cast<const uint32_t*>(s_rows[t] + g4);
-    }
-  };
-  constexpr int kStepOps = 2 * NT;  // memory instructions of one load_step
-
-  f32x4 acc[MT][NT];
-#pragma unroll
-  for (int m = 0; m < MT; ++m)
-#pragma unroll
-    for (int t = 0; t < NT; ++t) acc[m][t] = f32x4{0.f, 0.f, 0.f, 0.f};
-  uint32_t bad = 0u;
-
-  Stage st[S];
-  copy_chunk(0);
-#pragma unroll
-  for (int s2 = 0; s2 < S; ++s2) load_step(st[s2], s2);
-  __syncthreads();  // chunk 0 has landed (the barrier waits for this wavefront's loads)
-
-#pragma unroll 1
-  for (int c = 0; c < n_chunks; ++c) {
-    // the copies of the next chunk go out first: the S load_steps below are younger
-    if (c + 1 < n_chunks) copy_chunk(c + 1);
-    const u32x4* planes = ws_lds + (size_t)(c & 1) * (kWsBufferBytes / 16);
-    const uint8_t* bsc = reinterpret_cast<const uint8_t*>(planes) + S * MT * 4096;
-#pragma unroll
-    for (int s2 = 0; s2 < S; ++s2) {
-      const int step = c * S + s2;
-      if (step < nsteps && has_unit) {  // uniform
-        const int g = step * 4 + lq;
-        const bool in_k = g < groups;
-        const int g4 = min(step * 4, groups - 4);
-        i32x8 wa[NT];
-        int sa[NT];
-#pragma unroll
-        for (int t = 0; t < NT; ++t) {
-          // the dword holds groups g4 .. g4 + 3; g4 < 4 step only in the last, partial step
-          const uint32_t sbw = in_k ? (st[s2].sc[t] >> (8 * (g - g4))) & 0xFFu : 127u;
-          bad |= (uint32_t)((sbw - kScaleLo) > (kScaleHi - kScaleLo));
-          u32x4 w = st[s2].w[t];
-          if (!in_k) w = u32x4{0u, 0u, 0u, 0u};
-          bad |= fp4x8_nonfinite(w[0]) | fp4x8_nonfinite(w[1]) | fp4x8_nonfinite(w[2]) |
-                 fp4x8_nonfinite(w[3]);
-          sa[t] = (int)sbw - 1;
-          wa[t] = fp4_operand(w);
-        }
-#pragma unroll
-        for (int m = 0; m < MT; ++m) {
-          if (m >= n_live) break;  // uniform
-          const u32x4* pl = planes + (size_t)((s2 * MT + m) * 4) * 64 + lane;
-          const u32x4 h0 = pl[0], h1 = pl[64], l0 = pl[128], l1 = pl[192];
-          int sbh = bsc[(s2 * MT + m) * 64 + ln * 4 + lq];
-          if (!in_k) sbh = 127;
-          bad |= (uint32_t)(sbh == 0);
-          const int sbl = sbh - 4;
-          const i32x8 bh = fp8_operand(h0, h1);
-          const i32x8 bl = fp8_operand(l0, l1);
-          // the two MFMAs of an accumulator are kept NT instructions apart
-#pragma unroll
-          for (int t = 0; t < NT; ++t)
-            acc[m][t] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wa[t], bh, acc[m][t], 4, 0,
-                                                                         0, sa[t], 0, sbh);
-#pragma unroll
-          for (int t = 0; t < NT; ++t)
-            acc[m][t] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wa[t], bl, acc[m][t], 4, 0,
-                                                                         0, sa[t], 0, sbl);
-        }
-      }
-      load_step(st[s2], step + S);  // branch-free: past the end it re-reads the last groups
-    }
-    // This wavefront's copies have landed once at most S * kStepOps memory
-    // instructions are outstanding (they complete in order); a smaller count
-    // only waits longer.  vmcnt is a 6-bit field split over bits 3:0 and 15:14.
-    constexpr int kKeep = S * kStepOps - 4;
-    __builtin_amdgcn_s_waitcnt((kKeep & 15) | ((kKeep >> 4) << 14) | 0x0F70);
-    __builtin_amdgcn_s_barrier();  // everyone's copies of chunk c + 1 are in; chunk c's buffer is free
-    __asm__ volatile("" ::: "memory");
-  }
-  if (!has_unit) return;
-
-  // ---- epilogue; the exact path where the fast one was outside its domain -------
-  // (a scale byte 0 among a column's blocks marks rows outside the range: the
-  // whole unit is redone, from the bf16 rows)
-  const bool redo = __ballot(bad != 0u) != 0ull;
-#pragma unroll
-  for (int m = 0; m < MT; ++m) {
-    if (m >= n_live) break;
-    const int flat = row_flat[m * 16 + ln];
-    const int srow = row0 + m * 16 + ln;
-    if (redo) {
-      const uint16_t* a_row = nullptr;
-      if (flat >= 0) a_row = p.A + (size_t)(STAGE == 0 ? flat / p.top_k : srow) * (size_t)K;
-      exact_unit_global<NT>(w_rows, s_rows, a_row, K, lane, acc[m]);
-    }
-    if (STAGE == 0) {
-      uint2 packed[NT / 2] = {};
-      if (flat >= 0) epilogue_tile<STAGE, NT>(p, e, acc[m], col0, flat, srow, lq, packed);
-      if (p.actq != nullptr)
-        store_split_act(p, col0[0], col0[1], flat, srow, lane, packed[0], packed[1]);
-    } else {
-      // Transposed through this wavefront's part of the (now idle) operand
-      // buffers, so that one atomic instruction adds 64 consecutive columns of
-      // one token instead of 4 x 4 scattered columns of 16 tokens.
-      constexpr int kRowStride = 16 * NT + 4;  // floats; the pad spreads the rows over the banks
-      float* tr = reinterpret_cast<float*>(ws_lds) + (size_t)wave * 16 * kRowStride;
-#pragma unroll
-      for (int t = 0; t < NT; ++t)
-        *reinterpret_cast<f32x4*>(tr + ln * kRowStride + t * 16 + 4 * lq) = acc[m][t];
-      const int c = col0[0] + lane;  // the unit's 16 NT columns are consecutive
-      const float b = p.bias != nullptr ? p.bias[(size_t)e * (size_t)p.ncols + c] : 0.0f;
-#pragma unroll 4
-      for (int i = 0; i < 16; ++i) {
-        const int fi = row_flat[m * 16 + i];  // uniform
-        if (fi < 0) continue;
-        const float v = tr[i * kRowStride + lane];
-        unsafeAtomicAdd(p.out + (size_t)(fi / p.top_k) * (size_t)p.ncols + c, (v + b) * p.topk_w[fi]);
-      }
-    }
-  }
-}
-
-// ---------------------------------------------------------------------------
 // Wide tile kernel (workspace path): up to 128 sorted rows of one expert per
 // workgroup, so that the preparation of a weight tile (code points, inf/NaN and
 // scale-range checks) is shared by 16 MFMAs and every LDS operand read by 8.
@@ -1895,9 +1656,7 @@ StagePlan plan_stage(const GemmArgs& g) {
 }
 
 // The wide kernel takes split rows and reads weight scale bytes sixteen at a time.
-bool wide_kernel_applies(const GemmArgs& g) {
-  return g.Aq != nullptr && g.K >= 512 && env_int("VK_MOE_WIDE", 1) != 0;
-}
+bool wide_kernel_applies(const GemmArgs& g) { return g.Aq != nullptr && g.K >= 512; }
 
 template <int STAGE>
 void launch_stage(const GemmArgs& g, const StagePlan& pl, hipStream_t stream) {
@@ -1933,22 +1692,6 @@ void launch_stage(const GemmArgs& g, const StagePlan& pl, hipStream_t stream) {
       const dim3 grid_wide((wide_units + kWideWaves - 1) / kWideWaves,
                            (g.num_blocks * g.block_size + win - 1) / win);
       hipLaunchKernelGGL(kern, grid_wide, dim3(64 * kWideWaves), kWideLdsBytes, stream, g);
-      return;
-    }
-  }
-  if (g.Aq != nullptr && g.K >= 128) {  // the kernel reads weight scale bytes four at a time
-    auto* kern = tile_ws_kernel<STAGE>;
-    static const bool configured = [kern] {
-      const hipError_t err = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                                 hipFuncAttributeMaxDynamicSharedMemorySize,
-                                                 2 * kWsBufferBytes);
-      if (err != hipSuccess) (void)hipGetLastError();
-      return err == hipSuccess;
-    }();
-    if (configured) {
-      const int ws_units = STAGE == 0 ? g.ncols / (8 * kWsNT) : g.ncols / (16 * kWsNT);
-      const dim3 grid_ws((ws_units + kWsWaves - 1) / kWsWaves, grid.y);
-      hipLaunchKernelGGL(kern, grid_ws, dim3(64 * kWsWaves), 2 * kWsBufferBytes, stream, g);
       return;
     }
   }
@@ -2069,23 +1812,30 @@ void launch_fused_moe(const FusedMoeArgs& a, hipStream_t stream) {
   const StagePlan p0 = plan_stage<0>(g0), p1 = plan_stage<1>(g1);
   Workspace w;
   bool combine = false;
+  bool split_act_between = false;
   if (carve_workspace(a, w) && env_int("VK_MOE_PRESPLIT", 1) != 0) {
-    const bool tile0 = p0.variant != kMoeVariantResident, tile1 = p1.variant != kMoeVariantResident;
-    if (tile0) {
+    // the wide kernel takes a stage that runs as a tile kernel with K >= 512
+    const bool wide0 = p0.variant != kMoeVariantResident && g0.K >= 512;
+    const bool wide1 = p1.variant != kMoeVariantResident && g1.K >= 512;
+    if (wide0) {
       const long long pieces = (long long)a.M * split_row_k(a.hidden) / 8;
       hipLaunchKernelGGL(split_rows_kernel, dim3((unsigned)((pieces + 255) / 256)), dim3(256), 0,
                          stream, a.A, w.a_q, w.a_s, pieces, a.hidden);
       g0.Aq = w.a_q;
       g0.As = w.a_s;
     }
-    if (tile0 && tile1) {
-      g0.actq = w.act_q;
-      g0.actqs = w.act_s;
+    if (wide1) {
       g1.Aq = w.act_q;
       g1.As = w.act_s;
-      // The second stage stores its rows and a last pass sums them per token (the
-      // wide kernel only; far cheaper than one atomic per row and column).
-      if (wide_kernel_applies(g1) && env_int("VK_MOE_COMBINE", 1) != 0) {
+      if (wide0) {  // the first stage's epilogue writes act in split form as well
+        g0.actq = w.act_q;
+        g0.actqs = w.act_s;
+      } else {
+        split_act_between = true;
+      }
+      // The second stage stores its rows and a last pass sums them per token (far
+      // cheaper than one atomic per row and column).
+      if (env_int("VK_MOE_COMBINE", 1) != 0) {
         combine = true;
         g1.y = w.y;
         g1.pos = w.pos;
@@ -2101,6 +1851,11 @@ void launch_fused_moe(const FusedMoeArgs& a, hipStream_t stream) {
     g0.zero_count = (long long)a.M * a.hidden;
   }
   launch_stage<0>(g0, p0, stream);
+  if (split_act_between) {  // every sorted row, padding rows included (they hold old data)
+    const long long pieces = (long long)a.EM * split_row_k(a.ispp) / 8;
+    hipLaunchKernelGGL(split_rows_kernel, dim3((unsigned)((pieces + 255) / 256)), dim3(256), 0, stream,
+                       a.act, w.act_q, w.act_s, pieces, a.ispp);
+  }
   launch_stage<1>(g1, p1, stream);
   if (combine) {
     const dim3 grid((unsigned)((a.hidden / 4 + 255) / 256), (unsigned)a.M);
