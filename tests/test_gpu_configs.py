@@ -257,6 +257,37 @@ def test_tile_kernels_block_sizes(bs, use_workspace):
     _check(cfg, T, w, A, lg, sample=32, block_size=bs, use_workspace=use_workspace)
 
 
+@pytest.mark.parametrize("T,use_workspace", [(16, True), (300, True), (300, False)])
+def test_expert_map_keeps_local_experts_only(T, use_workspace):
+    """Expert parallelism: a rank that owns half the experts (in permuted local order)
+    adds only their contributions; selections of the other experts have no sorted row,
+    which the combine pass of the workspace path must skip."""
+    cfg = synth.CONFIGS["c1"]
+    seed = 1800
+    w = _weights(cfg, 1500)
+    A, lg = _inputs(cfg, T, seed)
+    rng = np.random.default_rng(seed)
+    local_n = cfg.E // 2
+    owned = rng.permutation(cfg.E)[:local_n]
+    emap = np.full(cfg.E, -1, dtype=np.int32)
+    emap[owned] = np.arange(local_n, dtype=np.int32)
+    own = to_dev(owned.astype(np.int64))
+    fe = ve.FusedExperts(w.w13[own].contiguous(), w.w13_scale[own].contiguous(),
+                         w.w2[own].contiguous(), w.w2_scale[own].contiguous(),
+                         expert_map=to_dev(emap), local_num_experts=local_n,
+                         scratch=ve.CaptureSafeScratch())
+    fe.use_workspace = use_workspace
+    ids, tw = fe.route(to_dev(lg), cfg.top_k, True)
+    bs = ve.default_block_size(T, cfg.top_k)
+    out = fe.apply(to_dev(A, torch.bfloat16), ids, tw, block_size=bs).cpu().numpy()
+    ids_np, tw_np = ids.cpu().numpy(), tw.cpu().numpy()
+    tw_local = np.where(emap[ids_np] >= 0, tw_np, np.float32(0.0)).astype(np.float32)
+    c = cpu_layer(A, w.numpy(), ids_np, tw_local, threads=16)
+    max_rel, rel_l2, nf = error_metrics(out, c["out"])
+    print(f"c1 T={T} expert map: max_abs/rms={max_rel:.3e} rel_l2={rel_l2:.3e}")
+    assert nf and max_rel <= MAX_ABS_TOL and rel_l2 <= REL_L2_TOL
+
+
 def test_second_stage_alone_on_the_workspace_path():
     """Small hidden, large intermediate, decode-sized batch: the first stage runs as the
     decode kernel, the second (K = 4096) as the workspace tile kernel, whose split rows

@@ -367,6 +367,10 @@ class FusedExperts:
         self.swiglu_limit, self.beta, self.linear_beta = swiglu_limit, beta, linear_beta
         self.expert_map = expert_map
         self.local_n = _local_n(local_num_experts, E)
+        # routing indices are global: with a map, as many experts as the map has entries
+        self.global_E = E if expert_map is None else int(expert_map.numel())
+        if expert_map is not None and (expert_map.dtype != torch.int32 or not expert_map.is_cuda):
+            raise ValueError("expert_map must be an int32 device tensor")
         self.scratch = scratch or _scratch
 
     # -- routing ------------------------------------------------------------
@@ -388,7 +392,7 @@ class FusedExperts:
         torch = self.torch
         M, top_k = topk_ids.shape
         dev = topk_ids.device
-        num_experts = self.E if num_experts is None else num_experts
+        num_experts = self.global_E if num_experts is None else num_experts
         max_em = _align_em_bound(M, top_k, self.local_n, block_size)
         cap_m = max(M, max_tokens or 0)
         cap = _align_em_bound(cap_m, top_k, self.local_n, block_size)
