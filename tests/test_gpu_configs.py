@@ -215,10 +215,13 @@ def test_config4_ragged(T):
 
 # ---- epilogue variants, block sizes ---------------------------------------------
 
+@pytest.mark.parametrize("T", [8, 200])
 @pytest.mark.parametrize("variant", ["bias", "limit", "situ", "situ_bias"])
-def test_epilogue_variants(variant):
+def test_epilogue_variants(variant, T):
+    """T = 8: the decode kernels; T = 200 (800 routed rows): the tile kernels of the
+    workspace path, whose second stage adds its bias before the combine pass."""
     cfg = synth.CONFIGS["c1"]
-    T, seed = 8, 1500
+    seed = 1500
     w = _weights(cfg, seed)
     A, lg = _inputs(cfg, T, seed)
     b13 = (synth.rand_normal((cfg.E, 2 * cfg.I), seed, 21) * 0.5).astype(np.float32)
@@ -233,7 +236,7 @@ def test_epilogue_variants(variant):
     if "situ" in variant:
         gpu_kw.update(activation="situ", beta=3.0, linear_beta=20.0)
         cpu_kw.update(activation=1, beta=3.0, linear_beta=20.0)
-    _check(cfg, T, w, A, lg, gpu_kw=gpu_kw, cpu_kw=cpu_kw)
+    _check(cfg, T, w, A, lg, sample=32 if T > 32 else None, gpu_kw=gpu_kw, cpu_kw=cpu_kw)
 
 
 @pytest.mark.parametrize("bs", [16, 32, 64, 128])
