@@ -1381,10 +1381,11 @@ __global__ __launch_bounds__(64 * kWideWaves) void tile_wide_kernel(GemmArgs p) 
         auto step = [&](auto i_c) {
           constexpr int i = decltype(i_c)::value;
           constexpr int j = i % R, jn = (j + 1) % R, jp = (j + 2) % R, cb = i & 1, nb = cb ^ 1;
-          // Steps past the last one (nsteps is rounded up here) only keep the sequence
-          // of memory operations, hence the counted waits, the same.
+          // The unrolled body stops at the last step (uniform): a step's counted waits
+          // look back at earlier operations only.
           const int c = c0 + i;
-          const bool work = has_unit && c < nsteps;  // uniform
+          if (c >= nsteps) return;
+          const bool work = has_unit;  // uniform
           // The weights of step c + 1 (and, when that is a first step of three, their
           // scale bytes) were issued in step c - 2; since then: the early row pieces of
           // that step (and row scales) and all of step c - 1.
