@@ -58,8 +58,10 @@ def test_config0_tiny():
     _check_layer(synth.CONFIGS["c0"], 16)
 
 
-@pytest.mark.parametrize("T", [1, 8, 32, 64])
+@pytest.mark.parametrize("T", [1, 8, 32, 64, 128, 129])
 def test_config1_decode(T):
+    """Up to 128 tokens (512 routed rows) the decode kernels run; 129 is the first batch
+    of the tile kernels."""
     _check_layer(synth.CONFIGS["c1"], T)
 
 
