@@ -1656,8 +1656,23 @@ StagePlan plan_stage(const GemmArgs& g) {
   return pl;
 }
 
-// The wide kernel takes split rows and reads weight scale bytes sixteen at a time.
-bool wide_kernel_applies(const GemmArgs& g) { return g.Aq != nullptr && g.K >= 512; }
+// True when the device grants the wide kernel its LDS (asked once per stage).
+template <int STAGE>
+bool wide_kernel_ready() {
+  static const bool configured = [] {
+    const hipError_t err = hipFuncSetAttribute(reinterpret_cast<const void*>(tile_wide_kernel<STAGE>),
+                                               hipFuncAttributeMaxDynamicSharedMemorySize,
+                                               kWideLdsBytes);
+    if (err != hipSuccess) (void)hipGetLastError();  // not left for the next caller to find
+    return err == hipSuccess;
+  }();
+  return configured;
+}
+
+// The wide kernel takes split rows (launch_fused_moe sets Aq only where it applies: a
+// tile-kernel stage with K >= 512, whose scale bytes it reads sixteen at a time, on a
+// device that grants its LDS).
+bool wide_kernel_applies(const GemmArgs& g) { return g.Aq != nullptr; }
 
 template <int STAGE>
 void launch_stage(const GemmArgs& g, const StagePlan& pl, hipStream_t stream) {
@@ -1679,22 +1694,13 @@ void launch_stage(const GemmArgs& g, const StagePlan& pl, hipStream_t stream) {
   const int group_rows = tile_group_rows(g.block_size, 16 * kTileMT);
   const dim3 grid((units + kTileWaves - 1) / kTileWaves, g.num_blocks * (g.block_size / group_rows));
   if (wide_kernel_applies(g)) {
-    auto* kern = tile_wide_kernel<STAGE>;
-    static const bool configured = [kern] {
-      const hipError_t err = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                                 hipFuncAttributeMaxDynamicSharedMemorySize,
-                                                 kWideLdsBytes);
-      if (err != hipSuccess) (void)hipGetLastError();
-      return err == hipSuccess;
-    }();
-    if (configured) {
-      const int wide_units = STAGE == 0 ? g.ncols / (8 * kWideNT) : g.ncols / (16 * kWideNT);
-      const int win = wide_window_rows(g.block_size);
-      const dim3 grid_wide((wide_units + kWideWaves - 1) / kWideWaves,
-                           (g.num_blocks * g.block_size + win - 1) / win);
-      hipLaunchKernelGGL(kern, grid_wide, dim3(64 * kWideWaves), kWideLdsBytes, stream, g);
-      return;
-    }
+    const int wide_units = STAGE == 0 ? g.ncols / (8 * kWideNT) : g.ncols / (16 * kWideNT);
+    const int win = wide_window_rows(g.block_size);
+    const dim3 grid_wide((wide_units + kWideWaves - 1) / kWideWaves,
+                         (g.num_blocks * g.block_size + win - 1) / win);
+    hipLaunchKernelGGL((tile_wide_kernel<STAGE>), grid_wide, dim3(64 * kWideWaves), kWideLdsBytes,
+                       stream, g);
+    return;
   }
   hipLaunchKernelGGL((tile_gemm_kernel<STAGE>), grid, dim3(64 * kTileWaves), 0, stream, g);
 }
@@ -1816,8 +1822,8 @@ void launch_fused_moe(const FusedMoeArgs& a, hipStream_t stream) {
   bool split_act_between = false;
   if (carve_workspace(a, w) && env_int("VK_MOE_PRESPLIT", 1) != 0) {
     // the wide kernel takes a stage that runs as a tile kernel with K >= 512
-    const bool wide0 = p0.variant != kMoeVariantResident && g0.K >= 512;
-    const bool wide1 = p1.variant != kMoeVariantResident && g1.K >= 512;
+    const bool wide0 = p0.variant != kMoeVariantResident && g0.K >= 512 && wide_kernel_ready<0>();
+    const bool wide1 = p1.variant != kMoeVariantResident && g1.K >= 512 && wide_kernel_ready<1>();
     if (wide0) {
       const long long pieces = (long long)a.M * split_row_k(a.hidden) / 8;
       hipLaunchKernelGGL(split_rows_kernel, dim3((unsigned)((pieces + 255) / 256)), dim3(256), 0,
