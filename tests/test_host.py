@@ -48,7 +48,7 @@ def test_default_block_size():
     assert ve.default_block_size(33) == 64 and ve.default_block_size(8192) == 64
     # with top_k: by routed rows, as the library splits its kernels
     assert ve.default_block_size(64, 4) == 16 and ve.default_block_size(128, 4) == 16
-    assert ve.default_block_size(129, 4) == 64 and ve.default_block_size(2047, 8) == 64
+    assert ve.default_block_size(129, 4) == 128 and ve.default_block_size(2047, 8) == 128
     assert ve.default_block_size(2048, 8) == 128 and ve.default_block_size(16384, 8) == 128
 
 

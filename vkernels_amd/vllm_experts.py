@@ -312,15 +312,15 @@ def default_block_size(M: int, top_k: int | None = None) -> int:
     (vllm_experts.py:846).  With top_k given the split follows the library's own
     (M * top_k <= 512 routed rows run the decode kernel, which makes a pass per 16
     rows: blocks of 16 tell it the passes of every expert exactly and pad least;
-    16384 routed rows and more take blocks of 128)."""
+    larger batches take blocks of 128)."""
     if top_k is not None:
         n = M * top_k
         if n <= 512:
             return 16
-        # prefill: a workgroup of the tile kernel takes 128 sorted rows of one expert;
-        # blocks of 128 give every expert windows of its own (measured +8 % at 32768
-        # routed rows over 256 experts)
-        return 128 if n >= 16384 else 64
+        # beyond: a workgroup of the tile kernel takes 128 sorted rows of one expert;
+        # blocks of 128 give every expert windows of its own (measured: 0.5 to 8 %
+        # faster than blocks of 64 from 16 to 770 rows per expert)
+        return 128
     return 16 if M <= 32 else 64
 
 
