@@ -252,7 +252,7 @@ def test_block_sizes(bs):
 @pytest.mark.parametrize("bs", [16, 48, 80, 128])
 def test_tile_kernels_block_sizes(bs, use_workspace):
     """The tile kernels (more than 512 routed rows) with and without the caller's workspace,
-    for block sizes below, above and not dividing their 64-row groups."""
+    for block sizes below, above and not dividing their 64- and 128-row groups."""
     cfg = synth.CONFIGS["c1"]
     T, seed = 160, 1700
     w = _weights(cfg, 1500)
