@@ -163,6 +163,16 @@ void vk_hip_fused_moe_mxfp4_ex(
     void* workspace, size_t workspace_bytes, unsigned flags, void* stream);
 
 /*
+ * Additive: per-device set-up that the launchers otherwise do on their first
+ * call (the dynamic-LDS limits of the GEMM kernels, the developer knobs of the environment).  Call it
+ * once per device, with that device current, before capturing a HIP graph
+ * that contains the entry points of this library.  Returns VK_OK or a
+ * VK_ERROR_* code.  No counterpart in the reference, whose launcher reads its
+ * one environment knob on first use (src/c/vkernels/kernels/moe_fused.hip:1520-1523).
+ */
+int vk_hip_init(void);
+
+/*
  * Additive: the two stages of vk_hip_fused_moe_mxfp4 as separate launches,
  * for callers that place work between them (a tensor-parallel all-reduce, a
  * profiler's events).  Device counterparts of the reference's stage split,

@@ -1,9 +1,13 @@
 """Compile libvkernels_hip.so for gfx950 with hipcc, in-tree.
 
-    python -m vkernels_amd.build
+    python -m vkernels_amd.build [--changed]
 
 hipcc cross-compiles without a GPU.  The library lands next to this file,
-where the loader looks first.
+where the loader looks first.  Every translation unit is compiled to an
+object file under ``vkernels_amd/build/`` (in parallel) and the objects are
+linked; ``--changed`` recompiles only the units whose sources are newer than
+their object (a developer convenience: ``build()`` itself always compiles
+everything).
 """
 from __future__ import annotations
 
@@ -11,11 +15,13 @@ import os
 import shutil
 import subprocess
 import sys
+from concurrent.futures import ThreadPoolExecutor
 from pathlib import Path
 
 PKG = Path(__file__).resolve().parent
 CSRC = PKG / "csrc"
 INCLUDE = PKG.parent / "include"
+OBJ = PKG / "build"
 LIB = PKG / "libvkernels_hip.so"
 
 SOURCES = ["moe_route.hip", "moe_align.hip", "moe_dequant.hip", "moe_gemm.hip", "hip_capi.cpp"]
@@ -23,7 +29,7 @@ SOURCES = ["moe_route.hip", "moe_align.hip", "moe_dequant.hip", "moe_gemm.hip", 
 # -packed-fp32-ops off: hipcc must not form packed fp32 arithmetic.
 # No fast-math: the router relies on IEEE division and un-contracted arithmetic.
 FLAGS = [
-    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared", "-fno-lto",
+    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fno-lto",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
 ]
 
@@ -35,9 +41,7 @@ def hipcc() -> str:
     raise RuntimeError("hipcc not found")
 
 
-def build(verbose: bool = False) -> Path:
-    cmd = [hipcc(), *FLAGS, f"-I{INCLUDE}", f"-I{CSRC}", "-x", "hip",
-           *[str(CSRC / s) for s in SOURCES], "-o", str(LIB)]
+def _run(cmd, verbose):
     if verbose:
         print(" ".join(cmd), flush=True)
     res = subprocess.run(cmd, capture_output=True, text=True)
@@ -47,8 +51,33 @@ def build(verbose: bool = False) -> Path:
         raise RuntimeError(f"hipcc failed:\n{err}")
     if verbose and err.strip():
         print(err, file=sys.stderr)
+
+
+def _stale(src: Path, obj: Path) -> bool:
+    if not obj.is_file():
+        return True
+    deps = [src, *CSRC.glob("*.hpp"), *INCLUDE.glob("*.h")]
+    return any(d.stat().st_mtime > obj.stat().st_mtime for d in deps)
+
+
+def build(verbose: bool = False, only_changed: bool = False) -> Path:
+    cc = hipcc()
+    OBJ.mkdir(exist_ok=True)
+    jobs = []
+    objects = []
+    for name in SOURCES:
+        src, obj = CSRC / name, OBJ / (Path(name).stem + ".o")
+        objects.append(str(obj))
+        if only_changed and not _stale(src, obj):
+            continue
+        jobs.append([cc, *FLAGS, f"-I{INCLUDE}", f"-I{CSRC}", "-x", "hip", "-c", str(src),
+                     "-o", str(obj)])
+    with ThreadPoolExecutor(max_workers=min(8, max(1, len(jobs)))) as pool:
+        list(pool.map(lambda cmd: _run(cmd, verbose), jobs))
+    _run([cc, "--offload-arch=gfx950", "-shared", "-fPIC", "-fno-lto", *objects, "-o", str(LIB)],
+         verbose)
     return LIB
 
 
 if __name__ == "__main__":
-    print(build(verbose=True))
+    print(build(verbose=True, only_changed="--changed" in sys.argv[1:]))

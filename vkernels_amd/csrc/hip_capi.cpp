@@ -110,6 +110,38 @@ void vk_hip_fused_moe_mxfp4_ws(
                             workspace_bytes, 0u, stream);
 }
 
+namespace {
+
+// After the launches of a void entry point: a launch the runtime refused is
+// recorded for vk_last_error() (peeked, so hipGetLastError() still reports it
+// to the caller as the conventions promise).
+void note_launch_error(const char* who) {
+  const hipError_t err = hipPeekAtLastError();
+  if (err != hipSuccess)
+    vk_set_last_error(VK_ERROR_INTERNAL,
+                      (std::string(who) + ": launch failed: " + hipGetErrorString(err)).c_str());
+}
+
+vk::FusedMoeArgs fused_args(
+    const uint16_t* A, const uint8_t* w13, const uint8_t* w13_scale,
+    const uint8_t* w2, const uint8_t* w2_scale, const float* topk_w,
+    uint16_t* act_scratch, float* out, int M, int hidden, int ispp, int top_k,
+    const int32_t* sorted_ids, const int32_t* expert_ids, int EM, float swiglu_limit,
+    int activation, float beta, float linear_beta, const float* b13, const float* b2,
+    int block_size, void* workspace, size_t workspace_bytes, unsigned flags) {
+  vk::FusedMoeArgs a{};
+  a.workspace = workspace; a.workspace_bytes = workspace_bytes; a.flags = flags;
+  a.A = A; a.w13 = w13; a.w13_scale = w13_scale; a.w2 = w2; a.w2_scale = w2_scale;
+  a.topk_w = topk_w; a.act = act_scratch; a.out = out;
+  a.sorted_ids = sorted_ids; a.expert_ids = expert_ids; a.b13 = b13; a.b2 = b2;
+  a.M = M; a.hidden = hidden; a.ispp = ispp; a.top_k = top_k; a.EM = EM;
+  a.block_size = block_size; a.swiglu_limit = swiglu_limit; a.beta = beta;
+  a.linear_beta = linear_beta; a.activation = activation;
+  return a;
+}
+
+}  // namespace
+
 void vk_hip_fused_moe_mxfp4_ex(
     const uint16_t* A, const uint8_t* w13, const uint8_t* w13_scale,
     const uint8_t* w2, const uint8_t* w2_scale,
@@ -123,16 +155,19 @@ void vk_hip_fused_moe_mxfp4_ex(
     void* workspace, size_t workspace_bytes, unsigned flags, void* stream) {
   (void)topk_ids;
   if (M <= 0 || EM <= 0) return;  // nothing routed: out is left as it is
-  vk::FusedMoeArgs a{};
-  a.workspace = workspace; a.workspace_bytes = workspace_bytes; a.flags = flags;
-  a.A = A; a.w13 = w13; a.w13_scale = w13_scale; a.w2 = w2; a.w2_scale = w2_scale;
-  a.topk_w = topk_w; a.act = act_scratch; a.out = out;
-  a.sorted_ids = sorted_ids; a.expert_ids = expert_ids; a.b13 = b13; a.b2 = b2;
-  a.M = M; a.hidden = hidden; a.ispp = ispp; a.top_k = top_k; a.EM = EM;
-  a.block_size = block_size; a.swiglu_limit = swiglu_limit; a.beta = beta;
-  a.linear_beta = linear_beta; a.activation = activation;
+  const vk::FusedMoeArgs a =
+      fused_args(A, w13, w13_scale, w2, w2_scale, topk_w, act_scratch, out, M, hidden, ispp,
+                 top_k, sorted_ids, expert_ids, EM, swiglu_limit, activation, beta, linear_beta,
+                 b13, b2, block_size, workspace, workspace_bytes, flags);
   if (!layer_args_ok("vk_hip_fused_moe_mxfp4", true, true, a)) return;
   vk::launch_fused_moe(a, static_cast<hipStream_t>(stream));
+  note_launch_error("vk_hip_fused_moe_mxfp4");
+}
+
+int vk_hip_init(void) {
+  if (!vk::prepare_moe_kernels())
+    return fail(VK_ERROR_UNSUPPORTED, "vk_hip_init: the device refuses a kernel its LDS");
+  return VK_OK;
 }
 
 void vk_hip_moe_gateup_mxfp4(
@@ -150,6 +185,7 @@ void vk_hip_moe_gateup_mxfp4(
   a.linear_beta = linear_beta; a.activation = activation;
   if (!layer_args_ok("vk_hip_moe_gateup_mxfp4", true, false, a)) return;
   vk::launch_moe_gateup(a, static_cast<hipStream_t>(stream));
+  note_launch_error("vk_hip_moe_gateup_mxfp4");
 }
 
 void vk_hip_moe_down_mxfp4(
@@ -166,6 +202,7 @@ void vk_hip_moe_down_mxfp4(
   a.block_size = block_size;
   if (!layer_args_ok("vk_hip_moe_down_mxfp4", false, true, a)) return;
   vk::launch_moe_down(a, static_cast<hipStream_t>(stream));
+  note_launch_error("vk_hip_moe_down_mxfp4");
 }
 
 int vk_hip_moe_align_block_size(

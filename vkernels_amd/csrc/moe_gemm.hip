@@ -1549,18 +1549,19 @@ __global__ __launch_bounds__(256) void fill_i32_kernel(int32_t* dst, int32_t val
 // (selections whose expert is not local have pos < 0).  One thread per 4 columns.
 __global__ __launch_bounds__(256) void combine_kernel(const float* __restrict__ y,
                                                       const int32_t* __restrict__ pos,
-                                                      float* __restrict__ out, int top_k, int ncols,
-                                                      int overwrite) {
-  const int t = blockIdx.y;
+                                                      float* __restrict__ out, int M, int top_k,
+                                                      int ncols, int overwrite) {
   const int c = (blockIdx.x * blockDim.x + threadIdx.x) * 4;
   if (c >= ncols) return;
-  f32x4 sum = {0.f, 0.f, 0.f, 0.f};
-  for (int s = 0; s < top_k; ++s) {
-    const int r = pos[t * top_k + s];  // uniform
-    if (r >= 0) sum += *reinterpret_cast<const f32x4*>(y + (size_t)r * (size_t)ncols + c);
+  for (int t = blockIdx.y; t < M; t += gridDim.y) {  // grid.y is capped at 65535
+    f32x4 sum = {0.f, 0.f, 0.f, 0.f};
+    for (int s = 0; s < top_k; ++s) {
+      const int r = pos[t * top_k + s];  // uniform
+      if (r >= 0) sum += *reinterpret_cast<const f32x4*>(y + (size_t)r * (size_t)ncols + c);
+    }
+    f32x4* o = reinterpret_cast<f32x4*>(out + (size_t)t * (size_t)ncols + c);
+    *o = overwrite ? sum : *o + sum;
   }
-  f32x4* o = reinterpret_cast<f32x4*>(out + (size_t)t * (size_t)ncols + c);
-  *o = overwrite ? sum : *o + sum;
 }
 
 // bf16 rows [R, K] -> split rows (see GemmArgs::Aq), zero blocks between K and
@@ -1593,11 +1594,6 @@ __global__ __launch_bounds__(256) void split_rows_kernel(const uint16_t* __restr
   }
 }
 
-int env_int(const char* name, int fallback) {
-  const char* v = getenv(name);
-  return (v != nullptr && *v != 0) ? atoi(v) : fallback;
-}
-
 int num_compute_units() {
   static const int cus = [] {
     int dev = 0, n = 0;
@@ -1609,25 +1605,61 @@ int num_compute_units() {
   return cus;
 }
 
+// Developer overrides of the launch shapes, read from the environment once per
+// process (0 / negative = the library's own choice).  VK_MOE_VARIANT, VK_MOE_NT,
+// VK_MOE_DEPTH, VK_MOE_WAVES: shape of the resident kernel; VK_MOE_WGS: its grid;
+// VK_MOE_PRESPLIT=0 / VK_MOE_COMBINE=0: ignore the workspace / add with atomics.
+struct DebugKnobs {
+  int variant, nt, depth, waves, wgs, presplit, combine;
+};
+
+const DebugKnobs& debug_knobs() {
+  static const DebugKnobs knobs = [] {
+    auto env_int = [](const char* name, int fallback) {
+      const char* v = getenv(name);
+      return (v != nullptr && *v != 0) ? atoi(v) : fallback;
+    };
+    DebugKnobs k;
+    k.variant = env_int("VK_MOE_VARIANT", -1);
+    k.nt = env_int("VK_MOE_NT", 0);
+    k.depth = env_int("VK_MOE_DEPTH", 0);
+    k.waves = env_int("VK_MOE_WAVES", 0);
+    k.wgs = env_int("VK_MOE_WGS", num_compute_units());
+    k.presplit = env_int("VK_MOE_PRESPLIT", 1);
+    k.combine = env_int("VK_MOE_COMBINE", 1);
+    return k;
+  }();
+  return knobs;
+}
+
 constexpr size_t kResidentLdsLimit = 150 * 1024;  // dynamic LDS the resident kernel may ask for
 
-// False when the device refuses the kernel its dynamic LDS (the caller then
-// takes the other variant).
+// True when the device grants the kernel its dynamic LDS (asked once per kernel;
+// a refusal makes the caller take the other variant).
 template <int STAGE, int WAVES, int NT, int D>
-bool launch_resident(const GemmArgs& g, size_t lds, hipStream_t stream) {
-  auto* kern = stream_resident_kernel<STAGE, WAVES, NT, D>;
-  static const bool configured = [kern] {
-    const hipError_t err = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                               hipFuncAttributeMaxDynamicSharedMemorySize,
-                                               (int)kResidentLdsLimit);
+bool resident_kernel_ready() {
+  static const bool configured = [] {
+    const hipError_t err = hipFuncSetAttribute(
+        reinterpret_cast<const void*>(stream_resident_kernel<STAGE, WAVES, NT, D>),
+        hipFuncAttributeMaxDynamicSharedMemorySize, (int)kResidentLdsLimit);
     if (err != hipSuccess) (void)hipGetLastError();  // not left for the next caller to find
     return err == hipSuccess;
   }();
-  if (!configured) return false;
-  const int wgs = env_int("VK_MOE_WGS", num_compute_units());
-  hipLaunchKernelGGL(kern, dim3(wgs), dim3(64 * WAVES), lds, stream, g);
+  return configured;
+}
+
+template <int STAGE, int WAVES, int NT, int D>
+bool launch_resident(const GemmArgs& g, size_t lds, hipStream_t stream) {
+  if (!resident_kernel_ready<STAGE, WAVES, NT, D>()) return false;
+  hipLaunchKernelGGL((stream_resident_kernel<STAGE, WAVES, NT, D>), dim3(debug_knobs().wgs),
+                     dim3(64 * WAVES), lds, stream, g);
   return true;
 }
+
+// The instantiations of the resident kernel: X(stage, wavefronts, tiles, depth).
+#define VK_RESIDENT_VARIANTS(X) \
+  X(0, 8, 2, 2) X(0, 8, 2, 4) X(0, 8, 2, 6) X(0, 4, 2, 4) X(0, 4, 2, 8) \
+  X(1, 8, 2, 4) X(1, 8, 1, 4) X(1, 8, 1, 6) X(1, 8, 1, 8) X(1, 8, 1, 12)
 
 // Launch shape of one stage.  variant kMoeVariantLds = the tile kernel.
 struct StagePlan {
@@ -1639,10 +1671,11 @@ template <int STAGE>
 StagePlan plan_stage(const GemmArgs& g) {
   const MoeTile tile = pick_moe_tile(g.n_flat, g.K, g.ncols, STAGE);
   StagePlan pl;
-  pl.variant = env_int("VK_MOE_VARIANT", tile.variant);
-  pl.nt = env_int("VK_MOE_NT", tile.nt);
-  pl.depth = env_int("VK_MOE_DEPTH", tile.depth);
-  pl.waves = env_int("VK_MOE_WAVES", tile.waves);
+  const DebugKnobs& knobs = debug_knobs();
+  pl.variant = knobs.variant >= 0 ? knobs.variant : tile.variant;
+  pl.nt = knobs.nt > 0 ? knobs.nt : tile.nt;
+  pl.depth = knobs.depth > 0 ? knobs.depth : tile.depth;
+  pl.waves = knobs.waves > 0 ? knobs.waves : tile.waves;
   const int groups = g.K / 32;
   const int nsteps = (groups + 3) / 4;
   // operand planes + block scales + one weight-scale region per wavefront
@@ -1677,17 +1710,13 @@ bool wide_kernel_applies(const GemmArgs& g) { return g.Aq != nullptr; }
 template <int STAGE>
 void launch_stage(const GemmArgs& g, const StagePlan& pl, hipStream_t stream) {
   if (pl.variant == kMoeVariantResident) {
-#define VK_RESIDENT(W_, NT_, D_) \
-  if (pl.waves == W_ && pl.nt == NT_ && pl.depth == D_ && \
-      launch_resident<STAGE, W_, NT_, D_>(g, pl.resident_lds, stream)) \
-    return
-    if constexpr (STAGE == 0) {
-      VK_RESIDENT(8, 2, 2); VK_RESIDENT(8, 2, 4); VK_RESIDENT(8, 2, 6);
-      VK_RESIDENT(4, 2, 4); VK_RESIDENT(4, 2, 8);
-    } else {
-      VK_RESIDENT(8, 2, 4); VK_RESIDENT(8, 1, 4); VK_RESIDENT(8, 1, 6); VK_RESIDENT(8, 1, 8);
-      VK_RESIDENT(8, 1, 12);
-    }
+#define VK_RESIDENT(S_, W_, NT_, D_) \
+  if constexpr (STAGE == S_) { \
+    if (pl.waves == W_ && pl.nt == NT_ && pl.depth == D_ && \
+        launch_resident<S_, W_, NT_, D_>(g, pl.resident_lds, stream)) \
+      return; \
+  }
+    VK_RESIDENT_VARIANTS(VK_RESIDENT)
 #undef VK_RESIDENT
   }
   const int units = STAGE == 0 ? g.ncols / (8 * kTileNT) : g.ncols / (16 * kTileNT);
@@ -1797,6 +1826,15 @@ size_t fused_moe_workspace_bytes(int M, int hidden, int ispp, int top_k, int EM)
   return workspace_layout(M, hidden, ispp, top_k, EM).total();
 }
 
+bool prepare_moe_kernels() {
+  bool ok = wide_kernel_ready<0>() && wide_kernel_ready<1>();
+#define VK_READY(S_, W_, NT_, D_) ok = resident_kernel_ready<S_, W_, NT_, D_>() && ok;
+  VK_RESIDENT_VARIANTS(VK_READY)
+#undef VK_READY
+  (void)debug_knobs();
+  return ok;
+}
+
 void launch_moe_gateup(const FusedMoeArgs& a, hipStream_t stream) {
   if (a.M <= 0 || a.EM <= 0 || a.block_size <= 0) return;
   const GemmArgs g = gateup_args(a);
@@ -1820,7 +1858,7 @@ void launch_fused_moe(const FusedMoeArgs& a, hipStream_t stream) {
   Workspace w;
   bool combine = false;
   bool split_act_between = false;
-  if (carve_workspace(a, w) && env_int("VK_MOE_PRESPLIT", 1) != 0) {
+  if (carve_workspace(a, w) && debug_knobs().presplit != 0) {
     // the wide kernel takes a stage that runs as a tile kernel with K >= 512
     const bool wide0 = p0.variant != kMoeVariantResident && g0.K >= 512 && wide_kernel_ready<0>();
     const bool wide1 = p1.variant != kMoeVariantResident && g1.K >= 512 && wide_kernel_ready<1>();
@@ -1842,7 +1880,7 @@ void launch_fused_moe(const FusedMoeArgs& a, hipStream_t stream) {
       }
       // The second stage stores its rows and a last pass sums them per token (far
       // cheaper than one atomic per row and column).
-      if (env_int("VK_MOE_COMBINE", 1) != 0) {
+      if (debug_knobs().combine != 0) {
         combine = true;
         g1.y = w.y;
         g1.pos = w.pos;
@@ -1865,8 +1903,8 @@ void launch_fused_moe(const FusedMoeArgs& a, hipStream_t stream) {
   }
   launch_stage<1>(g1, p1, stream);
   if (combine) {
-    const dim3 grid((unsigned)((a.hidden / 4 + 255) / 256), (unsigned)a.M);
-    hipLaunchKernelGGL(combine_kernel, grid, dim3(256), 0, stream, w.y, w.pos, a.out, a.top_k,
+    const dim3 grid((unsigned)((a.hidden / 4 + 255) / 256), (unsigned)(a.M < 65535 ? a.M : 65535));
+    hipLaunchKernelGGL(combine_kernel, grid, dim3(256), 0, stream, w.y, w.pos, a.out, a.M, a.top_k,
                        a.hidden, overwrite ? 1 : 0);
   }
 }

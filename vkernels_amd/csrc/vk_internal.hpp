@@ -49,4 +49,9 @@ void launch_fused_moe(const FusedMoeArgs& a, hipStream_t stream);
 void launch_moe_gateup(const FusedMoeArgs& a, hipStream_t stream);
 void launch_moe_down(const FusedMoeArgs& a, hipStream_t stream);
 
+// Per-kernel set-up that the launchers otherwise do on their first call (the
+// dynamic-LDS limits of the GEMM kernels), for callers that want it done before
+// a graph capture.  False when the device refuses a limit.
+bool prepare_moe_kernels();
+
 }  // namespace vk
