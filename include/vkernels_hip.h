@@ -164,13 +164,51 @@ void vk_hip_fused_moe_mxfp4_ex(
 
 /*
  * Additive: per-device set-up that the launchers otherwise do on their first
- * call (the dynamic-LDS limits of the GEMM kernels, the developer knobs of the environment).  Call it
+ * call (the dynamic-LDS limits of the GEMM kernels, the device address of the
+ * library's scratch array, the developer knobs of the environment).  Call it
  * once per device, with that device current, before capturing a HIP graph
  * that contains the entry points of this library.  Returns VK_OK or a
  * VK_ERROR_* code.  No counterpart in the reference, whose launcher reads its
  * one environment knob on first use (src/c/vkernels/kernels/moe_fused.hip:1520-1523).
  */
 int vk_hip_init(void);
+
+/*
+ * Additive: vk_hip_fused_moe_mxfp4_ex for callers that cannot allocate device
+ * memory and have no workspace to lend: code under HIP graph capture, tight
+ * serving loops, harnesses that forbid hipMalloc.  It has no counterpart in
+ * the reference.  The workspace is an array of
+ * vk_hip_static_scratch_bytes() (64 MiB) that the library itself holds in
+ * device memory on every GPU it runs on, from the loading of its code until
+ * the process ends; the call allocates nothing, frees nothing and does not
+ * synchronise.  Arguments and results are those of vk_hip_fused_moe_mxfp4_ex
+ * given a workspace of the size it asks for (the same kernels run).
+ *
+ * Returns VK_OK, VK_ERROR_INVALID_ARGUMENT for a contract violation, or
+ * VK_ERROR_OUT_OF_RANGE when vk_hip_fused_moe_mxfp4_workspace_bytes(M, hidden,
+ * ispp, top_k, EM) exceeds the array (nothing is launched; use
+ * vk_hip_fused_moe_mxfp4_ws with a workspace of the caller's).
+ *
+ * All calls on one GPU share that GPU's array: calls that may overlap on one
+ * GPU (different streams, different threads) race and must be ordered by the
+ * caller.  The array keeps the last call's contents; nothing in it has to start
+ * at zero, because every byte a call reads it has written before.  The array's
+ * device address is looked up on the first call on a device (or by
+ * vk_hip_init), which may load the library's code onto that device.
+ */
+size_t vk_hip_static_scratch_bytes(void);
+
+int vk_hip_fused_moe_mxfp4_static(
+    const uint16_t* A, const uint8_t* w13, const uint8_t* w13_scale,
+    const uint8_t* w2, const uint8_t* w2_scale,
+    const int32_t* topk_ids, const float* topk_w,
+    uint16_t* act_scratch, float* out,
+    int M, int hidden, int ispp, int top_k,
+    const int32_t* sorted_ids, const int32_t* expert_ids,
+    int EM, float swiglu_limit,
+    int activation, float beta, float linear_beta,
+    const float* b13, const float* b2, int block_size,
+    unsigned flags, void* stream);
 
 /*
  * Additive: the two stages of vk_hip_fused_moe_mxfp4 as separate launches,

@@ -24,7 +24,8 @@ INCLUDE = PKG.parent / "include"
 OBJ = PKG / "build"
 LIB = PKG / "libvkernels_hip.so"
 
-SOURCES = ["moe_route.hip", "moe_align.hip", "moe_dequant.hip", "moe_gemm.hip", "hip_capi.cpp"]
+SOURCES = ["moe_route.hip", "moe_align.hip", "moe_dequant.hip", "moe_gemm.hip", "static_scratch.hip",
+           "hip_capi.cpp"]
 
 # -packed-fp32-ops off: hipcc must not form packed fp32 arithmetic.
 # No fast-math: the router relies on IEEE division and un-contracted arithmetic.

@@ -165,8 +165,57 @@ void vk_hip_fused_moe_mxfp4_ex(
 }
 
 int vk_hip_init(void) {
+  hipError_t err = hipSuccess;
+  if (vk::static_scratch_ptr(&err) == nullptr)
+    return fail(VK_ERROR_INTERNAL,
+                (std::string("vk_hip_init: the library's scratch array has no device address: ") +
+                 hipGetErrorString(err)).c_str());
   if (!vk::prepare_moe_kernels())
     return fail(VK_ERROR_UNSUPPORTED, "vk_hip_init: the device refuses a kernel its LDS");
+  return VK_OK;
+}
+
+size_t vk_hip_static_scratch_bytes(void) { return vk::static_scratch_bytes(); }
+
+int vk_hip_fused_moe_mxfp4_static(
+    const uint16_t* A, const uint8_t* w13, const uint8_t* w13_scale,
+    const uint8_t* w2, const uint8_t* w2_scale,
+    const int32_t* topk_ids, const float* topk_w,
+    uint16_t* act_scratch, float* out,
+    int M, int hidden, int ispp, int top_k,
+    const int32_t* sorted_ids, const int32_t* expert_ids,
+    int EM, float swiglu_limit,
+    int activation, float beta, float linear_beta,
+    const float* b13, const float* b2, int block_size,
+    unsigned flags, void* stream) {
+  (void)topk_ids;
+  if (M <= 0 || EM <= 0) return VK_OK;  // nothing routed: out is left as it is
+  vk::FusedMoeArgs a =
+      fused_args(A, w13, w13_scale, w2, w2_scale, topk_w, act_scratch, out, M, hidden, ispp,
+                 top_k, sorted_ids, expert_ids, EM, swiglu_limit, activation, beta, linear_beta,
+                 b13, b2, block_size, nullptr, 0, flags);
+  if (!layer_args_ok("vk_hip_fused_moe_mxfp4_static", true, true, a))
+    return VK_ERROR_INVALID_ARGUMENT;
+  const size_t need = vk::fused_moe_workspace_bytes(M, hidden, ispp, top_k, EM);
+  if (need > vk::static_scratch_bytes())
+    return fail(VK_ERROR_OUT_OF_RANGE,
+                ("vk_hip_fused_moe_mxfp4_static: this call needs " + std::to_string(need) +
+                 " bytes of scratch, the library holds " +
+                 std::to_string(vk::static_scratch_bytes()) +
+                 "; use vk_hip_fused_moe_mxfp4_ws with a caller-owned workspace").c_str());
+  hipError_t err = hipSuccess;
+  a.workspace = vk::static_scratch_ptr(&err);
+  if (a.workspace == nullptr)
+    return fail(VK_ERROR_INTERNAL,
+                (std::string("vk_hip_fused_moe_mxfp4_static: the library's scratch array has no "
+                             "device address: ") + hipGetErrorString(err)).c_str());
+  a.workspace_bytes = vk::static_scratch_bytes();
+  vk::launch_fused_moe(a, static_cast<hipStream_t>(stream));
+  const hipError_t launched = hipPeekAtLastError();
+  if (launched != hipSuccess)
+    return fail(VK_ERROR_INTERNAL,
+                (std::string("vk_hip_fused_moe_mxfp4_static: launch failed: ") +
+                 hipGetErrorString(launched)).c_str());
   return VK_OK;
 }
 

@@ -54,4 +54,10 @@ void launch_moe_down(const FusedMoeArgs& a, hipStream_t stream);
 // a graph capture.  False when the device refuses a limit.
 bool prepare_moe_kernels();
 
+// The library-held workspace of vk_hip_fused_moe_mxfp4_static
+// (static_scratch.hip): its size, and the address of the current device's copy.
+constexpr size_t kStaticScratchBytes = (size_t)64 << 20;
+size_t static_scratch_bytes();
+void* static_scratch_ptr(hipError_t* err);
+
 }  // namespace vk
