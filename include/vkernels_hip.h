@@ -163,6 +163,56 @@ void vk_hip_fused_moe_mxfp4_ex(
     void* workspace, size_t workspace_bytes, unsigned flags, void* stream);
 
 /*
+ * Additive: weights prepacked at load time for the prefill-sized kernels, in
+ * the spirit of the reference's `kmajor` layout option
+ * (src/c/vkernels/kernels/moe_fused.hpp:315-343): a caller that keeps a second
+ * copy of the expert weights in the layout the matrix cores consume gets the
+ * FP4-rate path for batches of more than 512 routed rows.
+ *
+ * vk_hip_moe_prepack_weights rewrites [num_experts, rows, K/2] packed E2M1
+ * codes and [num_experts, rows, K/32] ue8m0 scales (stage 0: w13 with rows =
+ * 2*ispp, gate rows first, K = hidden; stage 1: w2 with rows = hidden, K =
+ * ispp) into `packed`, vk_hip_moe_prepack_bytes(...) bytes of 16-byte aligned
+ * device memory: per expert, per unit of 128 weight rows (stage 0: 64 gate
+ * rows and the 64 up rows of the same columns), per K step of 128, the unit's
+ * 8 operand tiles of 64 lanes x 16 bytes in lane order (codes moved onto the
+ * OCP FP4 code points), then 8 scale bytes per lane (decremented by one); then
+ * one flag byte per unit marking units whose weights hold an inf/NaN code or a
+ * scale byte outside [64, 190] (computed from the raw weights by the exact
+ * path).  Returns VK_OK or a VK_ERROR_* code.
+ *
+ * vk_hip_fused_moe_mxfp4_prepacked is vk_hip_fused_moe_mxfp4_ex with the two
+ * packed buffers (NULL, NULL = vk_hip_fused_moe_mxfp4_ex exactly) and the
+ * number of experts in the weight tensors.  The raw weights are still required:
+ * decode-sized calls and the exact path read them.  On the packed path the bf16
+ * activations are multiplied as a sum of three FP6 (E2M3) terms per block of 32
+ * along K (exact unless an element lies more than 2^-13 below its block's
+ * largest); VK_HIP_MOE_SPLIT2 selects two terms (error at most 2^-10 of the
+ * block's largest per element, two thirds of the matrix-core work).
+ * The workspace size is vk_hip_fused_moe_mxfp4_workspace_bytes(...), as for _ws.
+ */
+#define VK_HIP_MOE_SPLIT2 2u
+
+size_t vk_hip_moe_prepack_bytes(int32_t num_experts, int32_t rows, int32_t K, int32_t stage);
+
+int vk_hip_moe_prepack_weights(const uint8_t* w, const uint8_t* w_scale, int32_t num_experts,
+                               int32_t rows, int32_t K, int32_t stage, void* packed,
+                               size_t packed_bytes, void* stream);
+
+void vk_hip_fused_moe_mxfp4_prepacked(
+    const uint16_t* A, const uint8_t* w13, const uint8_t* w13_scale,
+    const uint8_t* w2, const uint8_t* w2_scale,
+    const int32_t* topk_ids, const float* topk_w,
+    uint16_t* act_scratch, float* out,
+    int M, int hidden, int ispp, int top_k,
+    const int32_t* sorted_ids, const int32_t* expert_ids,
+    int EM, float swiglu_limit,
+    int activation, float beta, float linear_beta,
+    const float* b13, const float* b2, int block_size,
+    void* workspace, size_t workspace_bytes, unsigned flags,
+    const void* w13_packed, const void* w2_packed, int num_experts, void* stream);
+
+/*
  * Additive: per-device set-up that the launchers otherwise do on their first
  * call (the dynamic-LDS limits of the GEMM kernels, the device address of the
  * library's scratch array, the developer knobs of the environment).  Call it
@@ -232,6 +282,35 @@ void vk_hip_moe_down_mxfp4(
     const float* b2, int block_size, void* stream);
 
 /*
+ * Additive: vk_hip_moe_down_mxfp4 with the optional arguments of the fused
+ * entry points: a caller-owned workspace (size as for vk_hip_fused_moe_mxfp4_ws),
+ * flags (VK_HIP_MOE_OVERWRITE_OUT, VK_HIP_MOE_SPLIT2) and the prepacked down
+ * weights (NULL = raw weights only).  It runs the second stage exactly as the
+ * fused call does for the same arguments, so a tensor-parallel caller can sum
+ * `act` contributions between the stages and a test can feed the second stage
+ * chosen `act` rows.  Device counterpart of moe_down_cpu + moe_combine_cpu,
+ * src/c/vkernels/kernels/moe_fused.hpp:259-283.
+ */
+void vk_hip_moe_down_mxfp4_ex(
+    const uint16_t* act, const uint8_t* w2, const uint8_t* w2_scale,
+    const float* topk_w, float* out, int M, int hidden, int ispp, int top_k,
+    const int32_t* sorted_ids, const int32_t* expert_ids, int EM,
+    const float* b2, int block_size, void* workspace, size_t workspace_bytes, unsigned flags,
+    const void* w2_packed, int num_experts, void* stream);
+
+/*
+ * Additive, for tests: bf16 rows [rows, K] -> the split rows the prefill-sized
+ * kernels multiply: per row `terms` (2 or 3) planes of Kp = K rounded up to 128
+ * bytes; a plane is Kp/32 blocks of 32 bytes: the 32 FP6 (E2M3) codes of the
+ * term (code i at bit 6 i), the term's scale byte (e-2-4t for term t, e the
+ * block's largest exponent field), 7 zero bytes.  row_flags[r] = 1 when a block
+ * of the row is outside the range of the split (inf/NaN, scale byte outside
+ * [64 + 4 (terms-1), 190]).  `split` holds rows * terms * Kp bytes.
+ */
+int vk_hip_split_rows_fp6(const uint16_t* x, int32_t rows, int32_t K, int32_t terms, void* split,
+                          uint8_t* row_flags, void* stream);
+
+/*
  * On-device alignment of the routing table: stable bucket of the flat indices
  * by (local) expert, each expert padded to a multiple of block_size.
  * Replaces vk_hip_moe_align_block_size,
@@ -280,13 +359,17 @@ int vk_hip_moe_route_topk(const float* logits, int32_t T, int32_t E,
 
 /*
  * Additive: dequantise an [N, K] tile of packed weights to bf16 with the
- * same device routine the GEMM kernels use, written transposed as [K][N].
+ * decode routines of the device library, written transposed as [K][N].
  * Device counterpart of dequant_weight_tile,
  * src/c/vkernels/kernels/moe_fused.hpp:217-235 (moe_fused.cpp:141-174), for
  * bit-exact checks of the weight decode.  group_size must be 32.
- * fast != 0 selects the hardware-conversion path the GEMM kernels take for
- * ordinary tiles (valid for finite codes and scale bytes 3..252); fast == 0
- * the exact integer path they fall back to.
+ * fast == 0 selects the integer-exact routine (every code, every scale byte):
+ * the one the GEMM kernels' exact path multiplies by.  fast != 0 selects the
+ * hardware conversion v_cvt_scalef32_pk_bf16_fp4 on the remapped codes (finite
+ * codes, scale bytes 3..252); the GEMM kernels' fast paths do not call it: the
+ * matrix cores decode the same remapped codes and decremented scale bytes
+ * themselves, and those values are pinned by the one-hot tests of the second
+ * stage instead.
  */
 int vk_hip_dequant_weight_tile(const uint8_t* packed, const uint8_t* scale,
                                uint16_t* out_bf16, int32_t N, int32_t K,

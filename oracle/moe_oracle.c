@@ -81,6 +81,59 @@ static inline float bf16_to_float(uint16_t v) {
 }
 
 /* ---------------------------------------------------------------------- */
+/* optional model of the GPU's activation operands (NOT in the reference)  */
+/* ---------------------------------------------------------------------- */
+
+/*
+ * The prefill kernels feed the matrix cores the bf16 activations as a sum of
+ * FP6 (E2M3) terms per block of 32 along K: with e the largest exponent field
+ * of the block and s = 2^(e-2-127),
+ *     t0 = Q(a / s) * s,  t1 = Q((a - t0) / (s/16)) * (s/16),
+ *     t2 = Q((a - t0 - t1) / (s/256)) * (s/256),          a' = t0 + t1 (+ t2),
+ * Q = round to nearest even on the E2M3 grid, saturating at +-7.5.  With the
+ * model switched on (terms = 2 or 3) the grouped GEMMs multiply a' instead of
+ * a, so a test can tell the error of that representation (model vs reference
+ * arithmetic, both on the CPU) from the error of the GPU's accumulation (GPU
+ * vs model).  terms = 0, the default, is the reference's arithmetic.
+ */
+static int g_act_model = 0;
+
+void vko_set_act_model(int terms) { g_act_model = (terms == 2 || terms == 3) ? terms : 0; }
+
+static float e2m3_round(float v) {
+  const float a = fabsf(v);
+  float q;
+  if (a < 2.0f) q = nearbyintf(a * 8.0f) * 0.125f;        /* subnormals and [1, 2): steps of 1/8 */
+  else if (a < 4.0f) q = nearbyintf(a * 4.0f) * 0.25f;
+  else q = nearbyintf(a * 2.0f) * 0.5f;
+  if (q > 7.5f) q = 7.5f;
+  return v < 0.0f ? -q : q;
+}
+
+/* a' for one block of 32 bf16 values (finite; blocks of zeros stay zeros). */
+void vko_act_model_block32(const uint16_t* a, float* out, int terms) {
+  int emax = 0;
+  for (int k = 0; k < 32; ++k) {
+    const int e = (a[k] >> 7) & 0xFF;
+    if (e > emax) emax = e;
+  }
+  if (emax == 0) {
+    for (int k = 0; k < 32; ++k) out[k] = 0.0f;
+    return;
+  }
+  const float s = ldexpf(1.0f, emax - 2 - 127);
+  for (int k = 0; k < 32; ++k) {
+    const float x = bits_to_float((uint32_t)a[k] << 16);
+    float sum = 0.0f, st = s;
+    for (int t = 0; t < terms; ++t) {
+      sum += e2m3_round((x - sum) / st) * st; /* exact: every term is a few bits of x */
+      st *= 0.0625f;
+    }
+    out[k] = sum;
+  }
+}
+
+/* ---------------------------------------------------------------------- */
 /* weight-tile dequantisation                                              */
 /* ---------------------------------------------------------------------- */
 
@@ -222,9 +275,14 @@ static void grouped_gemm(const uint16_t* A, int gather, const uint8_t* W,
               gather ? A + (size_t)(flat / top_k) * a_stride + k_base + k0
                      : A + (size_t)(row0 + r) * a_stride + k_base + k0;
           float dot[BLK_N];
+          float amodel[BLK_K];
+          if (g_act_model != 0) {
+            vko_act_model_block32(arow, amodel, g_act_model);
+            vko_act_model_block32(arow + 32, amodel + 32, g_act_model);
+          }
           for (int n = 0; n < BLK_N; ++n) dot[n] = 0.0f;
           for (int k = 0; k < BLK_K; ++k) {
-            const float a = bf16_to_float(arow[k]);
+            const float a = g_act_model != 0 ? amodel[k] : bf16_to_float(arow[k]);
             const float* wrow = tile_f + (size_t)k * BLK_N;
             for (int n = 0; n < BLK_N; ++n) dot[n] += a * wrow[n];
           }

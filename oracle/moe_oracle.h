@@ -135,6 +135,12 @@ float vko_route_exp(float x);
  * single-threaded behaviour; results are identical for any value). */
 void vko_set_threads(int n);
 
+/* Not in the reference: terms = 2 or 3: the grouped GEMMs multiply the sum of
+ * that many FP6 (E2M3) terms per activation block of 32 that the GPU's prefill
+ * kernels use; 0 (default) = the reference's arithmetic. */
+void vko_set_act_model(int terms);
+void vko_act_model_block32(const uint16_t* a, float* out, int terms);
+
 #ifdef __cplusplus
 }
 #endif

@@ -12,7 +12,7 @@ from pathlib import Path
 import numpy as np
 
 __all__ = [
-    "HERE", "build", "lib", "ref_lib", "have_ref", "set_threads",
+    "HERE", "build", "lib", "ref_lib", "have_ref", "set_threads", "set_act_model", "act_model_block32",
     "fp4nib_to_f32bits", "ue8m0_to_float", "f32bits_to_bf16",
     "dequant_weight_tile", "moe_align_block_size",
     "moe_align_block_size_with_map", "align_max_em", "align_em_bound",
@@ -73,6 +73,22 @@ def have_ref() -> bool:
 
 def set_threads(n: int) -> None:
     lib().vko_set_threads(int(n))
+
+
+def set_act_model(terms: int) -> None:
+    """2 or 3: the GEMMs multiply the sum of that many FP6 (E2M3) terms per
+    activation block of 32, the representation the GPU's prefill kernels use;
+    0: the reference's arithmetic."""
+    lib().vko_set_act_model(int(terms))
+
+
+def act_model_block32(a_bits, terms: int = 2) -> np.ndarray:
+    """The modelled values of one block of 32 bf16 bit patterns."""
+    a = np.ascontiguousarray(a_bits, dtype=np.uint16)
+    assert a.size == 32
+    out = np.empty(32, dtype=np.float32)
+    lib().vko_act_model_block32(_P(a.ctypes.data), _P(out.ctypes.data), int(terms))
+    return out
 
 
 def _ptr(a):

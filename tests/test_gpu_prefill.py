@@ -1,0 +1,443 @@
+"""GPU parity of the prefill-sized path on prepacked weights (FP4 x FP6 scaled MFMA),
+through the C ABI.
+
+Bit-exact: the prepacked layout, the split rows (against the oracle's model of the
+activation operands), and the weight values the matrix cores multiply by (one-hot
+activation rows through the second stage, every kernel family).
+Layer output: against the oracle within the contract's tolerance, and against the
+oracle run with the same activation representation (`oracle.set_act_model`) within a
+ten times tighter one, which isolates the GPU's accumulation from the representation.
+"""
+from __future__ import annotations
+
+import ctypes
+
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from vkernels_amd import synth
+from vkernels_amd import vllm_experts as ve
+
+import test_gpu_configs as cfgs
+from gpu_util import MAX_ABS_TOL, REL_L2_TOL, cpu_layer, dev, error_metrics, to_dev
+
+pytestmark = pytest.mark.gpu
+
+_P, _I, _F = ctypes.c_void_p, ctypes.c_int, ctypes.c_float
+
+# GPU against the oracle that multiplies the same activation representation: what is
+# left is the order of the fp32 sums and bf16 roundings of act that fall the other way
+MODEL_REL_L2_TOL = 5e-4
+MODEL_MAX_ABS_TOL = 5e-3
+
+
+# ---- the prepacked layout ---------------------------------------------------------
+
+def _prepack_reference(w, ws, stage):
+    """numpy restatement of the packed layout documented in include/vkernels_hip.h."""
+    E, rows, kb = w.shape
+    K = kb * 2
+    ncols = rows // 2 if stage == 0 else rows
+    units = ncols // 64 if stage == 0 else (ncols + 127) // 128
+    ksteps = (K + 127) // 128
+    out = np.zeros((E, units, ksteps, 8704), dtype=np.uint8)
+    flags = np.zeros((E, units), dtype=np.uint8)
+    lo, hi = w & 15, w >> 4
+    remap = lambda c: c + np.where((c & 6) != 0, 2, 0).astype(np.uint8)
+    nonfinite = ((lo & 6) == 6) | ((hi & 6) == 6)
+    for e in range(E):
+        for u in range(units):
+            for t in range(4):
+                for n in range(32):
+                    row = (t >> 1) * ncols + u * 64 + (t & 1) * 32 + n if stage == 0 else u * 128 + t * 32 + n
+                    if row >= rows:
+                        for ks in range(ksteps):
+                            out[e, u, ks, 8192:].reshape(64, 2, 4)[[n, n + 32], :, t] = 127
+                        continue
+                    if nonfinite[e, row].any() or (ws[e, row] < 64).any() or (ws[e, row] > 190).any():
+                        flags[e, u] = 1
+                    for g in range(ksteps * 4):
+                        ks, half, hh = g // 4, (g // 2) % 2, g % 2
+                        lane = n + 32 * hh
+                        sc_view = out[e, u, ks, 8192:].reshape(64, 2, 4)
+                        if g * 32 >= K:
+                            sc_view[lane, half, t] = 127
+                            continue
+                        piece = w[e, row, g * 16:(g + 1) * 16]
+                        packed = remap(piece & 15) | (remap(piece >> 4) << 4)
+                        off = ((half * 4 + t) * 64 + lane) * 16
+                        out[e, u, ks, off:off + 16] = packed
+                        sc_view[lane, half, t] = (int(ws[e, row, g]) - 1) & 0xFF
+    return out, flags
+
+
+@pytest.mark.parametrize("stage,rows,K", [(0, 256, 192), (1, 192, 128), (1, 128, 320)])
+def test_prepack_layout_bitwise(hip_lib, stage, rows, K):
+    size_fn, pack_fn, _ = ve.resolve_prepack_fns(hip_lib)
+    E = 3
+    rng = np.random.default_rng(stage * 100 + rows)
+    fin = np.array(synth.FINITE_CODES, dtype=np.uint8)
+    w = (fin[rng.integers(0, 12, (E, rows, K // 2))] | (fin[rng.integers(0, 12, (E, rows, K // 2))] << 4)).astype(np.uint8)
+    ws = rng.integers(64, 191, (E, rows, K // 32)).astype(np.uint8)
+    w[1, 7, 3] = 0x6E           # an inf code: its unit is flagged
+    ws[2, rows - 1, 0] = 63     # a scale byte below the range: its unit is flagged
+    ws[0, 40, 1] = 191          # above the range
+    n = int(size_fn(E, rows, K, stage))
+    buf = torch.zeros(n, dtype=torch.uint8, device=dev())
+    st = pack_fn(to_dev(w).data_ptr(), to_dev(ws).data_ptr(), E, rows, K, stage, buf.data_ptr(), n, None)
+    assert st == 0, ve.last_error(hip_lib)
+    torch.cuda.synchronize()
+    ref, flags = _prepack_reference(w, ws, stage)
+    got = buf.cpu().numpy()
+    body = ref.size
+    flagged = np.repeat(flags.ravel().astype(bool), ref.shape[2] * 8704)
+    # flagged units are never read in packed form; the others must match byte for byte
+    assert np.array_equal(got[:body][~flagged], ref.ravel()[~flagged])
+    f_off = (body + 255) // 256 * 256
+    assert np.array_equal(got[f_off:f_off + flags.size], flags.ravel())
+    assert flags.sum() == 3
+
+
+# ---- the split rows ------------------------------------------------------------------
+
+def _decode_fp6(codes24):
+    """[..., 24] bytes -> [..., 32] floats (E2M3, code i at bit 6 i)."""
+    b = codes24.astype(np.uint64)
+    bits = np.zeros(codes24.shape[:-1] + (3,), dtype=np.uint64)
+    for i in range(3):
+        for j in range(8):
+            bits[..., i] |= b[..., 8 * i + j] << np.uint64(8 * j)
+    vals = np.zeros(codes24.shape[:-1] + (32,), dtype=np.float64)
+    for i in range(32):
+        bit = 6 * i
+        word, sh = bit // 64, bit % 64
+        c = (bits[..., word] >> np.uint64(sh))
+        if sh > 58:
+            c |= bits[..., word + 1] << np.uint64(64 - sh)
+        c = (c & np.uint64(63)).astype(np.int64)
+        e, m = (c >> 3) & 3, c & 7
+        v = np.where(e == 0, m / 8.0, np.ldexp(1.0 + m / 8.0, e - 1))
+        vals[..., i] = np.where(c & 32, -v, v)
+    return vals
+
+
+@pytest.mark.parametrize("terms", [2, 3])
+def test_split_rows_match_the_oracle_model(hip_lib, terms):
+    fn = hip_lib.vk_hip_split_rows_fp6
+    fn.restype = _I
+    fn.argtypes = [_P, _I, _I, _I, _P, _P, _P]
+    rows, K = 24, 2880
+    kp = (K + 127) // 128 * 128
+    x = synth.make_activations(rows, K, 77 + terms)
+    xf = synth.bf16_bits_to_f32(x)
+    x[1] = synth.f32_to_bf16_bits(xf[1] * np.float32(2.0 ** 40))
+    x[2] = synth.f32_to_bf16_bits(xf[2] * np.float32(2.0 ** -40))
+    x[3, 64:96] = 0                      # a block of zeros
+    x[4, 100] = 0x7F80                   # inf: the row is flagged
+    x[5, 7] = 0x7FC0                     # NaN
+    x[6] = synth.f32_to_bf16_bits(xf[6] * np.float32(2.0 ** 90))    # scale byte above 190
+    x[7] = synth.f32_to_bf16_bits(xf[7] * np.float32(2.0 ** -70))   # below the range
+    x[8, 5] = 0x40FF                     # 7.96875: saturates the first term
+    out = torch.zeros(rows * terms * kp, dtype=torch.uint8, device=dev())
+    flags = torch.full((rows,), 9, dtype=torch.uint8, device=dev())
+    st = fn(to_dev(x).data_ptr(), rows, K, terms, out.data_ptr(), flags.data_ptr(), None)
+    assert st == 0, ve.last_error(hip_lib)
+    torch.cuda.synchronize()
+    fl = flags.cpu().numpy()
+    assert list(np.nonzero(fl)[0]) == [4, 5, 6, 7], fl
+    blocks = out.cpu().numpy().reshape(rows, terms, kp // 32, 32)
+    vals = _decode_fp6(blocks[..., :24])                        # [rows, terms, nblk, 32]
+    scale = np.ldexp(1.0, blocks[..., 24].astype(np.int64) - 127)
+    assert not blocks[..., 25:].any()
+    total = (vals * scale[..., None]).sum(axis=1)                # [rows, nblk, 32]
+    for r in range(rows):
+        if fl[r]:
+            continue
+        for b in range(kp // 32):
+            if b * 32 >= K:
+                assert not total[r, b].any()
+                continue
+            model = oracle.act_model_block32(x[r, b * 32:(b + 1) * 32], terms).astype(np.float64)
+            assert np.array_equal(total[r, b], model), (r, b)
+    # three terms resolve 2^-13 of the block's largest: exact but for the elements below
+    # 2^-5 of it (a few percent of a normal block), which are off by at most 2^-14 of it
+    if terms == 3:
+        exact = synth.bf16_bits_to_f32(x[9:]).astype(np.float64).reshape(rows - 9, K // 32, 32)
+        err = np.abs(total[9:, :K // 32] - exact)
+        big = np.abs(exact).max(axis=2, keepdims=True)
+        assert (err <= 2.0 ** -14 * big).all()
+        assert not err[np.abs(exact) >= 2.0 ** -5 * big].any()
+        assert np.count_nonzero(err) < 0.03 * err.size
+
+
+# ---- the weight values the kernels multiply by ---------------------------------------
+
+def _down_ex(lib):
+    fn = lib.vk_hip_moe_down_mxfp4_ex
+    fn.restype = None
+    fn.argtypes = [_P] * 5 + [_I] * 4 + [_P, _P, _I, _P, _I, _P, ctypes.c_size_t, ctypes.c_uint, _P, _I, _P]
+    return fn
+
+
+@pytest.mark.parametrize("path", ["packed3", "packed2", "workspace", "plain", "resident"])
+def test_onehot_rows_read_back_the_dequantised_weights(hip_lib, path):
+    """act rows with a single 1.0 at column k, routing weight 1: out[t, :] is column k of
+    the expert's dequantised W2, so every value the GEMM multiplies by is compared with the
+    oracle bit for bit.  Expert 0: the 12 finite codes with scale bytes 64, 65, 127, 189,
+    190 (the scaled-MFMA path); expert 1: all 16 codes and scale bytes 0, 1, 63, 191, 200,
+    255 (flagged: the exact path)."""
+    E, H = 2, 192
+    I = 256 if path == "resident" else 576
+    M = E * I
+    rng = np.random.default_rng(11)
+    fin = np.array(synth.FINITE_CODES, dtype=np.uint8)
+    w2 = np.zeros((E, H, I // 2), dtype=np.uint8)
+    w2[0] = fin[rng.integers(0, 12, (H, I // 2))] | (fin[rng.integers(0, 12, (H, I // 2))] << 4)
+    w2[1] = rng.integers(0, 256, (H, I // 2)).astype(np.uint8)
+    keep = np.ones(H, dtype=bool)
+    keep[[5, 77]] = False                                          # rows that keep their inf/NaN codes
+    lo, hi = w2[1] & 15, w2[1] >> 4
+    lo[keep] = fin[lo[keep] % 12]
+    hi[keep] = fin[hi[keep] % 12]
+    w2[1] = lo | (hi << 4)
+    w2s = np.zeros((E, H, I // 32), dtype=np.uint8)
+    w2s[0] = np.array([64, 65, 127, 189, 190], dtype=np.uint8)[rng.integers(0, 5, (H, I // 32))]
+    w2s[1] = np.array([0, 1, 63, 191, 200, 255], dtype=np.uint8)[rng.integers(0, 6, (H, I // 32))]
+    ids = (np.arange(M) // I).astype(np.int32).reshape(M, 1)
+    fe = ve.FusedExperts(to_dev(np.zeros((E, 2 * I, H // 2), np.uint8)), to_dev(np.zeros((E, 2 * I, H // 32), np.uint8)),
+                         to_dev(w2), to_dev(w2s), scratch=ve.CaptureSafeScratch(), prepack=path.startswith("packed"))
+    bs = 16 if path == "resident" else 128
+    sids, eids, out_em, max_em = fe.align(to_dev(ids), bs)
+    torch.cuda.synchronize()
+    s_np = sids.cpu().numpy()
+    act = np.zeros((max_em, I), dtype=np.uint16)
+    real = np.nonzero(s_np < M)[0]
+    act[real, s_np[real] % I] = 0x3F80                              # 1.0
+    d_act = to_dev(act)
+    tw = torch.ones((M, 1), dtype=torch.float32, device=dev())
+    out = torch.full((M, H), float("nan"), dtype=torch.float32, device=dev())
+    ws, need = None, 0
+    if path != "plain" and path != "resident":
+        need = int(fe.ws_bytes_fn(M, H, I, 1, max_em))
+        ws = torch.empty(need, dtype=torch.uint8, device=dev())
+    flags = ve.MOE_OVERWRITE_OUT | (ve.MOE_SPLIT2 if path == "packed2" else 0)
+    hip_lib.vk_set_last_error(0, b"")
+    _down_ex(hip_lib)(d_act.data_ptr(), fe.w2.data_ptr(), fe.w2_scale.data_ptr(), tw.data_ptr(),
+                      out.data_ptr(), M, H, I, 1, sids.data_ptr(), eids.data_ptr(), max_em, None, bs,
+                      None if ws is None else ws.data_ptr(), need, flags,
+                      None if fe.w2_packed is None else fe.w2_packed.data_ptr(), E, None)
+    torch.cuda.synchronize()
+    assert hip_lib.vk_last_error_code() == 0, ve.last_error(hip_lib)
+    got = out.cpu().numpy()
+    # expected: the oracle's second stage on the same act
+    eids16 = np.repeat(eids.cpu().numpy(), bs // 16).astype(np.int32)
+    partial = oracle.moe_down(act, w2, w2s, s_np, eids16, M, I, 0, I, H, 1, max_em)
+    tws = oracle.gather_sorted_weights(tw.cpu().numpy(), s_np)
+    exp = oracle.moe_combine(partial, None, tws, s_np, eids16, M, H, 1, max_em)
+    same = (got == exp) | (np.isnan(got) & np.isnan(exp))
+    assert same.all(), f"{path}: {np.count_nonzero(~same)} values differ, first at {np.argwhere(~same)[:5]}"
+    # and the expectation is the dequantisation table itself for the finite expert
+    table = synth.bf16_bits_to_f32(oracle.dequant_weight_tile(w2[0], w2s[0], H, I))   # [I, H]
+    assert np.array_equal(exp[:I], table)
+    assert np.isnan(exp[I:, 5]).all() and np.isfinite(exp[I:, 6]).all()
+
+
+# ---- the layer -------------------------------------------------------------------------
+
+def _edge_tokens(g, n_flat, top_k, want, seed):
+    """Tokens whose sorted rows sit where a tile kernel breaks: first and last routed row
+    of windows of 128, rows either side of 32-row tile boundaries, the last row of an
+    expert's segment, rows of the most and the least popular expert; then random ones."""
+    sids, eids, bs = g["sids"], g["eids"], g["bs"]
+    routed = np.nonzero(sids < n_flat)[0]
+    rows = set()
+    win = routed // 128
+    first = routed[np.r_[True, win[1:] != win[:-1]]]
+    last = routed[np.r_[win[1:] != win[:-1], True]]
+    rng = np.random.default_rng(seed)
+    for arr in (first, last):
+        rows.update(rng.choice(arr, min(arr.size, 24), replace=False).tolist())
+    edge = routed[np.isin(routed % 32, (0, 31))]
+    rows.update(rng.choice(edge, min(edge.size, 24), replace=False).tolist())
+    expert_of_row = np.repeat(eids, bs)[routed]
+    counts = np.bincount(expert_of_row[expert_of_row >= 0])
+    live = np.nonzero(counts)[0]
+    for e in (live[np.argmax(counts[live])], live[np.argmin(counts[live])]):
+        er = routed[expert_of_row == e]
+        rows.update(er[[0, -1]].tolist())
+    tokens = set((sids[list(rows)] // top_k).tolist())
+    T = n_flat // top_k
+    extra = rng.permutation(T)
+    for t in extra:
+        if len(tokens) >= want:
+            break
+        tokens.add(int(t))
+    return np.sort(np.fromiter(tokens, dtype=np.int64))
+
+
+def _check_prefill(cfg, T, w, A_bits, logits, terms=3, sample=128, wn=None, gpu_kw=None, cpu_kw=None,
+                   block_size=None, contract_only=False):
+    gpu_kw = dict(gpu_kw or {})
+    gpu_kw.update(prepack=True, split_terms=terms)
+    g = cfgs._run_gpu(cfg, w, A_bits, logits, block_size, True, **gpu_kw)
+    ids, tw = oracle.route_topk(logits, cfg.top_k, True)
+    assert np.array_equal(g["ids"], ids) and np.array_equal(g["tw"].view(np.uint32), tw.view(np.uint32))
+    rows = np.arange(T) if sample is None or sample >= T else \
+        _edge_tokens(g, T * cfg.top_k, cfg.top_k, sample, T)
+    wn = w.numpy() if wn is None else wn
+    c = cpu_layer(A_bits[rows], wn, ids[rows], tw[rows], threads=16, **(cpu_kw or {}))
+    max_rel, rel_l2, nf = error_metrics(g["out"][rows], c["out"])
+    oracle.set_act_model(terms)
+    try:
+        cm = cpu_layer(A_bits[rows], wn, ids[rows], tw[rows], threads=16, **(cpu_kw or {}))
+    finally:
+        oracle.set_act_model(0)
+    m_rel, m_l2, m_nf = error_metrics(g["out"][rows], cm["out"])
+    print(f"{cfg.name} T={T} terms={terms} rows checked {rows.size}: vs oracle max_abs/rms={max_rel:.3e} "
+          f"rel_l2={rel_l2:.3e}; vs oracle with the same operands max_abs/rms={m_rel:.3e} rel_l2={m_l2:.3e}")
+    assert nf and max_rel <= MAX_ABS_TOL and rel_l2 <= REL_L2_TOL
+    if not contract_only:
+        assert m_nf and m_rel <= MODEL_MAX_ABS_TOL and m_l2 <= MODEL_REL_L2_TOL
+    if terms == 3 and not contract_only:  # three terms: ten times inside the contract on their own
+        assert max_rel <= MAX_ABS_TOL / 4 and rel_l2 <= REL_L2_TOL / 10
+    return g, wn
+
+
+@pytest.mark.parametrize("terms", [3, 2])
+@pytest.mark.parametrize("T", [200, 513])
+def test_config1_prepacked(T, terms):
+    cfg = synth.CONFIGS["c1"]
+    w = cfgs._weights(cfg, 1500)
+    A, lg = cfgs._inputs(cfg, T, 1900 + T)
+    _check_prefill(cfg, T, w, A, lg, terms=terms)
+
+
+def test_config2_zipf_prepacked():
+    cfg = synth.CONFIGS["c2"]
+    w = cfgs._weights(cfg)
+    wn = None
+    for T in (4096, 512):
+        A, lg = cfgs._inputs(cfg, T, 2000)
+        _, wn = _check_prefill(cfg, T, w, A, lg, wn=wn)
+
+
+@pytest.mark.parametrize("T", [4096, 16384])
+def test_config3_prepacked(T):
+    cfg = synth.CONFIGS["c3"]
+    w = cfgs._weights(cfg)
+    A, lg = cfgs._inputs(cfg, T, 3000)
+    g, wn = _check_prefill(cfg, T, w, A, lg, sample=160)
+    assert np.all(np.isfinite(g["out"]))
+    if T == 4096:   # the two-term option on the same inputs
+        _check_prefill(cfg, T, w, A, lg, terms=2, sample=64, wn=wn)
+
+
+@pytest.mark.parametrize("T", [1000, 8191])
+def test_config4_prepacked(T):
+    """Block scales of 2^+-20 and all-zero blocks: single terms dominate the outputs, so the
+    end-to-end figure is held to the contract only (see the stage-wise tests of the raw path)."""
+    cfg = synth.CONFIGS["c4"]
+    key = ("c4x", 4000)
+    if key not in cfgs._WEIGHTS:
+        cfgs._WEIGHTS.clear()
+        cfgs._WEIGHTS[key] = cfgs._extreme_weights(cfg, 4000)
+    w = cfgs._WEIGHTS[key]
+    A, lg = cfgs._inputs(cfg, T, 4000)
+    _check_prefill(cfg, T, w, A, lg, contract_only=True)
+
+
+@pytest.mark.parametrize("variant", ["bias", "limit", "situ_bias"])
+def test_epilogue_variants_prepacked(variant):
+    cfg = synth.CONFIGS["c1"]
+    T, seed = 200, 1500
+    w = cfgs._weights(cfg, seed)
+    A, lg = cfgs._inputs(cfg, T, seed)
+    b13 = (synth.rand_normal((cfg.E, 2 * cfg.I), seed, 21) * 0.5).astype(np.float32)
+    b2 = (synth.rand_normal((cfg.E, cfg.H), seed, 22) * 0.5).astype(np.float32)
+    gpu_kw, cpu_kw = {}, {}
+    if "bias" in variant:
+        gpu_kw.update(b13=to_dev(b13), b2=to_dev(b2))
+        cpu_kw.update(b13=b13, b2=b2)
+    if variant == "limit":
+        gpu_kw.update(swiglu_limit=1.5)
+        cpu_kw.update(swiglu_limit=1.5)
+    if "situ" in variant:
+        gpu_kw.update(activation="situ", beta=3.0, linear_beta=20.0)
+        cpu_kw.update(activation=1, beta=3.0, linear_beta=20.0)
+    _check_prefill(cfg, T, w, A, lg, sample=48, gpu_kw=gpu_kw, cpu_kw=cpu_kw)
+
+
+@pytest.mark.parametrize("bs", [16, 48, 64, 80, 128])
+def test_block_sizes_prepacked(bs):
+    cfg = synth.CONFIGS["c1"]
+    T, seed = 160, 1700
+    w = cfgs._weights(cfg, 1500)
+    A, lg = cfgs._inputs(cfg, T, seed)
+    _check_prefill(cfg, T, w, A, lg, sample=48, block_size=bs)
+
+
+def test_values_outside_the_range_prepacked():
+    """inf/NaN codes and out-of-range scale bytes in some experts (flagged units: exact
+    path) and rows with inf, NaN, huge and tiny values (flagged rows: their segments take
+    the exact path); everything else on the fast path, in one call."""
+    cfg = synth.MoEConfig("t", 256, 512, 8, 2, (300,), "uniform")
+    T, seed = 300, 4300
+    w = synth.make_weights(cfg.E, cfg.H, cfg.I, seed, device=dev())
+    r = synth.rand_u63(w.w13[0].numel(), seed, 32, dev()).reshape(w.w13[0].shape)
+    w.w13[0][(r >> 10) % 4096 == 0] = 0x6E
+    r = synth.rand_u63(w.w2[1].numel(), seed, 33, dev()).reshape(w.w2[1].shape)
+    w.w2[1][(r >> 10) % 8192 == 0] = 0x7F
+    w.w2_scale[2][::7, 1] = 200
+    w.w13_scale[3][::5, 0] = 2
+    A, lg = cfgs._inputs(cfg, T, seed)
+    A = A.copy()
+    A[0, 5] = 0x7F80
+    A[1, 7] = 0x7FC0
+    A[2, :] = synth.f32_to_bf16_bits(synth.bf16_bits_to_f32(A[2, :]) * np.float32(2.0 ** 80))
+    A[3, :] = synth.f32_to_bf16_bits(synth.bf16_bits_to_f32(A[3, :]) * np.float32(2.0 ** -90))
+    A[4, :] = 0
+    g = cfgs._run_gpu(cfg, w, A, lg, None, True, prepack=True)
+    ids, tw = oracle.route_topk(lg, cfg.top_k, True)
+    c = cpu_layer(A, w.numpy(), ids, tw, threads=16)
+    for t in range(T):   # row by row: the rows differ by many orders of magnitude
+        max_rel, rel_l2, nf = error_metrics(g["out"][t], c["out"][t])
+        assert nf and max_rel <= MAX_ABS_TOL and rel_l2 <= REL_L2_TOL, (t, max_rel, rel_l2)
+    finite_rows = np.all(np.isfinite(c["out"]), axis=1)
+    assert 0 < finite_rows.sum() < T
+
+
+def test_expert_map_prepacked():
+    cfg = synth.CONFIGS["c1"]
+    T, seed = 300, 1800
+    w = cfgs._weights(cfg, 1500)
+    A, lg = cfgs._inputs(cfg, T, seed)
+    rng = np.random.default_rng(seed)
+    local_n = cfg.E // 2
+    owned = rng.permutation(cfg.E)[:local_n]
+    emap = np.full(cfg.E, -1, dtype=np.int32)
+    emap[owned] = np.arange(local_n, dtype=np.int32)
+    own = to_dev(owned.astype(np.int64))
+    fe = ve.FusedExperts(w.w13[own].contiguous(), w.w13_scale[own].contiguous(),
+                         w.w2[own].contiguous(), w.w2_scale[own].contiguous(),
+                         expert_map=to_dev(emap), local_num_experts=local_n,
+                         scratch=ve.CaptureSafeScratch(), prepack=True)
+    ids, tw = fe.route(to_dev(lg), cfg.top_k, True)
+    out = fe.apply(to_dev(A, torch.bfloat16), ids, tw).cpu().numpy()
+    ids_np, tw_np = ids.cpu().numpy(), tw.cpu().numpy()
+    tw_local = np.where(emap[ids_np] >= 0, tw_np, np.float32(0.0)).astype(np.float32)
+    c = cpu_layer(A, w.numpy(), ids_np, tw_local, threads=16)
+    max_rel, rel_l2, nf = error_metrics(out, c["out"])
+    assert nf and max_rel <= MAX_ABS_TOL / 4 and rel_l2 <= REL_L2_TOL / 10, (max_rel, rel_l2)
+
+
+def test_prepacked_calls_are_deterministic():
+    """The packed path has no atomics: two calls give the same bits."""
+    cfg = synth.CONFIGS["c1"]
+    T = 300
+    w = cfgs._weights(cfg, 1500)
+    A, lg = cfgs._inputs(cfg, T, 1801)
+    a = cfgs._run_gpu(cfg, w, A, lg, None, True, prepack=True)["out"]
+    b = cfgs._run_gpu(cfg, w, A, lg, None, True, prepack=True)["out"]
+    assert np.array_equal(a.view(np.uint32), b.view(np.uint32))

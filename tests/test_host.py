@@ -227,13 +227,16 @@ def test_workspace_bytes(lib):
     assert f(0, 2880, 2880, 4, 64) == 0 and f(64, 2880, 2880, 4, 0) == 0
     M, H, I, k, EM = 4096, 7168, 2048, 8, 49152
     need = f(M, H, I, k, EM)
-    # both split copies (2 bytes per value) and their scale rows, the second stage's
-    # fp32 rows and the position of every flat index, with alignment slack
-    floor = 2 * M * H + M * H // 32 + 2 * EM * I + EM * I // 32 + 4 * EM * H + 4 * M * k
+    # enough for either path.  Raw weights: both split copies (2 bytes per value) and their
+    # scale rows; prepacked weights: three planes of a byte per value and a flag byte per
+    # row; either way the second stage's fp32 rows and the position of every flat index
+    raw = 2 * M * H + M * H // 32 + 2 * EM * I + EM * I // 32 + 4 * EM * H + 4 * M * k
+    packed = 3 * M * H + 3 * EM * I + M + EM + 4 * EM * H + 4 * M * k
+    floor = max(raw, packed)
     assert floor <= need <= floor + M * 16 + EM * 16 + 6 * 256
     assert f(M + 1, H, I, k, EM) > need and f(M, H, I, k, EM + 64) > need
     # rows are padded to whole K steps of 128
-    assert f(64, 2880, 2880, 4, 512) >= 2 * 64 * 2944 + 2 * 512 * 2944
+    assert f(64, 2880, 2880, 4, 512) >= 3 * 64 * 2944 + 3 * 512 * 2944
 
 
 def test_entry_points_reject_contract_violations_without_a_device(lib):

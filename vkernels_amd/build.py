@@ -24,7 +24,7 @@ INCLUDE = PKG.parent / "include"
 OBJ = PKG / "build"
 LIB = PKG / "libvkernels_hip.so"
 
-SOURCES = ["moe_route.hip", "moe_align.hip", "moe_dequant.hip", "moe_gemm.hip", "static_scratch.hip",
+SOURCES = ["moe_route.hip", "moe_align.hip", "moe_dequant.hip", "moe_gemm.hip", "moe_prefill.hip", "static_scratch.hip",
            "hip_capi.cpp"]
 
 # -packed-fp32-ops off: hipcc must not form packed fp32 arithmetic.

@@ -164,6 +164,104 @@ void vk_hip_fused_moe_mxfp4_ex(
   note_launch_error("vk_hip_fused_moe_mxfp4");
 }
 
+void vk_hip_fused_moe_mxfp4_prepacked(
+    const uint16_t* A, const uint8_t* w13, const uint8_t* w13_scale,
+    const uint8_t* w2, const uint8_t* w2_scale,
+    const int32_t* topk_ids, const float* topk_w,
+    uint16_t* act_scratch, float* out,
+    int M, int hidden, int ispp, int top_k,
+    const int32_t* sorted_ids, const int32_t* expert_ids,
+    int EM, float swiglu_limit,
+    int activation, float beta, float linear_beta,
+    const float* b13, const float* b2, int block_size,
+    void* workspace, size_t workspace_bytes, unsigned flags,
+    const void* w13_packed, const void* w2_packed, int num_experts, void* stream) {
+  (void)topk_ids;
+  if (M <= 0 || EM <= 0) return;  // nothing routed: out is left as it is
+  vk::FusedMoeArgs a =
+      fused_args(A, w13, w13_scale, w2, w2_scale, topk_w, act_scratch, out, M, hidden, ispp,
+                 top_k, sorted_ids, expert_ids, EM, swiglu_limit, activation, beta, linear_beta,
+                 b13, b2, block_size, workspace, workspace_bytes, flags);
+  if (!layer_args_ok("vk_hip_fused_moe_mxfp4_prepacked", true, true, a)) return;
+  if ((w13_packed == nullptr) != (w2_packed == nullptr) || (w13_packed != nullptr && num_experts <= 0)) {
+    vk_set_last_error(VK_ERROR_INVALID_ARGUMENT,
+                      "vk_hip_fused_moe_mxfp4_prepacked: both packed buffers (or neither) and a "
+                      "positive num_experts are required");
+    return;
+  }
+  a.w13_packed = static_cast<const uint8_t*>(w13_packed);
+  a.w2_packed = static_cast<const uint8_t*>(w2_packed);
+  a.num_experts = num_experts;
+  vk::launch_fused_moe(a, static_cast<hipStream_t>(stream));
+  note_launch_error("vk_hip_fused_moe_mxfp4_prepacked");
+}
+
+void vk_hip_moe_down_mxfp4_ex(
+    const uint16_t* act, const uint8_t* w2, const uint8_t* w2_scale,
+    const float* topk_w, float* out, int M, int hidden, int ispp, int top_k,
+    const int32_t* sorted_ids, const int32_t* expert_ids, int EM,
+    const float* b2, int block_size, void* workspace, size_t workspace_bytes, unsigned flags,
+    const void* w2_packed, int num_experts, void* stream) {
+  if (M <= 0 || EM <= 0) return;
+  vk::FusedMoeArgs a{};
+  a.w2 = w2; a.w2_scale = w2_scale; a.topk_w = topk_w;
+  a.act = const_cast<uint16_t*>(act); a.out = out;
+  a.sorted_ids = sorted_ids; a.expert_ids = expert_ids; a.b2 = b2;
+  a.M = M; a.hidden = hidden; a.ispp = ispp; a.top_k = top_k; a.EM = EM;
+  a.block_size = block_size;
+  a.workspace = workspace; a.workspace_bytes = workspace_bytes; a.flags = flags;
+  a.w2_packed = static_cast<const uint8_t*>(w2_packed);
+  a.num_experts = num_experts;
+  if (!layer_args_ok("vk_hip_moe_down_mxfp4_ex", false, true, a)) return;
+  if (w2_packed != nullptr && num_experts <= 0) {
+    vk_set_last_error(VK_ERROR_INVALID_ARGUMENT,
+                      "vk_hip_moe_down_mxfp4_ex: num_experts must be positive with packed weights");
+    return;
+  }
+  vk::launch_moe_down(a, static_cast<hipStream_t>(stream));
+  note_launch_error("vk_hip_moe_down_mxfp4_ex");
+}
+
+int vk_hip_split_rows_fp6(const uint16_t* x, int32_t rows, int32_t K, int32_t terms, void* split,
+                          uint8_t* row_flags, void* stream) {
+  if (rows < 0 || K <= 0 || K % 32 != 0)
+    return fail(VK_ERROR_INVALID_ARGUMENT, "rows must be >= 0 and K a positive multiple of 32");
+  if (terms != 2 && terms != 3)
+    return fail(VK_ERROR_INVALID_ARGUMENT, "terms must be 2 or 3");
+  if (rows == 0) return VK_OK;
+  if (x == nullptr || split == nullptr || row_flags == nullptr)
+    return fail(VK_ERROR_INVALID_ARGUMENT, "x/split/row_flags must not be null");
+  vk::launch_split_rows_fp6(x, rows, K, terms, static_cast<uint8_t*>(split), row_flags,
+                            static_cast<hipStream_t>(stream));
+  return VK_OK;
+}
+
+size_t vk_hip_moe_prepack_bytes(int32_t num_experts, int32_t rows, int32_t K, int32_t stage) {
+  if (stage != 0 && stage != 1) return 0;
+  return vk::moe_prepack_bytes(num_experts, rows, K, stage);
+}
+
+int vk_hip_moe_prepack_weights(const uint8_t* w, const uint8_t* w_scale, int32_t num_experts,
+                               int32_t rows, int32_t K, int32_t stage, void* packed,
+                               size_t packed_bytes, void* stream) {
+  if (stage != 0 && stage != 1)
+    return fail(VK_ERROR_INVALID_ARGUMENT, "stage must be 0 (gate/up weights) or 1 (down weights)");
+  if (num_experts <= 0 || rows <= 0 || K <= 0 || K % 64 != 0)
+    return fail(VK_ERROR_INVALID_ARGUMENT, "num_experts and rows must be positive, K a positive multiple of 64");
+  if (stage == 0 ? (rows % 128 != 0) : (rows % 64 != 0))
+    return fail(VK_ERROR_INVALID_ARGUMENT,
+                "rows must be 2 * ispp with ispp a multiple of 64 (stage 0) or a multiple of 64 (stage 1)");
+  if (w == nullptr || w_scale == nullptr || packed == nullptr)
+    return fail(VK_ERROR_INVALID_ARGUMENT, "w/w_scale/packed must not be null");
+  if ((reinterpret_cast<uintptr_t>(packed) & 15) != 0 || (reinterpret_cast<uintptr_t>(w) & 15) != 0)
+    return fail(VK_ERROR_INVALID_ARGUMENT, "w and packed must be 16-byte aligned");
+  if (packed_bytes < vk::moe_prepack_bytes(num_experts, rows, K, stage))
+    return fail(VK_ERROR_INVALID_ARGUMENT, "packed buffer smaller than vk_hip_moe_prepack_bytes()");
+  vk::launch_moe_prepack(w, w_scale, num_experts, rows, K, stage, static_cast<uint8_t*>(packed),
+                         static_cast<hipStream_t>(stream));
+  return VK_OK;
+}
+
 int vk_hip_init(void) {
   hipError_t err = hipSuccess;
   if (vk::static_scratch_ptr(&err) == nullptr)

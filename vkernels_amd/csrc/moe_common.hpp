@@ -1,0 +1,83 @@
+// moe_common.hpp — device helpers shared by the MoE GEMM translation units.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "mxfp4.hpp"
+
+namespace vk {
+
+// Scale bytes the scaled-MFMA paths take (weights and activation blocks); units
+// and rows outside go to the exact path.
+constexpr uint32_t kScaleLo = 64u, kScaleHi = 190u;
+
+__device__ __forceinline__ float act_value(int activation, float g, float u,
+                                           float limit, float beta,
+                                           float linear_beta) {
+  if (activation == 1) {
+    const float sig = 1.0f / (1.0f + expf(-g));
+    const float gate_out = beta * tanhf(g / beta) * sig;
+    const float up_out = linear_beta > 0.0f ? linear_beta * tanhf(u / linear_beta) : u;
+    return gate_out * up_out;
+  }
+  if (limit > 0.0f) {
+    if (g > limit) g = limit;
+    if (u > limit) u = limit;
+    if (u < -limit) u = -limit;
+  }
+  // v_exp_f32 / v_rcp_f32: about 1 ulp each, far inside the bf16 rounding that follows
+  return (g * __builtin_amdgcn_rcpf(1.0f + __expf(-g))) * u;
+}
+
+__device__ __forceinline__ bf16x8 as_bf16x8(u32x4 v) {
+  union { u32x4 u; bf16x8 b; } c;
+  c.u = v;
+  return c.b;
+}
+
+
+// Largest bf16 exponent field among the 8 values of v: the exponent of the
+// largest magnitude, found with packed 16-bit maxima.
+__device__ __forceinline__ uint32_t bf16x8_max_exponent(u32x4 v) {
+  typedef __attribute__((ext_vector_type(2))) unsigned short u16x2;
+  union { uint32_t u; u16x2 h; } a, b, c, d;
+  a.u = v[0] & 0x7FFF7FFFu;
+  b.u = v[1] & 0x7FFF7FFFu;
+  c.u = v[2] & 0x7FFF7FFFu;
+  d.u = v[3] & 0x7FFF7FFFu;
+  a.h = __builtin_elementwise_max(a.h, b.h);
+  c.h = __builtin_elementwise_max(c.h, d.h);
+  a.h = __builtin_elementwise_max(a.h, c.h);
+  const uint32_t m = max(a.u & 0xFFFFu, a.u >> 16);
+  return m >> 7;
+}
+
+// s_waitcnt immediate that waits until at most n vector-memory operations are
+// outstanding and for nothing else (vmcnt is split over bits 3:0 and 15:14).
+constexpr int vmcnt_only(int n) { return (n & 15) | ((n >> 4) << 14) | 0x0F70; }
+
+template <int N>
+struct IntC {
+  static constexpr int value = N;
+};
+
+// The DMA form of the global load: every lane's 16 (4) bytes at `src` go to LDS
+// at byte address lds_base + 16 (4) * lane.  Written as assembly because the
+// compiler makes every later LDS read wait for all DMA loads it has emitted
+// itself, and for every register load issued along with them: a ring that is
+// filled several steps ahead needs the counted waits of the kernel instead.
+__device__ __forceinline__ void dma_load_16(const void* src, uint32_t lds_base) {
+  __asm__ volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off"
+                   :
+                   : "s"(__builtin_amdgcn_readfirstlane(lds_base)), "v"(src)
+                   : "memory");
+}
+__device__ __forceinline__ void dma_load_4(const void* src, uint32_t lds_base) {
+  __asm__ volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, off"
+                   :
+                   : "s"(__builtin_amdgcn_readfirstlane(lds_base)), "v"(src)
+                   : "memory");
+}
+
+}  // namespace vk

@@ -40,6 +40,7 @@
 
 #include <type_traits>
 
+#include "moe_common.hpp"
 #include "moe_heuristics.hpp"
 #include "mxfp4.hpp"
 #include "vk_internal.hpp"
@@ -99,31 +100,6 @@ __host__ __device__ inline int split_scale_stride(int K) { return (K / 32 + 15) 
 
 // Values per term of a split row: K rounded up to a whole K step.
 __host__ __device__ inline int split_row_k(int K) { return (K + 127) & ~127; }
-
-__device__ __forceinline__ float act_value(int activation, float g, float u,
-                                           float limit, float beta,
-                                           float linear_beta) {
-  if (activation == 1) {
-    const float sig = 1.0f / (1.0f + expf(-g));
-    const float gate_out = beta * tanhf(g / beta) * sig;
-    const float up_out = linear_beta > 0.0f ? linear_beta * tanhf(u / linear_beta) : u;
-    return gate_out * up_out;
-  }
-  if (limit > 0.0f) {
-    if (g > limit) g = limit;
-    if (u > limit) u = limit;
-    if (u < -limit) u = -limit;
-  }
-  // v_exp_f32 / v_rcp_f32: about 1 ulp each, far inside the bf16 rounding that follows
-  return (g * __builtin_amdgcn_rcpf(1.0f + __expf(-g))) * u;
-}
-
-__device__ __forceinline__ bf16x8 as_bf16x8(u32x4 v) {
-  union { u32x4 u; bf16x8 b; } c;
-  c.u = v;
-  return c.b;
-}
-
 
 // Stage 0 of a call that was asked to overwrite `out`: every workgroup clears
 // its share (the stage does not use `out`; the next stage starts after this one).
@@ -262,7 +238,6 @@ __device__ __forceinline__ void unit_tiles(const GemmArgs& p, int e, int unit, i
 // ---------------------------------------------------------------------------
 constexpr int kMaxRuns = 512;   // runs the resident kernel can list in LDS
 constexpr int kScMax = 4;       // 16-byte scale pieces per lane: NT * K/32 <= 64 * kScMax
-constexpr uint32_t kScaleLo = 64u, kScaleHi = 190u;  // scale bytes the scaled MFMA path takes
 
 typedef __attribute__((ext_vector_type(8))) int i32x8;
 typedef __attribute__((ext_vector_type(4))) int i32x4;
@@ -354,22 +329,6 @@ __device__ __forceinline__ void exact_unit_global(const uint8_t* const (&w_rows)
       }
     }
   }
-}
-
-// Largest bf16 exponent field among the 8 values of v: the exponent of the
-// largest magnitude, found with packed 16-bit maxima.
-__device__ __forceinline__ uint32_t bf16x8_max_exponent(u32x4 v) {
-  typedef __attribute__((ext_vector_type(2))) unsigned short u16x2;
-  union { uint32_t u; u16x2 h; } a, b, c, d;
-  a.u = v[0] & 0x7FFF7FFFu;
-  b.u = v[1] & 0x7FFF7FFFu;
-  c.u = v[2] & 0x7FFF7FFFu;
-  d.u = v[3] & 0x7FFF7FFFu;
-  a.h = __builtin_elementwise_max(a.h, b.h);
-  c.h = __builtin_elementwise_max(c.h, d.h);
-  a.h = __builtin_elementwise_max(a.h, c.h);
-  const uint32_t m = max(a.u & 0xFFFFu, a.u >> 16);
-  return m >> 7;
 }
 
 // 8 bf16 values -> the 8 E4M3 leading parts of v / 2^(sb-127) and the 8 E4M3
@@ -1125,33 +1084,6 @@ __host__ __device__ inline int wide_window_rows(int block_size) {
   return kWideRows % block_size == 0 ? kWideRows : tile_group_rows(block_size, kWideRows);
 }
 
-// s_waitcnt immediate that waits until at most n vector-memory operations are
-// outstanding and for nothing else (vmcnt is split over bits 3:0 and 15:14).
-constexpr int vmcnt_only(int n) { return (n & 15) | ((n >> 4) << 14) | 0x0F70; }
-
-template <int N>
-struct IntC {
-  static constexpr int value = N;
-};
-
-// The DMA form of the global load: every lane's 16 (4) bytes at `src` go to LDS
-// at byte address lds_base + 16 (4) * lane.  Written as assembly because the
-// compiler makes every later LDS read wait for all DMA loads it has emitted
-// itself, and for every register load issued along with them: a ring that is
-// filled several steps ahead needs the counted waits of the kernel instead.
-__device__ __forceinline__ void dma_load_16(const void* src, uint32_t lds_base) {
-  __asm__ volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off"
-                   :
-                   : "s"(__builtin_amdgcn_readfirstlane(lds_base)), "v"(src)
-                   : "memory");
-}
-__device__ __forceinline__ void dma_load_4(const void* src, uint32_t lds_base) {
-  __asm__ volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, off"
-                   :
-                   : "s"(__builtin_amdgcn_readfirstlane(lds_base)), "v"(src)
-                   : "memory");
-}
-
 template <int STAGE>
 __global__ __launch_bounds__(64 * kWideWaves) void tile_wide_kernel(GemmArgs p) {
   constexpr int NT = kWideNT, MT = kWideMT, R = kWideRing;
@@ -1823,11 +1755,27 @@ GemmArgs down_args(const FusedMoeArgs& a) {
 
 size_t fused_moe_workspace_bytes(int M, int hidden, int ispp, int top_k, int EM) {
   if (M <= 0 || EM <= 0 || hidden <= 0 || ispp <= 0 || top_k <= 0) return 0;
-  return workspace_layout(M, hidden, ispp, top_k, EM).total();
+  // enough for either layout (raw weights, prepacked weights)
+  const size_t raw = workspace_layout(M, hidden, ispp, top_k, EM).total();
+  const size_t packed = mx_workspace_bytes(M, hidden, ispp, top_k, EM);
+  return raw > packed ? raw : packed;
+}
+
+void launch_fill_i32(int32_t* dst, int32_t value, int n, hipStream_t stream) {
+  if (n <= 0) return;
+  hipLaunchKernelGGL(fill_i32_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream, dst,
+                     value, n);
+}
+
+void launch_combine(const float* y, const int32_t* pos, float* out, int M, int top_k, int hidden,
+                    bool overwrite, hipStream_t stream) {
+  const dim3 grid((unsigned)((hidden / 4 + 255) / 256), (unsigned)(M < 65535 ? M : 65535));
+  hipLaunchKernelGGL(combine_kernel, grid, dim3(256), 0, stream, y, pos, out, M, top_k, hidden,
+                     overwrite ? 1 : 0);
 }
 
 bool prepare_moe_kernels() {
-  bool ok = wide_kernel_ready<0>() && wide_kernel_ready<1>();
+  bool ok = wide_kernel_ready<0>() && wide_kernel_ready<1>() && prepare_mx_kernels();
 #define VK_READY(S_, W_, NT_, D_) ok = resident_kernel_ready<S_, W_, NT_, D_>() && ok;
   VK_RESIDENT_VARIANTS(VK_READY)
 #undef VK_READY
@@ -1841,10 +1789,32 @@ void launch_moe_gateup(const FusedMoeArgs& a, hipStream_t stream) {
   launch_stage<0>(g, plan_stage<0>(g), stream);
 }
 
+// The second stage alone.  With a workspace (and packed weights) it runs as in the
+// fused call: act split by a pass of its own, rows stored and summed per token.
 void launch_moe_down(const FusedMoeArgs& a, hipStream_t stream) {
   if (a.M <= 0 || a.EM <= 0 || a.block_size <= 0) return;
-  const GemmArgs g = down_args(a);
-  launch_stage<1>(g, plan_stage<1>(g), stream);
+  GemmArgs g = down_args(a);
+  const StagePlan pl = plan_stage<1>(g);
+  const bool overwrite = (a.flags & 1u) != 0u;  // VK_HIP_MOE_OVERWRITE_OUT
+  if (pl.variant != kMoeVariantResident && debug_knobs().presplit != 0) {
+    if (a.w2_packed != nullptr && launch_moe_down_prepacked(a, stream)) return;
+    Workspace w;
+    if (carve_workspace(a, w) && g.K >= 512 && wide_kernel_ready<1>() && debug_knobs().combine != 0) {
+      const long long pieces = (long long)a.EM * split_row_k(a.ispp) / 8;
+      hipLaunchKernelGGL(split_rows_kernel, dim3((unsigned)((pieces + 255) / 256)), dim3(256), 0,
+                         stream, a.act, w.act_q, w.act_s, pieces, a.ispp);
+      g.Aq = w.act_q;
+      g.As = w.act_s;
+      g.y = w.y;
+      g.pos = w.pos;
+      launch_fill_i32(w.pos, -1, a.M * a.top_k, stream);
+      launch_stage<1>(g, pl, stream);
+      launch_combine(w.y, w.pos, a.out, a.M, a.top_k, a.hidden, overwrite, stream);
+      return;
+    }
+  }
+  if (overwrite) launch_fill_i32(reinterpret_cast<int32_t*>(a.out), 0, a.M * a.hidden, stream);
+  launch_stage<1>(g, pl, stream);
 }
 
 // Both stages.  With a workspace, a stage that runs as the tile kernel takes
@@ -1855,6 +1825,11 @@ void launch_fused_moe(const FusedMoeArgs& a, hipStream_t stream) {
   GemmArgs g0 = gateup_args(a);
   GemmArgs g1 = down_args(a);
   const StagePlan p0 = plan_stage<0>(g0), p1 = plan_stage<1>(g1);
+  // prefill-sized batches on prepacked weights: the FP4-rate kernels of moe_prefill.hip
+  if (a.w13_packed != nullptr && p0.variant != kMoeVariantResident &&
+      p1.variant != kMoeVariantResident && debug_knobs().presplit != 0 &&
+      launch_fused_moe_prepacked(a, stream))
+    return;
   Workspace w;
   bool combine = false;
   bool split_act_between = false;
@@ -1885,8 +1860,7 @@ void launch_fused_moe(const FusedMoeArgs& a, hipStream_t stream) {
         g1.y = w.y;
         g1.pos = w.pos;
         const int n = a.M * a.top_k;
-        hipLaunchKernelGGL(fill_i32_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream,
-                           w.pos, -1, n);
+        launch_fill_i32(w.pos, -1, n, stream);
       }
     }
   }
@@ -1903,9 +1877,7 @@ void launch_fused_moe(const FusedMoeArgs& a, hipStream_t stream) {
   }
   launch_stage<1>(g1, p1, stream);
   if (combine) {
-    const dim3 grid((unsigned)((a.hidden / 4 + 255) / 256), (unsigned)(a.M < 65535 ? a.M : 65535));
-    hipLaunchKernelGGL(combine_kernel, grid, dim3(256), 0, stream, w.y, w.pos, a.out, a.M, a.top_k,
-                       a.hidden, overwrite ? 1 : 0);
+    launch_combine(w.y, w.pos, a.out, a.M, a.top_k, a.hidden, overwrite, stream);
   }
 }
 

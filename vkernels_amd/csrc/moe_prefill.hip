@@ -1,0 +1,828 @@
+// moe_prefill.hip — the grouped GEMMs of the fused MXFP4 MoE layer for
+// prefill-sized batches, on weights prepacked at load time.
+//
+//   stage 0  act[r, 0:I]  = bf16(act_fn(A[tok(r)] . W13[e, 0:I]^T + b13, A[tok(r)] . W13[e, I:2I]^T + b13))
+//   stage 1  y[r, :]      = (act[r] . W2[e]^T + b2) * topk_w[flat(r)],  pos[flat(r)] = r
+//
+// (reference semantics: src/c/vkernels/kernels/moe_fused.cpp:235-564; the
+// per-token sum of the y rows is combine_kernel's, in moe_gemm.hip.)
+//
+// Arithmetic.  v_mfma_scale_f32_32x32x64_f8f6f4 with the weights as the FP4
+// (E2M1) operand and the activations as FP6 (E2M3) operands, both at the FP4
+// rate of the matrix cores.  The weight codes are moved onto the OCP code
+// points and their scale bytes decremented once, when the weights are
+// prepacked (mxfp4.hpp: the reference's decode table is half of OCP's).  A
+// bf16 activation is fed as a sum of TERMS FP6 terms per block of 32 along K:
+// with e the largest exponent field of the block and s = 2^(e-2-127),
+//     t0 = Q(a / s) s,  t1 = Q((a - t0) / (s/16)) (s/16),  t2 = Q((a - t0 - t1) / (s/256)) (s/256),
+// Q = round to nearest even on the E2M3 grid; one MFMA per term, the term's
+// scale byte being e-2, e-6, e-10.  Three terms represent a bf16 value exactly
+// unless it lies more than 2^-13 below the largest of its block; two terms
+// (VK_HIP_MOE_SPLIT2) leave an error of at most 2^-10 of the block's largest.
+// Units whose weights hold an inf/NaN code or a scale byte outside
+// [kScaleLo, kScaleHi] (flagged when the weights are prepacked) and segments
+// with a row whose blocks are outside the representable range (flagged when
+// the rows are split) are recomputed by exact_unit_mx: integer-exact
+// dequantisation of the raw weights, bf16 MFMAs, bf16 rows from global memory.
+//
+// Work split.  A workgroup of 4 wavefronts (one per SIMD, 512 registers each)
+// takes a window of 128 sorted rows -- cut into segments of consecutive blocks
+// of one expert -- against 4 weight units; a unit is 128 weight rows (stage 0:
+// 64 gate rows and the 64 up rows of the same columns, so the activation is
+// fused; stage 1: 128 consecutive rows) = 4 MFMA tiles of 32, private to one
+// wavefront: 4 x 4 accumulator tiles of 32 x 32 = 256 registers.  Per K step
+// of 128:
+//   * the split rows of the window (TERMS x 128 bytes per row) arrive in LDS
+//     by the DMA form of the global load, two steps ahead, as whole cache
+//     lines, the 16-byte pieces of a row rotated by the row index so that the
+//     MFMA operand reads are conflict-free; shared by the four wavefronts, one
+//     barrier per step;
+//   * the wavefront's weights arrive straight in registers, two steps ahead:
+//     the prepacked layout stores a unit's K step as 8 operand tiles of 64
+//     lanes x 16 bytes in lane order, then 8 scale bytes per lane, 8704
+//     contiguous bytes, so every load instruction reads 1 KiB contiguously;
+//   * every operand read from LDS (32 bytes per lane: 24 of codes, the block's
+//     scale byte, padding) feeds 4 MFMAs of 32 cycles; no vector arithmetic
+//     sits between them.
+// All loads are issued by inline assembly and waited for with counted
+// s_waitcnt, because each wavefront issues them in a fixed order.
+//
+// Workgroup ids are mapped to (window, unit group) so that the 32 workgroups
+// resident on one XCD at a time cover 4 windows x 8 unit groups or the like:
+// the rows of a window and the weights of an expert are then fetched into
+// that XCD's L2 once and shared.
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "moe_common.hpp"
+#include "vk_internal.hpp"
+
+namespace vk {
+namespace {
+
+typedef __attribute__((ext_vector_type(8))) int i32x8;
+typedef __attribute__((ext_vector_type(4))) int i32x4;
+typedef __attribute__((ext_vector_type(2))) uint32_t u32x2;
+typedef __attribute__((ext_vector_type(6))) uint32_t u32x6;
+typedef __attribute__((ext_vector_type(16))) float f32x16;
+typedef __attribute__((ext_vector_type(32))) float f32x32;
+typedef __attribute__((ext_vector_type(32))) __bf16 bf16x32;
+
+constexpr int kMxRows = 128;        // sorted rows per window
+constexpr int kMxUnitRows = 128;    // weight rows per unit
+constexpr int kMxWaves = 4;
+constexpr int kMxRing = 3;          // K steps of split rows in LDS
+constexpr int kMxStepBytes = 8704;  // prepacked bytes of one unit's K step: 8 KiB of codes + 512 of scales
+
+struct MxArgs {
+  const uint8_t* Wp;       // prepacked weights of the stage
+  const uint8_t* Wflags;   // [E, units]: 1 = the unit takes the exact path
+  const uint8_t* W;        // raw weights [E, rows_w, K/2] and scales [E, rows_w, K/32] (exact path)
+  const uint8_t* Ws;
+  const uint16_t* A;       // bf16 rows (exact path): stage 0 A [M, K], stage 1 act [EM, K]
+  const uint8_t* Aq;       // split rows: row r = TERMS planes of Kp bytes at r * TERMS * Kp
+  const uint8_t* row_bad;  // per row of Aq: 1 = outside the split's range
+  const int32_t* sorted_ids;
+  const int32_t* expert_ids;
+  const float* topk_w;
+  const float* bias;
+  uint16_t* act;           // stage 0 output [EM, ncols]
+  float* y;                // stage 1 output [EM, ncols]
+  int32_t* pos;            // stage 1: pos[flat] = sorted row
+  int n_flat, top_k, K, ncols, num_blocks, block_size;
+  float swiglu_limit, beta, linear_beta;
+  int activation;
+  int units, col_groups, windows;
+};
+
+__host__ __device__ inline int mx_kp(int K) { return (K + 127) & ~127; }
+__host__ __device__ inline int mx_units(int stage, int ncols) {
+  return stage == 0 ? ncols / 64 : (ncols + kMxUnitRows - 1) / kMxUnitRows;
+}
+// Row of W (within an expert) that lane row n of tile t of `unit` multiplies; the
+// caller checks it against the expert's row count (stage 1's last unit may be ragged).
+__host__ __device__ inline int mx_weight_row(int stage, int ncols, int unit, int t, int n) {
+  if (stage == 0) return (t >> 1) * ncols + unit * 64 + (t & 1) * 32 + n;
+  return unit * kMxUnitRows + t * 32 + n;
+}
+__host__ __device__ inline int mx_window_rows(int block_size) {
+  if (kMxRows % block_size == 0) return kMxRows;
+  for (int rows = kMxRows; rows > 16; rows -= 16)
+    if (block_size % rows == 0) return rows;
+  return 16;
+}
+
+// ---------------------------------------------------------------------------
+// Prepacking (load time).
+// ---------------------------------------------------------------------------
+
+// flags[e, unit] = 1 when a code of the unit's rows is inf/NaN or a scale byte
+// lies outside [kScaleLo, kScaleHi].  One workgroup per (unit, expert).
+__global__ __launch_bounds__(256) void prepack_flag_kernel(const uint8_t* __restrict__ W,
+                                                           const uint8_t* __restrict__ Ws,
+                                                           uint8_t* __restrict__ flags, int stage,
+                                                           int rows_w, int ncols, int K, int units) {
+  const int unit = blockIdx.x, e = blockIdx.y;
+  const int n = threadIdx.x & 127, part = threadIdx.x >> 7;  // two threads per row
+  const int row = mx_weight_row(stage, ncols, unit, n >> 5, n & 31);
+  int bad = 0;
+  if (row < rows_w) {
+    const size_t r = (size_t)e * (size_t)rows_w + (size_t)row;
+    const uint32_t* codes = reinterpret_cast<const uint32_t*>(W + r * (size_t)(K / 2));
+    const uint8_t* sc = Ws + r * (size_t)(K / 32);
+    uint32_t any = 0u;
+    for (int i = part; i < K / 8; i += 2) any |= fp4x8_nonfinite(codes[i]);
+    for (int g = part; g < K / 32; g += 2) any |= (uint32_t)(((uint32_t)sc[g] - kScaleLo) > (kScaleHi - kScaleLo));
+    bad = any != 0u;
+  }
+  bad = __syncthreads_or(bad);
+  if (threadIdx.x == 0) flags[(size_t)e * units + unit] = (uint8_t)(bad != 0);
+}
+
+// One workgroup per (K step, unit, expert): 512 pieces of 16 bytes (codes on the
+// OCP points) and 64 x 8 scale bytes (decremented), zero codes / neutral scales
+// where the unit or K is ragged.
+__global__ __launch_bounds__(256) void prepack_kernel(const uint8_t* __restrict__ W,
+                                                      const uint8_t* __restrict__ Ws,
+                                                      uint8_t* __restrict__ packed, int stage,
+                                                      int rows_w, int ncols, int K, int units,
+                                                      int ksteps) {
+  const int kstep = blockIdx.x, unit = blockIdx.y, e = blockIdx.z;
+  const int groups = K / 32;
+  uint8_t* dst = packed + (((size_t)e * units + unit) * (size_t)ksteps + kstep) * (size_t)kMxStepBytes;
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const int pc = threadIdx.x + 256 * i;  // [half][tile][lane]
+    const int half = pc >> 8, t = (pc >> 6) & 3, lane = pc & 63;
+    const int row = mx_weight_row(stage, ncols, unit, t, lane & 31);
+    const int g = kstep * 4 + half * 2 + (lane >> 5);
+    u32x4 v = {0u, 0u, 0u, 0u};
+    if (row < rows_w && g < groups) {
+      const size_t r = (size_t)e * (size_t)rows_w + (size_t)row;
+      v = *reinterpret_cast<const u32x4*>(W + r * (size_t)(K / 2) + (size_t)g * 16);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) v[j] = fp4x8_to_ocp_doubled(v[j]);
+    }
+    *reinterpret_cast<u32x4*>(dst + (size_t)pc * 16) = v;
+  }
+  if (threadIdx.x < 64) {
+    const int lane = threadIdx.x;
+    uint32_t s8[2] = {0u, 0u};
+#pragma unroll
+    for (int half = 0; half < 2; ++half)
+#pragma unroll
+      for (int t = 0; t < 4; ++t) {
+        const int row = mx_weight_row(stage, ncols, unit, t, lane & 31);
+        const int g = kstep * 4 + half * 2 + (lane >> 5);
+        uint32_t s = 127u;
+        if (row < rows_w && g < groups)
+          s = ((uint32_t)Ws[((size_t)e * (size_t)rows_w + (size_t)row) * (size_t)groups + g] - 1u) & 0xFFu;
+        s8[half] |= s << (8 * t);
+      }
+    *reinterpret_cast<u32x2*>(dst + 8192 + lane * 8) = u32x2{s8[0], s8[1]};
+  }
+}
+
+// ---------------------------------------------------------------------------
+// bf16 rows [rows, K] -> split rows: per row TERMS planes of Kp bytes, a plane =
+// Kp/32 blocks of 32 bytes: 24 bytes of FP6 codes (value i at bit 6 i), the
+// term's scale byte, 7 zero bytes.  Blocks between K and Kp are zero with a
+// neutral scale.  row_bad[r] = 1 when a block of the row is outside the range
+// (inf/NaN, or a scale byte the scaled MFMA path does not take).
+// One workgroup per row, one lane per block of 32.
+// ---------------------------------------------------------------------------
+template <int TERMS>
+__global__ __launch_bounds__(256) void split_rows_fp6_kernel(const uint16_t* __restrict__ x,
+                                                             uint8_t* __restrict__ xq,
+                                                             uint8_t* __restrict__ row_bad, int K) {
+  const int kp = mx_kp(K);
+  const size_t row = blockIdx.x;
+  uint8_t* qrow = xq + row * (size_t)(TERMS * kp);
+  int bad = 0;
+  for (int b = threadIdx.x; b < kp / 32; b += 256) {
+    union { u32x4 q[4]; bf16x32 v; uint32_t d[16]; } in;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) in.q[i] = u32x4{0u, 0u, 0u, 0u};
+    if (b * 32 < K) {
+      const u32x4* src = reinterpret_cast<const u32x4*>(x + row * (size_t)K + (size_t)b * 32);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) in.q[i] = src[i];
+    }
+    uint32_t emax = max(max(bf16x8_max_exponent(in.q[0]), bf16x8_max_exponent(in.q[1])),
+                        max(bf16x8_max_exponent(in.q[2]), bf16x8_max_exponent(in.q[3])));
+    uint32_t sb = emax - 2u;
+    if (emax == 0u) {  // a block of zeros (or bf16 subnormals, taken as zero)
+      sb = 127u;
+    } else if (sb < kScaleLo + 4u * (TERMS - 1) || sb > kScaleHi) {
+      bad = 1;
+      sb = 127u;
+    }
+    f32x32 rest;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      rest[2 * i] = __uint_as_float(in.d[i] << 16);
+      rest[2 * i + 1] = __uint_as_float(in.d[i] & 0xFFFF0000u);
+    }
+#pragma unroll
+    for (int t = 0; t < TERMS; ++t) {
+      const uint32_t st = sb - 4u * t;
+      const float scale = __uint_as_float(st << 23);
+      union { bf16x32 v; uint32_t d[16]; } r16;  // the remainder is exact in bf16
+#pragma unroll
+      for (int i = 0; i < 16; ++i)
+        r16.d[i] = (__float_as_uint(rest[2 * i]) >> 16) | (__float_as_uint(rest[2 * i + 1]) & 0xFFFF0000u);
+      const u32x6 codes = __builtin_amdgcn_cvt_scalef32_pk32_fp6_bf16(r16.v, scale);
+      if (t + 1 < TERMS) rest -= __builtin_amdgcn_cvt_scalef32_pk32_f32_fp6(codes, scale);
+      uint8_t* blk = qrow + (size_t)t * kp + (size_t)b * 32;
+      *reinterpret_cast<u32x4*>(blk) = u32x4{codes[0], codes[1], codes[2], codes[3]};
+      *reinterpret_cast<u32x4*>(blk + 16) = u32x4{codes[4], codes[5], st, 0u};
+    }
+  }
+  bad = __syncthreads_or(bad);
+  if (threadIdx.x == 0) row_bad[row] = (uint8_t)(bad != 0);
+}
+
+// ---------------------------------------------------------------------------
+// Exact path of one unit for the 32 rows of one row tile: acc[t] = C[weight row of
+// tile t][activation row lane % 32] in the accumulator layout of the 32 x 32 MFMAs.
+// a_row: the bf16 row of this lane's activation row, or null for a padding row.
+// ---------------------------------------------------------------------------
+template <int STAGE>
+__device__ __forceinline__ void exact_unit_mx(const MxArgs& p, int e, int unit, const uint16_t* a_row,
+                                              int lane, f32x16 (&acc)[4]) {
+  const int n = lane & 31, hh = lane >> 5;
+  const int rows_w = STAGE == 0 ? 2 * p.ncols : p.ncols;
+  const int K = p.K;
+  const uint8_t* w_row[4];
+  const uint8_t* s_row[4];
+#pragma unroll
+  for (int t = 0; t < 4; ++t) {
+    const int row = mx_weight_row(STAGE, p.ncols, unit, t, n);
+    w_row[t] = nullptr;
+    s_row[t] = nullptr;
+    if (row < rows_w) {
+      const size_t r = (size_t)e * (size_t)rows_w + (size_t)row;
+      w_row[t] = p.W + r * (size_t)(K / 2);
+      s_row[t] = p.Ws + r * (size_t)(K / 32);
+    }
+#pragma unroll
+    for (int i = 0; i < 16; ++i) acc[t][i] = 0.f;
+  }
+#pragma unroll 1
+  for (int s = 0; s < K / 16; ++s) {  // 16 values of K: lane half hh takes 8 of them
+    const int k = 16 * s + 8 * hh;
+    u32x4 av = {0u, 0u, 0u, 0u};
+    if (a_row != nullptr) av = *reinterpret_cast<const u32x4*>(a_row + k);
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+      u32x4 wv = {0u, 0u, 0u, 0u};
+      if (w_row[t] != nullptr)
+        wv = dequant8_exact(*reinterpret_cast<const uint32_t*>(w_row[t] + k / 2), s_row[t][k >> 5]);
+      acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_bf16x8(wv), as_bf16x8(av), acc[t], 0, 0, 0);
+    }
+  }
+}
+
+// Register load of 16 (8) bytes per lane at base + voff (+ an immediate), not
+// waited for: the caller counts it and passes the registers through wait_loads.
+template <int OFF>
+__device__ __forceinline__ void load16_nowait(u32x4& dst, uint32_t voff, const uint8_t* base) {
+  __asm__ volatile("global_load_dwordx4 %0, %1, %2 offset:%3" : "=&v"(dst) : "v"(voff), "s"(base), "n"(OFF) : "memory");
+}
+__device__ __forceinline__ void load8_nowait(u32x2& dst, uint32_t voff, const uint8_t* base) {
+  __asm__ volatile("global_load_dwordx2 %0, %1, %2" : "=&v"(dst) : "v"(voff), "s"(base) : "memory");
+}
+// The DMA form with a uniform base and a 32-bit offset per lane: 16 bytes per lane to
+// LDS at lds_base + 16 * lane.
+__device__ __forceinline__ void dma16_saddr(uint32_t voff, const uint8_t* base, uint32_t lds_base) {
+  __asm__ volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+                   :
+                   : "s"(__builtin_amdgcn_readfirstlane(lds_base)), "v"(voff), "s"(base)
+                   : "memory");
+}
+
+struct WeightStep {  // one K step of a unit in registers
+  u32x4 w[8];        // [half][tile]
+  u32x2 sc;          // per lane: the 4 tiles' scale bytes of half 0, of half 1
+};
+
+// Waits until at most N vector-memory operations are outstanding; the registers of
+// `ws` are operands so that no use of them moves above the wait.
+template <int N>
+__device__ __forceinline__ void wait_loads(WeightStep& ws) {
+  __asm__ volatile("s_waitcnt vmcnt(%[n])"
+                   : "+v"(ws.w[0]), "+v"(ws.w[1]), "+v"(ws.w[2]), "+v"(ws.w[3]), "+v"(ws.w[4]),
+                     "+v"(ws.w[5]), "+v"(ws.w[6]), "+v"(ws.w[7]), "+v"(ws.sc)
+                   : [n] "n"(N)
+                   : "memory");
+}
+
+__device__ __forceinline__ i32x8 fp4_operand_ocp(u32x4 w) {  // codes already on the OCP points
+  const i32x4 y = {(int)w[0], (int)w[1], (int)w[2], (int)w[3]};
+  return __builtin_shufflevector(y, y, 0, 1, 2, 3, -1, -1, -1, -1);
+}
+
+template <int T>
+__device__ __forceinline__ f32x16 mfma_fp4_fp6(u32x4 w, i32x8 b, f32x16 acc, uint32_t wscale) {
+  // A: FP4 (cbsz 4), scale byte T of wscale; B: FP6 E2M3 (blgp 2), scale = byte 0 of b[6]
+  return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fp4_operand_ocp(w), b, acc, 4, 2, T,
+                                                         (int)wscale, 0, b[6]);
+}
+
+template <int STAGE, int TERMS>
+__global__ __launch_bounds__(64 * kMxWaves) void tile_mx_kernel(MxArgs p) {
+  constexpr int R = kMxRing;
+  constexpr int kSlotBytes = kMxRows * TERMS * 128;
+  typedef __attribute__((address_space(3))) void* lds_ptr;
+  extern __shared__ u32x4 mx_lds[];
+  __shared__ int row_flat[kMxRows];
+  __shared__ int seg_hi[2];   // highest routed row index among rows 0..63 / 64..127 (or -1)
+  __shared__ int seg_bad[2];  // a routed row of the half is outside the split's range
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int ln = lane & 31;
+  const int hh = lane >> 5;
+
+  // ---- (window, unit group) of this workgroup: chunks of 32 consecutive tiles go to
+  // one XCD (workgroup ids go round-robin over the 8 XCDs), chunk after chunk ----
+  const int total = p.col_groups * p.windows;
+  const int slot = blockIdx.x >> 3;
+  const int logical = ((slot >> 5) * 8 + (blockIdx.x & 7)) * 32 + (slot & 31);
+  if (logical >= total) return;
+  const int window = logical / p.col_groups;
+  const int colg = logical - window * p.col_groups;
+
+  const int K = p.K;
+  const int Kp = mx_kp(K);
+  const int nsteps = Kp / 128;
+  const int unit_raw = colg * kMxWaves + wave;
+  const bool has_unit = unit_raw < p.units;
+  const int unit = has_unit ? unit_raw : 0;
+  const uint32_t lds_base = (uint32_t)(uintptr_t)(lds_ptr)mx_lds;
+  const uint8_t* lds_bytes = reinterpret_cast<const uint8_t*>(mx_lds);
+
+  // Vector-memory operations of a wavefront per K step (for step c + 2): 4 TERMS row
+  // copies, 8 weight loads, 1 scale load.
+  constexpr int kRowOps = 4 * TERMS;
+  constexpr int kOps = kRowOps + 9;
+
+  auto segment = [&](const int row0_, const int n_rows_, const int e_) {
+    // uniform by construction; said so, so that addresses built on them stay scalar
+    const int row0 = __builtin_amdgcn_readfirstlane(row0_);
+    const int n_rows = __builtin_amdgcn_readfirstlane(n_rows_);
+    const int e = __builtin_amdgcn_readfirstlane(e_);
+    __syncthreads();  // the previous segment is done with row_flat and the ring
+    if (tid < kMxRows) {
+      int f = -1;
+      if (tid < n_rows) {
+        f = p.sorted_ids[row0 + tid];
+        if (f < 0 || f >= p.n_flat) f = -1;
+      }
+      row_flat[tid] = f;
+      int bad = 0;
+      if (f >= 0) bad = p.row_bad[STAGE == 0 ? f / p.top_k : row0 + tid];
+      const unsigned long long routed = __ballot(f >= 0);
+      const unsigned long long any_bad = __ballot(bad != 0);
+      if (lane == 0) {
+        seg_hi[wave] = routed != 0ull ? 63 - (int)__builtin_clzll(routed) : -1;
+        seg_bad[wave] = any_bad != 0ull;
+      }
+    }
+    __syncthreads();
+    const int hi = seg_hi[1] >= 0 ? 64 + seg_hi[1] : seg_hi[0];
+    const int n_live = (hi + 32) >> 5;  // row tiles of 32 up to the last routed row
+    if (n_live == 0) return;            // uniform
+    const bool slow = (seg_bad[0] | seg_bad[1]) != 0 ||
+                      (has_unit && p.Wflags[(size_t)e * p.units + unit] != 0);  // uniform per wavefront
+
+    // ---- row copies: one instruction moves 8 rows x 128 bytes of one term.  Lane
+    // (r, c) = (lane / 8, lane % 8) copies piece c ^ r of its row, so LDS position c of
+    // row r holds piece c ^ (r & 7).  Wavefront w copies row tile w (32 rows).
+    uint32_t cp_off[4];
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      const int r = lane >> 3, c = lane & 7;
+      const int rl = wave * 32 + g * 8 + r;
+      const int f = row_flat[rl];
+      size_t grow;
+      if (STAGE == 0) grow = f >= 0 ? (size_t)(f / p.top_k) : 0;
+      else grow = rl < n_rows ? (size_t)(row0 + rl) : (size_t)row0;
+      cp_off[g] = (uint32_t)(grow * (size_t)(TERMS * Kp)) + 16u * (uint32_t)(c ^ r);
+    }
+    auto copy_rows = [&](int step, int d) {  // operation d (0 .. 4 TERMS - 1) of the step's row copies
+      const int term = d >> 2, g = d & 3;
+      const int k0 = min(step, nsteps - 1) * 128;  // past the end: the last step again
+      const uint32_t dst = lds_base + (uint32_t)((step % R) * kSlotBytes +
+                                                 ((wave * TERMS + term) * 32 + g * 8) * 128);
+      dma16_saddr(cp_off[g] + (uint32_t)(term * Kp + k0), p.Aq, dst);
+    };
+    // ---- weight loads
+    const uint8_t* wp_unit = p.Wp + ((size_t)e * p.units + unit) * (size_t)nsteps * (size_t)kMxStepBytes;
+    const uint32_t voff16 = (uint32_t)lane * 16u, voff8 = (uint32_t)lane * 8u;
+    auto load_weights = [&](WeightStep& ws, int step, int j) {  // operation j (0 .. 8)
+      const uint8_t* base = wp_unit + (size_t)min(step, nsteps - 1) * (size_t)kMxStepBytes;
+      switch (j) {
+        case 0: load16_nowait<0>(ws.w[0], voff16, base); break;
+        case 1: load16_nowait<1024>(ws.w[1], voff16, base); break;
+        case 2: load16_nowait<2048>(ws.w[2], voff16, base); break;
+        case 3: load16_nowait<3072>(ws.w[3], voff16, base); break;
+        case 4: load16_nowait<0>(ws.w[4], voff16, base + 4096); break;
+        case 5: load16_nowait<1024>(ws.w[5], voff16, base + 4096); break;
+        case 6: load16_nowait<2048>(ws.w[6], voff16, base + 4096); break;
+        case 7: load16_nowait<3072>(ws.w[7], voff16, base + 4096); break;
+        default: load8_nowait(ws.sc, voff8, base + 8192); break;
+      }
+    };
+    // operation k (0 .. kOps - 1) of what a K step issues for step `step`
+    auto issue = [&](WeightStep& ws, int step, int k) {
+      if (k < kRowOps) copy_rows(step, k);
+      else load_weights(ws, step, k - kRowOps);
+    };
+
+    // ---- operand reads: lane (ln, hh) takes block 2 half + hh of row ln of row tile m:
+    // pieces 2 blk and 2 blk + 1, at positions (2 blk) ^ (ln & 7) and that ^ 1.  The four
+    // lane-dependent offsets (half 0 / 1, first / second piece) are added to the slot's
+    // base once per K step; row tile and term are immediate offsets of the reads.
+    uint32_t rd_off[4];
+    {
+      const uint32_t pos0 = (uint32_t)(((2 * hh) ^ (ln & 7)) * 16);
+      rd_off[0] = (uint32_t)(ln * 128) + pos0;
+      rd_off[1] = (uint32_t)(ln * 128) + (pos0 ^ 16u);
+      rd_off[2] = (uint32_t)(ln * 128) + (pos0 ^ 64u);
+      rd_off[3] = (uint32_t)(ln * 128) + (pos0 ^ 80u);
+    }
+    struct SlotBase {
+      const uint8_t* b[4];
+    };
+    auto slot_base = [&](int slot_) {
+      SlotBase sb;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        uint32_t off = rd_off[j] + (uint32_t)(slot_ * kSlotBytes);
+        __asm__ volatile("" : "+v"(off));  // one register per base: nothing to precompute per tile
+        sb.b[j] = lds_bytes + off;
+      }
+      return sb;
+    };
+    auto read_operand = [&](const SlotBase& sb, int m, int term, int half) {
+      const int tile_off = ((m * TERMS + term) * 32) * 128;
+      const u32x4 lo = *reinterpret_cast<const u32x4*>(sb.b[2 * half] + tile_off);
+      const u32x4 hi4 = *reinterpret_cast<const u32x4*>(sb.b[2 * half + 1] + tile_off);
+      return i32x8{(int)lo[0], (int)lo[1], (int)lo[2], (int)lo[3],
+                   (int)hi4[0], (int)hi4[1], (int)hi4[2], (int)hi4[3]};
+    };
+
+    f32x16 acc[4][4];
+#pragma unroll
+    for (int m = 0; m < 4; ++m)
+#pragma unroll
+      for (int t = 0; t < 4; ++t)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) acc[m][t][i] = 0.f;
+
+    auto k_loop = [&](auto live_c) {
+      constexpr int LIVE = decltype(live_c)::value;
+      constexpr int Q = 2 * LIVE * TERMS;               // operand reads per step
+      constexpr int kPer = (kOps + Q - 1) / Q;          // memory operations issued per read
+      WeightStep ws[3];
+      // prologue: what steps -2 and -1 would issue
+#pragma unroll
+      for (int k = 0; k < kOps; ++k) issue(ws[0], 0, k);
+#pragma unroll
+      for (int k = 0; k < kOps; ++k) issue(ws[1], 1, k);
+
+      // one K step; i = c % 3 picks the register set of the step's weights
+      auto step = [&](auto i_c, const int c) {
+          constexpr int i = decltype(i_c)::value;
+          constexpr int in2 = (i + 2) % 3;
+          // everything issued for step c has landed once only what step c - 1 issued
+          // (for step c + 1) is outstanding
+          wait_loads<kOps>(ws[i]);
+          __builtin_amdgcn_s_barrier();
+          __asm__ volatile("" ::: "memory");
+          int slot_ = c % R;
+          __asm__ volatile("" : "+s"(slot_));
+          const SlotBase sb = slot_base(slot_);
+          i32x8 cur = read_operand(sb, 0, 0, 0);
+          int issued = 0;
+#pragma unroll
+          for (int q = 0; q < Q; ++q) {
+            const int half = q / (LIVE * TERMS), m = (q / TERMS) % LIVE, term = q % TERMS;
+            i32x8 nxt = cur;
+            if (q + 1 < Q) {
+              const int q1 = q + 1;
+              nxt = read_operand(sb, (q1 / TERMS) % LIVE, q1 % TERMS, q1 / (LIVE * TERMS));
+            }
+#pragma unroll
+            for (int k = 0; k < kPer; ++k)
+              if (issued + k < kOps) issue(ws[in2], c + 2, issued + k);
+            issued += kPer;
+            __builtin_amdgcn_sched_barrier(0);
+            {  // (a wavefront without a unit multiplies unit 0's weights and drops the result)
+              const uint32_t wsc = ws[i].sc[half];
+              acc[m][0] = mfma_fp4_fp6<0>(ws[i].w[half * 4 + 0], cur, acc[m][0], wsc);
+              acc[m][1] = mfma_fp4_fp6<1>(ws[i].w[half * 4 + 1], cur, acc[m][1], wsc);
+              acc[m][2] = mfma_fp4_fp6<2>(ws[i].w[half * 4 + 2], cur, acc[m][2], wsc);
+              acc[m][3] = mfma_fp4_fp6<3>(ws[i].w[half * 4 + 3], cur, acc[m][3], wsc);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            cur = nxt;
+          }
+      };
+      // three steps per pass of the loop body (no exit inside it), then the remainder
+      int c0 = 0;
+#pragma unroll 1
+      for (; c0 + 3 <= nsteps; c0 += 3) {
+        step(IntC<0>{}, c0);
+        step(IntC<1>{}, c0 + 1);
+        step(IntC<2>{}, c0 + 2);
+      }
+      if (c0 < nsteps) step(IntC<0>{}, c0);
+      if (c0 + 1 < nsteps) step(IntC<1>{}, c0 + 1);
+      // the loads issued past the last step write registers and the ring: let them land
+      wait_loads<0>(ws[0]);
+      wait_loads<0>(ws[1]);
+      wait_loads<0>(ws[2]);
+    };
+    if (n_live > 3) k_loop(IntC<4>{});
+    else if (n_live == 3) k_loop(IntC<3>{});
+    else if (n_live == 2) k_loop(IntC<2>{});
+    else k_loop(IntC<1>{});
+    __syncthreads();
+
+    if (STAGE == 1 && colg == 0 && tid < n_rows && row_flat[tid] >= 0) p.pos[row_flat[tid]] = row0 + tid;
+    if (!has_unit) return;
+
+    // ---- epilogue: lane (ln, hh) holds, of activation row 32 m + ln, the weight rows
+    // 8 (i / 4) + 4 hh + i % 4 of each tile ----
+#pragma unroll
+    for (int m = 0; m < 4; ++m) {
+      if (m >= n_live) break;
+      f32x16 (&tile)[4] = acc[m];
+      const int flat = row_flat[m * 32 + ln];
+      const int srow = row0 + m * 32 + ln;
+      if (slow) {
+        const uint16_t* a_row = nullptr;
+        if (flat >= 0) a_row = p.A + (size_t)(STAGE == 0 ? flat / p.top_k : srow) * (size_t)K;
+        exact_unit_mx<STAGE>(p, e, unit, a_row, lane, tile);
+      }
+      if (flat < 0) continue;
+      if (STAGE == 0) {
+        const float* bias = p.bias != nullptr ? p.bias + (size_t)e * (size_t)(2 * p.ncols) : nullptr;
+#pragma unroll
+        for (int tp = 0; tp < 2; ++tp)
+#pragma unroll
+          for (int rg = 0; rg < 4; ++rg) {
+            const int col = unit * 64 + tp * 32 + rg * 8 + hh * 4;
+            uint32_t packed[2];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+              float g = tile[tp][rg * 4 + i], u = tile[tp + 2][rg * 4 + i];
+              if (bias != nullptr) {
+                g += bias[col + i];
+                u += bias[p.ncols + col + i];
+              }
+              const uint32_t v = f32_to_bf16_bits(
+                  act_value(p.activation, g, u, p.swiglu_limit, p.beta, p.linear_beta));
+              if (i & 1) packed[i >> 1] |= v << 16;
+              else packed[i >> 1] = v;
+            }
+            *reinterpret_cast<uint2*>(p.act + (size_t)srow * (size_t)p.ncols + col) =
+                make_uint2(packed[0], packed[1]);
+          }
+      } else {
+        const float w = p.topk_w[flat];
+        float* yrow = p.y + (size_t)srow * (size_t)p.ncols;
+#pragma unroll
+        for (int t = 0; t < 4; ++t)
+#pragma unroll
+          for (int rg = 0; rg < 4; ++rg) {
+            const int col = unit * kMxUnitRows + t * 32 + rg * 8 + hh * 4;
+            if (col >= p.ncols) continue;  // the last unit may be ragged (ncols is a multiple of 64)
+            f32x4 v = {tile[t][rg * 4], tile[t][rg * 4 + 1], tile[t][rg * 4 + 2], tile[t][rg * 4 + 3]};
+            if (p.bias != nullptr)
+              v += *reinterpret_cast<const f32x4*>(p.bias + (size_t)e * (size_t)p.ncols + col);
+            *reinterpret_cast<f32x4*>(yrow + col) = v * w;
+          }
+      }
+    }
+  };
+
+  const int total_rows = p.num_blocks * p.block_size;
+  const int win = mx_window_rows(p.block_size);
+  int row = window * win;
+  const int win_end = min(row + win, total_rows);
+  while (row < win_end) {  // uniform
+    const int e = p.expert_ids[row / p.block_size];
+    int seg_end = min(win_end, (row / p.block_size + 1) * p.block_size);
+    while (seg_end < win_end && p.expert_ids[seg_end / p.block_size] == e)
+      seg_end = min(win_end, seg_end + p.block_size);
+    if (e >= 0) segment(row, seg_end - row, e);
+    row = seg_end;
+  }
+}
+
+template <int STAGE, int TERMS>
+bool mx_kernel_ready() {
+  static const bool configured = [] {
+    const hipError_t err = hipFuncSetAttribute(
+        reinterpret_cast<const void*>(tile_mx_kernel<STAGE, TERMS>),
+        hipFuncAttributeMaxDynamicSharedMemorySize, kMxRing * kMxRows * TERMS * 128);
+    if (err != hipSuccess) (void)hipGetLastError();  // not left for the next caller to find
+    return err == hipSuccess;
+  }();
+  return configured;
+}
+
+template <int STAGE, int TERMS>
+void launch_mx_stage_t(MxArgs g, hipStream_t stream) {
+  const int win = mx_window_rows(g.block_size);
+  g.units = mx_units(STAGE, g.ncols);
+  g.col_groups = (g.units + kMxWaves - 1) / kMxWaves;
+  g.windows = (g.num_blocks * g.block_size + win - 1) / win;
+  const long long total = (long long)g.col_groups * g.windows;
+  const unsigned grid = (unsigned)((total + 255) / 256 * 256);
+  hipLaunchKernelGGL((tile_mx_kernel<STAGE, TERMS>), dim3(grid), dim3(64 * kMxWaves),
+                     kMxRing * kMxRows * TERMS * 128, stream, g);
+}
+
+MxArgs mx_args(const FusedMoeArgs& a, int stage) {
+  MxArgs g{};
+  g.sorted_ids = a.sorted_ids;
+  g.expert_ids = a.expert_ids;
+  g.topk_w = a.topk_w;
+  g.act = a.act;
+  g.n_flat = a.M * a.top_k;
+  g.top_k = a.top_k;
+  g.num_blocks = a.EM / a.block_size;
+  g.block_size = a.block_size;
+  g.swiglu_limit = a.swiglu_limit;
+  g.beta = a.beta;
+  g.linear_beta = a.linear_beta;
+  g.activation = a.activation;
+  if (stage == 0) {
+    g.A = a.A; g.W = a.w13; g.Ws = a.w13_scale; g.bias = a.b13; g.K = a.hidden; g.ncols = a.ispp;
+  } else {
+    g.A = a.act; g.W = a.w2; g.Ws = a.w2_scale; g.bias = a.b2; g.K = a.ispp; g.ncols = a.hidden;
+  }
+  return g;
+}
+
+size_t align256(size_t n) { return (n + 255) & ~(size_t)255; }
+
+}  // namespace
+
+// ---- prepacked weights -------------------------------------------------------
+
+size_t moe_prepack_bytes(int num_experts, int rows, int K, int stage) {
+  if (num_experts <= 0 || rows <= 0 || K <= 0) return 0;
+  const int ncols = stage == 0 ? rows / 2 : rows;
+  const size_t units = (size_t)mx_units(stage, ncols);
+  return align256((size_t)num_experts * units * (size_t)(mx_kp(K) / 128) * kMxStepBytes) +
+         align256((size_t)num_experts * units);
+}
+
+void launch_moe_prepack(const uint8_t* w, const uint8_t* w_scale, int num_experts, int rows, int K,
+                        int stage, uint8_t* packed, hipStream_t stream) {
+  const int ncols = stage == 0 ? rows / 2 : rows;
+  const int units = mx_units(stage, ncols);
+  const int ksteps = mx_kp(K) / 128;
+  uint8_t* flags = packed + align256((size_t)num_experts * units * (size_t)ksteps * kMxStepBytes);
+  hipLaunchKernelGGL(prepack_flag_kernel, dim3(units, num_experts), dim3(256), 0, stream, w, w_scale,
+                     flags, stage, rows, ncols, K, units);
+  hipLaunchKernelGGL(prepack_kernel, dim3(ksteps, units, num_experts), dim3(256), 0, stream, w,
+                     w_scale, packed, stage, rows, ncols, K, units, ksteps);
+}
+
+// ---- workspace of the prepacked path -------------------------------------------
+//   split rows of A [M, 3 Kp(hidden)], of act [EM, 3 Kp(ispp)], their row flags,
+//   the second stage's rows y [EM, hidden] fp32, pos [M top_k].
+
+namespace {
+struct MxWorkspace {
+  size_t aq, cq, abad, cbad, y, pos;
+  size_t total() const { return aq + cq + abad + cbad + y + pos; }
+};
+MxWorkspace mx_workspace(int M, int hidden, int ispp, int top_k, int EM) {
+  MxWorkspace l;
+  l.aq = align256((size_t)M * 3 * mx_kp(hidden));
+  l.cq = align256((size_t)EM * 3 * mx_kp(ispp));
+  l.abad = align256((size_t)M);
+  l.cbad = align256((size_t)EM);
+  l.y = align256((size_t)EM * hidden * sizeof(float));
+  l.pos = align256((size_t)M * top_k * sizeof(int32_t));
+  return l;
+}
+}  // namespace
+
+size_t mx_workspace_bytes(int M, int hidden, int ispp, int top_k, int EM) {
+  return mx_workspace(M, hidden, ispp, top_k, EM).total();
+}
+
+bool prepare_mx_kernels() {
+  return mx_kernel_ready<0, 2>() && mx_kernel_ready<0, 3>() && mx_kernel_ready<1, 2>() &&
+         mx_kernel_ready<1, 3>();
+}
+
+namespace {
+
+struct MxPlan {
+  MxArgs g0, g1;
+  uint8_t *aq, *cq, *abad, *cbad;
+  float* y;
+  int32_t* pos;
+  bool two_terms;
+};
+
+// False when the prepacked path does not take the call (no packed weights, workspace
+// short or misaligned, split rows beyond the 32-bit offsets of the row copies, LDS refused).
+bool mx_plan(const FusedMoeArgs& a, bool need_stage0, MxPlan& pl) {
+  if ((need_stage0 && a.w13_packed == nullptr) || a.w2_packed == nullptr || a.workspace == nullptr)
+    return false;
+  const MxWorkspace l = mx_workspace(a.M, a.hidden, a.ispp, a.top_k, a.EM);
+  if (a.workspace_bytes < l.total() || (reinterpret_cast<uintptr_t>(a.workspace) & 15) != 0) return false;
+  if ((unsigned long long)a.EM * 3ull * mx_kp(a.ispp) >= (1ull << 32) ||
+      (unsigned long long)a.M * 3ull * mx_kp(a.hidden) >= (1ull << 32))
+    return false;
+  pl.two_terms = (a.flags & 2u) != 0u;  // VK_HIP_MOE_SPLIT2
+  if (pl.two_terms ? !(mx_kernel_ready<0, 2>() && mx_kernel_ready<1, 2>())
+                   : !(mx_kernel_ready<0, 3>() && mx_kernel_ready<1, 3>()))
+    return false;
+  uint8_t* base = static_cast<uint8_t*>(a.workspace);
+  pl.aq = base;
+  pl.cq = pl.aq + l.aq;
+  pl.abad = pl.cq + l.cq;
+  pl.cbad = pl.abad + l.abad;
+  pl.y = reinterpret_cast<float*>(pl.cbad + l.cbad);
+  pl.pos = reinterpret_cast<int32_t*>(pl.cbad + l.cbad + l.y);
+  pl.g0 = mx_args(a, 0);
+  pl.g1 = mx_args(a, 1);
+  const int units0 = mx_units(0, a.ispp), units1 = mx_units(1, a.hidden);
+  pl.g0.Wp = a.w13_packed;
+  pl.g0.Wflags = a.w13_packed == nullptr ? nullptr :
+      a.w13_packed + align256((size_t)a.num_experts * units0 * (size_t)(mx_kp(a.hidden) / 128) * kMxStepBytes);
+  pl.g1.Wp = a.w2_packed;
+  pl.g1.Wflags = a.w2_packed + align256((size_t)a.num_experts * units1 * (size_t)(mx_kp(a.ispp) / 128) * kMxStepBytes);
+  pl.g0.Aq = pl.aq; pl.g0.row_bad = pl.abad;
+  pl.g1.Aq = pl.cq; pl.g1.row_bad = pl.cbad;
+  pl.g1.y = pl.y; pl.g1.pos = pl.pos;
+  return true;
+}
+
+void mx_stage0(const FusedMoeArgs& a, const MxPlan& pl, hipStream_t stream) {
+  if (pl.two_terms) {
+    hipLaunchKernelGGL(split_rows_fp6_kernel<2>, dim3(a.M), dim3(256), 0, stream, a.A, pl.aq, pl.abad, a.hidden);
+    launch_mx_stage_t<0, 2>(pl.g0, stream);
+  } else {
+    hipLaunchKernelGGL(split_rows_fp6_kernel<3>, dim3(a.M), dim3(256), 0, stream, a.A, pl.aq, pl.abad, a.hidden);
+    launch_mx_stage_t<0, 3>(pl.g0, stream);
+  }
+}
+
+// split act (every sorted row; padding rows hold old data and are never routed) ->
+// second stage -> per-token sum
+void mx_stage1(const FusedMoeArgs& a, const MxPlan& pl, hipStream_t stream) {
+  launch_fill_i32(pl.pos, -1, a.M * a.top_k, stream);
+  if (pl.two_terms) {
+    hipLaunchKernelGGL(split_rows_fp6_kernel<2>, dim3(a.EM), dim3(256), 0, stream, a.act, pl.cq, pl.cbad, a.ispp);
+    launch_mx_stage_t<1, 2>(pl.g1, stream);
+  } else {
+    hipLaunchKernelGGL(split_rows_fp6_kernel<3>, dim3(a.EM), dim3(256), 0, stream, a.act, pl.cq, pl.cbad, a.ispp);
+    launch_mx_stage_t<1, 3>(pl.g1, stream);
+  }
+  launch_combine(pl.y, pl.pos, a.out, a.M, a.top_k, a.hidden, (a.flags & 1u) != 0u, stream);
+}
+
+}  // namespace
+
+// The whole layer on prepacked weights; false when the path does not take the call
+// (nothing has been enqueued then).
+bool launch_fused_moe_prepacked(const FusedMoeArgs& a, hipStream_t stream) {
+  MxPlan pl;
+  if (!mx_plan(a, true, pl)) return false;
+  mx_stage0(a, pl, stream);
+  mx_stage1(a, pl, stream);
+  return true;
+}
+
+// The second stage alone (act is the caller's), likewise.
+bool launch_moe_down_prepacked(const FusedMoeArgs& a, hipStream_t stream) {
+  MxPlan pl;
+  if (!mx_plan(a, false, pl)) return false;
+  mx_stage1(a, pl, stream);
+  return true;
+}
+
+// Test hook: the split rows of bf16 rows [rows, K] as the GEMM kernels read them.
+void launch_split_rows_fp6(const uint16_t* x, int rows, int K, int terms, uint8_t* xq, uint8_t* row_bad,
+                           hipStream_t stream) {
+  if (rows <= 0) return;
+  if (terms == 2)
+    hipLaunchKernelGGL(split_rows_fp6_kernel<2>, dim3(rows), dim3(256), 0, stream, x, xq, row_bad, K);
+  else
+    hipLaunchKernelGGL(split_rows_fp6_kernel<3>, dim3(rows), dim3(256), 0, stream, x, xq, row_bad, K);
+}
+
+}  // namespace vk

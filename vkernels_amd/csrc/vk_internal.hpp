@@ -40,6 +40,10 @@ struct FusedMoeArgs {
   void* workspace;         // optional, see fused_moe_workspace_bytes
   size_t workspace_bytes;
   unsigned flags;          // VK_HIP_MOE_* of vkernels_hip.h
+  // optional: the weights prepacked by launch_moe_prepack (both or neither)
+  const uint8_t* w13_packed;
+  const uint8_t* w2_packed;
+  int num_experts;         // experts in the weight tensors (needed with prepacked weights)
 };
 
 // Bytes of workspace with which launch_fused_moe runs its fastest path.
@@ -48,6 +52,24 @@ size_t fused_moe_workspace_bytes(int M, int hidden, int ispp, int top_k, int EM)
 void launch_fused_moe(const FusedMoeArgs& a, hipStream_t stream);
 void launch_moe_gateup(const FusedMoeArgs& a, hipStream_t stream);
 void launch_moe_down(const FusedMoeArgs& a, hipStream_t stream);
+
+// Pieces of the workspace path shared between the translation units.
+void launch_fill_i32(int32_t* dst, int32_t value, int n, hipStream_t stream);
+void launch_combine(const float* y, const int32_t* pos, float* out, int M, int top_k, int hidden,
+                    bool overwrite, hipStream_t stream);
+
+// Prepacked weights (moe_prefill.hip): bytes of the packed form of [num_experts, rows,
+// K/2] codes + [num_experts, rows, K/32] scales (stage 0: rows = 2 * ispp, gate rows
+// first; stage 1: rows = hidden), the packing launch, and the layer on packed weights.
+size_t moe_prepack_bytes(int num_experts, int rows, int K, int stage);
+void launch_moe_prepack(const uint8_t* w, const uint8_t* w_scale, int num_experts, int rows, int K,
+                        int stage, uint8_t* packed, hipStream_t stream);
+size_t mx_workspace_bytes(int M, int hidden, int ispp, int top_k, int EM);
+bool launch_fused_moe_prepacked(const FusedMoeArgs& a, hipStream_t stream);
+bool launch_moe_down_prepacked(const FusedMoeArgs& a, hipStream_t stream);
+void launch_split_rows_fp6(const uint16_t* x, int rows, int K, int terms, uint8_t* xq, uint8_t* row_bad,
+                           hipStream_t stream);
+bool prepare_mx_kernels();
 
 // Per-kernel set-up that the launchers otherwise do on their first call (the
 // dynamic-LDS limits of the GEMM kernels), for callers that want it done before

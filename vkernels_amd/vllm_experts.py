@@ -41,6 +41,7 @@ __all__ = [
     "resolve_moe_fn",
     "resolve_route_fn",
     "resolve_dequant_fn",
+    "resolve_prepack_fns",
 ]
 
 VK_OK = 0
@@ -246,6 +247,24 @@ def resolve_moe_ws_fn(lib):
 
 
 MOE_OVERWRITE_OUT = 1  # VK_HIP_MOE_OVERWRITE_OUT
+MOE_SPLIT2 = 2         # VK_HIP_MOE_SPLIT2
+
+
+def resolve_prepack_fns(lib):
+    """(vk_hip_moe_prepack_bytes, vk_hip_moe_prepack_weights, vk_hip_fused_moe_mxfp4_prepacked)
+    or (None, None, None) when the library predates them."""
+    size_fn = getattr(lib, "vk_hip_moe_prepack_bytes", None)
+    pack_fn = getattr(lib, "vk_hip_moe_prepack_weights", None)
+    moe_fn = getattr(lib, "vk_hip_fused_moe_mxfp4_prepacked", None)
+    if size_fn is None or pack_fn is None or moe_fn is None:
+        return None, None, None
+    size_fn.restype = ctypes.c_size_t
+    size_fn.argtypes = [_I, _I, _I, _I]
+    pack_fn.restype = _I
+    pack_fn.argtypes = [_P, _P, _I, _I, _I, _I, _P, ctypes.c_size_t, _P]
+    moe_fn.restype = None
+    moe_fn.argtypes = _MOE_ARGTYPES[:-1] + [_P, ctypes.c_size_t, ctypes.c_uint, _P, _P, _I, _P]
+    return size_fn, pack_fn, moe_fn
 
 
 def resolve_moe_ex_fn(lib):
@@ -335,7 +354,8 @@ class FusedExperts:
 
     def __init__(self, w13, w13_scale, w2, w2_scale, *, b13=None, b2=None, activation="swiglu",
                  swiglu_limit: float = 0.0, beta: float = 4.0, linear_beta: float = 25.0,
-                 expert_map=None, local_num_experts=None, scratch: CaptureSafeScratch | None = None):
+                 expert_map=None, local_num_experts=None, scratch: CaptureSafeScratch | None = None,
+                 prepack: bool = False, split_terms: int = 3):
         torch = _require_torch()
         self.torch = torch
         self.lib = load_libvkernels_hip()
@@ -372,6 +392,34 @@ class FusedExperts:
         if expert_map is not None and (expert_map.dtype != torch.int32 or not expert_map.is_cuda):
             raise ValueError("expert_map must be an int32 device tensor")
         self.scratch = scratch or _scratch
+        # a second copy of the weights in the layout of the prefill-sized kernels
+        # (load time; batches of more than 512 routed rows then run at the FP4 rate)
+        if split_terms not in (2, 3):
+            raise ValueError("split_terms must be 2 or 3")
+        self.split_terms = split_terms
+        self.w13_packed = self.w2_packed = None
+        self.moe_prepacked_fn = None
+        if prepack:
+            self.prepack()
+
+    def prepack(self):
+        """Build the prepacked copies of w13 and w2 (idempotent)."""
+        if self.w13_packed is not None:
+            return
+        torch = self.torch
+        size_fn, pack_fn, moe_fn = resolve_prepack_fns(self.lib)
+        if pack_fn is None:
+            raise RuntimeError("vk_hip_moe_prepack_weights not found in libvkernels_hip.so")
+        packed = []
+        for stage, (w, ws, rows, K) in enumerate(((self.w13, self.w13_scale, 2 * self.ispp, self.hidden),
+                                                  (self.w2, self.w2_scale, self.hidden, self.ispp))):
+            n = int(size_fn(self.E, rows, K, stage))
+            buf = torch.empty(n, dtype=torch.uint8, device=w.device)
+            st = pack_fn(_ptr(w), _ptr(ws), self.E, rows, K, stage, _ptr(buf), n, _stream(torch))
+            _check(self.lib, st, "vk_hip_moe_prepack_weights")
+            packed.append(buf)
+        self.w13_packed, self.w2_packed = packed
+        self.moe_prepacked_fn = moe_fn
 
     # -- routing ------------------------------------------------------------
     def route(self, logits, top_k: int, renormalize: bool = True):
@@ -392,6 +440,8 @@ class FusedExperts:
         torch = self.torch
         M, top_k = topk_ids.shape
         dev = topk_ids.device
+        if block_size <= 0 or block_size % 16 != 0:
+            raise ValueError(f"block_size must be a positive multiple of 16, got {block_size}")
         num_experts = self.global_E if num_experts is None else num_experts
         max_em = _align_em_bound(M, top_k, self.local_n, block_size)
         cap_m = max(M, max_tokens or 0)
@@ -419,6 +469,8 @@ class FusedExperts:
         top_k = topk_ids.shape[1]
         dev = hidden_states.device
         block_size = default_block_size(M, top_k) if block_size is None else block_size
+        if block_size <= 0 or block_size % 16 != 0:
+            raise ValueError(f"block_size must be a positive multiple of 16, got {block_size}")
         hidden_states = hidden_states.contiguous()
         topk_ids = topk_ids.to(torch.int32).contiguous()
         if topk_weights is None:
@@ -457,6 +509,9 @@ class FusedExperts:
                 _ptr(out_fp32), M, K, self.ispp, top_k, _ptr(sids), _ptr(eids), max_em,
                 float(self.swiglu_limit), self.activation, float(self.beta),
                 float(self.linear_beta), _ptr(self.b13), _ptr(self.b2), block_size)
+        # the entry points return void: a refused call (contract violation, launch error)
+        # leaves its message in the thread's error state, which is read back here
+        self.lib.vk_set_last_error(0, b"")
         if self.moe_ws_fn is not None and self.use_workspace:
             # the library splits the rows once per call into this workspace where its
             # tile kernels run (large batches, large K); held like the other scratch
@@ -465,9 +520,14 @@ class FusedExperts:
             cap_bytes = int(self.ws_bytes_fn(max(M, max_tokens or 0), K, self.ispp, top_k, cap))
             ws = self.scratch.get(("ws", K, self.ispp), need, dtype=torch.uint8, device=dev,
                                   capacity=cap_bytes, name="workspace")
-            if self.moe_ex_fn is not None:
-                self.moe_ex_fn(*args, _ptr(ws), need, MOE_OVERWRITE_OUT if overwrite else 0,
-                               _stream(torch))
+            flags = MOE_OVERWRITE_OUT if overwrite else 0
+            if self.w13_packed is not None:
+                if self.split_terms == 2:
+                    flags |= MOE_SPLIT2
+                self.moe_prepacked_fn(*args, _ptr(ws), need, flags, _ptr(self.w13_packed),
+                                      _ptr(self.w2_packed), self.E, _stream(torch))
+            elif self.moe_ex_fn is not None:
+                self.moe_ex_fn(*args, _ptr(ws), need, flags, _stream(torch))
             elif overwrite:
                 raise RuntimeError("overwrite=True needs vk_hip_fused_moe_mxfp4_ex")
             else:
@@ -476,6 +536,8 @@ class FusedExperts:
             raise RuntimeError("overwrite=True needs the workspace entry points")
         else:
             self.moe_fn(*args, _stream(torch))
+        if int(self.lib.vk_last_error_code()) != VK_OK:
+            raise RuntimeError(f"fused MoE call refused: {last_error(self.lib)}")
 
     def forward(self, hidden_states, router_logits, top_k: int, **kw):
         """Router + layer: returns (out fp32 [M, H], topk_ids, topk_w)."""
