@@ -1,28 +1,36 @@
 #!/usr/bin/env python3
 """Benchmark of the fused MXFP4 MoE layer on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c1:64]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c1:64] [--prefill c3:16384]
 
 A step is one pass of the whole hot path over one batch of synthetic tokens
-already resident in HBM: router -> on-device alignment -> clearing `out` ->
-gate/up grouped GEMM + SwiGLU -> down grouped GEMM + combine, all through the
-C ABI of libvkernels_hip.so on one stream.  The default workload is the
-decode-shaped layer the headline metric is quoted on (hidden 2880,
-intermediate 2880, 32 experts, top-4, T = 64).  Weight sets are rotated
-between steps so that the 256 MB Infinity Cache cannot serve the 423 MB of
-expert weights twice.
+already resident in HBM: router -> on-device alignment -> gate/up grouped GEMM
++ SwiGLU -> down grouped GEMM + combine, all through the C ABI of
+libvkernels_hip.so on one stream.
 
-One JSON line is printed.  `value` is tokens/s of the whole step.  `roofline`
-is for the dominant kernel (the gate/up GEMM, two thirds of the weight bytes):
-its algorithmic HBM bytes per launch divided by its mean duration, measured
-with events on the launch stream in a second loop of the same steps, against
-the 8 TB/s peak.  `cpu_baseline` times the reference's CPU oracle (or this
-repository's restatement when the reference build is absent) on the same
-workload on the host's cores.
+The metric has two halves, and one JSON line carries both:
+
+* the top-level fields are the decode-shaped workload the metric is quoted on
+  (hidden 2880, intermediate 2880, 32 experts, top-4, T = 64), HBM bound.
+  `roofline` is its dominant kernel (the gate/up GEMM, two thirds of the
+  weight bytes): algorithmic HBM bytes per launch over its mean duration,
+  measured with events on the launch stream in a second loop of the same
+  steps, against the 8 TB/s peak.  Weight sets are rotated between steps so
+  that the 256 MB Infinity Cache cannot serve the 423 MB of weights twice;
+* `prefill` is the prefill-shaped workload that is bound by the matrix cores
+  (hidden 7168, intermediate 2048, 256 experts, top-8, T = 16384) on weights
+  prepacked at load time: tokens/s of the whole step and a `roofline` whose
+  `achieved` is the layer's algorithmic flops (6 T k H I) over the mean
+  event-timed duration of the fused call, against the dense FP4 peak.
+
+`cpu_baseline` times the reference's CPU oracle (or this repository's
+restatement when the reference build is absent) on a bounded sample of the
+decode workload, single-threaded and on all host cores.
 """
 from __future__ import annotations
 
 import argparse
+import hashlib
 import json
 import os
 import sys
@@ -34,13 +42,7 @@ sys.path.insert(0, str(ROOT))
 
 HBM_PEAK_GBS = 8000.0
 FP4_PEAK_TFLOPS = 10100.0
-
-# HBM bytes per launch of the gate/up kernel from rocprofv3 FETCH_SIZE and
-# WRITE_SIZE counters (two runs of this script under --pmc, scaled by what the
-# same counters read for the 512 MiB copy of --copy-calibration: x2.0 and x1.0).
-# Counters cannot be read from inside this process, so the figure of the last
-# profiled build is recorded here per workload; null for the others.
-MEASURED_TRAFFIC = {"c1:64": 309.1e6}
+METRIC = "MoE layer tokens/s; % HBM BW roofline (decode), % FP4 MFMA peak (prefill)"
 
 
 def parse_args():
@@ -48,7 +50,12 @@ def parse_args():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--workload", default="c1:64", help="config:T, e.g. c1:64, c2:512")
+    ap.add_argument("--workload", default="c1:64", help="config:T of the top-level record, e.g. c1:64, c2:512")
+    ap.add_argument("--prefill", default="c3:16384",
+                    help="config:T of the `prefill` record (prepacked weights); 'none' skips it")
+    ap.add_argument("--split-terms", type=int, default=3, choices=(2, 3),
+                    help="FP6 terms per activation on the prepacked path")
+    ap.add_argument("--no-prepack", action="store_true", help="raw weights only, also for prefill sizes")
     ap.add_argument("--weight-sets", type=int, default=0, help="0 = enough to exceed 1 GiB")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--block-size", type=int, default=0)
@@ -58,71 +65,110 @@ def parse_args():
     return ap.parse_args()
 
 
-def cpu_baseline(cfg, T, seed, steps_budget_s=30.0):
-    """Reference CPU oracle on the same workload, single thread."""
+def sources_digest() -> str:
+    """Digest of the kernel sources: names the build a profile was taken on."""
+    h = hashlib.sha256()
+    for path in sorted((ROOT / "vkernels_amd" / "csrc").iterdir()):
+        h.update(path.name.encode())
+        h.update(path.read_bytes())
+    return h.hexdigest()[:16]
+
+
+def measured_traffic(workload: str):
+    """HBM bytes per launch of the workload's dominant kernel from the profiler's
+    FETCH_SIZE / WRITE_SIZE counters (profiles/traffic.json, written when the build
+    was profiled); None when the kernel sources have changed since."""
+    path = ROOT / "profiles" / "traffic.json"
+    if not path.is_file():
+        return None
+    try:
+        rec = json.loads(path.read_text()).get(workload)
+    except (OSError, ValueError):
+        return None
+    if not rec or rec.get("sources_sha16") != sources_digest():
+        return None
+    return rec.get("traffic_bytes")
+
+
+def cpu_baseline(cfg, T, seed, budget_s=12.0):
+    """Reference CPU oracle on a bounded sample of the workload: one thread (the
+    reference oracle is single-threaded) and all host cores (OpenMP over tiles,
+    bit-identical for any thread count)."""
     import numpy as np
     import oracle
     from vkernels_amd import synth
 
     use_ref = oracle.have_ref()
-    oracle.set_threads(1)
-    # bounded sample: enough tokens for about 10-30 s of single-core work
     t_cpu = min(T, 64)
     w = synth.make_weights(cfg.E, cfg.H, cfg.I, seed).numpy()
     A = synth.make_activations(t_cpu, cfg.H, seed)
     lg = synth.make_logits(cfg.logits, t_cpu, cfg.E, seed, A, cfg.H)
-    times = []
-    t_begin = time.perf_counter()
-    while len(times) < 3 and (not times or time.perf_counter() - t_begin < steps_budget_s):
-        t0 = time.perf_counter()
-        oracle.moe_layer(A, lg, *w, cfg.top_k, use_ref=use_ref)
-        times.append(time.perf_counter() - t0)
-    best = sorted(times)[len(times) // 2]
+
+    def timed(threads, ref):
+        oracle.set_threads(threads)
+        times = []
+        t_begin = time.perf_counter()
+        while len(times) < 3 and (not times or time.perf_counter() - t_begin < budget_s):
+            t0 = time.perf_counter()
+            oracle.moe_layer(A, lg, *w, cfg.top_k, use_ref=ref)
+            times.append(time.perf_counter() - t0)
+        return sorted(times)[len(times) // 2], len(times)
+
+    one, n_one = timed(1, use_ref)
+    cores = len(os.sched_getaffinity(0)) if hasattr(os, "sched_getaffinity") else (os.cpu_count() or 1)
+    cores = min(cores, int(os.environ.get("OMP_NUM_THREADS", cores) or cores))
+    many, n_many = timed(cores, False)  # the OpenMP build is this repository's restatement
+    oracle.set_threads(1)
     return {
-        "value": t_cpu / best, "unit": "tokens/s", "cores": 1,
+        "value": t_cpu / one, "unit": "tokens/s", "cores": 1,
         "kind": "reference" if use_ref else "port",
         "sample": f"{cfg.name} T={t_cpu}: router + align + fused layer, median of "
-                  f"{len(times)} runs, {best * 1e3:.1f} ms each",
+                  f"{n_one} runs, {one * 1e3:.1f} ms each",
+        "all_cores": {"value": t_cpu / many, "unit": "tokens/s", "cores": cores, "kind": "port",
+                      "sample": f"same sample, {many * 1e3:.1f} ms (median of {n_many})"},
+        "host_cpus": os.cpu_count(),
     }
 
 
-def main():
-    args = parse_args()
-    if args.gpus != 1:
-        print("bench.py: this build runs on one GPU; --gpus N with N > 1 is not supported "
-              "(no collectives are part of the fused MoE path)", file=sys.stderr)
-        sys.exit(2)
-
+def run_workload(args, workload, steps, warmup, prepack):
+    """Times one workload; returns the record's fields."""
     import numpy as np
     import torch
     from vkernels_amd import synth
     from vkernels_amd import vllm_experts as ve
 
-    name, t_str = args.workload.split(":")
+    name, t_str = workload.split(":")
     cfg = synth.CONFIGS[name]
     T = int(t_str)
     seed = synth.config_seed(cfg, T)
     dev = torch.device("cuda", 0)
-    torch.cuda.set_device(dev)
+    H, I, k = cfg.H, cfg.I, cfg.top_k
+    prefill = T * k > 512  # the library's own split between its decode and tile kernels
+    prepack = prepack and prefill
 
-    per_set = synth.algorithmic_bytes(cfg.H, cfg.I, cfg.E, cfg.top_k, 0, cfg.E)
+    per_set = synth.algorithmic_bytes(H, I, cfg.E, k, 0, cfg.E)
     n_sets = args.weight_sets or max(2, -(-(1 << 30) // per_set))
     n_sets = min(n_sets, 8)
+    if per_set > (1 << 30):
+        n_sets = 1  # one set is already several times the Infinity Cache
     experts = []
     for s in range(n_sets):
-        w = synth.make_weights(cfg.E, cfg.H, cfg.I, seed + 7919 * s, device=dev)
-        experts.append(ve.FusedExperts(w.w13, w.w13_scale, w.w2, w.w2_scale))
-    A_bits = synth.make_activations(T, cfg.H, seed)
-    logits_np = synth.make_logits(cfg.logits, T, cfg.E, seed, A_bits, cfg.H)
+        w = synth.make_weights(cfg.E, H, I, seed + 7919 * s, device=dev)
+        experts.append(ve.FusedExperts(w.w13, w.w13_scale, w.w2, w.w2_scale, prepack=prepack,
+                                       split_terms=args.split_terms))
+    A_bits = synth.make_activations(T, H, seed)
+    logits_np = synth.make_logits(cfg.logits, T, cfg.E, seed, A_bits, H)
     A = torch.from_numpy(A_bits.view(np.int16)).view(torch.bfloat16).to(dev)
     logits = torch.from_numpy(logits_np).to(dev)
-    out = torch.empty((T, cfg.H), dtype=torch.float32, device=dev)
-    bs = args.block_size or ve.default_block_size(T, cfg.top_k)
-    prefill = T * cfg.top_k > 512  # the library's own split between its decode and tile kernels
+    out = torch.empty((T, H), dtype=torch.float32, device=dev)
+    bs = args.block_size or ve.default_block_size(T, k)
+    lib = ve.load_libvkernels_hip()
+    lib.vk_hip_moe_gateup_mxfp4.restype = None
+    lib.vk_hip_moe_down_mxfp4.restype = None
 
     def step(i, events=None):
         fe = experts[i % n_sets]
-        ids, w = fe.route(logits, cfg.top_k, True)
+        ids, w = fe.route(logits, k, True)
         if events is None:
             fe.apply(A, ids, w, block_size=bs, out_fp32=out)
             return
@@ -141,35 +187,30 @@ def main():
         e0, e1, e2 = events
         e0.record()
         lib.vk_hip_moe_gateup_mxfp4(
-            ve._ptr(A), ve._ptr(fe.w13), ve._ptr(fe.w13_scale), ve._ptr(act), T, cfg.H, cfg.I,
-            cfg.top_k, ve._ptr(sids), ve._ptr(eids), max_em, ve._F(0.0), 0, ve._F(4.0),
+            ve._ptr(A), ve._ptr(fe.w13), ve._ptr(fe.w13_scale), ve._ptr(act), T, H, I,
+            k, ve._ptr(sids), ve._ptr(eids), max_em, ve._F(0.0), 0, ve._F(4.0),
             ve._F(25.0), None, bs, st)
         e1.record()
         lib.vk_hip_moe_down_mxfp4(
             ve._ptr(act), ve._ptr(fe.w2), ve._ptr(fe.w2_scale), ve._ptr(w), ve._ptr(out), T,
-            cfg.H, cfg.I, cfg.top_k, ve._ptr(sids), ve._ptr(eids), max_em, None, bs, st)
+            H, I, k, ve._ptr(sids), ve._ptr(eids), max_em, None, bs, st)
         e2.record()
 
-    lib = ve.load_libvkernels_hip()
-    lib.vk_hip_moe_gateup_mxfp4.restype = None
-    lib.vk_hip_moe_down_mxfp4.restype = None
-
-    for i in range(args.warmup):
+    for i in range(warmup):
         step(i)
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    for i in range(args.steps):
+    for i in range(steps):
         step(i)
     torch.cuda.synchronize()
-    elapsed = time.perf_counter() - t0
-    ms_per_step = elapsed / args.steps * 1e3
+    ms_per_step = (time.perf_counter() - t0) / steps * 1e3
 
     # Second loop: the same steps with events around each GEMM stage.
-    ev = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(args.steps)]
-    for i in range(min(args.warmup, 5)):
+    ev = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(steps)]
+    for i in range(min(warmup, 5)):
         step(i, ev[0])
     torch.cuda.synchronize()
-    for i in range(args.steps):
+    for i in range(steps):
         step(i, ev[i])
     torch.cuda.synchronize()
     gate_ms = sorted(e[0].elapsed_time(e[1]) for e in ev)
@@ -177,22 +218,27 @@ def main():
     gate_avg = sum(gate_ms) / len(gate_ms)
     down_avg = sum(down_ms) / len(down_ms)
 
-    # active experts from the actual routing
-    ids, _ = experts[0].route(logits, cfg.top_k, True)
-    active = int(torch.unique(ids).numel())
-    H, I, k = cfg.H, cfg.I, cfg.top_k
+    ids, _ = experts[0].route(logits, k, True)
+    active = int(torch.unique(ids).numel())  # from the actual routing
     gate_bytes = active * (I * H + I * H // 16) + 2 * T * H + 2 * T * k * I
     down_bytes = active * (H * I // 2 + H * I // 32) + 2 * T * k * I + 4 * T * H
     layer_bytes = synth.algorithmic_bytes(H, I, cfg.E, k, T, active)
     flops = synth.algorithmic_flops(H, I, k, T)
     if prefill:
-        # events[1]..[2] bracket the whole fused call (split pass + both grouped GEMMs)
         fused_tflops = flops / (down_avg * 1e-3) / 1e12
+        if prepack:
+            kernel = (f"vk_hip_fused_moe_mxfp4_prepacked (split_rows_fp6_kernel<{args.split_terms}> x2 + "
+                      f"tile_mx_kernel<0,{args.split_terms}> + tile_mx_kernel<1,{args.split_terms}> + combine_kernel)")
+            issued = float(args.split_terms)  # FP4-rate MFMAs per algorithmic product
+        else:
+            kernel = ("vk_hip_fused_moe_mxfp4_ex (split_rows_kernel + tile_wide_kernel<0> + "
+                      "tile_wide_kernel<1> + combine_kernel)")
+            issued = 4.0  # two FP8-rate MFMAs per product = four at the FP4 rate
         roofline = {
-            "bound": "mfma", "kernel": "vk_hip_fused_moe_mxfp4_ex (split_rows_kernel + tile_wide_kernel<0> "
-                                       "+ tile_wide_kernel<1> + combine_kernel)",
+            "bound": "mfma", "kernel": kernel,
             "achieved": fused_tflops, "peak": FP4_PEAK_TFLOPS, "unit": "TFLOP/s",
             "frac": fused_tflops / FP4_PEAK_TFLOPS, "traffic": None,
+            "matrix_rate_frac": issued * fused_tflops / FP4_PEAK_TFLOPS,
             "flops_per_launch": flops, "avg_launch_us": down_avg * 1e3,
             "median_launch_us": down_ms[len(down_ms) // 2] * 1e3,
         }
@@ -201,28 +247,21 @@ def main():
         roofline = {
             "bound": "hbm", "kernel": "stream_resident_kernel<0, ...> (gate/up grouped GEMM + SwiGLU)",
             "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-            "frac": achieved / HBM_PEAK_GBS, "traffic": MEASURED_TRAFFIC.get(args.workload),
+            "frac": achieved / HBM_PEAK_GBS, "traffic": measured_traffic(workload),
             "bytes_per_launch": gate_bytes, "avg_launch_us": gate_avg * 1e3,
             "median_launch_us": gate_ms[len(gate_ms) // 2] * 1e3,
         }
-
-    line = {
-        "metric": "MoE layer tokens/s; % HBM BW roofline (decode), % FP4 MFMA peak (prefill)",
+    rec = {
         "value": T / (ms_per_step * 1e-3),
         "unit": "tokens/s",
-        "n_gpus": 1,
-        "steps": args.steps,
-        "warmup": args.warmup,
+        "steps": steps,
+        "warmup": warmup,
         "ms_per_step": ms_per_step,
-        "higher_is_better": True,
-        "scaling": "weak",
-        "vs_baseline": None,
-        "dtype": "bf16",
-        "data": "synthetic",
         "config": {
             "workload": f"{cfg.name} T={T}: hidden {H}, intermediate {I}, {cfg.E} experts, "
                         f"top-{k}, MXFP4 weights, bf16 activations, {cfg.logits} routing",
             "block_size": bs, "active_experts": active, "weight_sets": n_sets,
+            "weights": "prepacked at load time (+ raw)" if prepack else "raw",
         },
         "roofline": roofline,
         "layer": {
@@ -233,7 +272,49 @@ def main():
             "down_kernel_gbs": None if prefill else down_bytes / (down_avg * 1e-3) / 1e9,
         },
     }
+    if prepack:
+        rec["config"]["split_terms"] = args.split_terms
+    del experts
+    torch.cuda.empty_cache()
+    return rec, cfg, T, seed
+
+
+def main():
+    args = parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on one GPU; --gpus N with N > 1 is not supported "
+              "(no collectives are part of the fused MoE path)", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    torch.cuda.set_device(torch.device("cuda", 0))
+
+    rec, cfg, T, seed = run_workload(args, args.workload, args.steps, args.warmup, not args.no_prepack)
+    line = {
+        "metric": METRIC,
+        "value": rec["value"],
+        "unit": rec["unit"],
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": rec["ms_per_step"],
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16",
+        "data": "synthetic",
+        "config": rec["config"],
+        "roofline": rec["roofline"],
+        "layer": rec["layer"],
+    }
+    if args.prefill != "none" and args.prefill != args.workload:
+        # fewer steps: a prefill step is milliseconds, and the default run must stay short
+        p_steps = max(5, min(args.steps, 20))
+        p_rec, _, _, _ = run_workload(args, args.prefill, p_steps, min(args.warmup, 3),
+                                      not args.no_prepack)
+        line["prefill"] = p_rec
     if args.copy_calibration:
+        dev = torch.device("cuda", 0)
         src = torch.empty(512 << 20, dtype=torch.uint8, device=dev).fill_(1)
         dst = torch.empty_like(src)
         for _ in range(3):

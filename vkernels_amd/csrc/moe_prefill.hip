@@ -53,6 +53,7 @@
 // that XCD's L2 once and shared.
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+#include <stdlib.h>
 
 #include "moe_common.hpp"
 #include "vk_internal.hpp"
@@ -93,6 +94,7 @@ struct MxArgs {
   float swiglu_limit, beta, linear_beta;
   int activation;
   int units, col_groups, windows;
+  int map_mode;  // experiment: 0 = chunks of 32 tiles per XCD, 1 = identity, n >= 2 = chunks of n tiles
 };
 
 __host__ __device__ inline int mx_kp(int K) { return (K + 127) & ~127; }
@@ -317,6 +319,16 @@ __device__ __forceinline__ void wait_loads(WeightStep& ws) {
                    : "memory");
 }
 
+// The same, and for the wavefront's LDS reads as well.
+template <int N>
+__device__ __forceinline__ void wait_loads_and_reads(WeightStep& ws) {
+  __asm__ volatile("s_waitcnt vmcnt(%[n]) lgkmcnt(0)"
+                   : "+v"(ws.w[0]), "+v"(ws.w[1]), "+v"(ws.w[2]), "+v"(ws.w[3]), "+v"(ws.w[4]),
+                     "+v"(ws.w[5]), "+v"(ws.w[6]), "+v"(ws.w[7]), "+v"(ws.sc)
+                   : [n] "n"(N)
+                   : "memory");
+}
+
 __device__ __forceinline__ i32x8 fp4_operand_ocp(u32x4 w) {  // codes already on the OCP points
   const i32x4 y = {(int)w[0], (int)w[1], (int)w[2], (int)w[3]};
   return __builtin_shufflevector(y, y, 0, 1, 2, 3, -1, -1, -1, -1);
@@ -349,7 +361,9 @@ __global__ __launch_bounds__(64 * kMxWaves) void tile_mx_kernel(MxArgs p) {
   // one XCD (workgroup ids go round-robin over the 8 XCDs), chunk after chunk ----
   const int total = p.col_groups * p.windows;
   const int slot = blockIdx.x >> 3;
-  const int logical = ((slot >> 5) * 8 + (blockIdx.x & 7)) * 32 + (slot & 31);
+  int logical = ((slot >> 5) * 8 + (blockIdx.x & 7)) * 32 + (slot & 31);
+  if (p.map_mode == 1) logical = blockIdx.x;
+  else if (p.map_mode >= 2) logical = ((slot / p.map_mode) * 8 + (blockIdx.x & 7)) * p.map_mode + (slot % p.map_mode);
   if (logical >= total) return;
   const int window = logical / p.col_groups;
   const int colg = logical - window * p.col_groups;
@@ -482,54 +496,78 @@ __global__ __launch_bounds__(64 * kMxWaves) void tile_mx_kernel(MxArgs p) {
 #pragma unroll
         for (int i = 0; i < 16; ++i) acc[m][t][i] = 0.f;
 
+    // The K loop, compiled once per number of live row tiles.  A step is Q groups of 4
+    // MFMAs (one operand of rows against the 4 weight tiles).  Software pipeline over the
+    // groups: while group q multiplies, the operand of group q + 1 is completed and the
+    // reads of group q + 2 are issued, across the step boundary as well, so the matrix pipe
+    // never waits for LDS.  Memory operations for step c + 2 are issued in groups 0 .. Q-3
+    // of step c.  After group Q-3 comes the step's one barrier: each wavefront has waited
+    // for its loads of step c + 1 (only the kOps operations of this step may be
+    // outstanding) and for its LDS reads of step c (all issued by then), so behind the
+    // barrier step c + 1 can be read and the slot of step c can take step c + 3.
     auto k_loop = [&](auto live_c) {
       constexpr int LIVE = decltype(live_c)::value;
-      constexpr int Q = 2 * LIVE * TERMS;               // operand reads per step
-      constexpr int kPer = (kOps + Q - 1) / Q;          // memory operations issued per read
+      constexpr int Q = 2 * LIVE * TERMS;                  // groups (operand reads) per step
+      constexpr int kPer = (kOps + Q - 3) / (Q - 2);       // memory operations per issuing group
+      auto group_operand = [&](const SlotBase& sb, int q) {
+        return read_operand(sb, (q / TERMS) % LIVE, q % TERMS, q / (LIVE * TERMS));
+      };
       WeightStep ws[3];
-      // prologue: what steps -2 and -1 would issue
+      // prologue: the loads of steps 0 and 1; step 0's have landed in every wavefront
+      // once only step 1's are outstanding
 #pragma unroll
       for (int k = 0; k < kOps; ++k) issue(ws[0], 0, k);
 #pragma unroll
       for (int k = 0; k < kOps; ++k) issue(ws[1], 1, k);
+      wait_loads<kOps>(ws[0]);
+      __builtin_amdgcn_s_barrier();
+      __asm__ volatile("" ::: "memory");
+      SlotBase sb = slot_base(0);
+      i32x8 cur = group_operand(sb, 0);
+      i32x8 nxt = group_operand(sb, 1);
 
       // one K step; i = c % 3 picks the register set of the step's weights
       auto step = [&](auto i_c, const int c) {
-          constexpr int i = decltype(i_c)::value;
-          constexpr int in2 = (i + 2) % 3;
-          // everything issued for step c has landed once only what step c - 1 issued
-          // (for step c + 1) is outstanding
-          wait_loads<kOps>(ws[i]);
-          __builtin_amdgcn_s_barrier();
-          __asm__ volatile("" ::: "memory");
-          int slot_ = c % R;
-          __asm__ volatile("" : "+s"(slot_));
-          const SlotBase sb = slot_base(slot_);
-          i32x8 cur = read_operand(sb, 0, 0, 0);
-          int issued = 0;
+        constexpr int i = decltype(i_c)::value;
+        constexpr int in1 = (i + 1) % 3, in2 = (i + 2) % 3;
+        int slot_next = (c + 1) % R;
+        __asm__ volatile("" : "+s"(slot_next));
+        const SlotBase sbn = slot_base(slot_next);
+        int issued = 0;
 #pragma unroll
-          for (int q = 0; q < Q; ++q) {
-            const int half = q / (LIVE * TERMS), m = (q / TERMS) % LIVE, term = q % TERMS;
-            i32x8 nxt = cur;
-            if (q + 1 < Q) {
-              const int q1 = q + 1;
-              nxt = read_operand(sb, (q1 / TERMS) % LIVE, q1 % TERMS, q1 / (LIVE * TERMS));
-            }
+        for (int q = 0; q < Q; ++q) {
+          const int half = q / (LIVE * TERMS), m = (q / TERMS) % LIVE;
+          const uint32_t wsc = ws[i].sc[half];
+          // (a wavefront without a unit multiplies unit 0's weights and drops the result)
+          acc[m][0] = mfma_fp4_fp6<0>(ws[i].w[half * 4 + 0], cur, acc[m][0], wsc);
+          __builtin_amdgcn_sched_barrier(0);
+          // reads of group q + 2; the last two groups read the next step's first two
+          const i32x8 pend = q + 2 < Q ? group_operand(sb, q + 2) : group_operand(sbn, q + 2 - Q);
+          __builtin_amdgcn_sched_barrier(0);
+          acc[m][1] = mfma_fp4_fp6<1>(ws[i].w[half * 4 + 1], cur, acc[m][1], wsc);
+          __builtin_amdgcn_sched_barrier(0);
+          if (q < Q - 2) {
 #pragma unroll
             for (int k = 0; k < kPer; ++k)
               if (issued + k < kOps) issue(ws[in2], c + 2, issued + k);
             issued += kPer;
-            __builtin_amdgcn_sched_barrier(0);
-            {  // (a wavefront without a unit multiplies unit 0's weights and drops the result)
-              const uint32_t wsc = ws[i].sc[half];
-              acc[m][0] = mfma_fp4_fp6<0>(ws[i].w[half * 4 + 0], cur, acc[m][0], wsc);
-              acc[m][1] = mfma_fp4_fp6<1>(ws[i].w[half * 4 + 1], cur, acc[m][1], wsc);
-              acc[m][2] = mfma_fp4_fp6<2>(ws[i].w[half * 4 + 2], cur, acc[m][2], wsc);
-              acc[m][3] = mfma_fp4_fp6<3>(ws[i].w[half * 4 + 3], cur, acc[m][3], wsc);
-            }
-            __builtin_amdgcn_sched_barrier(0);
-            cur = nxt;
           }
+          __builtin_amdgcn_sched_barrier(0);
+          acc[m][2] = mfma_fp4_fp6<2>(ws[i].w[half * 4 + 2], cur, acc[m][2], wsc);
+          __builtin_amdgcn_sched_barrier(0);
+          __asm__ volatile("" : "+v"(nxt));  // complete from here on (read a group ago)
+          __builtin_amdgcn_sched_barrier(0);
+          acc[m][3] = mfma_fp4_fp6<3>(ws[i].w[half * 4 + 3], cur, acc[m][3], wsc);
+          __builtin_amdgcn_sched_barrier(0);
+          if (q == Q - 3) {
+            wait_loads_and_reads<kOps>(ws[in1]);
+            __builtin_amdgcn_s_barrier();
+            __asm__ volatile("" ::: "memory");
+          }
+          cur = nxt;
+          nxt = pend;
+        }
+        sb = sbn;
       };
       // three steps per pass of the loop body (no exit inside it), then the remainder
       int c0 = 0;
@@ -643,7 +681,10 @@ void launch_mx_stage_t(MxArgs g, hipStream_t stream) {
   g.col_groups = (g.units + kMxWaves - 1) / kMxWaves;
   g.windows = (g.num_blocks * g.block_size + win - 1) / win;
   const long long total = (long long)g.col_groups * g.windows;
-  const unsigned grid = (unsigned)((total + 255) / 256 * 256);
+  static const int map_mode = [] { const char* v = getenv("VK_MOE_MX_MAP"); return v ? atoi(v) : 0; }();
+  g.map_mode = map_mode;
+  const long long period = map_mode >= 2 ? 8ll * map_mode : 256;
+  const unsigned grid = (unsigned)((total + period - 1) / period * period);
   hipLaunchKernelGGL((tile_mx_kernel<STAGE, TERMS>), dim3(grid), dim3(64 * kMxWaves),
                      kMxRing * kMxRows * TERMS * 128, stream, g);
 }
