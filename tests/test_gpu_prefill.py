@@ -21,7 +21,7 @@ from vkernels_amd import synth
 from vkernels_amd import vllm_experts as ve
 
 import test_gpu_configs as cfgs
-from gpu_util import MAX_ABS_TOL, REL_L2_TOL, cpu_layer, dev, error_metrics, to_dev
+from gpu_util import MAX_ABS_TOL, REL_L2_TOL, cpu_layer, dev, edge_tokens, error_metrics, to_dev
 
 pytestmark = pytest.mark.gpu
 
@@ -246,37 +246,6 @@ def test_onehot_rows_read_back_the_dequantised_weights(hip_lib, path):
 
 # ---- the layer -------------------------------------------------------------------------
 
-def _edge_tokens(g, n_flat, top_k, want, seed):
-    """Tokens whose sorted rows sit where a tile kernel breaks: first and last routed row
-    of windows of 128, rows either side of 32-row tile boundaries, the last row of an
-    expert's segment, rows of the most and the least popular expert; then random ones."""
-    sids, eids, bs = g["sids"], g["eids"], g["bs"]
-    routed = np.nonzero(sids < n_flat)[0]
-    rows = set()
-    win = routed // 128
-    first = routed[np.r_[True, win[1:] != win[:-1]]]
-    last = routed[np.r_[win[1:] != win[:-1], True]]
-    rng = np.random.default_rng(seed)
-    for arr in (first, last):
-        rows.update(rng.choice(arr, min(arr.size, 24), replace=False).tolist())
-    edge = routed[np.isin(routed % 32, (0, 31))]
-    rows.update(rng.choice(edge, min(edge.size, 24), replace=False).tolist())
-    expert_of_row = np.repeat(eids, bs)[routed]
-    counts = np.bincount(expert_of_row[expert_of_row >= 0])
-    live = np.nonzero(counts)[0]
-    for e in (live[np.argmax(counts[live])], live[np.argmin(counts[live])]):
-        er = routed[expert_of_row == e]
-        rows.update(er[[0, -1]].tolist())
-    tokens = set((sids[list(rows)] // top_k).tolist())
-    T = n_flat // top_k
-    extra = rng.permutation(T)
-    for t in extra:
-        if len(tokens) >= want:
-            break
-        tokens.add(int(t))
-    return np.sort(np.fromiter(tokens, dtype=np.int64))
-
-
 def _check_prefill(cfg, T, w, A_bits, logits, terms=3, sample=128, wn=None, gpu_kw=None, cpu_kw=None,
                    block_size=None, contract_only=False):
     gpu_kw = dict(gpu_kw or {})
@@ -285,7 +254,7 @@ def _check_prefill(cfg, T, w, A_bits, logits, terms=3, sample=128, wn=None, gpu_
     ids, tw = oracle.route_topk(logits, cfg.top_k, True)
     assert np.array_equal(g["ids"], ids) and np.array_equal(g["tw"].view(np.uint32), tw.view(np.uint32))
     rows = np.arange(T) if sample is None or sample >= T else \
-        _edge_tokens(g, T * cfg.top_k, cfg.top_k, sample, T)
+        edge_tokens(g, T * cfg.top_k, cfg.top_k, sample, T)
     wn = w.numpy() if wn is None else wn
     c = cpu_layer(A_bits[rows], wn, ids[rows], tw[rows], threads=16, **(cpu_kw or {}))
     max_rel, rel_l2, nf = error_metrics(g["out"][rows], c["out"])

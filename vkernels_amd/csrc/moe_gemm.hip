@@ -1135,12 +1135,13 @@ __global__ __launch_bounds__(64 * kWideWaves) void tile_wide_kernel(GemmArgs p) 
         if (f < 0 || f >= p.n_flat) f = -1;
       }
       row_flat[tid] = f;
-      const int cnt = (int)__popcll(__ballot(f >= 0));
-      if (lane == 0) wave_valid[wave] = cnt;
+      // one past the highest routed row of this half of the window (padding may stand
+      // anywhere among an expert's rows)
+      const unsigned long long routed = __ballot(f >= 0);
+      if (lane == 0) wave_valid[wave] = routed != 0ull ? 64 - (int)__builtin_clzll(routed) : 0;
     }
     __syncthreads();
-    // routed rows are a prefix of an expert's rows (padding follows them)
-    const int n_live = (wave_valid[0] + wave_valid[1] + 15) >> 4;
+    const int n_live = ((wave_valid[1] > 0 ? 64 + wave_valid[1] : wave_valid[0]) + 15) >> 4;
     if (n_live == 0) return;  // uniform
 
     const uint8_t* w_rows[NT];
