@@ -192,6 +192,12 @@ void vk_hip_fused_moe_mxfp4_ex(
  * The workspace size is vk_hip_fused_moe_mxfp4_workspace_bytes(...), as for _ws.
  */
 #define VK_HIP_MOE_SPLIT2 2u
+/* VK_HIP_MOE_W4A4: the W4A4 mode of the reference's orchestration ops
+ * (src/c/vkernels/kernels/moe_aux.hpp:1-25): both stages quantise their
+ * activations (A, then act) to MXFP4 exactly as mxfp4_moe_quant does and multiply
+ * FP4 by FP4, one matrix-core pass per product.  The layer then equals the
+ * reference's layer applied to the dequantised quantised activations. */
+#define VK_HIP_MOE_W4A4 4u
 
 size_t vk_hip_moe_prepack_bytes(int32_t num_experts, int32_t rows, int32_t K, int32_t stage);
 
@@ -309,6 +315,31 @@ void vk_hip_moe_down_mxfp4_ex(
  */
 int vk_hip_split_rows_fp6(const uint16_t* x, int32_t rows, int32_t K, int32_t terms, void* split,
                           uint8_t* row_flags, void* stream);
+
+/*
+ * Additive: device counterparts of the reference's MXFP4 MoE orchestration ops
+ * (CPU ABI src/c/vkernels/capi/capi.hpp:470-503, semantics
+ * src/c/vkernels/kernels/moe_aux.hpp:40-158), bit-identical to them:
+ *   vk_hip_mxfp4_moe_quant         A [M, hidden] bf16 -> packed [M, hidden/2] E2M1
+ *                                  codes (low nibble = even k) and scales
+ *                                  [M, hidden/32] ue8m0 (0xFF = zero group)
+ *   vk_hip_mxfp4_moe_sorted_quant  the same for row sorted_ids[r] / top_k of A per
+ *                                  sorted row r; padding rows (id outside
+ *                                  [0, M*top_k)) give zero codes and 0xFF scales
+ *   vk_hip_mxfp4_moe_scatter_reduce out[token, :] += partial[r, :] * topk_w[r] for
+ *                                  every routed sorted row r, in ascending r (gather
+ *                                  form: no atomics; workspace: M*top_k int32)
+ * group_size must be 32.  Return VK_OK or a VK_ERROR_* code.
+ */
+int vk_hip_mxfp4_moe_quant(const uint16_t* A, uint8_t* packed, uint8_t* scales, int32_t M,
+                           int32_t hidden, int32_t group_size, void* stream);
+int vk_hip_mxfp4_moe_sorted_quant(const uint16_t* A, const int32_t* sorted_ids, uint8_t* packed,
+                                  uint8_t* scales, int32_t M, int32_t hidden, int32_t group_size,
+                                  int32_t top_k, int32_t EM, void* stream);
+int vk_hip_mxfp4_moe_scatter_reduce(const float* partial, const float* topk_w,
+                                    const int32_t* sorted_ids, float* out, int32_t M, int32_t width,
+                                    int32_t top_k, int32_t EM, void* workspace,
+                                    size_t workspace_bytes, void* stream);
 
 /*
  * On-device alignment of the routing table: stable bucket of the flat indices

@@ -94,11 +94,13 @@ static inline float bf16_to_float(uint16_t v) {
  * model switched on (terms = 2 or 3) the grouped GEMMs multiply a' instead of
  * a, so a test can tell the error of that representation (model vs reference
  * arithmetic, both on the CPU) from the error of the GPU's accumulation (GPU
- * vs model).  terms = 0, the default, is the reference's arithmetic.
+ * vs model).  terms = 1 is the W4A4 mode: the activations are quantised to
+ * MXFP4 as the reference's mxfp4_moe_quant does (aux_oracle.c) and dequantised.
+ * terms = 0, the default, is the reference's arithmetic.
  */
 static int g_act_model = 0;
 
-void vko_set_act_model(int terms) { g_act_model = (terms == 2 || terms == 3) ? terms : 0; }
+void vko_set_act_model(int terms) { g_act_model = (terms >= 1 && terms <= 3) ? terms : 0; }
 
 static float e2m3_round(float v) {
   const float a = fabsf(v);
@@ -276,7 +278,10 @@ static void grouped_gemm(const uint16_t* A, int gather, const uint8_t* W,
                      : A + (size_t)(row0 + r) * a_stride + k_base + k0;
           float dot[BLK_N];
           float amodel[BLK_K];
-          if (g_act_model != 0) {
+          if (g_act_model == 1) {
+            vko_aux_model_block32(arow, amodel);
+            vko_aux_model_block32(arow + 32, amodel + 32);
+          } else if (g_act_model != 0) {
             vko_act_model_block32(arow, amodel, g_act_model);
             vko_act_model_block32(arow + 32, amodel + 32, g_act_model);
           }

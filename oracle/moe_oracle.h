@@ -141,6 +141,27 @@ void vko_set_threads(int n);
 void vko_set_act_model(int terms);
 void vko_act_model_block32(const uint16_t* a, float* out, int terms);
 
+/* ---- MXFP4 MoE orchestration ops (aux_oracle.c; moe_aux.cpp of the reference) ---- */
+uint8_t vko_aux_scale_byte(uint16_t amax_bits);
+void vko_mxfp4_moe_quant(const uint16_t* A, uint8_t* packed, uint8_t* scales, int M, int hidden,
+                         int group_size);
+void vko_mxfp4_moe_sorted_quant(const uint16_t* A, const int32_t* sorted_ids, uint8_t* packed,
+                                uint8_t* scales, int M, int hidden, int group_size, int top_k,
+                                int EM);
+void vko_mxfp4_moe_sort(const uint16_t* A, const int32_t* sorted_ids, uint16_t* A_sorted, int M,
+                        int hidden, int top_k, int EM);
+void vko_mxfp4_moe_sort_scales(const uint8_t* scales, const int32_t* sorted_ids,
+                               uint8_t* scales_sorted, int M, int n_groups, int top_k, int EM);
+void vko_mxfp4_moe_scatter_reduce(const float* partial, const float* topk_w,
+                                  const int32_t* sorted_ids, float* out, int M, int width,
+                                  int top_k, int EM);
+void vko_mxfp4_moe_scatter_reduce_q(const uint8_t* partial_q, const uint8_t* partial_s,
+                                    const float* topk_w, const int32_t* sorted_ids, float* out,
+                                    int M, int width, int top_k, int EM, int group_size);
+/* Not in the reference: the values a W4A4 layer multiplies for one group of 32 bf16
+ * activations (quantised as mxfp4_moe_quant does, then dequantised). */
+void vko_aux_model_block32(const uint16_t* a, float* out);
+
 #ifdef __cplusplus
 }
 #endif

@@ -19,6 +19,9 @@ __all__ = [
     "gather_sorted_weights", "fused_moe_mxfp4", "moe_gateup",
     "moe_act_epilogue", "moe_down", "moe_combine", "route_topk", "route_exp",
     "moe_layer",
+    "aux_scale_byte", "mxfp4_moe_quant", "mxfp4_moe_sorted_quant", "mxfp4_moe_sort",
+    "mxfp4_moe_sort_scales", "mxfp4_moe_scatter_reduce", "mxfp4_moe_scatter_reduce_q",
+    "mxfp4_dequant_act",
 ]
 
 HERE = Path(__file__).resolve().parent
@@ -87,7 +90,10 @@ def act_model_block32(a_bits, terms: int = 2) -> np.ndarray:
     a = np.ascontiguousarray(a_bits, dtype=np.uint16)
     assert a.size == 32
     out = np.empty(32, dtype=np.float32)
-    lib().vko_act_model_block32(_P(a.ctypes.data), _P(out.ctypes.data), int(terms))
+    if int(terms) == 1:   # the W4A4 mode: quantised as mxfp4_moe_quant does, then dequantised
+        lib().vko_aux_model_block32(_P(a.ctypes.data), _P(out.ctypes.data))
+    else:
+        lib().vko_act_model_block32(_P(a.ctypes.data), _P(out.ctypes.data), int(terms))
     return out
 
 
@@ -256,6 +262,90 @@ def moe_combine(partial, b2, topk_w_sorted, sorted_ids, expert_ids, M, hidden, t
     fn = ref_lib().vkref_moe_combine if use_ref else lib().vko_moe_combine
     fn(_ptr(partial), _ptr(b2), _ptr(tws), _ptr(sids), _ptr(eids), _ptr(out), M, hidden, top_k, EM)
     return out
+
+
+# ---- MXFP4 MoE orchestration ops (moe_aux.cpp of the reference) -------------------
+
+def _aux(name, use_ref):
+    return getattr(ref_lib(), "vkref_" + name) if use_ref else getattr(lib(), "vko_" + name)
+
+
+def aux_scale_byte(amax_bits: int) -> int:
+    fn = lib().vko_aux_scale_byte
+    fn.restype = _c.c_uint8
+    return int(fn(_c.c_uint16(int(amax_bits) & 0x7FFF)))
+
+
+def mxfp4_moe_quant(A, group_size=32, use_ref=False):
+    """(packed [M, hidden/2], scales [M, hidden/group_size]) of bf16 rows A [M, hidden]."""
+    A = _arr(A, np.uint16)
+    M, hidden = A.shape
+    packed = np.zeros((M, hidden // 2), dtype=np.uint8)
+    scales = np.zeros((M, hidden // group_size), dtype=np.uint8)
+    _aux("mxfp4_moe_quant", use_ref)(_ptr(A), _ptr(packed), _ptr(scales), M, hidden, group_size)
+    return packed, scales
+
+
+def mxfp4_moe_sorted_quant(A, sorted_ids, top_k, group_size=32, use_ref=False):
+    A = _arr(A, np.uint16); sids = _arr(sorted_ids, np.int32)
+    M, hidden = A.shape
+    EM = sids.size
+    packed = np.zeros((EM, hidden // 2), dtype=np.uint8)
+    scales = np.zeros((EM, hidden // group_size), dtype=np.uint8)
+    _aux("mxfp4_moe_sorted_quant", use_ref)(_ptr(A), _ptr(sids), _ptr(packed), _ptr(scales), M,
+                                            hidden, group_size, top_k, EM)
+    return packed, scales
+
+
+def mxfp4_moe_sort(A, sorted_ids, top_k, use_ref=False):
+    A = _arr(A, np.uint16); sids = _arr(sorted_ids, np.int32)
+    M, hidden = A.shape
+    out = np.zeros((sids.size, hidden), dtype=np.uint16)
+    _aux("mxfp4_moe_sort", use_ref)(_ptr(A), _ptr(sids), _ptr(out), M, hidden, top_k, sids.size)
+    return out
+
+
+def mxfp4_moe_sort_scales(scales, sorted_ids, top_k, use_ref=False):
+    scales = _arr(scales, np.uint8); sids = _arr(sorted_ids, np.int32)
+    M, ng = scales.shape
+    out = np.zeros((sids.size, ng), dtype=np.uint8)
+    _aux("mxfp4_moe_sort_scales", use_ref)(_ptr(scales), _ptr(sids), _ptr(out), M, ng, top_k, sids.size)
+    return out
+
+
+def mxfp4_moe_scatter_reduce(partial, topk_w_sorted, sorted_ids, M, top_k, out=None, use_ref=False):
+    partial = _arr(partial, np.float32); tws = _arr(topk_w_sorted, np.float32)
+    sids = _arr(sorted_ids, np.int32)
+    EM, width = partial.shape
+    if out is None:
+        out = np.zeros((M, width), dtype=np.float32)
+    _aux("mxfp4_moe_scatter_reduce", use_ref)(_ptr(partial), _ptr(tws), _ptr(sids), _ptr(out), M,
+                                              width, top_k, EM)
+    return out
+
+
+def mxfp4_moe_scatter_reduce_q(partial_q, partial_s, topk_w_sorted, sorted_ids, M, top_k,
+                               group_size=32, out=None, use_ref=False):
+    pq = _arr(partial_q, np.uint8); ps = _arr(partial_s, np.uint8)
+    tws = _arr(topk_w_sorted, np.float32); sids = _arr(sorted_ids, np.int32)
+    EM, width = pq.shape[0], pq.shape[1] * 2
+    if out is None:
+        out = np.zeros((M, width), dtype=np.float32)
+    _aux("mxfp4_moe_scatter_reduce_q", use_ref)(_ptr(pq), _ptr(ps), _ptr(tws), _ptr(sids), _ptr(out),
+                                                M, width, top_k, EM, group_size)
+    return out
+
+
+def mxfp4_dequant_act(packed, scales, group_size=32):
+    """float32 values of quantised activations: table value x 2^(s-127), 0xFF -> 0
+    (the W4A4 activation decode of tests/kernels/moe/test_moe_aux.cpp:53-69)."""
+    packed = np.asarray(packed, dtype=np.uint8); scales = np.asarray(scales, dtype=np.uint8)
+    table = np.array([fp4nib_to_f32bits(i) for i in range(16)], dtype=np.uint32).view(np.float32)
+    nib = np.stack([packed & 15, packed >> 4], axis=-1).reshape(packed.shape[0], -1)
+    sc = np.where(scales == 0xFF, np.float32(0.0),
+                  (scales.astype(np.uint32) << 23).view(np.float32)).astype(np.float32)
+    with np.errstate(invalid="ignore"):
+        return table[nib] * np.repeat(sc, group_size, axis=1)
 
 
 def route_topk(logits, top_k, renormalize=True):

@@ -9,6 +9,7 @@
 #include <cstddef>
 #include <cstdint>
 
+#include "vkernels/kernels/moe_aux.hpp"
 #include "vkernels/kernels/moe_fused.hpp"
 
 namespace vk = vkernels::kernels;
@@ -87,6 +88,42 @@ void vkref_dequant_weight_tile_ref(const uint8_t* packed, const uint8_t* scale,
                                    int stride_scale_n, int stride_scale_k) {
   vk::dequant_weight_tile_ref(packed, scale, out_bf16, N, K, group_size,
                               stride_packed, stride_scale_n, stride_scale_k);
+}
+
+
+// ---- moe_aux.cpp ----
+void vkref_mxfp4_moe_quant(const uint16_t* A, uint8_t* packed, uint8_t* scales, int M, int hidden,
+                           int group_size) {
+  vk::mxfp4_moe_quant(A, packed, scales, M, hidden, group_size);
+}
+
+void vkref_mxfp4_moe_sorted_quant(const uint16_t* A, const int32_t* sorted_ids, uint8_t* packed,
+                                  uint8_t* scales, int M, int hidden, int group_size, int top_k,
+                                  int EM) {
+  vk::mxfp4_moe_sorted_quant(A, sorted_ids, packed, scales, M, hidden, group_size, top_k, EM);
+}
+
+void vkref_mxfp4_moe_sort(const uint16_t* A, const int32_t* sorted_ids, uint16_t* A_sorted, int M,
+                          int hidden, int top_k, int EM) {
+  vk::mxfp4_moe_sort(A, sorted_ids, A_sorted, M, hidden, top_k, EM);
+}
+
+void vkref_mxfp4_moe_sort_scales(const uint8_t* scales, const int32_t* sorted_ids,
+                                 uint8_t* scales_sorted, int M, int n_groups, int top_k, int EM) {
+  vk::mxfp4_moe_sort_scales(scales, sorted_ids, scales_sorted, M, n_groups, top_k, EM);
+}
+
+void vkref_mxfp4_moe_scatter_reduce(const float* partial, const float* topk_w,
+                                    const int32_t* sorted_ids, float* out, int M, int width,
+                                    int top_k, int EM) {
+  vk::mxfp4_moe_scatter_reduce(partial, topk_w, sorted_ids, out, M, width, top_k, EM);
+}
+
+void vkref_mxfp4_moe_scatter_reduce_q(const uint8_t* partial_q, const uint8_t* partial_s,
+                                      const float* topk_w, const int32_t* sorted_ids, float* out,
+                                      int M, int width, int top_k, int EM, int group_size) {
+  vk::mxfp4_moe_scatter_reduce_q(partial_q, partial_s, topk_w, sorted_ids, out, M, width, top_k,
+                                 EM, group_size);
 }
 
 }  // extern "C"

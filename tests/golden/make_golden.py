@@ -84,6 +84,29 @@ def main():
     np.savez_compressed(OUT / "align_cases.npz", n=6, **cases)
     print("align cases written")
 
+    # moe_aux.cpp: activation quantisation (token and sorted order), routed combine, and the
+    # scale byte of every positive bf16 pattern as a group's largest value
+    M, hidden, top_k, E = 12, 128, 2, 4
+    A = synth.make_activations(M, hidden, 95)
+    A[0, :32] = 0
+    A[1, 40] = 0x7F80
+    A[2, :] = synth.f32_to_bf16_bits(synth.bf16_bits_to_f32(A[2, :]) * np.float32(2.0 ** -100))
+    ids = rng.integers(0, E, (M, top_k)).astype(np.int32)
+    sids, _, em = oracle.moe_align_block_size(ids, 16, E, use_ref=True)
+    sids = sids[:em]
+    packed, scales = oracle.mxfp4_moe_quant(A, use_ref=True)
+    spk, ssc = oracle.mxfp4_moe_sorted_quant(A, sids, top_k, use_ref=True)
+    partial = rng.standard_normal((em, 64)).astype(np.float32)
+    tws = rng.random(em).astype(np.float32)
+    reduced = oracle.mxfp4_moe_scatter_reduce(partial, tws, sids, M, top_k, use_ref=True)
+    pats = np.zeros((32768, 32), dtype=np.uint16)
+    pats[:, 0] = np.arange(32768, dtype=np.uint16)
+    scale_table = oracle.mxfp4_moe_quant(pats, use_ref=True)[1][:, 0]
+    np.savez_compressed(OUT / "aux_quant.npz", A=A, top_k=top_k, sorted_ids=sids, packed=packed,
+                        scales=scales, sorted_packed=spk, sorted_scales=ssc, partial=partial,
+                        topk_w_sorted=tws, reduced=reduced, scale_table=scale_table)
+    print("aux fixture written, EM", em)
+
 
 if __name__ == "__main__":
     main()

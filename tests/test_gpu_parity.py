@@ -91,7 +91,8 @@ def test_dequant_all_bytes_all_scales(hip_lib):
                 continue
             scale = np.full((N, K // 32), s, dtype=np.uint8)
             ref = oracle.dequant_weight_tile(packed, scale, N, K)
-            st = fn(d_packed.data_ptr(), to_dev(scale).data_ptr(), d_out.data_ptr(), N, K, 32,
+            d_scale = to_dev(scale)
+            st = fn(d_packed.data_ptr(), d_scale.data_ptr(), d_out.data_ptr(), N, K, 32,
                     K // 2, K // 32, 1, fast, None)
             assert st == 0
             torch.cuda.synchronize()
@@ -110,7 +111,8 @@ def test_router_matches_oracle_bitwise(hip_lib):
             lg[:, 1::2] = lg[:, 0::2]  # exact ties: the lower index must win
         ids = torch.zeros((T, k), dtype=torch.int32, device=dev())
         w = torch.zeros((T, k), dtype=torch.float32, device=dev())
-        st = fn(to_dev(lg).data_ptr(), T, E, k, 1, ids.data_ptr(), w.data_ptr(), None)
+        d_lg = to_dev(lg)
+        st = fn(d_lg.data_ptr(), T, E, k, 1, ids.data_ptr(), w.data_ptr(), None)
         assert st == 0
         torch.cuda.synchronize()
         rid, rw = oracle.route_topk(lg, k, True)

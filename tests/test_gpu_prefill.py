@@ -86,7 +86,8 @@ def test_prepack_layout_bitwise(hip_lib, stage, rows, K):
     ws[0, 40, 1] = 191          # above the range
     n = int(size_fn(E, rows, K, stage))
     buf = torch.zeros(n, dtype=torch.uint8, device=dev())
-    st = pack_fn(to_dev(w).data_ptr(), to_dev(ws).data_ptr(), E, rows, K, stage, buf.data_ptr(), n, None)
+    d_w, d_ws = to_dev(w), to_dev(ws)
+    st = pack_fn(d_w.data_ptr(), d_ws.data_ptr(), E, rows, K, stage, buf.data_ptr(), n, None)
     assert st == 0, ve.last_error(hip_lib)
     torch.cuda.synchronize()
     ref, flags = _prepack_reference(w, ws, stage)
@@ -142,7 +143,8 @@ def test_split_rows_match_the_oracle_model(hip_lib, terms):
     x[8, 5] = 0x40FF                     # 7.96875: saturates the first term
     out = torch.zeros(rows * terms * kp, dtype=torch.uint8, device=dev())
     flags = torch.full((rows,), 9, dtype=torch.uint8, device=dev())
-    st = fn(to_dev(x).data_ptr(), rows, K, terms, out.data_ptr(), flags.data_ptr(), None)
+    d_x = to_dev(x)
+    st = fn(d_x.data_ptr(), rows, K, terms, out.data_ptr(), flags.data_ptr(), None)
     assert st == 0, ve.last_error(hip_lib)
     torch.cuda.synchronize()
     fl = flags.cpu().numpy()

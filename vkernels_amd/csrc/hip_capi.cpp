@@ -236,6 +236,51 @@ int vk_hip_split_rows_fp6(const uint16_t* x, int32_t rows, int32_t K, int32_t te
   return VK_OK;
 }
 
+int vk_hip_mxfp4_moe_quant(const uint16_t* A, uint8_t* packed, uint8_t* scales, int32_t M,
+                           int32_t hidden, int32_t group_size, void* stream) {
+  if (group_size != 32) return fail(VK_ERROR_UNSUPPORTED, "group_size must be 32");
+  if (M < 0 || hidden < 0 || hidden % 32 != 0)
+    return fail(VK_ERROR_INVALID_ARGUMENT, "M and hidden must be non-negative, hidden a multiple of group_size");
+  if (M == 0 || hidden == 0) return VK_OK;
+  if (A == nullptr || packed == nullptr || scales == nullptr)
+    return fail(VK_ERROR_INVALID_ARGUMENT, "A/packed/scales must not be null");
+  vk::launch_mxfp4_quant(A, nullptr, packed, scales, M, hidden, 1, M, static_cast<hipStream_t>(stream));
+  return VK_OK;
+}
+
+int vk_hip_mxfp4_moe_sorted_quant(const uint16_t* A, const int32_t* sorted_ids, uint8_t* packed,
+                                  uint8_t* scales, int32_t M, int32_t hidden, int32_t group_size,
+                                  int32_t top_k, int32_t EM, void* stream) {
+  if (group_size != 32) return fail(VK_ERROR_UNSUPPORTED, "group_size must be 32");
+  if (M < 0 || hidden < 0 || EM < 0 || top_k <= 0 || hidden % 32 != 0)
+    return fail(VK_ERROR_INVALID_ARGUMENT,
+                "M, hidden, EM must be non-negative, top_k positive, hidden a multiple of group_size");
+  if (EM == 0 || hidden == 0) return VK_OK;
+  if (A == nullptr || sorted_ids == nullptr || packed == nullptr || scales == nullptr)
+    return fail(VK_ERROR_INVALID_ARGUMENT, "A/sorted_ids/packed/scales must not be null");
+  vk::launch_mxfp4_quant(A, sorted_ids, packed, scales, EM, hidden, top_k, M * top_k,
+                         static_cast<hipStream_t>(stream));
+  return VK_OK;
+}
+
+int vk_hip_mxfp4_moe_scatter_reduce(const float* partial, const float* topk_w,
+                                    const int32_t* sorted_ids, float* out, int32_t M, int32_t width,
+                                    int32_t top_k, int32_t EM, void* workspace,
+                                    size_t workspace_bytes, void* stream) {
+  if (M < 0 || width < 0 || EM < 0 || top_k <= 0 || width % 4 != 0)
+    return fail(VK_ERROR_INVALID_ARGUMENT,
+                "M, width, EM must be non-negative, top_k positive, width a multiple of 4");
+  if (M == 0 || width == 0 || EM == 0) return VK_OK;
+  if (partial == nullptr || topk_w == nullptr || sorted_ids == nullptr || out == nullptr)
+    return fail(VK_ERROR_INVALID_ARGUMENT, "partial/topk_w/sorted_ids/out must not be null");
+  if (workspace == nullptr || workspace_bytes < sizeof(int32_t) * (size_t)M * (size_t)top_k ||
+      (reinterpret_cast<uintptr_t>(workspace) & 3) != 0)
+    return fail(VK_ERROR_INVALID_ARGUMENT, "workspace must hold M * top_k int32 values");
+  vk::launch_mxfp4_scatter_reduce(partial, topk_w, sorted_ids, out, M, width, top_k, EM,
+                                  static_cast<int32_t*>(workspace), static_cast<hipStream_t>(stream));
+  return VK_OK;
+}
+
 size_t vk_hip_moe_prepack_bytes(int32_t num_experts, int32_t rows, int32_t K, int32_t stage) {
   if (stage != 0 && stage != 1) return 0;
   return vk::moe_prepack_bytes(num_experts, rows, K, stage);

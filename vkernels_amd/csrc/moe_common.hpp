@@ -26,8 +26,12 @@ __device__ __forceinline__ float act_value(int activation, float g, float u,
     if (u > limit) u = limit;
     if (u < -limit) u = -limit;
   }
-  // v_exp_f32 / v_rcp_f32: about 1 ulp each, far inside the bf16 rounding that follows
-  return (g * __builtin_amdgcn_rcpf(1.0f + __expf(-g))) * u;
+  // v_exp_f32 / v_rcp_f32: about 1 ulp each, far inside the bf16 rounding that follows.
+  // Below g = -87 the quotient is subnormal, which v_rcp_f32 flushes to zero (and an
+  // infinite u then gives NaN where g / (1 + e^-g) * u is an infinity): there the
+  // reciprocal is taken of the denominator scaled by 2^-64 and scaled back by a multiply.
+  const float s = g < -87.0f ? 0x1p-64f : 1.0f;
+  return (g * (__builtin_amdgcn_rcpf((1.0f + __expf(-g)) * s) * s)) * u;
 }
 
 __device__ __forceinline__ bf16x8 as_bf16x8(u32x4 v) {

@@ -245,13 +245,182 @@ __global__ __launch_bounds__(256) void split_rows_fp6_kernel(const uint16_t* __r
 }
 
 // ---------------------------------------------------------------------------
+// MXFP4 quantisation of activations, as the reference's mxfp4_moe_quant does
+// (src/c/vkernels/kernels/moe_aux.cpp:99-139), per group of 32 bf16 values:
+//   amax = the largest magnitude (a NaN never is, an inf is);
+//   amax zero or non-finite: scale byte 0xFF and zero codes; else
+//   scale byte s = clamp(ceil(log2(amax / 3)) + 127, 1, 254): with amax = 1.m x 2^x that
+//   is the exponent field of amax, less one when m <= 1.5 (amax / 3 is a power of two
+//   only for m = 1.5), at least 1;
+//   code = nearest of {0, .25, 1, 1.5, 2, 3} to |a| / 2^(s-127), ties to the larger
+//   (thresholds .125, .625, 1.25, 1.75, 2.5), sign bit set when a / scale < 0.
+// d: the 32 values, two per dword; codes: 4 dwords, low nibble = even k.
+// ---------------------------------------------------------------------------
+__device__ __forceinline__ void quant_group32(const uint32_t (&d)[16], uint32_t& sb, uint32_t (&codes)[4]) {
+  // (bit patterns of non-negative floats order like the floats; a NaN counts as zero)
+  uint32_t bits = 0u;
+#pragma unroll
+  for (int i = 0; i < 16; ++i) {
+    uint32_t lo = d[i] & 0x7FFFu, hi = (d[i] >> 16) & 0x7FFFu;
+    if (lo > 0x7F80u) lo = 0u;
+    if (hi > 0x7F80u) hi = 0u;
+    bits = max(bits, max(lo, hi));
+  }
+  const uint32_t ex = bits >> 7, mant = bits & 0x7Fu;
+  if (ex == 0xFFu || bits == 0u) {
+    sb = 0xFFu;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) codes[j] = 0u;
+    return;
+  }
+  int s = (int)ex - (mant <= 0x40u ? 1 : 0);
+  if (ex == 0u || s < 1) s = 1;
+  sb = (uint32_t)s;
+  // a / 2^(s-127) as a product with 2^(127-s), exact (the rounding at underflow included)
+  const float inv = s <= 253 ? __uint_as_float((uint32_t)(254 - s) << 23) : __uint_as_float(0x00400000u);
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    uint32_t word = 0u;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const uint32_t dw = d[j * 4 + (i >> 1)];
+      const float a = __uint_as_float((i & 1) ? (dw & 0xFFFF0000u) : (dw << 16));
+      const float x = __fmul_rn(a, inv);
+      const float v = fabsf(x);
+      uint32_t mag = 5u;              // also what a NaN gets: every comparison is false
+      if (v < 0.125f) mag = 0u;
+      else if (v < 0.625f) mag = 1u;
+      else if (v < 1.25f) mag = 2u;
+      else if (v < 1.75f) mag = 3u;
+      else if (v < 2.5f) mag = 4u;
+      if (x < 0.0f) mag |= 8u;
+      word |= mag << (4 * i);
+    }
+    codes[j] = word;
+  }
+}
+
+// Packed codes [rows, K/2] and scale bytes [rows, K/32] of bf16 rows: row r of the output
+// is x[r] (sorted_ids null) or x[sorted_ids[r] / top_k], a padding row (id outside
+// [0, n_flat)) giving zero codes and 0xFF scales (mxfp4_moe_sorted_quant,
+// moe_aux.cpp:171-209).  One lane per group of 32.
+__global__ __launch_bounds__(256) void mxfp4_quant_kernel(const uint16_t* __restrict__ x,
+                                                          const int32_t* __restrict__ sorted_ids,
+                                                          uint8_t* __restrict__ packed,
+                                                          uint8_t* __restrict__ scales, int K,
+                                                          int top_k, int n_flat) {
+  const size_t row = blockIdx.x;
+  const uint16_t* src = x + row * (size_t)K;
+  bool pad = false;
+  if (sorted_ids != nullptr) {
+    const int flat = sorted_ids[row];
+    pad = flat < 0 || flat >= n_flat;
+    src = x + (size_t)(pad ? 0 : flat / top_k) * (size_t)K;
+  }
+  for (int g = threadIdx.x; g < K / 32; g += 256) {
+    union { u32x4 q[4]; uint32_t d[16]; } in;
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      in.q[i] = pad ? u32x4{0u, 0u, 0u, 0u} : reinterpret_cast<const u32x4*>(src + (size_t)g * 32)[i];
+    uint32_t sb, codes[4];
+    quant_group32(in.d, sb, codes);
+    *reinterpret_cast<u32x4*>(packed + row * (size_t)(K / 2) + (size_t)g * 16) =
+        u32x4{codes[0], codes[1], codes[2], codes[3]};
+    scales[row * (size_t)(K / 32) + g] = (uint8_t)sb;
+  }
+}
+
+// The same quantisation as the split rows of the W4A4 mode: one plane of Kp bytes per
+// row, a block = the 32 codes moved onto the OCP code points (16 bytes), the scale byte
+// less one, 15 zero bytes; zero groups get a neutral scale.  row_bad[r] = 1 when a scale
+// byte is outside the range the scaled MFMA path takes.
+__global__ __launch_bounds__(256) void quant_rows_w4_kernel(const uint16_t* __restrict__ x,
+                                                            uint8_t* __restrict__ xq,
+                                                            uint8_t* __restrict__ row_bad, int K) {
+  const int kp = mx_kp(K);
+  const size_t row = blockIdx.x;
+  uint8_t* qrow = xq + row * (size_t)kp;
+  int bad = 0;
+  for (int b = threadIdx.x; b < kp / 32; b += 256) {
+    union { u32x4 q[4]; uint32_t d[16]; } in;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) in.q[i] = u32x4{0u, 0u, 0u, 0u};
+    if (b * 32 < K) {
+      const u32x4* src = reinterpret_cast<const u32x4*>(x + row * (size_t)K + (size_t)b * 32);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) in.q[i] = src[i];
+    }
+    uint32_t sb, codes[4];
+    quant_group32(in.d, sb, codes);
+    uint32_t st = 127u;
+    if (sb != 0xFFu) {
+      st = sb - 1u;
+      if (st < kScaleLo || st > kScaleHi) bad = 1;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) codes[j] = fp4x8_to_ocp_doubled(codes[j]);
+    }
+    uint8_t* blk = qrow + (size_t)b * 32;
+    *reinterpret_cast<u32x4*>(blk) = u32x4{codes[0], codes[1], codes[2], codes[3]};
+    *reinterpret_cast<u32x4*>(blk + 16) = u32x4{st, 0u, 0u, 0u};
+  }
+  bad = __syncthreads_or(bad);
+  if (threadIdx.x == 0) row_bad[row] = (uint8_t)(bad != 0);
+}
+
+// pos[flat] = sorted row of every routed flat index (the others keep their -1).
+__global__ __launch_bounds__(256) void invert_sorted_ids_kernel(const int32_t* __restrict__ sorted_ids,
+                                                                int32_t* __restrict__ pos, int EM,
+                                                                int n_flat) {
+  const int r = blockIdx.x * blockDim.x + threadIdx.x;
+  if (r >= EM) return;
+  const int flat = sorted_ids[r];
+  if (flat >= 0 && flat < n_flat) pos[flat] = r;
+}
+
+// Routed combine in gather form (mxfp4_moe_scatter_reduce, moe_aux.cpp:265-285):
+// out[t, :] += partial[r, :] * topk_w[r] over the token's sorted rows r in ascending
+// order, which is the order the reference's loop over r adds them in; the product and
+// the sum are rounded separately, as there.  One thread per 4 columns.
+__global__ __launch_bounds__(256) void scatter_reduce_kernel(const float* __restrict__ partial,
+                                                             const float* __restrict__ topk_w,
+                                                             const int32_t* __restrict__ pos,
+                                                             float* __restrict__ out, int M, int width,
+                                                             int top_k) {
+  const int c = (blockIdx.x * blockDim.x + threadIdx.x) * 4;
+  if (c >= width) return;
+  for (int t = blockIdx.y; t < M; t += gridDim.y) {
+    f32x4* o = reinterpret_cast<f32x4*>(out + (size_t)t * (size_t)width + c);
+    f32x4 sum = *o;
+    int last = -1;
+    for (int s = 0; s < top_k; ++s) {   // the next larger sorted row of this token (top_k is small)
+      int r = 0x7FFFFFFF;
+      for (int j = 0; j < top_k; ++j) {
+        const int rj = pos[t * top_k + j];
+        if (rj > last && rj < r) r = rj;
+      }
+      if (r == 0x7FFFFFFF) break;
+      last = r;
+      const f32x4 p = *reinterpret_cast<const f32x4*>(partial + (size_t)r * (size_t)width + c);
+      const float w = topk_w[r];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        float prod = p[i] * w;
+        asm volatile("" : "+v"(prod));   // the rounded product is a value of its own: no fused multiply-add
+        sum[i] += prod;
+      }
+    }
+    *o = sum;
+  }
+}
+
+// ---------------------------------------------------------------------------
 // Exact path of one unit for the 32 rows of one row tile: acc[t] = C[weight row of
 // tile t][activation row lane % 32] in the accumulator layout of the 32 x 32 MFMAs.
 // a_row: the bf16 row of this lane's activation row, or null for a padding row.
-// ---------------------------------------------------------------------------
+// q_row (W4A4 mode): the row's quantised plane instead; its values are decoded exactly.
 template <int STAGE>
 __device__ __forceinline__ void exact_unit_mx(const MxArgs& p, int e, int unit, const uint16_t* a_row,
-                                              int lane, f32x16 (&acc)[4]) {
+                                              const uint8_t* q_row, int lane, f32x16 (&acc)[4]) {
   const int n = lane & 31, hh = lane >> 5;
   const int rows_w = STAGE == 0 ? 2 * p.ncols : p.ncols;
   const int K = p.K;
@@ -275,6 +444,12 @@ __device__ __forceinline__ void exact_unit_mx(const MxArgs& p, int e, int unit, 
     const int k = 16 * s + 8 * hh;
     u32x4 av = {0u, 0u, 0u, 0u};
     if (a_row != nullptr) av = *reinterpret_cast<const u32x4*>(a_row + k);
+    if (q_row != nullptr) {  // 8 codes of block k / 32 back on the reference's code points
+      const uint8_t* blk = q_row + (size_t)(k >> 5) * 32;
+      uint32_t c = *reinterpret_cast<const uint32_t*>(blk + ((k & 31) >> 1));
+      c -= (c & 0x44444444u) >> 1;
+      av = dequant8_exact(c, ((uint32_t)blk[16] + 1u) & 0xFFu);
+    }
 #pragma unroll
     for (int t = 0; t < 4; ++t) {
       u32x4 wv = {0u, 0u, 0u, 0u};
@@ -334,11 +509,17 @@ __device__ __forceinline__ i32x8 fp4_operand_ocp(u32x4 w) {  // codes already on
   return __builtin_shufflevector(y, y, 0, 1, 2, 3, -1, -1, -1, -1);
 }
 
-template <int T>
-__device__ __forceinline__ f32x16 mfma_fp4_fp6(u32x4 w, i32x8 b, f32x16 acc, uint32_t wscale) {
-  // A: FP4 (cbsz 4), scale byte T of wscale; B: FP6 E2M3 (blgp 2), scale = byte 0 of b[6]
-  return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fp4_operand_ocp(w), b, acc, 4, 2, T,
-                                                         (int)wscale, 0, b[6]);
+// One scaled MFMA: A = FP4 (cbsz 4) with scale byte T of wscale.  B = the operand read
+// from LDS: FP6 E2M3 (blgp 2, scale in byte 0 of b[6]) or, in the W4A4 mode, FP4 (blgp 4,
+// codes in b[0..3], scale in byte 0 of b[4]).
+template <int T, bool W4A4>
+__device__ __forceinline__ f32x16 mfma_fp4_act(u32x4 w, i32x8 b, f32x16 acc, uint32_t wscale) {
+  if constexpr (W4A4)
+    return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fp4_operand_ocp(w), b, acc, 4, 4, T,
+                                                           (int)wscale, 0, b[4]);
+  else
+    return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fp4_operand_ocp(w), b, acc, 4, 2, T,
+                                                           (int)wscale, 0, b[6]);
 }
 
 template <int STAGE, int TERMS>
@@ -539,12 +720,12 @@ __global__ __launch_bounds__(64 * kMxWaves) void tile_mx_kernel(MxArgs p) {
           const int half = q / (LIVE * TERMS), m = (q / TERMS) % LIVE;
           const uint32_t wsc = ws[i].sc[half];
           // (a wavefront without a unit multiplies unit 0's weights and drops the result)
-          acc[m][0] = mfma_fp4_fp6<0>(ws[i].w[half * 4 + 0], cur, acc[m][0], wsc);
+          acc[m][0] = mfma_fp4_act<0, TERMS == 1>(ws[i].w[half * 4 + 0], cur, acc[m][0], wsc);
           __builtin_amdgcn_sched_barrier(0);
           // reads of group q + 2; the last two groups read the next step's first two
           const i32x8 pend = q + 2 < Q ? group_operand(sb, q + 2) : group_operand(sbn, q + 2 - Q);
           __builtin_amdgcn_sched_barrier(0);
-          acc[m][1] = mfma_fp4_fp6<1>(ws[i].w[half * 4 + 1], cur, acc[m][1], wsc);
+          acc[m][1] = mfma_fp4_act<1, TERMS == 1>(ws[i].w[half * 4 + 1], cur, acc[m][1], wsc);
           __builtin_amdgcn_sched_barrier(0);
           if (q < Q - 2) {
 #pragma unroll
@@ -553,11 +734,11 @@ __global__ __launch_bounds__(64 * kMxWaves) void tile_mx_kernel(MxArgs p) {
             issued += kPer;
           }
           __builtin_amdgcn_sched_barrier(0);
-          acc[m][2] = mfma_fp4_fp6<2>(ws[i].w[half * 4 + 2], cur, acc[m][2], wsc);
+          acc[m][2] = mfma_fp4_act<2, TERMS == 1>(ws[i].w[half * 4 + 2], cur, acc[m][2], wsc);
           __builtin_amdgcn_sched_barrier(0);
           __asm__ volatile("" : "+v"(nxt));  // complete from here on (read a group ago)
           __builtin_amdgcn_sched_barrier(0);
-          acc[m][3] = mfma_fp4_fp6<3>(ws[i].w[half * 4 + 3], cur, acc[m][3], wsc);
+          acc[m][3] = mfma_fp4_act<3, TERMS == 1>(ws[i].w[half * 4 + 3], cur, acc[m][3], wsc);
           __builtin_amdgcn_sched_barrier(0);
           if (q == Q - 3) {
             wait_loads_and_reads<kOps>(ws[in1]);
@@ -584,10 +765,11 @@ __global__ __launch_bounds__(64 * kMxWaves) void tile_mx_kernel(MxArgs p) {
       wait_loads<0>(ws[1]);
       wait_loads<0>(ws[2]);
     };
+    // (one plane per row: a step of one row tile would be shorter than the pipeline)
     if (n_live > 3) k_loop(IntC<4>{});
     else if (n_live == 3) k_loop(IntC<3>{});
-    else if (n_live == 2) k_loop(IntC<2>{});
-    else k_loop(IntC<1>{});
+    else if (n_live == 2 || TERMS == 1) k_loop(IntC<2>{});
+    else if constexpr (TERMS > 1) k_loop(IntC<1>{});
     __syncthreads();
 
     if (STAGE == 1 && colg == 0 && tid < n_rows && row_flat[tid] >= 0) p.pos[row_flat[tid]] = row0 + tid;
@@ -603,8 +785,13 @@ __global__ __launch_bounds__(64 * kMxWaves) void tile_mx_kernel(MxArgs p) {
       const int srow = row0 + m * 32 + ln;
       if (slow) {
         const uint16_t* a_row = nullptr;
-        if (flat >= 0) a_row = p.A + (size_t)(STAGE == 0 ? flat / p.top_k : srow) * (size_t)K;
-        exact_unit_mx<STAGE>(p, e, unit, a_row, lane, tile);
+        const uint8_t* q_row = nullptr;
+        if (flat >= 0) {
+          const size_t grow = (size_t)(STAGE == 0 ? flat / p.top_k : srow);
+          if (TERMS == 1) q_row = p.Aq + grow * (size_t)Kp;
+          else a_row = p.A + grow * (size_t)K;
+        }
+        exact_unit_mx<STAGE>(p, e, unit, a_row, q_row, lane, tile);
       }
       if (flat < 0) continue;
       if (STAGE == 0) {
@@ -763,8 +950,8 @@ size_t mx_workspace_bytes(int M, int hidden, int ispp, int top_k, int EM) {
 }
 
 bool prepare_mx_kernels() {
-  return mx_kernel_ready<0, 2>() && mx_kernel_ready<0, 3>() && mx_kernel_ready<1, 2>() &&
-         mx_kernel_ready<1, 3>();
+  return mx_kernel_ready<0, 1>() && mx_kernel_ready<0, 2>() && mx_kernel_ready<0, 3>() &&
+         mx_kernel_ready<1, 1>() && mx_kernel_ready<1, 2>() && mx_kernel_ready<1, 3>();
 }
 
 namespace {
@@ -774,7 +961,7 @@ struct MxPlan {
   uint8_t *aq, *cq, *abad, *cbad;
   float* y;
   int32_t* pos;
-  bool two_terms;
+  int terms;  // FP6 terms per activation (2, 3) or 1 = the W4A4 mode (MXFP4 activations)
 };
 
 // False when the prepacked path does not take the call (no packed weights, workspace
@@ -787,9 +974,10 @@ bool mx_plan(const FusedMoeArgs& a, bool need_stage0, MxPlan& pl) {
   if ((unsigned long long)a.EM * 3ull * mx_kp(a.ispp) >= (1ull << 32) ||
       (unsigned long long)a.M * 3ull * mx_kp(a.hidden) >= (1ull << 32))
     return false;
-  pl.two_terms = (a.flags & 2u) != 0u;  // VK_HIP_MOE_SPLIT2
-  if (pl.two_terms ? !(mx_kernel_ready<0, 2>() && mx_kernel_ready<1, 2>())
-                   : !(mx_kernel_ready<0, 3>() && mx_kernel_ready<1, 3>()))
+  pl.terms = (a.flags & 4u) != 0u ? 1 : (a.flags & 2u) != 0u ? 2 : 3;  // VK_HIP_MOE_W4A4, _SPLIT2
+  if (!(pl.terms == 1 ? mx_kernel_ready<0, 1>() && mx_kernel_ready<1, 1>()
+        : pl.terms == 2 ? mx_kernel_ready<0, 2>() && mx_kernel_ready<1, 2>()
+                        : mx_kernel_ready<0, 3>() && mx_kernel_ready<1, 3>()))
     return false;
   uint8_t* base = static_cast<uint8_t*>(a.workspace);
   pl.aq = base;
@@ -813,7 +1001,10 @@ bool mx_plan(const FusedMoeArgs& a, bool need_stage0, MxPlan& pl) {
 }
 
 void mx_stage0(const FusedMoeArgs& a, const MxPlan& pl, hipStream_t stream) {
-  if (pl.two_terms) {
+  if (pl.terms == 1) {
+    hipLaunchKernelGGL(quant_rows_w4_kernel, dim3(a.M), dim3(256), 0, stream, a.A, pl.aq, pl.abad, a.hidden);
+    launch_mx_stage_t<0, 1>(pl.g0, stream);
+  } else if (pl.terms == 2) {
     hipLaunchKernelGGL(split_rows_fp6_kernel<2>, dim3(a.M), dim3(256), 0, stream, a.A, pl.aq, pl.abad, a.hidden);
     launch_mx_stage_t<0, 2>(pl.g0, stream);
   } else {
@@ -826,7 +1017,10 @@ void mx_stage0(const FusedMoeArgs& a, const MxPlan& pl, hipStream_t stream) {
 // second stage -> per-token sum
 void mx_stage1(const FusedMoeArgs& a, const MxPlan& pl, hipStream_t stream) {
   launch_fill_i32(pl.pos, -1, a.M * a.top_k, stream);
-  if (pl.two_terms) {
+  if (pl.terms == 1) {
+    hipLaunchKernelGGL(quant_rows_w4_kernel, dim3(a.EM), dim3(256), 0, stream, a.act, pl.cq, pl.cbad, a.ispp);
+    launch_mx_stage_t<1, 1>(pl.g1, stream);
+  } else if (pl.terms == 2) {
     hipLaunchKernelGGL(split_rows_fp6_kernel<2>, dim3(a.EM), dim3(256), 0, stream, a.act, pl.cq, pl.cbad, a.ispp);
     launch_mx_stage_t<1, 2>(pl.g1, stream);
   } else {
@@ -864,6 +1058,27 @@ void launch_split_rows_fp6(const uint16_t* x, int rows, int K, int terms, uint8_
     hipLaunchKernelGGL(split_rows_fp6_kernel<2>, dim3(rows), dim3(256), 0, stream, x, xq, row_bad, K);
   else
     hipLaunchKernelGGL(split_rows_fp6_kernel<3>, dim3(rows), dim3(256), 0, stream, x, xq, row_bad, K);
+}
+
+// ---- MXFP4 orchestration ops (device counterparts of moe_aux.cpp) -----------------
+
+void launch_mxfp4_quant(const uint16_t* A, const int32_t* sorted_ids, uint8_t* packed, uint8_t* scales,
+                        int rows, int hidden, int top_k, int n_flat, hipStream_t stream) {
+  if (rows <= 0 || hidden <= 0) return;
+  hipLaunchKernelGGL(mxfp4_quant_kernel, dim3(rows), dim3(256), 0, stream, A, sorted_ids, packed, scales,
+                     hidden, top_k, n_flat);
+}
+
+void launch_mxfp4_scatter_reduce(const float* partial, const float* topk_w, const int32_t* sorted_ids,
+                                 float* out, int M, int width, int top_k, int EM, int32_t* pos,
+                                 hipStream_t stream) {
+  if (M <= 0 || width <= 0 || EM <= 0) return;
+  launch_fill_i32(pos, -1, M * top_k, stream);
+  hipLaunchKernelGGL(invert_sorted_ids_kernel, dim3((unsigned)((EM + 255) / 256)), dim3(256), 0, stream,
+                     sorted_ids, pos, EM, M * top_k);
+  const dim3 grid((unsigned)((width / 4 + 255) / 256), (unsigned)(M < 65535 ? M : 65535));
+  hipLaunchKernelGGL(scatter_reduce_kernel, grid, dim3(256), 0, stream, partial, topk_w, pos, out, M,
+                     width, top_k);
 }
 
 }  // namespace vk

@@ -71,6 +71,14 @@ void launch_split_rows_fp6(const uint16_t* x, int rows, int K, int terms, uint8_
                            hipStream_t stream);
 bool prepare_mx_kernels();
 
+// MXFP4 orchestration ops (moe_prefill.hip): activation quantisation in the ABI layout
+// (sorted_ids null = token order), routed combine in gather form (pos: M * top_k ints).
+void launch_mxfp4_quant(const uint16_t* A, const int32_t* sorted_ids, uint8_t* packed, uint8_t* scales,
+                        int rows, int hidden, int top_k, int n_flat, hipStream_t stream);
+void launch_mxfp4_scatter_reduce(const float* partial, const float* topk_w, const int32_t* sorted_ids,
+                                 float* out, int M, int width, int top_k, int EM, int32_t* pos,
+                                 hipStream_t stream);
+
 // Per-kernel set-up that the launchers otherwise do on their first call (the
 // dynamic-LDS limits of the GEMM kernels), for callers that want it done before
 // a graph capture.  False when the device refuses a limit.

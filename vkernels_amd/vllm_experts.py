@@ -248,6 +248,7 @@ def resolve_moe_ws_fn(lib):
 
 MOE_OVERWRITE_OUT = 1  # VK_HIP_MOE_OVERWRITE_OUT
 MOE_SPLIT2 = 2         # VK_HIP_MOE_SPLIT2
+MOE_W4A4 = 4           # VK_HIP_MOE_W4A4
 
 
 def resolve_prepack_fns(lib):
@@ -355,7 +356,7 @@ class FusedExperts:
     def __init__(self, w13, w13_scale, w2, w2_scale, *, b13=None, b2=None, activation="swiglu",
                  swiglu_limit: float = 0.0, beta: float = 4.0, linear_beta: float = 25.0,
                  expert_map=None, local_num_experts=None, scratch: CaptureSafeScratch | None = None,
-                 prepack: bool = False, split_terms: int = 3):
+                 prepack: bool = False, split_terms: int = 3, w4a4: bool = False):
         torch = _require_torch()
         self.torch = torch
         self.lib = load_libvkernels_hip()
@@ -397,6 +398,11 @@ class FusedExperts:
         if split_terms not in (2, 3):
             raise ValueError("split_terms must be 2 or 3")
         self.split_terms = split_terms
+        # W4A4: batches of more than 512 routed rows quantise their activations to MXFP4 as
+        # the reference's mxfp4_moe_quant does (needs the prepacked weights)
+        self.w4a4 = bool(w4a4)
+        if self.w4a4 and not prepack:
+            raise ValueError("w4a4=True needs prepack=True")
         self.w13_packed = self.w2_packed = None
         self.moe_prepacked_fn = None
         if prepack:
@@ -522,7 +528,9 @@ class FusedExperts:
                                   capacity=cap_bytes, name="workspace")
             flags = MOE_OVERWRITE_OUT if overwrite else 0
             if self.w13_packed is not None:
-                if self.split_terms == 2:
+                if self.w4a4:
+                    flags |= MOE_W4A4
+                elif self.split_terms == 2:
                     flags |= MOE_SPLIT2
                 self.moe_prepacked_fn(*args, _ptr(ws), need, flags, _ptr(self.w13_packed),
                                       _ptr(self.w2_packed), self.E, _stream(torch))
