@@ -56,6 +56,9 @@ def parse_args():
     ap.add_argument("--split-terms", type=int, default=3, choices=(2, 3),
                     help="FP6 terms per activation on the prepacked path")
     ap.add_argument("--no-prepack", action="store_true", help="raw weights only, also for prefill sizes")
+    ap.add_argument("--no-modes", action="store_true",
+                    help="skip the prefill record's other arithmetic modes (2 <-> 3 terms, W4A4)")
+    ap.add_argument("--w4a4", action="store_true", help="top-level record in the W4A4 mode (prefill sizes)")
     ap.add_argument("--weight-sets", type=int, default=0, help="0 = enough to exceed 1 GiB")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--block-size", type=int, default=0)
@@ -130,8 +133,11 @@ def cpu_baseline(cfg, T, seed, budget_s=12.0):
     }
 
 
-def run_workload(args, workload, steps, warmup, prepack):
-    """Times one workload; returns the record's fields."""
+def run_workload(args, workload, steps, warmup, prepack, split_terms=None, w4a4=False):
+    """Times one workload; returns the record's fields.  split_terms / w4a4 choose the
+    arithmetic of the prepacked path (default: args.split_terms FP6 terms per bf16
+    activation; w4a4: activations quantised to MXFP4 as the reference's mxfp4_moe_quant
+    does, one FP4 x FP4 MFMA per product)."""
     import numpy as np
     import torch
     from vkernels_amd import synth
@@ -145,6 +151,7 @@ def run_workload(args, workload, steps, warmup, prepack):
     H, I, k = cfg.H, cfg.I, cfg.top_k
     prefill = T * k > 512  # the library's own split between its decode and tile kernels
     prepack = prepack and prefill
+    terms = split_terms or args.split_terms
 
     per_set = synth.algorithmic_bytes(H, I, cfg.E, k, 0, cfg.E)
     n_sets = args.weight_sets or max(2, -(-(1 << 30) // per_set))
@@ -155,7 +162,7 @@ def run_workload(args, workload, steps, warmup, prepack):
     for s in range(n_sets):
         w = synth.make_weights(cfg.E, H, I, seed + 7919 * s, device=dev)
         experts.append(ve.FusedExperts(w.w13, w.w13_scale, w.w2, w.w2_scale, prepack=prepack,
-                                       split_terms=args.split_terms))
+                                       split_terms=terms, w4a4=w4a4 and prepack))
     A_bits = synth.make_activations(T, H, seed)
     logits_np = synth.make_logits(cfg.logits, T, cfg.E, seed, A_bits, H)
     A = torch.from_numpy(A_bits.view(np.int16)).view(torch.bfloat16).to(dev)
@@ -226,10 +233,14 @@ def run_workload(args, workload, steps, warmup, prepack):
     flops = synth.algorithmic_flops(H, I, k, T)
     if prefill:
         fused_tflops = flops / (down_avg * 1e-3) / 1e12
-        if prepack:
-            kernel = (f"vk_hip_fused_moe_mxfp4_prepacked (split_rows_fp6_kernel<{args.split_terms}> x2 + "
-                      f"tile_mx_kernel<0,{args.split_terms}> + tile_mx_kernel<1,{args.split_terms}> + combine_kernel)")
-            issued = float(args.split_terms)  # FP4-rate MFMAs per algorithmic product
+        if prepack and w4a4:
+            kernel = ("vk_hip_fused_moe_mxfp4_prepacked, W4A4 (quant_rows_w4_kernel x2 + tile_mx_kernel<0,1> + "
+                      "tile_mx_kernel<1,1> + combine_kernel)")
+            issued = 1.0
+        elif prepack:
+            kernel = (f"vk_hip_fused_moe_mxfp4_prepacked (split_rows_fp6_kernel<{terms}> x2 + "
+                      f"tile_mx_kernel<0,{terms}> + tile_mx_kernel<1,{terms}> + combine_kernel)")
+            issued = float(terms)  # FP4-rate MFMAs per algorithmic product
         else:
             kernel = ("vk_hip_fused_moe_mxfp4_ex (split_rows_kernel + tile_wide_kernel<0> + "
                       "tile_wide_kernel<1> + combine_kernel)")
@@ -273,7 +284,9 @@ def run_workload(args, workload, steps, warmup, prepack):
         },
     }
     if prepack:
-        rec["config"]["split_terms"] = args.split_terms
+        rec["config"]["activations"] = ("MXFP4 (reference mxfp4_moe_quant), one FP4 x FP4 MFMA per product"
+                                        if w4a4 else f"bf16 as {terms} FP6 E2M3 terms per block of 32")
+        rec["config"]["split_terms"] = 1 if w4a4 else terms
     del experts
     torch.cuda.empty_cache()
     return rec, cfg, T, seed
@@ -289,7 +302,8 @@ def main():
     import torch
     torch.cuda.set_device(torch.device("cuda", 0))
 
-    rec, cfg, T, seed = run_workload(args, args.workload, args.steps, args.warmup, not args.no_prepack)
+    rec, cfg, T, seed = run_workload(args, args.workload, args.steps, args.warmup, not args.no_prepack,
+                                     w4a4=args.w4a4)
     line = {
         "metric": METRIC,
         "value": rec["value"],
@@ -312,6 +326,19 @@ def main():
         p_steps = max(5, min(args.steps, 20))
         p_rec, _, _, _ = run_workload(args, args.prefill, p_steps, min(args.warmup, 3),
                                       not args.no_prepack)
+        if not args.no_prepack and not args.no_modes:
+            # the same workload in the path's other two arithmetic modes (see `activations`)
+            p_rec["other_modes"] = {}
+            for key, kw in (("fp6_terms_%d" % (5 - args.split_terms), dict(split_terms=5 - args.split_terms)),
+                            ("w4a4", dict(w4a4=True))):
+                m_rec, _, _, _ = run_workload(args, args.prefill, p_steps, min(args.warmup, 3), True, **kw)
+                p_rec["other_modes"][key] = {
+                    "value": m_rec["value"], "ms_per_step": m_rec["ms_per_step"],
+                    "activations": m_rec["config"]["activations"],
+                    "fused_call_us": m_rec["roofline"]["avg_launch_us"],
+                    "frac": m_rec["roofline"]["frac"],
+                    "matrix_rate_frac": m_rec["roofline"]["matrix_rate_frac"],
+                }
         line["prefill"] = p_rec
     if args.copy_calibration:
         dev = torch.device("cuda", 0)

@@ -221,13 +221,46 @@ void vk_hip_fused_moe_mxfp4_prepacked(
 /*
  * Additive: per-device set-up that the launchers otherwise do on their first
  * call (the dynamic-LDS limits of the GEMM kernels, the device address of the
- * library's scratch array, the developer knobs of the environment).  Call it
+ * library's scratch array, the tuning store of the launch shapes).  Call it
  * once per device, with that device current, before capturing a HIP graph
  * that contains the entry points of this library.  Returns VK_OK or a
  * VK_ERROR_* code.  No counterpart in the reference, whose launcher reads its
  * one environment knob on first use (src/c/vkernels/kernels/moe_fused.hip:1520-1523).
  */
 int vk_hip_init(void);
+
+/*
+ * Additive: the launch-shape heuristics of the MoE kernels, as the reference
+ * keeps its GEMM ones (candidate table
+ * src/c/vkernels/kernels/common/heuristics.hpp:20-61; tuning store
+ * src/c/vkernels/core/tuning.hpp:11-25, consulted before the compiled-in rules).
+ *
+ * vk_hip_moe_default_block_size: the alignment block the kernels like best for
+ * M tokens routed to top_k experts each (what to pass to
+ * vk_hip_moe_align_block_size and on to the layer).  Any multiple of 16 works.
+ *
+ * A launch shape is four ints {variant, wavefronts, tiles, depth}.
+ * vk_hip_moe_tile_candidates writes up to `capacity` shapes that stage 0
+ * (gate/up) or 1 (down) can be launched at and returns how many there are.
+ * vk_hip_moe_tile_query writes the shape a call of this problem size (blocks =
+ * EM / block_size) would be planned with and returns 1 when it comes from the tuning store, 0 from the
+ * compiled-in rules (a launcher still falls back to the tile kernels where a
+ * shape does not fit the device's LDS).
+ * vk_hip_moe_tile_set puts a record for (stage, K, ncols, bucket of n_flat)
+ * into the process's store (shape null: removes it); VK_ERROR_INVALID_ARGUMENT
+ * for a shape that is not a candidate.  vk_hip_moe_tuning_load reads
+ * <dir>/moe_fused.gfx950.tune (dir null: $VKERNELS_TUNING_CACHE, default
+ * ~/.cache/vkernels/tuning, "off" = none; also read on first use) and returns
+ * the number of records taken.  vk_hip_moe_tuning_dump writes the store as the
+ * text of such a file into buf (at most capacity bytes, always terminated) and
+ * returns the length the whole text needs.
+ */
+int vk_hip_moe_default_block_size(int M, int top_k);
+int vk_hip_moe_tile_candidates(int stage, int* shapes, int capacity);
+int vk_hip_moe_tile_query(int stage, int K, int ncols, int n_flat, int blocks, int* shape);
+int vk_hip_moe_tile_set(int stage, int K, int ncols, int n_flat, const int* shape);
+int vk_hip_moe_tuning_load(const char* dir);
+size_t vk_hip_moe_tuning_dump(char* buf, size_t capacity);
 
 /*
  * Additive: vk_hip_fused_moe_mxfp4_ex for callers that cannot allocate device

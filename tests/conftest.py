@@ -9,6 +9,11 @@ if str(ROOT) not in sys.path:
     sys.path.insert(0, str(ROOT))
 
 
+# a tuning store on the machine must not change what the tests launch (the reference's
+# test main does the same: tests/test_main.cpp:21-26)
+os.environ["VKERNELS_TUNING_CACHE"] = "off"
+
+
 def pytest_configure(config):
     config.addinivalue_line("markers", "gpu: needs a real MI355X (run with -m gpu)")
 

@@ -230,3 +230,20 @@ def test_call_sequence_under_graph_capture(hip_lib, T, prepack):
         c = cpu_layer(a_bits[rows], w.numpy(), rid[rows], rtw[rows], threads=16)
         max_rel, rel_l2, nf = error_metrics(got[rows], c["out"])
         assert nf and max_rel <= MAX_ABS_TOL and rel_l2 <= REL_L2_TOL, (seed, max_rel, rel_l2)
+
+
+def test_apply_hands_back_bf16_on_request(hip_lib):
+    """The reference's serving class returns the layer in the activations' type
+    (src/python/vkernels/vllm_experts.py:1092): output_dtype gives that, as the rounded
+    fp32 result; an empty batch keeps its shape and type."""
+    cfg = synth.CONFIGS["c0"]
+    w = cfgs._weights(cfg, 77)
+    fe = ve.FusedExperts(w.w13, w.w13_scale, w.w2, w.w2_scale)
+    a_bits, l_np = cfgs._inputs(cfg, 16, 78)
+    A = to_dev(a_bits, torch.bfloat16)
+    ids, tw = fe.route(to_dev(l_np), cfg.top_k, True)
+    full = fe.apply(A, ids, tw)
+    half = fe.apply(A, ids, tw, output_dtype=torch.bfloat16)
+    assert half.dtype == torch.bfloat16 and torch.equal(half, full.to(torch.bfloat16))
+    none = fe.apply(A[:0], ids[:0], tw[:0], output_dtype=torch.bfloat16)
+    assert none.dtype == torch.bfloat16 and tuple(none.shape) == (0, cfg.H)

@@ -288,3 +288,60 @@ def test_synth_is_deterministic_and_prefix_stable():
     lg = synth.make_logits("zipf", 512, 128, 3)
     top = np.bincount(np.argsort(-lg, axis=1)[:, :4].ravel(), minlength=128)
     assert top.max() > 6 * np.median(top)
+
+
+# ---- launch-shape heuristics and the tuning store (reference: kernels/common/heuristics.hpp:20-61,
+# core/tuning.hpp:11-25; tests/core/test_tuning.cpp reads the same format) ----
+def test_tile_candidates_and_compiled_in_rules():
+    for stage in (0, 1):
+        cands = ve.moe_tile_candidates(stage)
+        assert len(cands) == 6 and len(set(cands)) == 6
+        assert (0, 4, 4, 0) in cands                      # the tile kernels
+        for n_flat, K, ncols in [(1, 2880, 2880), (256, 2880, 2880), (512, 7168, 2048), (513, 2880, 2880),
+                                 (131072, 7168, 2048), (64, 256, 512)]:
+            shape, stored = ve.moe_tile_query(stage, K, ncols, n_flat)
+            assert not stored and shape in cands, (stage, n_flat, shape)   # selectors return table entries only
+            # the decode kernels up to 512 routed rows, where a pass's rows fit LDS and registers
+            assert (shape[0] == 2) == (n_flat <= 512 and K <= (4096 if stage == 0 else 3072))
+    assert ve.moe_tile_query(0, 2880, 2880, 128, blocks=136)[0] == (2, 4, 2, 8)     # many runs
+    assert ve.moe_tile_query(0, 2880, 2880, 128, blocks=40)[0] == (2, 8, 2, 4)
+    assert ve.moe_tile_query(0, 4096, 1536, 6)[0] == (2, 4, 2, 8)                   # rows of K = 4096
+    assert ve.moe_tile_query(0, 256, 512, 32)[0] == (2, 8, 2, 2) and ve.moe_tile_query(1, 512, 256, 32)[0] == (2, 8, 1, 4)
+    assert ve.default_block_size(0, 4) == 16 and ve.default_block_size(1 << 20, 32) == 128
+
+
+def test_tuning_store_round_trip(tmp_path):
+    lib = ve.load_libvkernels_hip()
+    key = (0, 2880, 2880, 200)
+    before, _ = ve.moe_tile_query(*key)
+    other = next(c for c in ve.moe_tile_candidates(0) if c != before and c[0] == 2)
+    try:
+        ve.moe_tile_set(*key, other)
+        assert ve.moe_tile_query(*key) == (other, True)
+        assert ve.moe_tile_query(0, 2880, 2880, 129) == (other, True)      # same bucket of 256 rows
+        assert ve.moe_tile_query(0, 2880, 2880, 128)[1] is False           # the next bucket down
+        assert ve.moe_tile_query(1, 2880, 2880, 200)[1] is False
+        with pytest.raises(ValueError):
+            ve.moe_tile_set(*key, (2, 8, 3, 4))                            # not a compiled shape
+        with pytest.raises(ValueError):
+            ve.moe_tile_set(1, 2880, 2880, 200, other)                     # a stage-0 shape for stage 1
+        text = ve.moe_tuning_dump()
+        assert text.startswith("# vk-native-tuning/2\n") and "key=0,2880,2880,256\n" in text
+        (tmp_path / "moe_fused.gfx950.tune").write_text(
+            text.replace("key=0,2880,2880,256", "key=0,4096,1536,64")
+            + "garbage line\nkey=1,4096\nwaves=8\n"                          # malformed key: skipped
+            + "key=1,1536,4096,64\nvariant=2\nwaves=8\nnt=7\ndepth=4\n"      # not compiled: skipped
+            + "key=1,1536,4096,512\nvariant=2\nwaves=8\nnt=1\n"              # incomplete: skipped
+            + "# comment\n\nkey=1,1536,4096,32\nvariant=2\nwaves=8\nnt=1\ndepth=12\n")
+        assert ve.moe_tuning_load(str(tmp_path)) == 2
+        assert ve.moe_tile_query(0, 4096, 1536, 40) == (other, True)
+        assert ve.moe_tile_query(1, 1536, 4096, 17) == ((2, 8, 1, 12), True)
+        assert ve.moe_tile_query(1, 1536, 4096, 64)[1] is False and ve.moe_tile_query(1, 1536, 4096, 512)[1] is False
+        assert ve.moe_tile_query(*key) == (other, True)                    # a record set by hand survives a load
+        assert ve.moe_tuning_load(str(tmp_path / "nowhere")) == 0          # no file: the file's records go
+        assert ve.moe_tile_query(1, 1536, 4096, 17)[1] is False
+    finally:
+        ve.moe_tile_set(*key, None)
+        ve.moe_tuning_load(str(tmp_path / "nowhere"))
+    assert ve.moe_tile_query(*key) == (before, False)
+    assert lib.vk_hip_moe_tile_set(2, 64, 64, 1, None) == ve.VK_ERROR_INVALID_ARGUMENT

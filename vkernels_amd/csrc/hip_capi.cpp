@@ -5,9 +5,11 @@
 
 #include <hip/hip_runtime.h>
 
+#include <cstring>
 #include <string>
 
 #include "vk_internal.hpp"
+#include "moe_tuning.hpp"
 
 namespace {
 
@@ -316,6 +318,58 @@ int vk_hip_init(void) {
   if (!vk::prepare_moe_kernels())
     return fail(VK_ERROR_UNSUPPORTED, "vk_hip_init: the device refuses a kernel its LDS");
   return VK_OK;
+}
+
+int vk_hip_moe_default_block_size(int M, int top_k) {
+  return vk::moe_default_block_size(M < 0 ? 0 : M, top_k < 0 ? 0 : top_k);
+}
+
+int vk_hip_moe_tile_candidates(int stage, int* shapes, int capacity) {
+  size_t n = 0;
+  const vk::MoeTileCandidate* table = vk::moe_tile_candidates(&n);
+  int count = 0;
+  for (size_t i = 0; i < n; ++i) {
+    if (table[i].stage != stage) continue;
+    if (shapes != nullptr && count < capacity) {
+      const vk::MoeTile& t = table[i].tile;
+      const int row[4] = {t.variant, t.waves, t.nt, t.depth};
+      for (int j = 0; j < 4; ++j) shapes[4 * count + j] = row[j];
+    }
+    ++count;
+  }
+  return count;
+}
+
+int vk_hip_moe_tile_query(int stage, int K, int ncols, int n_flat, int blocks, int* shape) {
+  vk::MoeTile t;
+  const bool stored = vk::moe_tuning_find(stage, K, ncols, n_flat, &t);
+  if (!stored) t = vk::pick_moe_tile(n_flat, K, ncols, stage, blocks);
+  if (shape != nullptr) {
+    shape[0] = t.variant; shape[1] = t.waves; shape[2] = t.nt; shape[3] = t.depth;
+  }
+  return stored ? 1 : 0;
+}
+
+int vk_hip_moe_tile_set(int stage, int K, int ncols, int n_flat, const int* shape) {
+  vk::MoeTile t{};
+  if (shape != nullptr) t = vk::MoeTile{shape[0], shape[1], shape[2], shape[3]};
+  if (!vk::moe_tuning_set(stage, K, ncols, n_flat, shape != nullptr ? &t : nullptr))
+    return fail(VK_ERROR_INVALID_ARGUMENT,
+                "vk_hip_moe_tile_set: stage must be 0 or 1, sizes positive, and the shape one of "
+                "vk_hip_moe_tile_candidates");
+  return VK_OK;
+}
+
+int vk_hip_moe_tuning_load(const char* dir) { return vk::moe_tuning_load(dir); }
+
+size_t vk_hip_moe_tuning_dump(char* buf, size_t capacity) {
+  const std::string text = vk::moe_tuning_dump("vk_hip_moe_tuning_dump");
+  if (buf != nullptr && capacity > 0) {
+    const size_t n = text.size() < capacity - 1 ? text.size() : capacity - 1;
+    memcpy(buf, text.data(), n);
+    buf[n] = 0;
+  }
+  return text.size() + 1;
 }
 
 size_t vk_hip_static_scratch_bytes(void) { return vk::static_scratch_bytes(); }

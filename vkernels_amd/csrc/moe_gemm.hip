@@ -42,6 +42,7 @@
 
 #include "moe_common.hpp"
 #include "moe_heuristics.hpp"
+#include "moe_tuning.hpp"
 #include "mxfp4.hpp"
 #include "vk_internal.hpp"
 
@@ -360,6 +361,12 @@ __device__ __forceinline__ void split_bf16x8(u32x4 v, uint32_t sb, uint2& hi, ui
   lo = make_uint2(l[0].u, l[1].u);
 }
 
+// 16-byte pieces of a row that a lane of the resident kernel holds in registers while it
+// stages a pass (every wavefront takes every WAVES-th group of 32 values): workgroups of
+// 8 wavefronts, two to a SIMD, hold K <= 3072; workgroups of 4, with a SIMD's whole
+// register file each, K <= 4096.
+__host__ __device__ constexpr int resident_batch(int waves) { return waves == 4 ? 32 : 96 / waves; }
+
 template <int STAGE, int WAVES, int NT, int D>
 __global__ __launch_bounds__(64 * WAVES) void stream_resident_kernel(GemmArgs p) {
   extern __shared__ u32x4 b_lds[];  // [nsteps][2][2][64] operand planes, block scales, weight scales
@@ -606,7 +613,7 @@ __global__ __launch_bounds__(64 * WAVES) void stream_resident_kernel(GemmArgs p)
         // the loads, so that the wait below counts only the row loads), then
         // the wait for the slowest wavefront of the previous pass.  The weight
         // loads so stay in flight while the rows are split and written.
-        constexpr int kBatch = 96 / WAVES;  // pieces per lane: K <= 3072 in one batch
+        constexpr int kBatch = resident_batch(WAVES);  // pieces per lane, all of K in one batch
         const int n_pieces = (nsteps * 4 + WAVES - 1) / WAVES;  // the launcher keeps it <= kBatch
         const int sd = lane & 3;
         const int sj = lane >> 2;
@@ -1538,33 +1545,6 @@ int num_compute_units() {
   return cus;
 }
 
-// Developer overrides of the launch shapes, read from the environment once per
-// process (0 / negative = the library's own choice).  VK_MOE_VARIANT, VK_MOE_NT,
-// VK_MOE_DEPTH, VK_MOE_WAVES: shape of the resident kernel; VK_MOE_WGS: its grid;
-// VK_MOE_PRESPLIT=0 / VK_MOE_COMBINE=0: ignore the workspace / add with atomics.
-struct DebugKnobs {
-  int variant, nt, depth, waves, wgs, presplit, combine;
-};
-
-const DebugKnobs& debug_knobs() {
-  static const DebugKnobs knobs = [] {
-    auto env_int = [](const char* name, int fallback) {
-      const char* v = getenv(name);
-      return (v != nullptr && *v != 0) ? atoi(v) : fallback;
-    };
-    DebugKnobs k;
-    k.variant = env_int("VK_MOE_VARIANT", -1);
-    k.nt = env_int("VK_MOE_NT", 0);
-    k.depth = env_int("VK_MOE_DEPTH", 0);
-    k.waves = env_int("VK_MOE_WAVES", 0);
-    k.wgs = env_int("VK_MOE_WGS", num_compute_units());
-    k.presplit = env_int("VK_MOE_PRESPLIT", 1);
-    k.combine = env_int("VK_MOE_COMBINE", 1);
-    return k;
-  }();
-  return knobs;
-}
-
 constexpr size_t kResidentLdsLimit = 150 * 1024;  // dynamic LDS the resident kernel may ask for
 
 // True when the device grants the kernel its dynamic LDS (asked once per kernel;
@@ -1584,15 +1564,10 @@ bool resident_kernel_ready() {
 template <int STAGE, int WAVES, int NT, int D>
 bool launch_resident(const GemmArgs& g, size_t lds, hipStream_t stream) {
   if (!resident_kernel_ready<STAGE, WAVES, NT, D>()) return false;
-  hipLaunchKernelGGL((stream_resident_kernel<STAGE, WAVES, NT, D>), dim3(debug_knobs().wgs),
+  hipLaunchKernelGGL((stream_resident_kernel<STAGE, WAVES, NT, D>), dim3(num_compute_units()),
                      dim3(64 * WAVES), lds, stream, g);
   return true;
 }
-
-// The instantiations of the resident kernel: X(stage, wavefronts, tiles, depth).
-#define VK_RESIDENT_VARIANTS(X) \
-  X(0, 8, 2, 2) X(0, 8, 2, 4) X(0, 8, 2, 6) X(0, 4, 2, 4) X(0, 4, 2, 8) \
-  X(1, 8, 2, 4) X(1, 8, 1, 4) X(1, 8, 1, 6) X(1, 8, 1, 8) X(1, 8, 1, 12)
 
 // Launch shape of one stage.  variant kMoeVariantLds = the tile kernel.
 struct StagePlan {
@@ -1602,13 +1577,15 @@ struct StagePlan {
 
 template <int STAGE>
 StagePlan plan_stage(const GemmArgs& g) {
-  const MoeTile tile = pick_moe_tile(g.n_flat, g.K, g.ncols, STAGE);
+  // a record of the tuning store first, then the compiled-in rules
+  MoeTile tile;
+  if (!moe_tuning_find(STAGE, g.K, g.ncols, g.n_flat, &tile))
+    tile = pick_moe_tile(g.n_flat, g.K, g.ncols, STAGE, g.num_blocks);
   StagePlan pl;
-  const DebugKnobs& knobs = debug_knobs();
-  pl.variant = knobs.variant >= 0 ? knobs.variant : tile.variant;
-  pl.nt = knobs.nt > 0 ? knobs.nt : tile.nt;
-  pl.depth = knobs.depth > 0 ? knobs.depth : tile.depth;
-  pl.waves = knobs.waves > 0 ? knobs.waves : tile.waves;
+  pl.variant = tile.variant;
+  pl.nt = tile.nt;
+  pl.depth = tile.depth;
+  pl.waves = tile.waves;
   const int groups = g.K / 32;
   const int nsteps = (groups + 3) / 4;
   // operand planes + block scales + one weight-scale region per wavefront
@@ -1617,7 +1594,7 @@ StagePlan plan_stage(const GemmArgs& g) {
   if (pl.resident_lds > kResidentLdsLimit || g.num_blocks > kMaxRuns ||
       pl.nt * groups > 64 * kScMax ||
       (res_units + pl.waves - 1) / pl.waves > 64 ||  // one bit per unit in a wavefront's redo mask
-      nsteps * 4 > 96)  // the rows are staged in one batch of 96 / waves pieces
+      nsteps * 4 > resident_batch(pl.waves) * pl.waves)  // the rows are staged in one batch
     pl.variant = kMoeVariantLds;
   return pl;
 }
@@ -1780,7 +1757,8 @@ bool prepare_moe_kernels() {
 #define VK_READY(S_, W_, NT_, D_) ok = resident_kernel_ready<S_, W_, NT_, D_>() && ok;
   VK_RESIDENT_VARIANTS(VK_READY)
 #undef VK_READY
-  (void)debug_knobs();
+  MoeTile unused;
+  (void)moe_tuning_find(0, 64, 64, 1, &unused);  // reads the tuning store now rather than on the first launch
   return ok;
 }
 
@@ -1797,10 +1775,10 @@ void launch_moe_down(const FusedMoeArgs& a, hipStream_t stream) {
   GemmArgs g = down_args(a);
   const StagePlan pl = plan_stage<1>(g);
   const bool overwrite = (a.flags & 1u) != 0u;  // VK_HIP_MOE_OVERWRITE_OUT
-  if (pl.variant != kMoeVariantResident && debug_knobs().presplit != 0) {
+  if (pl.variant != kMoeVariantResident) {
     if (a.w2_packed != nullptr && launch_moe_down_prepacked(a, stream)) return;
     Workspace w;
-    if (carve_workspace(a, w) && g.K >= 512 && wide_kernel_ready<1>() && debug_knobs().combine != 0) {
+    if (carve_workspace(a, w) && g.K >= 512 && wide_kernel_ready<1>()) {
       const long long pieces = (long long)a.EM * split_row_k(a.ispp) / 8;
       hipLaunchKernelGGL(split_rows_kernel, dim3((unsigned)((pieces + 255) / 256)), dim3(256), 0,
                          stream, a.act, w.act_q, w.act_s, pieces, a.ispp);
@@ -1828,13 +1806,13 @@ void launch_fused_moe(const FusedMoeArgs& a, hipStream_t stream) {
   const StagePlan p0 = plan_stage<0>(g0), p1 = plan_stage<1>(g1);
   // prefill-sized batches on prepacked weights: the FP4-rate kernels of moe_prefill.hip
   if (a.w13_packed != nullptr && p0.variant != kMoeVariantResident &&
-      p1.variant != kMoeVariantResident && debug_knobs().presplit != 0 &&
+      p1.variant != kMoeVariantResident &&
       launch_fused_moe_prepacked(a, stream))
     return;
   Workspace w;
   bool combine = false;
   bool split_act_between = false;
-  if (carve_workspace(a, w) && debug_knobs().presplit != 0) {
+  if (carve_workspace(a, w)) {
     // the wide kernel takes a stage that runs as a tile kernel with K >= 512
     const bool wide0 = p0.variant != kMoeVariantResident && g0.K >= 512 && wide_kernel_ready<0>();
     const bool wide1 = p1.variant != kMoeVariantResident && g1.K >= 512 && wide_kernel_ready<1>();
@@ -1856,13 +1834,10 @@ void launch_fused_moe(const FusedMoeArgs& a, hipStream_t stream) {
       }
       // The second stage stores its rows and a last pass sums them per token (far
       // cheaper than one atomic per row and column).
-      if (debug_knobs().combine != 0) {
-        combine = true;
-        g1.y = w.y;
-        g1.pos = w.pos;
-        const int n = a.M * a.top_k;
-        launch_fill_i32(w.pos, -1, n, stream);
-      }
+      combine = true;
+      g1.y = w.y;
+      g1.pos = w.pos;
+      launch_fill_i32(w.pos, -1, a.M * a.top_k, stream);
     }
   }
   const bool overwrite = (a.flags & 1u) != 0u;  // VK_HIP_MOE_OVERWRITE_OUT

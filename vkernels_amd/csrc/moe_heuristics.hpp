@@ -1,10 +1,13 @@
-// moe_heuristics.hpp — launch shapes of the MoE grouped GEMMs for gfx950.
+// moe_heuristics.hpp — launch shapes of the MoE grouped GEMMs for gfx950, as data.
 //
-// Same role as the GEMM candidate table of the reference
-// (src/c/vkernels/kernels/common/heuristics.hpp:20-61), which has no MoE
-// entries of its own: a small table of launch shapes and a pure function
-// that picks one from the problem size on the host.
+// Same layering as the reference's GEMM candidates
+// (src/c/vkernels/kernels/common/heuristics.hpp:20-61, which has no MoE entries of its
+// own): the table of shapes that are compiled and were swept, and a selector that only
+// ever returns entries of it.  The selector is consulted after the tuning store
+// (moe_tuning.hpp), the way the reference's selectors are (core/tuning.hpp:1-9).
 #pragma once
+
+#include <cstddef>
 
 namespace vk {
 
@@ -13,31 +16,105 @@ enum { kMoeVariantLds = 0, kMoeVariantResident = 2 };
 struct MoeTile {
   int variant;  // kMoeVariantResident: one workgroup per compute unit, the
                 // activation rows of a run resident in LDS (decode);
-                // kMoeVariantLds: activation rows staged through LDS chunk by chunk
+                // kMoeVariantLds: the tile kernels (rows staged through LDS)
   int waves;    // wavefronts per workgroup
   int nt;       // 16-row weight tiles per wavefront
   int depth;    // K steps in flight per wavefront (resident variant)
 };
 
-// n_flat = tokens * top_k routed rows in the call, K / ncols the GEMM's
-// reduction and output widths, stage 0 = gate/up, 1 = down.  The number of
-// experts is not known to the launcher, so the split is on the routed rows
-// alone: a decode batch leaves most experts with at most one 16-row tile.
+inline bool operator==(const MoeTile& a, const MoeTile& b) {
+  return a.variant == b.variant && a.waves == b.waves && a.nt == b.nt && a.depth == b.depth;
+}
+
+// Every shape a stage can be launched at: the instantiations of the resident kernel
+// (X(stage, wavefronts, tiles, depth) — moe_gemm.hip instantiates exactly these) and
+// the tile kernels as one more entry.  The sweep (vkernels_amd/tune_moe.py) times each
+// of these for a stage and a problem size.
+#define VK_RESIDENT_VARIANTS(X) \
+  X(0, 8, 2, 2) X(0, 8, 2, 4) X(0, 8, 2, 6) X(0, 4, 2, 4) X(0, 4, 2, 8) \
+  X(1, 8, 2, 4) X(1, 8, 1, 4) X(1, 8, 1, 6) X(1, 8, 1, 8) X(1, 8, 1, 12)
+
+struct MoeTileCandidate {
+  int stage;
+  MoeTile tile;
+};
+
+inline const MoeTileCandidate* moe_tile_candidates(size_t* count) {
+  static const MoeTileCandidate table[] = {
+#define VK_CANDIDATE(S_, W_, NT_, D_) {S_, {kMoeVariantResident, W_, NT_, D_}},
+      VK_RESIDENT_VARIANTS(VK_CANDIDATE)
+#undef VK_CANDIDATE
+      {0, {kMoeVariantLds, 4, 4, 0}},
+      {1, {kMoeVariantLds, 4, 4, 0}},
+  };
+  *count = sizeof(table) / sizeof(table[0]);
+  return table;
+}
+
+inline bool is_moe_tile_candidate(int stage, const MoeTile& tile) {
+  size_t n = 0;
+  const MoeTileCandidate* table = moe_tile_candidates(&n);
+  for (size_t i = 0; i < n; ++i)
+    if (table[i].stage == stage && table[i].tile == tile) return true;
+  return false;
+}
+
+// Routed rows up to which a call runs the resident (decode) kernels: beyond, most
+// experts have several 16-row passes and the tile kernels, which keep a 128-row window
+// per workgroup, read each weight byte once per window instead of once per pass.
+constexpr int kMoeDecodeMaxRows = 512;
+
+// One row of the decision table: the first row whose bounds hold decides.
+struct MoeTileRule {
+  int stage;
+  int max_rows;    // n_flat <= max_rows
+  int max_k;       // K <= max_k
+  int min_blocks;  // blocks of the call (EM / block_size, an upper bound of the runs) >= min_blocks
+  MoeTile tile;
+};
+
+// n_flat = tokens * top_k routed rows in the call, K / ncols the GEMM's reduction and
+// output widths, stage 0 = gate/up, 1 = down, blocks = EM / block_size.  The number of
+// experts is not known to the launcher: the split between the kernel families is on the
+// routed rows alone, and `blocks` stands for the number of runs where that matters.
 //
-// Decode: the units of a run are shared by (compute units / runs) workgroups
-// of 8 wavefronts, so a stage wants at least ~3 units per wavefront or the
-// last round leaves most wavefronts idle.  Gate/up units are a gate tile and
-// its up tile (nt = 2, ispp / 16 units per expert); the down stage, with half
-// the weight rows, takes single tiles (nt = 1) and keeps the bytes in flight
-// per wavefront with a deeper pipeline.
-inline MoeTile pick_moe_tile(int n_flat, int K, int ncols, int stage) {
-  (void)K;
-  (void)ncols;
-  if (n_flat <= 512) {
-    if (stage == 1) return MoeTile{kMoeVariantResident, 8, 1, 8};
-    return MoeTile{kMoeVariantResident, 8, 2, 4};
-  }
+// Decode: the units of a run are shared by (compute units / runs) workgroups of 8
+// wavefronts, so a stage wants at least ~3 units per wavefront or the last round leaves
+// most wavefronts idle.  Gate/up units are a gate tile and its up tile (nt = 2,
+// ispp / 16 units per expert); the down stage, with half the weight rows, takes single
+// tiles (nt = 1) and keeps the bytes in flight per wavefront with a deeper pipeline.
+// Rows (each from the sweep table profiles/moe_decode_tile_sweep.md):
+//  - K <= 1024: a unit is a few steps long, and steps in flight past its end are
+//    wasted loads: the shallowest pipelines (256x512x8x2: 12.1 against 13.8 us);
+//  - many runs (more than 64 blocks: 2880x2880x128x4 from T = 32): each workgroup has a
+//    run to itself and few units, and 4 wavefronts with 8 steps in flight each keep more
+//    bytes in flight per wavefront (157 against 165 us, 214 against 229 us);
+//  - 3072 < K <= 4096 (4096x1536x64x6 gate/up): the rows of a pass fit LDS and registers
+//    only with 4 wavefronts per workgroup;
+//  - otherwise (8, 2, 4) / (8, 1, 8), within 2 % of the best of every other point swept.
+inline MoeTile pick_moe_tile(int n_flat, int K, int ncols, int stage, int blocks) {
+  (void)ncols;  // no swept point separates on it: the units per wavefront follow from it, not the shape
+  static const MoeTileRule rules[] = {
+      {0, kMoeDecodeMaxRows, 1024, 0, {kMoeVariantResident, 8, 2, 2}},
+      {0, kMoeDecodeMaxRows, 3072, 65, {kMoeVariantResident, 4, 2, 8}},
+      {0, kMoeDecodeMaxRows, 3072, 0, {kMoeVariantResident, 8, 2, 4}},
+      {0, kMoeDecodeMaxRows, 4096, 0, {kMoeVariantResident, 4, 2, 8}},
+      {1, kMoeDecodeMaxRows, 1024, 0, {kMoeVariantResident, 8, 1, 4}},
+      {1, kMoeDecodeMaxRows, 3072, 0, {kMoeVariantResident, 8, 1, 8}},
+  };
+  for (const MoeTileRule& r : rules)
+    if (r.stage == stage && n_flat <= r.max_rows && K <= r.max_k && blocks >= r.min_blocks) return r.tile;
   return MoeTile{kMoeVariantLds, 4, 4, 0};
+}
+
+// Alignment block the library's kernels like best for a batch of M tokens routed to
+// top_k experts each.  Decode kernel: a pass per 16 rows, and blocks of 16 tell it the
+// passes of every expert exactly and pad least.  Tile kernels: a workgroup takes a
+// window of 128 sorted rows of one expert, so blocks of 128 give every expert windows of
+// its own (0.5 to 8 % faster than blocks of 64 from 16 to 770 rows per expert).
+inline int moe_default_block_size(int M, int top_k) {
+  const long long n = (long long)M * (long long)top_k;
+  return n <= kMoeDecodeMaxRows ? 16 : 128;
 }
 
 }  // namespace vk

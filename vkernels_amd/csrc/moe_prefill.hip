@@ -94,7 +94,6 @@ struct MxArgs {
   float swiglu_limit, beta, linear_beta;
   int activation;
   int units, col_groups, windows;
-  int map_mode;  // experiment: 0 = chunks of 32 tiles per XCD, 1 = identity, n >= 2 = chunks of n tiles
 };
 
 __host__ __device__ inline int mx_kp(int K) { return (K + 127) & ~127; }
@@ -542,9 +541,7 @@ __global__ __launch_bounds__(64 * kMxWaves) void tile_mx_kernel(MxArgs p) {
   // one XCD (workgroup ids go round-robin over the 8 XCDs), chunk after chunk ----
   const int total = p.col_groups * p.windows;
   const int slot = blockIdx.x >> 3;
-  int logical = ((slot >> 5) * 8 + (blockIdx.x & 7)) * 32 + (slot & 31);
-  if (p.map_mode == 1) logical = blockIdx.x;
-  else if (p.map_mode >= 2) logical = ((slot / p.map_mode) * 8 + (blockIdx.x & 7)) * p.map_mode + (slot % p.map_mode);
+  const int logical = ((slot >> 5) * 8 + (blockIdx.x & 7)) * 32 + (slot & 31);
   if (logical >= total) return;
   const int window = logical / p.col_groups;
   const int colg = logical - window * p.col_groups;
@@ -868,10 +865,7 @@ void launch_mx_stage_t(MxArgs g, hipStream_t stream) {
   g.col_groups = (g.units + kMxWaves - 1) / kMxWaves;
   g.windows = (g.num_blocks * g.block_size + win - 1) / win;
   const long long total = (long long)g.col_groups * g.windows;
-  static const int map_mode = [] { const char* v = getenv("VK_MOE_MX_MAP"); return v ? atoi(v) : 0; }();
-  g.map_mode = map_mode;
-  const long long period = map_mode >= 2 ? 8ll * map_mode : 256;
-  const unsigned grid = (unsigned)((total + period - 1) / period * period);
+  const unsigned grid = (unsigned)((total + 255) / 256 * 256);  // whole chunks of 32 tiles for each of 8 XCDs
   hipLaunchKernelGGL((tile_mx_kernel<STAGE, TERMS>), dim3(grid), dim3(64 * kMxWaves),
                      kMxRing * kMxRows * TERMS * 128, stream, g);
 }

@@ -327,21 +327,72 @@ def _stream(torch):
 _scratch = CaptureSafeScratch()
 
 
-def default_block_size(M: int, top_k: int | None = None) -> int:
+def default_block_size(M: int, top_k: int | None = None, lib=None) -> int:
     """The reference's policy: 16-row alignment for decode batches, 64 above
-    (vllm_experts.py:846).  With top_k given the split follows the library's own
-    (M * top_k <= 512 routed rows run the decode kernel, which makes a pass per 16
-    rows: blocks of 16 tell it the passes of every expert exactly and pad least;
-    larger batches take blocks of 128)."""
+    (vllm_experts.py:846).  With top_k given the library is asked what its kernels
+    like best (vk_hip_moe_default_block_size: 16 while M * top_k routed rows run the
+    decode kernels, blocks of 128 for the tile kernels' windows beyond)."""
     if top_k is not None:
-        n = M * top_k
-        if n <= 512:
-            return 16
-        # beyond: a workgroup of the tile kernel takes 128 sorted rows of one expert;
-        # blocks of 128 give every expert windows of its own (measured: 0.5 to 8 %
-        # faster than blocks of 64 from 16 to 770 rows per expert)
-        return 128
+        lib = load_libvkernels_hip() if lib is None else lib
+        fn = getattr(lib, "vk_hip_moe_default_block_size", None)
+        if fn is None:
+            raise RuntimeError("the loaded libvkernels_hip has no vk_hip_moe_default_block_size; "
+                               "pass block_size, or call default_block_size(M) for the reference's policy")
+        fn.restype, fn.argtypes = _I, [_I, _I]
+        return int(fn(int(M), int(top_k)))
     return 16 if M <= 32 else 64
+
+
+# ---- launch shapes: candidates, the tuning store, queries (vkernels_hip.h) ----
+def moe_tile_candidates(stage: int, lib=None) -> list[tuple[int, int, int, int]]:
+    """(variant, wavefronts, tiles, depth) of every shape the stage can be launched at."""
+    lib = load_libvkernels_hip() if lib is None else lib
+    fn = lib.vk_hip_moe_tile_candidates
+    fn.restype, fn.argtypes = _I, [_I, _P, _I]
+    n = int(fn(stage, None, 0))
+    buf = (ctypes.c_int * (4 * n))()
+    fn(stage, buf, n)
+    return [tuple(buf[4 * i:4 * i + 4]) for i in range(n)]
+
+
+def moe_tile_query(stage: int, K: int, ncols: int, n_flat: int, blocks: int | None = None, lib=None):
+    """((variant, wavefronts, tiles, depth), from_store) a call of this size is planned
+    with; blocks = EM / block_size (default: one block per 16 routed rows)."""
+    lib = load_libvkernels_hip() if lib is None else lib
+    fn = lib.vk_hip_moe_tile_query
+    fn.restype, fn.argtypes = _I, [_I, _I, _I, _I, _I, _P]
+    buf = (ctypes.c_int * 4)()
+    blocks = (n_flat + 15) // 16 if blocks is None else blocks
+    stored = int(fn(stage, K, ncols, n_flat, blocks, buf))
+    return tuple(buf), bool(stored)
+
+
+def moe_tile_set(stage: int, K: int, ncols: int, n_flat: int, shape, lib=None) -> None:
+    """Puts (shape None: removes) the record of this problem in the process's tuning store."""
+    lib = load_libvkernels_hip() if lib is None else lib
+    fn = lib.vk_hip_moe_tile_set
+    fn.restype, fn.argtypes = _I, [_I, _I, _I, _I, _P]
+    buf = None if shape is None else (ctypes.c_int * 4)(*shape)
+    if fn(stage, K, ncols, n_flat, buf) != VK_OK:
+        raise ValueError(last_error(lib))
+
+
+def moe_tuning_load(directory: str | None = None, lib=None) -> int:
+    lib = load_libvkernels_hip() if lib is None else lib
+    fn = lib.vk_hip_moe_tuning_load
+    fn.restype, fn.argtypes = _I, [ctypes.c_char_p]
+    return int(fn(None if directory is None else os.fsencode(directory)))
+
+
+def moe_tuning_dump(lib=None) -> str:
+    """The process's tuning store as the text of a moe_fused.gfx950.tune file."""
+    lib = load_libvkernels_hip() if lib is None else lib
+    fn = lib.vk_hip_moe_tuning_dump
+    fn.restype, fn.argtypes = ctypes.c_size_t, [ctypes.c_char_p, ctypes.c_size_t]
+    need = int(fn(None, 0))
+    buf = ctypes.create_string_buffer(need)
+    fn(buf, need)
+    return buf.value.decode()
 
 
 class FusedExperts:
@@ -465,9 +516,11 @@ class FusedExperts:
 
     # -- the layer --------------------------------------------------------------
     def apply(self, hidden_states, topk_ids, topk_weights=None, *, block_size: int | None = None,
-              max_tokens: int | None = None, out_fp32=None):
+              max_tokens: int | None = None, out_fp32=None, output_dtype=None):
         """hidden_states [M, H] bf16, topk_ids [M, k] int32, topk_weights [M, k]
-        fp32 (None = ones).  Returns fp32 [M, H]."""
+        fp32 (None = ones).  Returns the fp32 [M, H] result, or, with output_dtype
+        (say torch.bfloat16, what the reference's apply hands back,
+        src/python/vkernels/vllm_experts.py:1092), that result cast."""
         torch = self.torch
         M, K = hidden_states.shape
         if K != self.hidden:
@@ -490,12 +543,11 @@ class FusedExperts:
         overwrite = self.moe_ex_fn is not None and self.use_workspace and M > 0
         if not overwrite:
             out_fp32.zero_()
-        if M == 0:
-            return out_fp32
-        sids, eids, _, max_em = self.align(topk_ids, block_size, max_tokens=max_tokens)
-        self.fused_call(hidden_states, topk_ids, topk_weights, sids, eids, max_em, block_size,
-                        out_fp32, max_tokens=max_tokens, overwrite=overwrite)
-        return out_fp32
+        if M > 0:
+            sids, eids, _, max_em = self.align(topk_ids, block_size, max_tokens=max_tokens)
+            self.fused_call(hidden_states, topk_ids, topk_weights, sids, eids, max_em, block_size,
+                            out_fp32, max_tokens=max_tokens, overwrite=overwrite)
+        return out_fp32 if output_dtype is None else out_fp32.to(output_dtype)
 
     def fused_call(self, hidden_states, topk_ids, topk_weights, sids, eids, max_em: int,
                    block_size: int, out_fp32, *, max_tokens: int | None = None,
