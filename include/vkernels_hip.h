@@ -375,6 +375,58 @@ int vk_hip_mxfp4_moe_scatter_reduce(const float* partial, const float* topk_w,
                                     size_t workspace_bytes, void* stream);
 
 /*
+ * Additive: the layer as four stages with an explicit boundary between the
+ * linear GEMMs and the elementwise epilogues, for tensor-parallel callers that
+ * sum (all-reduce) the fp32 pre-activations of their K slices between them.
+ * Device counterparts of the reference's stage split
+ * (src/c/vkernels/kernels/moe_fused.hpp:103-125; HIP declarations :259-283
+ * moe_gateup_preact / moe_act_epilogue / moe_down_preact / moe_combine, which the
+ * reference's C ABI does not export), with block_size as one more argument
+ * (the reference's are fixed at 16) and the stream last:
+ *
+ *   vk_hip_moe_gateup_preact  gate_up[r, 0:ispp] = A[token(r), k_base : k_base +
+ *       hidden_k] . w13[e, 0:ispp]^T, gate_up[r, ispp:2*ispp] likewise with the up
+ *       rows, fp32 [EM, 2*ispp]; A rows are `hidden` wide, w13 / w13_scale are the
+ *       rank's shard [E, 2*ispp, hidden_k/2] / [E, 2*ispp, hidden_k/32]
+ *   (caller: all-reduce gate_up)
+ *   vk_hip_moe_act_epilogue   act[r, :] = activation(gate_up[r] + b13[e]), bf16
+ *       [EM, ispp]
+ *   vk_hip_moe_down_preact    partial[r, :] = act[r, k_base : k_base + ispp_k] .
+ *       w2[e]^T, fp32 [EM, hidden]; act rows are `ispp` wide, w2 / w2_scale the
+ *       shard [E, hidden, ispp_k/2] / [E, hidden, ispp_k/32]
+ *   (caller: all-reduce partial)
+ *   vk_hip_moe_combine        out[token, :] += (partial[r, :] + b2[e, :]) *
+ *       topk_w_sorted[r] over the token's sorted rows in ascending r: the sum
+ *       the reference forms, bit for bit (gather form, no atomics; workspace:
+ *       M*top_k int32 of device memory); topk_w_sorted is [EM], the routing
+ *       weight of every sorted row (out accumulates: zero it first)
+ *
+ * With k_base = 0 and the full K the four calls compute what
+ * vk_hip_fused_moe_mxfp4 computes.  Only routed rows (sorted id in
+ * [0, M*top_k), block with an expert) are written or read.  hidden_k and ispp_k
+ * must be multiples of 64, k_base and the row widths multiples of 8 (rows are
+ * read 16 bytes at a time).  The GEMM stages take raw weights and run the
+ * decode kernels or the plain tile kernels.  Return VK_OK or a VK_ERROR_* code;
+ * asynchronous on `stream`, no allocation.
+ */
+int vk_hip_moe_gateup_preact(const uint16_t* A, const uint8_t* w13, const uint8_t* w13_scale,
+                             const int32_t* sorted_ids, const int32_t* expert_ids, float* gate_up,
+                             int M, int hidden, int ispp, int top_k, int EM, int k_base, int hidden_k,
+                             int block_size, void* stream);
+int vk_hip_moe_act_epilogue(const float* gate_up, const float* b13, uint16_t* act,
+                            const int32_t* sorted_ids, const int32_t* expert_ids, int M, int top_k,
+                            int EM, int ispp, float swiglu_limit, int activation, float beta,
+                            float linear_beta, int block_size, void* stream);
+int vk_hip_moe_down_preact(const uint16_t* act, const uint8_t* w2, const uint8_t* w2_scale,
+                           const int32_t* sorted_ids, const int32_t* expert_ids, float* partial, int M,
+                           int ispp, int hidden, int top_k, int EM, int k_base, int ispp_k,
+                           int block_size, void* stream);
+int vk_hip_moe_combine(const float* partial, const float* b2, const float* topk_w_sorted,
+                       const int32_t* sorted_ids, const int32_t* expert_ids, float* out, int M,
+                       int hidden, int top_k, int EM, int block_size, void* workspace,
+                       size_t workspace_bytes, void* stream);
+
+/*
  * On-device alignment of the routing table: stable bucket of the flat indices
  * by (local) expert, each expert padded to a multiple of block_size.
  * Replaces vk_hip_moe_align_block_size,

@@ -345,3 +345,38 @@ def test_tuning_store_round_trip(tmp_path):
         ve.moe_tuning_load(str(tmp_path / "nowhere"))
     assert ve.moe_tile_query(*key) == (before, False)
     assert lib.vk_hip_moe_tile_set(2, 64, 64, 1, None) == ve.VK_ERROR_INVALID_ARGUMENT
+
+
+def test_stage_entry_points_reject_contract_violations_without_a_device():
+    """The four stages of the tensor-parallel split validate on the host and launch
+    nothing for a refused or an empty call."""
+    lib = ve.load_libvkernels_hip()
+    P, I, F = ctypes.c_void_p, ctypes.c_int, ctypes.c_float
+    gu = lib.vk_hip_moe_gateup_preact
+    gu.restype, gu.argtypes = I, [P] * 6 + [I] * 8 + [P]
+    dn = lib.vk_hip_moe_down_preact
+    dn.restype, dn.argtypes = I, [P] * 6 + [I] * 8 + [P]
+    ep = lib.vk_hip_moe_act_epilogue
+    ep.restype, ep.argtypes = I, [P] * 5 + [I] * 4 + [F, I, F, F, I, P]
+    cb = lib.vk_hip_moe_combine
+    cb.restype, cb.argtypes = I, [P] * 6 + [I] * 5 + [P, ctypes.c_size_t, P]
+    bad = ve.VK_ERROR_INVALID_ARGUMENT
+    nil = (None,) * 6
+    #                         M  hidden ispp k  EM  k_base k_dim bs
+    assert gu(*nil, 0, 256, 512, 2, 0, 0, 256, 16, None) == 0             # nothing routed
+    assert gu(*nil, 4, 256, 512, 2, 32, 0, 256, 16, None) == bad          # null buffers
+    assert "null" in ve.last_error(lib)
+    assert gu(*nil, 4, 256, 512, 2, 32, 4, 128, 16, None) == bad          # k_base not a multiple of 8
+    assert gu(*nil, 4, 256, 512, 2, 32, 0, 96, 16, None) == bad           # slice not a multiple of 64
+    assert gu(*nil, 4, 256, 512, 2, 32, 192, 128, 16, None) == bad        # slice past the row
+    assert gu(*nil, 4, 256, 512, 2, 32, 0, 256, 24, None) == bad          # block size
+    assert gu(*nil, 4, 256, 512, 0, 32, 0, 256, 16, None) == bad          # top_k
+    assert dn(*nil, 4, 512, 256, 2, 32, 0, 512, 16, None) == bad
+    assert dn(*nil, 4, 512, 250, 2, 32, 0, 512, 16, None) == bad          # output width
+    assert dn(*nil, 0, 512, 256, 2, 0, 0, 512, 16, None) == 0
+    assert ep(None, None, None, None, None, 4, 2, 32, 512, 0.0, 0, 4.0, 25.0, 16, None) == bad
+    assert ep(None, None, None, None, None, 4, 2, 32, 512, 0.0, 5, 4.0, 25.0, 16, None) == bad   # activation
+    assert ep(None, None, None, None, None, 0, 2, 0, 512, 0.0, 0, 4.0, 25.0, 16, None) == 0
+    assert cb(*nil, 4, 256, 2, 32, 16, None, 0, None) == bad
+    assert cb(*nil, 4, 254, 2, 32, 16, None, 0, None) == bad
+    assert cb(*nil, 0, 256, 2, 0, 16, None, 0, None) == 0

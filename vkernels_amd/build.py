@@ -25,7 +25,7 @@ OBJ = PKG / "build"
 LIB = PKG / "libvkernels_hip.so"
 
 SOURCES = ["moe_route.hip", "moe_align.hip", "moe_dequant.hip", "moe_gemm.hip", "moe_prefill.hip", "static_scratch.hip",
-           "moe_tuning.cpp",
+           "moe_tuning.cpp", "moe_stages.hip",
            "hip_capi.cpp"]
 
 # -packed-fp32-ops off: hipcc must not form packed fp32 arithmetic.

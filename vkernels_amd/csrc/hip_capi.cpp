@@ -283,6 +283,105 @@ int vk_hip_mxfp4_moe_scatter_reduce(const float* partial, const float* topk_w,
   return VK_OK;
 }
 
+namespace {
+
+// Shape rules the stage entry points share; null when they hold.
+const char* stage_shape_error(int M, int width_a, int ncols, int top_k, int EM, int k_base, int k_dim,
+                              int block_size) {
+  if (M < 0 || EM < 0) return "M and EM must not be negative";
+  if (width_a <= 0 || ncols <= 0 || ncols % 64 != 0 || width_a % 8 != 0)
+    return "row widths must be positive, the output width a multiple of 64, the input width of 8";
+  if (top_k <= 0) return "top_k must be positive";
+  if (k_dim <= 0 || k_dim % 64 != 0 || k_base < 0 || k_base % 8 != 0 || k_base + k_dim > width_a)
+    return "the K slice must be a multiple of 64 wide, start at a multiple of 8 and lie inside the rows";
+  if (block_size <= 0 || block_size % 16 != 0 || EM % block_size != 0)
+    return "block_size must be a multiple of 16 and divide EM";
+  return nullptr;
+}
+
+int stage_launch_status(const char* who) {
+  note_launch_error(who);
+  return vk_last_error_code() == VK_OK ? VK_OK : VK_ERROR_INTERNAL;
+}
+
+}  // namespace
+
+int vk_hip_moe_gateup_preact(const uint16_t* A, const uint8_t* w13, const uint8_t* w13_scale,
+                             const int32_t* sorted_ids, const int32_t* expert_ids, float* gate_up,
+                             int M, int hidden, int ispp, int top_k, int EM, int k_base, int hidden_k,
+                             int block_size, void* stream) {
+  if (const char* why = stage_shape_error(M, hidden, ispp, top_k, EM, k_base, hidden_k, block_size))
+    return fail(VK_ERROR_INVALID_ARGUMENT, (std::string("vk_hip_moe_gateup_preact: ") + why).c_str());
+  if (M == 0 || EM == 0) return VK_OK;
+  if (A == nullptr || w13 == nullptr || w13_scale == nullptr || sorted_ids == nullptr ||
+      expert_ids == nullptr || gate_up == nullptr)
+    return fail(VK_ERROR_INVALID_ARGUMENT, "vk_hip_moe_gateup_preact: buffers must not be null");
+  vk_set_last_error(VK_OK, "");
+  vk::launch_moe_preact(0, A, w13, w13_scale, sorted_ids, expert_ids, gate_up, M, hidden, ispp, top_k, EM,
+                        k_base, hidden_k, block_size, static_cast<hipStream_t>(stream));
+  return stage_launch_status("vk_hip_moe_gateup_preact");
+}
+
+int vk_hip_moe_act_epilogue(const float* gate_up, const float* b13, uint16_t* act,
+                            const int32_t* sorted_ids, const int32_t* expert_ids, int M, int top_k,
+                            int EM, int ispp, float swiglu_limit, int activation, float beta,
+                            float linear_beta, int block_size, void* stream) {
+  if (M < 0 || EM < 0 || top_k <= 0 || ispp <= 0 || ispp % 4 != 0 || block_size <= 0 ||
+      EM % block_size != 0)
+    return fail(VK_ERROR_INVALID_ARGUMENT,
+                "vk_hip_moe_act_epilogue: M, EM non-negative, top_k positive, ispp a positive multiple "
+                "of 4, block_size a divisor of EM");
+  if (activation != VK_MOE_SWIGLU && activation != VK_MOE_SITU)
+    return fail(VK_ERROR_INVALID_ARGUMENT, "vk_hip_moe_act_epilogue: unknown activation");
+  if (M == 0 || EM == 0) return VK_OK;
+  if (gate_up == nullptr || act == nullptr || sorted_ids == nullptr || expert_ids == nullptr)
+    return fail(VK_ERROR_INVALID_ARGUMENT, "vk_hip_moe_act_epilogue: buffers must not be null");
+  vk_set_last_error(VK_OK, "");
+  vk::launch_moe_act_epilogue(gate_up, b13, act, sorted_ids, expert_ids, M, top_k, EM, ispp, block_size,
+                              swiglu_limit, activation, beta, linear_beta,
+                              static_cast<hipStream_t>(stream));
+  return stage_launch_status("vk_hip_moe_act_epilogue");
+}
+
+int vk_hip_moe_down_preact(const uint16_t* act, const uint8_t* w2, const uint8_t* w2_scale,
+                           const int32_t* sorted_ids, const int32_t* expert_ids, float* partial, int M,
+                           int ispp, int hidden, int top_k, int EM, int k_base, int ispp_k,
+                           int block_size, void* stream) {
+  if (const char* why = stage_shape_error(M, ispp, hidden, top_k, EM, k_base, ispp_k, block_size))
+    return fail(VK_ERROR_INVALID_ARGUMENT, (std::string("vk_hip_moe_down_preact: ") + why).c_str());
+  if (M == 0 || EM == 0) return VK_OK;
+  if (act == nullptr || w2 == nullptr || w2_scale == nullptr || sorted_ids == nullptr ||
+      expert_ids == nullptr || partial == nullptr)
+    return fail(VK_ERROR_INVALID_ARGUMENT, "vk_hip_moe_down_preact: buffers must not be null");
+  vk_set_last_error(VK_OK, "");
+  vk::launch_moe_preact(1, act, w2, w2_scale, sorted_ids, expert_ids, partial, M, ispp, hidden, top_k, EM,
+                        k_base, ispp_k, block_size, static_cast<hipStream_t>(stream));
+  return stage_launch_status("vk_hip_moe_down_preact");
+}
+
+int vk_hip_moe_combine(const float* partial, const float* b2, const float* topk_w_sorted,
+                       const int32_t* sorted_ids, const int32_t* expert_ids, float* out, int M,
+                       int hidden, int top_k, int EM, int block_size, void* workspace,
+                       size_t workspace_bytes, void* stream) {
+  if (M < 0 || EM < 0 || top_k <= 0 || hidden <= 0 || hidden % 4 != 0 || block_size <= 0 ||
+      EM % block_size != 0)
+    return fail(VK_ERROR_INVALID_ARGUMENT,
+                "vk_hip_moe_combine: M, EM non-negative, top_k positive, hidden a positive multiple of "
+                "4, block_size a divisor of EM");
+  if (M == 0 || EM == 0) return VK_OK;
+  if (partial == nullptr || topk_w_sorted == nullptr || sorted_ids == nullptr || expert_ids == nullptr ||
+      out == nullptr)
+    return fail(VK_ERROR_INVALID_ARGUMENT, "vk_hip_moe_combine: buffers must not be null");
+  if (workspace == nullptr || workspace_bytes < sizeof(int32_t) * (size_t)M * (size_t)top_k ||
+      (reinterpret_cast<uintptr_t>(workspace) & 3) != 0)
+    return fail(VK_ERROR_INVALID_ARGUMENT, "vk_hip_moe_combine: workspace must hold M * top_k int32 values");
+  vk_set_last_error(VK_OK, "");
+  vk::launch_moe_combine_sorted(partial, b2, topk_w_sorted, sorted_ids, expert_ids, out, M, hidden, top_k,
+                                EM, block_size, static_cast<int32_t*>(workspace),
+                                static_cast<hipStream_t>(stream));
+  return stage_launch_status("vk_hip_moe_combine");
+}
+
 size_t vk_hip_moe_prepack_bytes(int32_t num_experts, int32_t rows, int32_t K, int32_t stage) {
   if (stage != 0 && stage != 1) return 0;
   return vk::moe_prepack_bytes(num_experts, rows, K, stage);

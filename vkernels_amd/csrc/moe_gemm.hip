@@ -77,6 +77,12 @@ struct GemmArgs {
   // then sums each token's rows.
   float* y;
   int32_t* pos;
+  // Optional: the stage's linear part alone (tensor-parallel callers sum it over ranks
+  // before the epilogue): stage 0 stores preact[srow, c] = gate and preact[srow, ncols + c]
+  // = up of every routed sorted row (row width 2 ncols), stage 1 preact[srow, c] (width
+  // ncols); no bias, no activation, no routing weight.
+  float* preact;
+  int a_stride;             // elements between rows of A (K, or the full width of a K slice)
   int n_flat;               // M * top_k
   int top_k;
   int K;                    // hidden (stage 0) or ispp (stage 1)
@@ -123,6 +129,16 @@ template <int STAGE, int NT>
 __device__ __forceinline__ void epilogue_tile(const GemmArgs& p, int e, const f32x4 (&acc)[NT],
                                               const int (&col0)[NT], int flat, int srow, int lq,
                                               uint2* packed_out = nullptr) {
+  if (p.preact != nullptr) {  // the linear part alone, as fp32
+    const int width = STAGE == 0 ? 2 * p.ncols : p.ncols;
+    float* row = p.preact + (size_t)srow * (size_t)width;
+#pragma unroll
+    for (int t = 0; t < NT; ++t) {
+      const int c = col0[t] + 4 * lq + ((STAGE == 0 && t >= NT / 2) ? p.ncols : 0);
+      *reinterpret_cast<f32x4*>(row + c) = acc[t];
+    }
+    return;
+  }
   if (STAGE == 0) {
 #pragma unroll
     for (int t = 0; t < NT / 2; ++t) {
@@ -620,7 +636,7 @@ __global__ __launch_bounds__(64 * WAVES) void stream_resident_kernel(GemmArgs p)
         const uint16_t* src =
             p.A + (size_t)(st_flat >= 0 ? (STAGE == 0 ? st_flat / p.top_k
                                                       : run_row0 + tile * 16 + sj)
-                                        : 0) * (size_t)K;
+                                        : 0) * (size_t)p.a_stride;
         u32x4 v[kBatch];
 #pragma unroll
         for (int it = 0; it < kBatch; ++it) {
@@ -781,7 +797,7 @@ __global__ __launch_bounds__(64 * WAVES) void stream_resident_kernel(GemmArgs p)
         if (redo != 0ull) {
           const uint16_t* a_row = nullptr;
           if (my_flat >= 0)
-            a_row = p.A + (size_t)(STAGE == 0 ? my_flat / p.top_k : srow) * (size_t)K;
+            a_row = p.A + (size_t)(STAGE == 0 ? my_flat / p.top_k : srow) * (size_t)p.a_stride;
           while (redo != 0ull) {
             const int idx = __builtin_ctzll(redo);
             redo &= redo - 1ull;
@@ -906,7 +922,7 @@ __global__ __launch_bounds__(64 * kTileWaves, 2) void tile_gemm_kernel(GemmArgs 
   const int sr = tid >> 2, sd = tid & 3;
   const int sflat = row_flat[sr];
   const uint16_t* src =
-      p.A + (size_t)(sflat >= 0 ? (STAGE == 0 ? sflat / p.top_k : row0 + sr) : 0) * (size_t)K;
+      p.A + (size_t)(sflat >= 0 ? (STAGE == 0 ? sflat / p.top_k : row0 + sr) : 0) * (size_t)p.a_stride;
   const int sm = sr >> 4, sn = sr & 15;
 
   f32x4 acc[MT][NT];
@@ -1036,7 +1052,7 @@ __global__ __launch_bounds__(64 * kTileWaves, 2) void tile_gemm_kernel(GemmArgs 
     const int srow = row0 + m * 16 + ln;
     if (redo) {
       const uint16_t* a_row = nullptr;
-      if (flat >= 0) a_row = p.A + (size_t)(STAGE == 0 ? flat / p.top_k : srow) * (size_t)K;
+      if (flat >= 0) a_row = p.A + (size_t)(STAGE == 0 ? flat / p.top_k : srow) * (size_t)p.a_stride;
       exact_unit_global<NT>(w_rows, s_rows, a_row, K, lane, acc[m]);
     }
     uint2 packed[NT / 2] = {};
@@ -1422,7 +1438,7 @@ __global__ __launch_bounds__(64 * kWideWaves) void tile_wide_kernel(GemmArgs p) 
       const int srow = row0 + m * 16 + ln;
       if (redo) {
         const uint16_t* a_row = nullptr;
-        if (flat >= 0) a_row = p.A + (size_t)(STAGE == 0 ? flat / p.top_k : srow) * (size_t)K;
+        if (flat >= 0) a_row = p.A + (size_t)(STAGE == 0 ? flat / p.top_k : srow) * (size_t)p.a_stride;
         exact_unit_global<NT>(w_rows, s_rows, a_row, K, lane, acc[m]);
       }
       if (STAGE == 0) {
@@ -1714,6 +1730,7 @@ GemmArgs gateup_args(const FusedMoeArgs& a) {
   g.Ws = a.w13_scale;
   g.bias = a.b13;
   g.K = a.hidden;
+  g.a_stride = a.hidden;
   g.ncols = a.ispp;
   return g;
 }
@@ -1725,6 +1742,7 @@ GemmArgs down_args(const FusedMoeArgs& a) {
   g.Ws = a.w2_scale;
   g.bias = a.b2;
   g.K = a.ispp;
+  g.a_stride = a.ispp;
   g.ncols = a.hidden;
   return g;
 }
@@ -1766,6 +1784,36 @@ void launch_moe_gateup(const FusedMoeArgs& a, hipStream_t stream) {
   if (a.M <= 0 || a.EM <= 0 || a.block_size <= 0) return;
   const GemmArgs g = gateup_args(a);
   launch_stage<0>(g, plan_stage<0>(g), stream);
+}
+
+// The linear part of a stage for one K slice (tensor-parallel ranks; the reference's
+// moe_gateup_preact / moe_down_preact, src/c/vkernels/kernels/moe_fused.hpp:259-283):
+// rows of `a` are a_stride wide and the slice starts at column k_base of each; w / w_scale
+// are the rank's shard [E, rows, k_dim / 2] and [E, rows, k_dim / 32].  stage 0: rows =
+// 2 * ncols, preact [EM, 2 * ncols] (gate columns, then up columns); stage 1: rows =
+// ncols, preact [EM, ncols].  Routed rows are written, the others left as they are.
+// Runs the decode kernel or the plain tile kernel (no workspace, raw weights).
+void launch_moe_preact(int stage, const uint16_t* a, const uint8_t* w, const uint8_t* w_scale,
+                       const int32_t* sorted_ids, const int32_t* expert_ids, float* preact, int M,
+                       int a_stride, int ncols, int top_k, int EM, int k_base, int k_dim, int block_size,
+                       hipStream_t stream) {
+  if (M <= 0 || EM <= 0 || block_size <= 0) return;
+  GemmArgs g{};
+  g.A = a + k_base;
+  g.a_stride = a_stride;
+  g.W = w;
+  g.Ws = w_scale;
+  g.sorted_ids = sorted_ids;
+  g.expert_ids = expert_ids;
+  g.preact = preact;
+  g.n_flat = M * top_k;
+  g.top_k = top_k;
+  g.K = k_dim;
+  g.ncols = ncols;
+  g.num_blocks = EM / block_size;
+  g.block_size = block_size;
+  if (stage == 0) launch_stage<0>(g, plan_stage<0>(g), stream);
+  else launch_stage<1>(g, plan_stage<1>(g), stream);
 }
 
 // The second stage alone.  With a workspace (and packed weights) it runs as in the

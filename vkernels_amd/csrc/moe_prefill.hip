@@ -366,52 +366,6 @@ __global__ __launch_bounds__(256) void quant_rows_w4_kernel(const uint16_t* __re
   if (threadIdx.x == 0) row_bad[row] = (uint8_t)(bad != 0);
 }
 
-// pos[flat] = sorted row of every routed flat index (the others keep their -1).
-__global__ __launch_bounds__(256) void invert_sorted_ids_kernel(const int32_t* __restrict__ sorted_ids,
-                                                                int32_t* __restrict__ pos, int EM,
-                                                                int n_flat) {
-  const int r = blockIdx.x * blockDim.x + threadIdx.x;
-  if (r >= EM) return;
-  const int flat = sorted_ids[r];
-  if (flat >= 0 && flat < n_flat) pos[flat] = r;
-}
-
-// Routed combine in gather form (mxfp4_moe_scatter_reduce, moe_aux.cpp:265-285):
-// out[t, :] += partial[r, :] * topk_w[r] over the token's sorted rows r in ascending
-// order, which is the order the reference's loop over r adds them in; the product and
-// the sum are rounded separately, as there.  One thread per 4 columns.
-__global__ __launch_bounds__(256) void scatter_reduce_kernel(const float* __restrict__ partial,
-                                                             const float* __restrict__ topk_w,
-                                                             const int32_t* __restrict__ pos,
-                                                             float* __restrict__ out, int M, int width,
-                                                             int top_k) {
-  const int c = (blockIdx.x * blockDim.x + threadIdx.x) * 4;
-  if (c >= width) return;
-  for (int t = blockIdx.y; t < M; t += gridDim.y) {
-    f32x4* o = reinterpret_cast<f32x4*>(out + (size_t)t * (size_t)width + c);
-    f32x4 sum = *o;
-    int last = -1;
-    for (int s = 0; s < top_k; ++s) {   // the next larger sorted row of this token (top_k is small)
-      int r = 0x7FFFFFFF;
-      for (int j = 0; j < top_k; ++j) {
-        const int rj = pos[t * top_k + j];
-        if (rj > last && rj < r) r = rj;
-      }
-      if (r == 0x7FFFFFFF) break;
-      last = r;
-      const f32x4 p = *reinterpret_cast<const f32x4*>(partial + (size_t)r * (size_t)width + c);
-      const float w = topk_w[r];
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        float prod = p[i] * w;
-        asm volatile("" : "+v"(prod));   // the rounded product is a value of its own: no fused multiply-add
-        sum[i] += prod;
-      }
-    }
-    *o = sum;
-  }
-}
-
 // ---------------------------------------------------------------------------
 // Exact path of one unit for the 32 rows of one row tile: acc[t] = C[weight row of
 // tile t][activation row lane % 32] in the accumulator layout of the 32 x 32 MFMAs.
@@ -1061,18 +1015,6 @@ void launch_mxfp4_quant(const uint16_t* A, const int32_t* sorted_ids, uint8_t* p
   if (rows <= 0 || hidden <= 0) return;
   hipLaunchKernelGGL(mxfp4_quant_kernel, dim3(rows), dim3(256), 0, stream, A, sorted_ids, packed, scales,
                      hidden, top_k, n_flat);
-}
-
-void launch_mxfp4_scatter_reduce(const float* partial, const float* topk_w, const int32_t* sorted_ids,
-                                 float* out, int M, int width, int top_k, int EM, int32_t* pos,
-                                 hipStream_t stream) {
-  if (M <= 0 || width <= 0 || EM <= 0) return;
-  launch_fill_i32(pos, -1, M * top_k, stream);
-  hipLaunchKernelGGL(invert_sorted_ids_kernel, dim3((unsigned)((EM + 255) / 256)), dim3(256), 0, stream,
-                     sorted_ids, pos, EM, M * top_k);
-  const dim3 grid((unsigned)((width / 4 + 255) / 256), (unsigned)(M < 65535 ? M : 65535));
-  hipLaunchKernelGGL(scatter_reduce_kernel, grid, dim3(256), 0, stream, partial, topk_w, pos, out, M,
-                     width, top_k);
 }
 
 }  // namespace vk

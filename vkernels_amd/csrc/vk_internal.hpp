@@ -75,6 +75,18 @@ bool prepare_mx_kernels();
 // (sorted_ids null = token order), routed combine in gather form (pos: M * top_k ints).
 void launch_mxfp4_quant(const uint16_t* A, const int32_t* sorted_ids, uint8_t* packed, uint8_t* scales,
                         int rows, int hidden, int top_k, int n_flat, hipStream_t stream);
+void launch_moe_preact(int stage, const uint16_t* a, const uint8_t* w, const uint8_t* w_scale,
+                       const int32_t* sorted_ids, const int32_t* expert_ids, float* preact, int M,
+                       int a_stride, int ncols, int top_k, int EM, int k_base, int k_dim, int block_size,
+                       hipStream_t stream);
+void launch_moe_act_epilogue(const float* gate_up, const float* b13, uint16_t* act,
+                             const int32_t* sorted_ids, const int32_t* expert_ids, int M, int top_k, int EM,
+                             int ispp, int block_size, float swiglu_limit, int activation, float beta,
+                             float linear_beta, hipStream_t stream);
+void launch_moe_combine_sorted(const float* partial, const float* bias, const float* w_sorted,
+                               const int32_t* sorted_ids, const int32_t* expert_ids, float* out, int M,
+                               int width, int top_k, int EM, int block_size, int32_t* pos,
+                               hipStream_t stream);
 void launch_mxfp4_scatter_reduce(const float* partial, const float* topk_w, const int32_t* sorted_ids,
                                  float* out, int M, int width, int top_k, int EM, int32_t* pos,
                                  hipStream_t stream);
