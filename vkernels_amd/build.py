@@ -62,24 +62,37 @@ def _stale(src: Path, obj: Path) -> bool:
     return any(d.stat().st_mtime > obj.stat().st_mtime for d in deps)
 
 
-def build(verbose: bool = False, only_changed: bool = False) -> Path:
+def build(verbose: bool = False, only_changed: bool = False, out_dir: Path | None = None,
+          defines: tuple[str, ...] = ()) -> Path:
+    """Compiles every translation unit and links libvkernels_hip.so in the package
+    directory.  With out_dir the objects and the library go there instead (a build with
+    extra -D defines, say the profiling build, beside the product build, not over it)."""
     cc = hipcc()
-    OBJ.mkdir(exist_ok=True)
+    obj_dir = OBJ if out_dir is None else Path(out_dir) / "obj"
+    lib = LIB if out_dir is None else Path(out_dir) / LIB.name
+    obj_dir.mkdir(parents=True, exist_ok=True)
     jobs = []
     objects = []
     for name in SOURCES:
-        src, obj = CSRC / name, OBJ / (Path(name).stem + ".o")
+        src, obj = CSRC / name, obj_dir / (Path(name).stem + ".o")
         objects.append(str(obj))
         if only_changed and not _stale(src, obj):
             continue
-        jobs.append([cc, *FLAGS, f"-I{INCLUDE}", f"-I{CSRC}", "-x", "hip", "-c", str(src),
-                     "-o", str(obj)])
+        jobs.append([cc, *FLAGS, *(f"-D{d}" for d in defines), f"-I{INCLUDE}", f"-I{CSRC}", "-x", "hip",
+                     "-c", str(src), "-o", str(obj)])
     with ThreadPoolExecutor(max_workers=min(8, max(1, len(jobs)))) as pool:
         list(pool.map(lambda cmd: _run(cmd, verbose), jobs))
-    _run([cc, "--offload-arch=gfx950", "-shared", "-fPIC", "-fno-lto", *objects, "-o", str(LIB)],
+    _run([cc, "--offload-arch=gfx950", "-shared", "-fPIC", "-fno-lto", *objects, "-o", str(lib)],
          verbose)
-    return LIB
+    return lib
 
 
 if __name__ == "__main__":
-    print(build(verbose=True, only_changed="--changed" in sys.argv[1:]))
+    import argparse
+    ap = argparse.ArgumentParser(description="build libvkernels_hip.so for gfx950")
+    ap.add_argument("--changed", action="store_true", help="recompile only what is older than its sources")
+    ap.add_argument("--out", default=None, help="directory for the objects and the library (default: in tree)")
+    ap.add_argument("--define", action="append", default=[], help="extra -D for every translation unit")
+    ap.add_argument("--quiet", action="store_true")
+    a = ap.parse_args()
+    print(build(verbose=not a.quiet, only_changed=a.changed, out_dir=a.out, defines=tuple(a.define)))

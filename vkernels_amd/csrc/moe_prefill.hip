@@ -94,7 +94,26 @@ struct MxArgs {
   float swiglu_limit, beta, linear_beta;
   int activation;
   int units, col_groups, windows;
+#ifdef VK_MX_TRACE
+  unsigned long long* trace;  // 8 values per workgroup (see MX_TRACE)
+#endif
 };
+
+// Profiling build only (-DVK_MX_TRACE, `python -m vkernels_amd.build --define VK_MX_TRACE
+// --out DIR`): thread 0 of every workgroup stores the 100 MHz clock at a few points of the
+// kernel (0 entry, 1 rows listed, 2 K loop done, 3 barrier passed, 5 first row tile stored,
+// 4 epilogue done; 6, 7 = the hardware ids of its compute unit) into a buffer the caller
+// hands to vk_debug_mx_trace(buffer, stage), 8 values per workgroup;
+// vkernels_amd/mx_trace.py runs a workload on such a build and prints the phases.  Not
+// compiled into the library.
+#ifdef VK_MX_TRACE
+unsigned long long* g_mx_trace = nullptr;
+int g_mx_trace_stage = 1;
+#define MX_TRACE(slot_) \
+  do { if (p.trace != nullptr && threadIdx.x == 0) p.trace[(size_t)blockIdx.x * 8 + (slot_)] = wall_clock64(); } while (0)
+#else
+#define MX_TRACE(slot_) do {} while (0)
+#endif
 
 __host__ __device__ inline int mx_kp(int K) { return (K + 127) & ~127; }
 __host__ __device__ inline int mx_units(int stage, int ncols) {
@@ -497,6 +516,13 @@ __global__ __launch_bounds__(64 * kMxWaves) void tile_mx_kernel(MxArgs p) {
   const int slot = blockIdx.x >> 3;
   const int logical = ((slot >> 5) * 8 + (blockIdx.x & 7)) * 32 + (slot & 31);
   if (logical >= total) return;
+  MX_TRACE(0);
+#ifdef VK_MX_TRACE
+  if (p.trace != nullptr && threadIdx.x == 0) {
+    p.trace[(size_t)blockIdx.x * 8 + 6] = __builtin_amdgcn_s_getreg((4 << 0) | (0 << 6) | (31 << 11));  // HW_ID
+    p.trace[(size_t)blockIdx.x * 8 + 7] = __builtin_amdgcn_s_getreg((20 << 0) | (0 << 6) | (31 << 11)); // XCC_ID
+  }
+#endif
   const int window = logical / p.col_groups;
   const int colg = logical - window * p.col_groups;
 
@@ -540,6 +566,7 @@ __global__ __launch_bounds__(64 * kMxWaves) void tile_mx_kernel(MxArgs p) {
     const int hi = seg_hi[1] >= 0 ? 64 + seg_hi[1] : seg_hi[0];
     const int n_live = (hi + 32) >> 5;  // row tiles of 32 up to the last routed row
     if (n_live == 0) return;            // uniform
+    MX_TRACE(1);
     const bool slow = (seg_bad[0] | seg_bad[1]) != 0 ||
                       (has_unit && p.Wflags[(size_t)e * p.units + unit] != 0);  // uniform per wavefront
 
@@ -721,19 +748,46 @@ __global__ __launch_bounds__(64 * kMxWaves) void tile_mx_kernel(MxArgs p) {
     else if (n_live == 3) k_loop(IntC<3>{});
     else if (n_live == 2 || TERMS == 1) k_loop(IntC<2>{});
     else if constexpr (TERMS > 1) k_loop(IntC<1>{});
+    MX_TRACE(2);
     __syncthreads();
+    MX_TRACE(3);
 
     if (STAGE == 1 && colg == 0 && tid < n_rows && row_flat[tid] >= 0) p.pos[row_flat[tid]] = row0 + tid;
     if (!has_unit) return;
 
     // ---- epilogue: lane (ln, hh) holds, of activation row 32 m + ln, the weight rows
-    // 8 (i / 4) + 4 hh + i % 4 of each tile ----
+    // 8 (i / 4) + 4 hh + i % 4 of each tile: a few columns of 32 different rows.  Stored
+    // like that, every store instruction touches 64 cache lines; instead the values of 32
+    // rows go through a staging area of the wavefront's own in the ring (free after the
+    // barrier above) and leave as whole lines: 4 rows x 256 bytes (8 rows x 128 bytes in
+    // stage 0) per store instruction ----
+    uint8_t* stage_lds = reinterpret_cast<uint8_t*>(mx_lds) + wave * (R * kSlotBytes / kMxWaves);
+    auto wave_fence = [] {  // LDS operations of a wavefront execute in order; this keeps the compiler's too
+      __asm__ volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    };
+    // The routing weights of this lane's four rows, loaded and waited for here: a load
+    // still pending when the stores begin makes every later wait for it (at the joins of
+    // the branches below) a wait for the stores issued in between, a round trip to memory
+    // per group of stores.
+    float w_row[4] = {0.f, 0.f, 0.f, 0.f};
+    if (STAGE == 1) {
+#pragma unroll
+      for (int m = 0; m < 4; ++m) {
+        const int f = m < n_live ? row_flat[m * 32 + ln] : -1;
+        if (f >= 0) w_row[m] = p.topk_w[f];
+      }
+      __asm__ volatile("s_waitcnt vmcnt(0)"
+                       : "+v"(w_row[0]), "+v"(w_row[1]), "+v"(w_row[2]), "+v"(w_row[3])
+                       :
+                       : "memory");
+    }
 #pragma unroll
     for (int m = 0; m < 4; ++m) {
       if (m >= n_live) break;
       f32x16 (&tile)[4] = acc[m];
       const int flat = row_flat[m * 32 + ln];
       const int srow = row0 + m * 32 + ln;
+      const unsigned long long routed = __ballot(flat >= 0);  // bit r (< 32): row 32 m + r is routed
       if (slow) {
         const uint16_t* a_row = nullptr;
         const uint8_t* q_row = nullptr;
@@ -744,46 +798,97 @@ __global__ __launch_bounds__(64 * kMxWaves) void tile_mx_kernel(MxArgs p) {
         }
         exact_unit_mx<STAGE>(p, e, unit, a_row, q_row, lane, tile);
       }
-      if (flat < 0) continue;
       if (STAGE == 0) {
-        const float* bias = p.bias != nullptr ? p.bias + (size_t)e * (size_t)(2 * p.ncols) : nullptr;
+        constexpr int kPitch = 144;  // 64 bf16 of a row + 16: rows stay 16-byte aligned
+        // 128 activation values per lane and row tile: the plain SwiGLU (no bias, no
+        // clamp), which is what serving runs, gets a loop of its own without a branch per
+        // value; the same act_value with its parameters known at compile time.
+        auto act_rows = [&](auto plain_c) {
+          constexpr bool kPlain = decltype(plain_c)::value != 0;
+          const float* bias = p.bias != nullptr ? p.bias + (size_t)e * (size_t)(2 * p.ncols) : nullptr;
 #pragma unroll
-        for (int tp = 0; tp < 2; ++tp)
+          for (int tp = 0; tp < 2; ++tp)
 #pragma unroll
-          for (int rg = 0; rg < 4; ++rg) {
-            const int col = unit * 64 + tp * 32 + rg * 8 + hh * 4;
-            uint32_t packed[2];
+            for (int rg = 0; rg < 4; ++rg) {
+              const int cl = tp * 32 + rg * 8 + hh * 4;  // column within the unit's 64
+              const int col = unit * 64 + cl;
+              uint32_t packed[2];
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {
-              float g = tile[tp][rg * 4 + i], u = tile[tp + 2][rg * 4 + i];
-              if (bias != nullptr) {
-                g += bias[col + i];
-                u += bias[p.ncols + col + i];
+              for (int i = 0; i < 4; ++i) {
+                float g = tile[tp][rg * 4 + i], u = tile[tp + 2][rg * 4 + i];
+                float a;
+                if constexpr (kPlain) {
+                  a = act_value(0, g, u, 0.0f, 0.0f, 0.0f);
+                } else {
+                  if (bias != nullptr) {
+                    g += bias[col + i];
+                    u += bias[p.ncols + col + i];
+                  }
+                  a = act_value(p.activation, g, u, p.swiglu_limit, p.beta, p.linear_beta);
+                }
+                const uint32_t v = f32_to_bf16_bits(a);
+                if (i & 1) packed[i >> 1] |= v << 16;
+                else packed[i >> 1] = v;
               }
-              const uint32_t v = f32_to_bf16_bits(
-                  act_value(p.activation, g, u, p.swiglu_limit, p.beta, p.linear_beta));
-              if (i & 1) packed[i >> 1] |= v << 16;
-              else packed[i >> 1] = v;
+              *reinterpret_cast<uint2*>(stage_lds + ln * kPitch + cl * 2) = make_uint2(packed[0], packed[1]);
             }
-            *reinterpret_cast<uint2*>(p.act + (size_t)srow * (size_t)p.ncols + col) =
-                make_uint2(packed[0], packed[1]);
-          }
+        };
+        if (flat >= 0) {
+          if (p.activation == 0 && !(p.swiglu_limit > 0.0f) && p.bias == nullptr) act_rows(IntC<1>{});
+          else act_rows(IntC<0>{});
+        }
+        wave_fence();
+        u32x4 v[4];  // all the reads, one wait, then the stores: 8 rows x 128 bytes per instruction
+#pragma unroll
+        for (int pass = 0; pass < 4; ++pass)
+          v[pass] = *reinterpret_cast<const u32x4*>(stage_lds + (pass * 8 + (lane >> 3)) * kPitch + (lane & 7) * 16);
+        wave_fence();
+#pragma unroll
+        for (int pass = 0; pass < 4; ++pass) {
+          const int r = pass * 8 + (lane >> 3), piece = lane & 7;
+          if ((routed >> r) & 1ull)
+            *reinterpret_cast<u32x4*>(p.act + (size_t)(row0 + m * 32 + r) * (size_t)p.ncols + unit * 64 +
+                                      piece * 8) = v[pass];
+        }
       } else {
-        const float w = p.topk_w[flat];
-        float* yrow = p.y + (size_t)srow * (size_t)p.ncols;
+        constexpr int kPitch = 272;  // 64 floats of a row + 16 bytes
+        const float w = w_row[m];
 #pragma unroll
-        for (int t = 0; t < 4; ++t)
+        for (int tp = 0; tp < 2; ++tp) {  // tiles 2 tp, 2 tp + 1: 64 columns
+          if (flat >= 0) {
 #pragma unroll
-          for (int rg = 0; rg < 4; ++rg) {
-            const int col = unit * kMxUnitRows + t * 32 + rg * 8 + hh * 4;
-            if (col >= p.ncols) continue;  // the last unit may be ragged (ncols is a multiple of 64)
-            f32x4 v = {tile[t][rg * 4], tile[t][rg * 4 + 1], tile[t][rg * 4 + 2], tile[t][rg * 4 + 3]};
-            if (p.bias != nullptr)
-              v += *reinterpret_cast<const f32x4*>(p.bias + (size_t)e * (size_t)p.ncols + col);
-            *reinterpret_cast<f32x4*>(yrow + col) = v * w;
+            for (int tl = 0; tl < 2; ++tl)
+#pragma unroll
+              for (int rg = 0; rg < 4; ++rg) {
+                const int t = 2 * tp + tl;
+                const int cl = tl * 32 + rg * 8 + hh * 4;
+                const int col = unit * kMxUnitRows + tp * 64 + cl;
+                f32x4 v = {tile[t][rg * 4], tile[t][rg * 4 + 1], tile[t][rg * 4 + 2], tile[t][rg * 4 + 3]};
+                if (p.bias != nullptr && col < p.ncols)
+                  v += *reinterpret_cast<const f32x4*>(p.bias + (size_t)e * (size_t)p.ncols + col);
+                *reinterpret_cast<f32x4*>(stage_lds + ln * kPitch + cl * 4) = v * w;
+              }
           }
+          wave_fence();
+          f32x4 v[8];  // all the reads, one wait, then the stores: 4 rows x 256 bytes per instruction
+#pragma unroll
+          for (int pass = 0; pass < 8; ++pass)
+            v[pass] = *reinterpret_cast<const f32x4*>(stage_lds + (pass * 4 + (lane >> 4)) * kPitch + (lane & 15) * 16);
+          wave_fence();
+          const int col = unit * kMxUnitRows + tp * 64 + (lane & 15) * 4;
+          if (col < p.ncols) {  // (the last unit may be ragged: ncols is a multiple of 64)
+#pragma unroll
+            for (int pass = 0; pass < 8; ++pass) {
+              const int r = pass * 4 + (lane >> 4);
+              if ((routed >> r) & 1ull)
+                *reinterpret_cast<f32x4*>(p.y + (size_t)(row0 + m * 32 + r) * (size_t)p.ncols + col) = v[pass];
+            }
+          }
+        }
       }
+      if (m == 0) MX_TRACE(5);
     }
+    MX_TRACE(4);
   };
 
   const int total_rows = p.num_blocks * p.block_size;
@@ -820,6 +925,9 @@ void launch_mx_stage_t(MxArgs g, hipStream_t stream) {
   g.windows = (g.num_blocks * g.block_size + win - 1) / win;
   const long long total = (long long)g.col_groups * g.windows;
   const unsigned grid = (unsigned)((total + 255) / 256 * 256);  // whole chunks of 32 tiles for each of 8 XCDs
+#ifdef VK_MX_TRACE
+  g.trace = STAGE == g_mx_trace_stage ? g_mx_trace : nullptr;
+#endif
   hipLaunchKernelGGL((tile_mx_kernel<STAGE, TERMS>), dim3(grid), dim3(64 * kMxWaves),
                      kMxRing * kMxRows * TERMS * 128, stream, g);
 }
@@ -1016,5 +1124,12 @@ void launch_mxfp4_quant(const uint16_t* A, const int32_t* sorted_ids, uint8_t* p
   hipLaunchKernelGGL(mxfp4_quant_kernel, dim3(rows), dim3(256), 0, stream, A, sorted_ids, packed, scales,
                      hidden, top_k, n_flat);
 }
+
+#ifdef VK_MX_TRACE
+extern "C" void vk_debug_mx_trace(void* buffer, int stage) {
+  g_mx_trace = static_cast<unsigned long long*>(buffer);
+  g_mx_trace_stage = stage;
+}
+#endif
 
 }  // namespace vk
