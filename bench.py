@@ -56,6 +56,8 @@ def parse_args():
     ap.add_argument("--split-terms", type=int, default=3, choices=(2, 3),
                     help="FP6 terms per activation on the prepacked path")
     ap.add_argument("--no-prepack", action="store_true", help="raw weights only, also for prefill sizes")
+    ap.add_argument("--no-workspace", action="store_true",
+                    help="call the reference's own symbol (no workspace, raw weights)")
     ap.add_argument("--no-modes", action="store_true",
                     help="skip the prefill record's other arithmetic modes (2 <-> 3 terms, W4A4)")
     ap.add_argument("--w4a4", action="store_true", help="top-level record in the W4A4 mode (prefill sizes)")
@@ -150,7 +152,7 @@ def run_workload(args, workload, steps, warmup, prepack, split_terms=None, w4a4=
     dev = torch.device("cuda", 0)
     H, I, k = cfg.H, cfg.I, cfg.top_k
     prefill = T * k > 512  # the library's own split between its decode and tile kernels
-    prepack = prepack and prefill
+    prepack = prepack and prefill and not args.no_workspace
     terms = split_terms or args.split_terms
 
     per_set = synth.algorithmic_bytes(H, I, cfg.E, k, 0, cfg.E)
@@ -163,6 +165,8 @@ def run_workload(args, workload, steps, warmup, prepack, split_terms=None, w4a4=
         w = synth.make_weights(cfg.E, H, I, seed + 7919 * s, device=dev)
         experts.append(ve.FusedExperts(w.w13, w.w13_scale, w.w2, w.w2_scale, prepack=prepack,
                                        split_terms=terms, w4a4=w4a4 and prepack))
+        if args.no_workspace:
+            experts[-1].use_workspace = False
     A_bits = synth.make_activations(T, H, seed)
     logits_np = synth.make_logits(cfg.logits, T, cfg.E, seed, A_bits, H)
     A = torch.from_numpy(A_bits.view(np.int16)).view(torch.bfloat16).to(dev)
@@ -185,7 +189,9 @@ def run_workload(args, workload, steps, warmup, prepack, split_terms=None, w4a4=
         if prefill:
             events[0].record()
             events[1].record()
-            fe.fused_call(A, ids, w, sids, eids, max_em, bs, out, overwrite=True)
+            if args.no_workspace:
+                out.zero_()
+            fe.fused_call(A, ids, w, sids, eids, max_em, bs, out, overwrite=not args.no_workspace)
             events[2].record()
             return
         out.zero_()
@@ -241,6 +247,9 @@ def run_workload(args, workload, steps, warmup, prepack, split_terms=None, w4a4=
             kernel = (f"vk_hip_fused_moe_mxfp4_prepacked (split_rows_fp6_kernel<{terms}> x2 + "
                       f"tile_mx_kernel<0,{terms}> + tile_mx_kernel<1,{terms}> + combine_kernel)")
             issued = float(terms)  # FP4-rate MFMAs per algorithmic product
+        elif args.no_workspace:
+            kernel = "vk_hip_fused_moe_mxfp4 (clear of out + tile_gemm_kernel<0> + tile_gemm_kernel<1>, atomics)"
+            issued = 4.0
         else:
             kernel = ("vk_hip_fused_moe_mxfp4_ex (split_rows_kernel + tile_wide_kernel<0> + "
                       "tile_wide_kernel<1> + combine_kernel)")

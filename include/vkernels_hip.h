@@ -242,8 +242,8 @@ int vk_hip_init(void);
  * A launch shape is four ints {variant, wavefronts, tiles, depth}.
  * vk_hip_moe_tile_candidates writes up to `capacity` shapes that stage 0
  * (gate/up) or 1 (down) can be launched at and returns how many there are.
- * vk_hip_moe_tile_query writes the shape a call of this problem size (blocks =
- * EM / block_size) would be planned with and returns 1 when it comes from the tuning store, 0 from the
+ * vk_hip_moe_tile_query writes the shape a call of this problem size would be
+ * planned with and returns 1 when it comes from the tuning store, 0 from the
  * compiled-in rules (a launcher still falls back to the tile kernels where a
  * shape does not fit the device's LDS).
  * vk_hip_moe_tile_set puts a record for (stage, K, ncols, bucket of n_flat)
@@ -257,7 +257,7 @@ int vk_hip_init(void);
  */
 int vk_hip_moe_default_block_size(int M, int top_k);
 int vk_hip_moe_tile_candidates(int stage, int* shapes, int capacity);
-int vk_hip_moe_tile_query(int stage, int K, int ncols, int n_flat, int blocks, int* shape);
+int vk_hip_moe_tile_query(int stage, int K, int ncols, int n_flat, int* shape);
 int vk_hip_moe_tile_set(int stage, int K, int ncols, int n_flat, const int* shape);
 int vk_hip_moe_tuning_load(const char* dir);
 size_t vk_hip_moe_tuning_dump(char* buf, size_t capacity);

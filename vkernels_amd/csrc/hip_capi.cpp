@@ -439,10 +439,10 @@ int vk_hip_moe_tile_candidates(int stage, int* shapes, int capacity) {
   return count;
 }
 
-int vk_hip_moe_tile_query(int stage, int K, int ncols, int n_flat, int blocks, int* shape) {
+int vk_hip_moe_tile_query(int stage, int K, int ncols, int n_flat, int* shape) {
   vk::MoeTile t;
   const bool stored = vk::moe_tuning_find(stage, K, ncols, n_flat, &t);
-  if (!stored) t = vk::pick_moe_tile(n_flat, K, ncols, stage, blocks);
+  if (!stored) t = vk::pick_moe_tile(n_flat, K, ncols, stage);
   if (shape != nullptr) {
     shape[0] = t.variant; shape[1] = t.waves; shape[2] = t.nt; shape[3] = t.depth;
   }

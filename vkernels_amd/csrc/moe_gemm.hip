@@ -1596,7 +1596,7 @@ StagePlan plan_stage(const GemmArgs& g) {
   // a record of the tuning store first, then the compiled-in rules
   MoeTile tile;
   if (!moe_tuning_find(STAGE, g.K, g.ncols, g.n_flat, &tile))
-    tile = pick_moe_tile(g.n_flat, g.K, g.ncols, STAGE, g.num_blocks);
+    tile = pick_moe_tile(g.n_flat, g.K, g.ncols, STAGE);
   StagePlan pl;
   pl.variant = tile.variant;
   pl.nt = tile.nt;

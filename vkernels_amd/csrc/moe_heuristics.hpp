@@ -67,16 +67,15 @@ constexpr int kMoeDecodeMaxRows = 512;
 // One row of the decision table: the first row whose bounds hold decides.
 struct MoeTileRule {
   int stage;
-  int max_rows;    // n_flat <= max_rows
-  int max_k;       // K <= max_k
-  int min_blocks;  // blocks of the call (EM / block_size, an upper bound of the runs) >= min_blocks
+  int max_rows;  // n_flat <= max_rows
+  int max_k;     // K <= max_k
   MoeTile tile;
 };
 
 // n_flat = tokens * top_k routed rows in the call, K / ncols the GEMM's reduction and
-// output widths, stage 0 = gate/up, 1 = down, blocks = EM / block_size.  The number of
-// experts is not known to the launcher: the split between the kernel families is on the
-// routed rows alone, and `blocks` stands for the number of runs where that matters.
+// output widths, stage 0 = gate/up, 1 = down.  Neither the number of experts nor the
+// number of runs is known to the launcher (EM may be the caller's upper bound), so the
+// split between the kernel families is on the routed rows alone.
 //
 // Decode: the units of a run are shared by (compute units / runs) workgroups of 8
 // wavefronts, so a stage wants at least ~3 units per wavefront or the last round leaves
@@ -86,24 +85,25 @@ struct MoeTileRule {
 // Rows (each from the sweep table profiles/moe_decode_tile_sweep.md):
 //  - K <= 1024: a unit is a few steps long, and steps in flight past its end are
 //    wasted loads: the shallowest pipelines (256x512x8x2: 12.1 against 13.8 us);
-//  - many runs (more than 64 blocks: 2880x2880x128x4 from T = 32): each workgroup has a
-//    run to itself and few units, and 4 wavefronts with 8 steps in flight each keep more
-//    bytes in flight per wavefront (157 against 165 us, 214 against 229 us);
 //  - 3072 < K <= 4096 (4096x1536x64x6 gate/up): the rows of a pass fit LDS and registers
-//    only with 4 wavefronts per workgroup;
-//  - otherwise (8, 2, 4) / (8, 1, 8), within 2 % of the best of every other point swept.
-inline MoeTile pick_moe_tile(int n_flat, int K, int ncols, int stage, int blocks) {
+//    only with 4 wavefronts per workgroup (41 against 69 us at T = 1, 107 against 176 us
+//    at T = 32 for the tile kernel, which is what runs beyond K = 4096);
+//  - otherwise (8, 2, 4) / (8, 1, 8), within 2 % of the best of every other point swept
+//    but one: with 128 experts and 32 tokens or more, uniformly routed, (4, 2, 8) is 3 to
+//    7 % faster for gate/up; the number of runs that makes it so is not known here, and
+//    with skewed routing (27 active experts of 128) the same shape is 20 % slower, so
+//    that choice is left to the tuning store.
+inline MoeTile pick_moe_tile(int n_flat, int K, int ncols, int stage) {
   (void)ncols;  // no swept point separates on it: the units per wavefront follow from it, not the shape
   static const MoeTileRule rules[] = {
-      {0, kMoeDecodeMaxRows, 1024, 0, {kMoeVariantResident, 8, 2, 2}},
-      {0, kMoeDecodeMaxRows, 3072, 65, {kMoeVariantResident, 4, 2, 8}},
-      {0, kMoeDecodeMaxRows, 3072, 0, {kMoeVariantResident, 8, 2, 4}},
-      {0, kMoeDecodeMaxRows, 4096, 0, {kMoeVariantResident, 4, 2, 8}},
-      {1, kMoeDecodeMaxRows, 1024, 0, {kMoeVariantResident, 8, 1, 4}},
-      {1, kMoeDecodeMaxRows, 3072, 0, {kMoeVariantResident, 8, 1, 8}},
+      {0, kMoeDecodeMaxRows, 1024, {kMoeVariantResident, 8, 2, 2}},
+      {0, kMoeDecodeMaxRows, 3072, {kMoeVariantResident, 8, 2, 4}},
+      {0, kMoeDecodeMaxRows, 4096, {kMoeVariantResident, 4, 2, 8}},
+      {1, kMoeDecodeMaxRows, 1024, {kMoeVariantResident, 8, 1, 4}},
+      {1, kMoeDecodeMaxRows, 3072, {kMoeVariantResident, 8, 1, 8}},
   };
   for (const MoeTileRule& r : rules)
-    if (r.stage == stage && n_flat <= r.max_rows && K <= r.max_k && blocks >= r.min_blocks) return r.tile;
+    if (r.stage == stage && n_flat <= r.max_rows && K <= r.max_k) return r.tile;
   return MoeTile{kMoeVariantLds, 4, 4, 0};
 }
 

@@ -88,9 +88,8 @@ def main() -> None:
             ids, tw = fe_sets[0].route(logits, k, True)
             out = torch.zeros((T, H), dtype=torch.float32, device=dev)
             bs = ve.default_block_size(T, k)
-            blocks = fe_sets[0].align(ids, bs)[3] // bs
             for stage, K, ncols in ((0, H, I), (1, I, H)):
-                rule, _ = ve.moe_tile_query(stage, K, ncols, T * k, blocks)
+                rule, _ = ve.moe_tile_query(stage, K, ncols, T * k)
                 times = {}
                 for cand in ve.moe_tile_candidates(stage):
                     ve.moe_tile_set(stage, K, ncols, T * k, cand)

@@ -355,15 +355,13 @@ def moe_tile_candidates(stage: int, lib=None) -> list[tuple[int, int, int, int]]
     return [tuple(buf[4 * i:4 * i + 4]) for i in range(n)]
 
 
-def moe_tile_query(stage: int, K: int, ncols: int, n_flat: int, blocks: int | None = None, lib=None):
-    """((variant, wavefronts, tiles, depth), from_store) a call of this size is planned
-    with; blocks = EM / block_size (default: one block per 16 routed rows)."""
+def moe_tile_query(stage: int, K: int, ncols: int, n_flat: int, lib=None):
+    """((variant, wavefronts, tiles, depth), from_store) a call of this size is planned with."""
     lib = load_libvkernels_hip() if lib is None else lib
     fn = lib.vk_hip_moe_tile_query
-    fn.restype, fn.argtypes = _I, [_I, _I, _I, _I, _I, _P]
+    fn.restype, fn.argtypes = _I, [_I, _I, _I, _I, _P]
     buf = (ctypes.c_int * 4)()
-    blocks = (n_flat + 15) // 16 if blocks is None else blocks
-    stored = int(fn(stage, K, ncols, n_flat, blocks, buf))
+    stored = int(fn(stage, K, ncols, n_flat, buf))
     return tuple(buf), bool(stored)
 
 
