@@ -501,6 +501,7 @@ __global__ __launch_bounds__(64 * kMxWaves) void tile_mx_kernel(MxArgs p) {
   typedef __attribute__((address_space(3))) void* lds_ptr;
   extern __shared__ u32x4 mx_lds[];
   __shared__ int row_flat[kMxRows];
+  __shared__ float row_w[kMxRows];  // stage 1: the routing weight of every row (0 where none is routed)
   __shared__ int seg_hi[2];   // highest routed row index among rows 0..63 / 64..127 (or -1)
   __shared__ int seg_bad[2];  // a routed row of the half is outside the split's range
 
@@ -540,6 +541,11 @@ __global__ __launch_bounds__(64 * kMxWaves) void tile_mx_kernel(MxArgs p) {
   constexpr int kRowOps = 4 * TERMS;
   constexpr int kOps = kRowOps + 9;
 
+  // the rows of this workgroup's window
+  const int total_rows = p.num_blocks * p.block_size;
+  const int win = mx_window_rows(p.block_size);
+  const int win_end = min(window * win + win, total_rows);
+
   auto segment = [&](const int row0_, const int n_rows_, const int e_) {
     // uniform by construction; said so, so that addresses built on them stay scalar
     const int row0 = __builtin_amdgcn_readfirstlane(row0_);
@@ -555,6 +561,7 @@ __global__ __launch_bounds__(64 * kMxWaves) void tile_mx_kernel(MxArgs p) {
       row_flat[tid] = f;
       int bad = 0;
       if (f >= 0) bad = p.row_bad[STAGE == 0 ? f / p.top_k : row0 + tid];
+      if (STAGE == 1) row_w[tid] = f >= 0 ? p.topk_w[f] : 0.f;  // (in flight together with the flag)
       const unsigned long long routed = __ballot(f >= 0);
       const unsigned long long any_bad = __ballot(bad != 0);
       if (lane == 0) {
@@ -765,22 +772,6 @@ __global__ __launch_bounds__(64 * kMxWaves) void tile_mx_kernel(MxArgs p) {
     auto wave_fence = [] {  // LDS operations of a wavefront execute in order; this keeps the compiler's too
       __asm__ volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
     };
-    // The routing weights of this lane's four rows, loaded and waited for here: a load
-    // still pending when the stores begin makes every later wait for it (at the joins of
-    // the branches below) a wait for the stores issued in between, a round trip to memory
-    // per group of stores.
-    float w_row[4] = {0.f, 0.f, 0.f, 0.f};
-    if (STAGE == 1) {
-#pragma unroll
-      for (int m = 0; m < 4; ++m) {
-        const int f = m < n_live ? row_flat[m * 32 + ln] : -1;
-        if (f >= 0) w_row[m] = p.topk_w[f];
-      }
-      __asm__ volatile("s_waitcnt vmcnt(0)"
-                       : "+v"(w_row[0]), "+v"(w_row[1]), "+v"(w_row[2]), "+v"(w_row[3])
-                       :
-                       : "memory");
-    }
 #pragma unroll
     for (int m = 0; m < 4; ++m) {
       if (m >= n_live) break;
@@ -851,39 +842,58 @@ __global__ __launch_bounds__(64 * kMxWaves) void tile_mx_kernel(MxArgs p) {
                                       piece * 8) = v[pass];
         }
       } else {
+        // A wavefront runs alone on its SIMD, so every branch and every predicate of this
+        // code is paid in full; it is therefore specialised, per row tile, on what is
+        // uniform: a bias or none, and whether the tile's 32 rows all belong to this
+        // workgroup's window.  Then rows that are not routed are stored like the others
+        // (with a routing weight of zero): nothing reads them (pos never points at them),
+        // and a later segment of this window, if they are its rows, overwrites them.
         constexpr int kPitch = 272;  // 64 floats of a row + 16 bytes
-        const float w = w_row[m];
+        // (from LDS, put there when the rows were listed: a load from memory still pending
+        // when the stores begin makes every later wait for it a wait for those stores)
+        const float w = row_w[m * 32 + ln];
+        auto store_rows = [&](auto bias_c, auto guard_c) {
+          constexpr bool kBias = decltype(bias_c)::value != 0, kGuard = decltype(guard_c)::value != 0;
 #pragma unroll
-        for (int tp = 0; tp < 2; ++tp) {  // tiles 2 tp, 2 tp + 1: 64 columns
-          if (flat >= 0) {
+          for (int tp = 0; tp < 2; ++tp) {  // tiles 2 tp, 2 tp + 1: 64 columns
+            const int col0 = unit * kMxUnitRows + tp * 64;
+            if (col0 >= p.ncols) break;  // uniform: the last unit may be ragged (ncols is a multiple of 64)
 #pragma unroll
             for (int tl = 0; tl < 2; ++tl)
 #pragma unroll
               for (int rg = 0; rg < 4; ++rg) {
                 const int t = 2 * tp + tl;
                 const int cl = tl * 32 + rg * 8 + hh * 4;
-                const int col = unit * kMxUnitRows + tp * 64 + cl;
                 f32x4 v = {tile[t][rg * 4], tile[t][rg * 4 + 1], tile[t][rg * 4 + 2], tile[t][rg * 4 + 3]};
-                if (p.bias != nullptr && col < p.ncols)
-                  v += *reinterpret_cast<const f32x4*>(p.bias + (size_t)e * (size_t)p.ncols + col);
+                if constexpr (kBias)
+                  v += *reinterpret_cast<const f32x4*>(p.bias + (size_t)e * (size_t)p.ncols + col0 + cl);
                 *reinterpret_cast<f32x4*>(stage_lds + ln * kPitch + cl * 4) = v * w;
               }
-          }
-          wave_fence();
-          f32x4 v[8];  // all the reads, one wait, then the stores: 4 rows x 256 bytes per instruction
+            wave_fence();
+            f32x4 v[8];  // all the reads, one wait, then the stores: 4 rows x 256 bytes per instruction
 #pragma unroll
-          for (int pass = 0; pass < 8; ++pass)
-            v[pass] = *reinterpret_cast<const f32x4*>(stage_lds + (pass * 4 + (lane >> 4)) * kPitch + (lane & 15) * 16);
-          wave_fence();
-          const int col = unit * kMxUnitRows + tp * 64 + (lane & 15) * 4;
-          if (col < p.ncols) {  // (the last unit may be ragged: ncols is a multiple of 64)
+            for (int pass = 0; pass < 8; ++pass)
+              v[pass] = *reinterpret_cast<const f32x4*>(stage_lds + (pass * 4 + (lane >> 4)) * kPitch + (lane & 15) * 16);
+            wave_fence();
+            float* dst = p.y + (size_t)(row0 + m * 32 + (lane >> 4)) * (size_t)p.ncols + col0 + (lane & 15) * 4;
 #pragma unroll
             for (int pass = 0; pass < 8; ++pass) {
-              const int r = pass * 4 + (lane >> 4);
-              if ((routed >> r) & 1ull)
-                *reinterpret_cast<f32x4*>(p.y + (size_t)(row0 + m * 32 + r) * (size_t)p.ncols + col) = v[pass];
+              if constexpr (kGuard) {
+                if ((routed >> (pass * 4 + (lane >> 4))) & 1ull) *reinterpret_cast<f32x4*>(dst) = v[pass];
+              } else {
+                *reinterpret_cast<f32x4*>(dst) = v[pass];
+              }
+              dst += 4 * (size_t)p.ncols;
             }
           }
+        };
+        const bool inside = row0 + m * 32 + 32 <= win_end;  // uniform
+        if (p.bias == nullptr) {
+          if (inside) store_rows(IntC<0>{}, IntC<0>{});
+          else store_rows(IntC<0>{}, IntC<1>{});
+        } else {
+          if (inside) store_rows(IntC<1>{}, IntC<0>{});
+          else store_rows(IntC<1>{}, IntC<1>{});
         }
       }
       if (m == 0) MX_TRACE(5);
@@ -891,10 +901,7 @@ __global__ __launch_bounds__(64 * kMxWaves) void tile_mx_kernel(MxArgs p) {
     MX_TRACE(4);
   };
 
-  const int total_rows = p.num_blocks * p.block_size;
-  const int win = mx_window_rows(p.block_size);
   int row = window * win;
-  const int win_end = min(row + win, total_rows);
   while (row < win_end) {  // uniform
     const int e = p.expert_ids[row / p.block_size];
     int seg_end = min(win_end, (row / p.block_size + 1) * p.block_size);
