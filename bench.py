@@ -53,8 +53,9 @@ def parse_args():
     ap.add_argument("--workload", default="c1:64", help="config:T of the top-level record, e.g. c1:64, c2:512")
     ap.add_argument("--prefill", default="c3:16384",
                     help="config:T of the `prefill` record (prepacked weights); 'none' skips it")
-    ap.add_argument("--split-terms", type=int, default=3, choices=(2, 3),
-                    help="FP6 terms per activation on the prepacked path")
+    ap.add_argument("--split-terms", type=int, default=0, choices=(0, 2, 3),
+                    help="FP6 terms per activation on the prepacked path: 0 = the library's default "
+                         "(3 in the first stage, 2 in the second), 2 or 3 = that many in both")
     ap.add_argument("--no-prepack", action="store_true", help="raw weights only, also for prefill sizes")
     ap.add_argument("--no-workspace", action="store_true",
                     help="call the reference's own symbol (no workspace, raw weights)")
@@ -153,7 +154,7 @@ def run_workload(args, workload, steps, warmup, prepack, split_terms=None, w4a4=
     H, I, k = cfg.H, cfg.I, cfg.top_k
     prefill = T * k > 512  # the library's own split between its decode and tile kernels
     prepack = prepack and prefill and not args.no_workspace
-    terms = split_terms or args.split_terms
+    terms = args.split_terms if split_terms is None else split_terms   # 0 = the library's default
 
     per_set = synth.algorithmic_bytes(H, I, cfg.E, k, 0, cfg.E)
     n_sets = args.weight_sets or max(2, -(-(1 << 30) // per_set))
@@ -164,7 +165,7 @@ def run_workload(args, workload, steps, warmup, prepack, split_terms=None, w4a4=
     for s in range(n_sets):
         w = synth.make_weights(cfg.E, H, I, seed + 7919 * s, device=dev)
         experts.append(ve.FusedExperts(w.w13, w.w13_scale, w.w2, w.w2_scale, prepack=prepack,
-                                       split_terms=terms, w4a4=w4a4 and prepack))
+                                       split_terms=terms or None, w4a4=w4a4 and prepack))
         if args.no_workspace:
             experts[-1].use_workspace = False
     A_bits = synth.make_activations(T, H, seed)
@@ -244,9 +245,10 @@ def run_workload(args, workload, steps, warmup, prepack, split_terms=None, w4a4=
                       "tile_mx_kernel<1,1> + combine_kernel)")
             issued = 1.0
         elif prepack:
-            kernel = (f"vk_hip_fused_moe_mxfp4_prepacked (split_rows_fp6_kernel<{terms}> x2 + "
-                      f"tile_mx_kernel<0,{terms}> + tile_mx_kernel<1,{terms}> + combine_kernel)")
-            issued = float(terms)  # FP4-rate MFMAs per algorithmic product
+            t0, t1 = (terms, terms) if terms else (3, 2)
+            kernel = (f"vk_hip_fused_moe_mxfp4_prepacked (split_rows_fp6_kernel<{t0}> + tile_mx_kernel<0,{t0}> + "
+                      f"split_rows_fp6_kernel<{t1}> + tile_mx_kernel<1,{t1}> + combine_kernel)")
+            issued = (2.0 * t0 + t1) / 3.0  # FP4-rate MFMAs per algorithmic product (2/3 of them in stage 0)
         elif args.no_workspace:
             kernel = "vk_hip_fused_moe_mxfp4 (clear of out + tile_gemm_kernel<0> + tile_gemm_kernel<1>, atomics)"
             issued = 4.0
@@ -293,9 +295,11 @@ def run_workload(args, workload, steps, warmup, prepack, split_terms=None, w4a4=
         },
     }
     if prepack:
-        rec["config"]["activations"] = ("MXFP4 (reference mxfp4_moe_quant), one FP4 x FP4 MFMA per product"
-                                        if w4a4 else f"bf16 as {terms} FP6 E2M3 terms per block of 32")
-        rec["config"]["split_terms"] = 1 if w4a4 else terms
+        rec["config"]["activations"] = (
+            "MXFP4 (reference mxfp4_moe_quant), one FP4 x FP4 MFMA per product" if w4a4 else
+            f"bf16 as {terms} FP6 E2M3 terms per block of 32 in both stages" if terms else
+            "bf16 as FP6 E2M3 terms per block of 32: 3 in the first stage, 2 in the second")
+        rec["config"]["split_terms"] = [1, 1] if w4a4 else [terms, terms] if terms else [3, 2]
     del experts
     torch.cuda.empty_cache()
     return rec, cfg, T, seed
@@ -338,8 +342,10 @@ def main():
         if not args.no_prepack and not args.no_modes:
             # the same workload in the path's other two arithmetic modes (see `activations`)
             p_rec["other_modes"] = {}
-            for key, kw in (("fp6_terms_%d" % (5 - args.split_terms), dict(split_terms=5 - args.split_terms)),
-                            ("w4a4", dict(w4a4=True))):
+            others = [("fp6_terms_%d" % t, dict(split_terms=t)) for t in (3, 2) if t != args.split_terms]
+            if args.split_terms:
+                others.insert(0, ("fp6_terms_3_2", dict(split_terms=0)))
+            for key, kw in others + [("w4a4", dict(w4a4=True))]:
                 m_rec, _, _, _ = run_workload(args, args.prefill, p_steps, min(args.warmup, 3), True, **kw)
                 p_rec["other_modes"][key] = {
                     "value": m_rec["value"], "ms_per_step": m_rec["ms_per_step"],

@@ -185,13 +185,20 @@ void vk_hip_fused_moe_mxfp4_ex(
  * packed buffers (NULL, NULL = vk_hip_fused_moe_mxfp4_ex exactly) and the
  * number of experts in the weight tensors.  The raw weights are still required:
  * decode-sized calls and the exact path read them.  On the packed path the bf16
- * activations are multiplied as a sum of three FP6 (E2M3) terms per block of 32
- * along K (exact unless an element lies more than 2^-13 below its block's
- * largest); VK_HIP_MOE_SPLIT2 selects two terms (error at most 2^-10 of the
- * block's largest per element, two thirds of the matrix-core work).
+ * activations are multiplied as a sum of FP6 (E2M3) terms per block of 32 along K,
+ * each term with a block scale of its own: three terms (exact unless an element
+ * lies more than 2^-13 below its block's largest) in the first stage, whose
+ * error passes through the activation function and the second GEMM, and two
+ * terms (error at most 2^-10 of the block's largest per element) in the second:
+ * 5e-4 relative L2 of the layer against the reference's bf16 arithmetic.
+ * VK_HIP_MOE_SPLIT3 selects three terms in both stages (7e-5; 12 % more
+ * matrix-core work), VK_HIP_MOE_SPLIT2 two in both (1.4e-3, worst element 1e-2
+ * of the RMS: inside the reference's tolerance of 5e-3 / 2e-2, with less margin;
+ * 25 % less work).
  * The workspace size is vk_hip_fused_moe_mxfp4_workspace_bytes(...), as for _ws.
  */
 #define VK_HIP_MOE_SPLIT2 2u
+#define VK_HIP_MOE_SPLIT3 8u
 /* VK_HIP_MOE_W4A4: the W4A4 mode of the reference's orchestration ops
  * (src/c/vkernels/kernels/moe_aux.hpp:1-25): both stages quantise their
  * activations (A, then act) to MXFP4 exactly as mxfp4_moe_quant does and multiply

@@ -100,7 +100,13 @@ static inline float bf16_to_float(uint16_t v) {
  */
 static int g_act_model = 0;
 
-void vko_set_act_model(int terms) { g_act_model = (terms >= 1 && terms <= 3) ? terms : 0; }
+static int g_act_model_down = 0; /* the second stage's, when it differs (terms = first + 16 * second) */
+
+void vko_set_act_model(int terms) {
+  const int first = terms & 15, second = terms >> 4;
+  g_act_model = (first >= 1 && first <= 3) ? first : 0;
+  g_act_model_down = (second >= 1 && second <= 3) ? second : g_act_model;
+}
 
 static float e2m3_round(float v) {
   const float a = fabsf(v);
@@ -112,26 +118,30 @@ static float e2m3_round(float v) {
   return v < 0.0f ? -q : q;
 }
 
-/* a' for one block of 32 bf16 values (finite; blocks of zeros stay zeros). */
+/* a' for one block of 32 bf16 values (finite; blocks of zeros stay zeros).  Every term
+ * has a scale of its own, set as the first one's is: from the largest exponent field of
+ * what the terms before it left (exact in bf16), less 2, and not below 2^(64-127). */
 void vko_act_model_block32(const uint16_t* a, float* out, int terms) {
-  int emax = 0;
+  float rest[32];
   for (int k = 0; k < 32; ++k) {
-    const int e = (a[k] >> 7) & 0xFF;
-    if (e > emax) emax = e;
+    rest[k] = bits_to_float((uint32_t)a[k] << 16);
+    out[k] = 0.0f;
   }
-  if (emax == 0) {
-    for (int k = 0; k < 32; ++k) out[k] = 0.0f;
-    return;
-  }
-  const float s = ldexpf(1.0f, emax - 2 - 127);
-  for (int k = 0; k < 32; ++k) {
-    const float x = bits_to_float((uint32_t)a[k] << 16);
-    float sum = 0.0f, st = s;
-    for (int t = 0; t < terms; ++t) {
-      sum += e2m3_round((x - sum) / st) * st; /* exact: every term is a few bits of x */
-      st *= 0.0625f;
+  for (int t = 0; t < terms; ++t) {
+    int emax = 0;
+    for (int k = 0; k < 32; ++k) {
+      const int e = (int)((float_to_bits(rest[k]) >> 23) & 0xFF); /* bf16 and fp32 share the exponent field */
+      if (e > emax) emax = e;
     }
-    out[k] = sum;
+    if (emax == 0) break; /* nothing left (bf16 subnormals count as zero) */
+    int sb = emax - 2;
+    if (sb < 64) sb = 64;
+    const float st = ldexpf(1.0f, sb - 127);
+    for (int k = 0; k < 32; ++k) {
+      const float term = e2m3_round(rest[k] / st) * st; /* exact: a few bits of the value */
+      out[k] += term;
+      rest[k] -= term;
+    }
   }
 }
 
@@ -278,16 +288,17 @@ static void grouped_gemm(const uint16_t* A, int gather, const uint8_t* W,
                      : A + (size_t)(row0 + r) * a_stride + k_base + k0;
           float dot[BLK_N];
           float amodel[BLK_K];
-          if (g_act_model == 1) {
+          const int model = gather ? g_act_model : g_act_model_down;
+          if (model == 1) {
             vko_aux_model_block32(arow, amodel);
             vko_aux_model_block32(arow + 32, amodel + 32);
-          } else if (g_act_model != 0) {
-            vko_act_model_block32(arow, amodel, g_act_model);
-            vko_act_model_block32(arow + 32, amodel + 32, g_act_model);
+          } else if (model != 0) {
+            vko_act_model_block32(arow, amodel, model);
+            vko_act_model_block32(arow + 32, amodel + 32, model);
           }
           for (int n = 0; n < BLK_N; ++n) dot[n] = 0.0f;
           for (int k = 0; k < BLK_K; ++k) {
-            const float a = g_act_model != 0 ? amodel[k] : bf16_to_float(arow[k]);
+            const float a = model != 0 ? amodel[k] : bf16_to_float(arow[k]);
             const float* wrow = tile_f + (size_t)k * BLK_N;
             for (int n = 0; n < BLK_N; ++n) dot[n] += a * wrow[n];
           }

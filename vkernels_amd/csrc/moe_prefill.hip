@@ -243,14 +243,22 @@ __global__ __launch_bounds__(256) void split_rows_fp6_kernel(const uint16_t* __r
       rest[2 * i] = __uint_as_float(in.d[i] << 16);
       rest[2 * i + 1] = __uint_as_float(in.d[i] & 0xFFFF0000u);
     }
+    uint32_t st = sb;
 #pragma unroll
     for (int t = 0; t < TERMS; ++t) {
-      const uint32_t st = sb - 4u * t;
-      const float scale = __uint_as_float(st << 23);
-      union { bf16x32 v; uint32_t d[16]; } r16;  // the remainder is exact in bf16
+      union { bf16x32 v; uint32_t d[16]; u32x4 q[4]; } r16;  // the remainder is exact in bf16
 #pragma unroll
       for (int i = 0; i < 16; ++i)
         r16.d[i] = (__float_as_uint(rest[2 * i]) >> 16) | (__float_as_uint(rest[2 * i + 1]) & 0xFFFF0000u);
+      if (t > 0) {
+        // a scale of the term's own, set as the first one's: from the largest exponent
+        // field of what is left (at most 2^-4 of the previous term's scale, usually less:
+        // then the term resolves a bit more), and not below the range of the path
+        const uint32_t er = max(max(bf16x8_max_exponent(r16.q[0]), bf16x8_max_exponent(r16.q[1])),
+                                max(bf16x8_max_exponent(r16.q[2]), bf16x8_max_exponent(r16.q[3])));
+        st = er >= kScaleLo + 2u ? er - 2u : kScaleLo;
+      }
+      const float scale = __uint_as_float(st << 23);
       const u32x6 codes = __builtin_amdgcn_cvt_scalef32_pk32_fp6_bf16(r16.v, scale);
       if (t + 1 < TERMS) rest -= __builtin_amdgcn_cvt_scalef32_pk32_f32_fp6(codes, scale);
       uint8_t* blk = qrow + (size_t)t * kp + (size_t)b * 32;
@@ -1024,7 +1032,9 @@ struct MxPlan {
   uint8_t *aq, *cq, *abad, *cbad;
   float* y;
   int32_t* pos;
-  int terms;  // FP6 terms per activation (2, 3) or 1 = the W4A4 mode (MXFP4 activations)
+  // FP6 terms per activation in the first and in the second stage (2 or 3), or 1 and 1 =
+  // the W4A4 mode (MXFP4 activations)
+  int terms0, terms1;
 };
 
 // False when the prepacked path does not take the call (no packed weights, workspace
@@ -1037,11 +1047,17 @@ bool mx_plan(const FusedMoeArgs& a, bool need_stage0, MxPlan& pl) {
   if ((unsigned long long)a.EM * 3ull * mx_kp(a.ispp) >= (1ull << 32) ||
       (unsigned long long)a.M * 3ull * mx_kp(a.hidden) >= (1ull << 32))
     return false;
-  pl.terms = (a.flags & 4u) != 0u ? 1 : (a.flags & 2u) != 0u ? 2 : 3;  // VK_HIP_MOE_W4A4, _SPLIT2
-  if (!(pl.terms == 1 ? mx_kernel_ready<0, 1>() && mx_kernel_ready<1, 1>()
-        : pl.terms == 2 ? mx_kernel_ready<0, 2>() && mx_kernel_ready<1, 2>()
-                        : mx_kernel_ready<0, 3>() && mx_kernel_ready<1, 3>()))
-    return false;
+  // VK_HIP_MOE_W4A4; _SPLIT2; _SPLIT3; default: three terms where the error passes through
+  // the activation function and the second GEMM, two in the second stage
+  if ((a.flags & 4u) != 0u) pl.terms0 = pl.terms1 = 1;
+  else if ((a.flags & 2u) != 0u) pl.terms0 = pl.terms1 = 2;
+  else if ((a.flags & 8u) != 0u) pl.terms0 = pl.terms1 = 3;
+  else { pl.terms0 = 3; pl.terms1 = 2; }
+  const bool ready0 = !need_stage0 || (pl.terms0 == 1 ? mx_kernel_ready<0, 1>()
+                                       : pl.terms0 == 2 ? mx_kernel_ready<0, 2>() : mx_kernel_ready<0, 3>());
+  const bool ready1 = pl.terms1 == 1 ? mx_kernel_ready<1, 1>()
+                      : pl.terms1 == 2 ? mx_kernel_ready<1, 2>() : mx_kernel_ready<1, 3>();
+  if (!ready0 || !ready1) return false;
   uint8_t* base = static_cast<uint8_t*>(a.workspace);
   pl.aq = base;
   pl.cq = pl.aq + l.aq;
@@ -1064,10 +1080,10 @@ bool mx_plan(const FusedMoeArgs& a, bool need_stage0, MxPlan& pl) {
 }
 
 void mx_stage0(const FusedMoeArgs& a, const MxPlan& pl, hipStream_t stream) {
-  if (pl.terms == 1) {
+  if (pl.terms0 == 1) {
     hipLaunchKernelGGL(quant_rows_w4_kernel, dim3(a.M), dim3(256), 0, stream, a.A, pl.aq, pl.abad, a.hidden);
     launch_mx_stage_t<0, 1>(pl.g0, stream);
-  } else if (pl.terms == 2) {
+  } else if (pl.terms0 == 2) {
     hipLaunchKernelGGL(split_rows_fp6_kernel<2>, dim3(a.M), dim3(256), 0, stream, a.A, pl.aq, pl.abad, a.hidden);
     launch_mx_stage_t<0, 2>(pl.g0, stream);
   } else {
@@ -1080,10 +1096,10 @@ void mx_stage0(const FusedMoeArgs& a, const MxPlan& pl, hipStream_t stream) {
 // second stage -> per-token sum
 void mx_stage1(const FusedMoeArgs& a, const MxPlan& pl, hipStream_t stream) {
   launch_fill_i32(pl.pos, -1, a.M * a.top_k, stream);
-  if (pl.terms == 1) {
+  if (pl.terms1 == 1) {
     hipLaunchKernelGGL(quant_rows_w4_kernel, dim3(a.EM), dim3(256), 0, stream, a.act, pl.cq, pl.cbad, a.ispp);
     launch_mx_stage_t<1, 1>(pl.g1, stream);
-  } else if (pl.terms == 2) {
+  } else if (pl.terms1 == 2) {
     hipLaunchKernelGGL(split_rows_fp6_kernel<2>, dim3(a.EM), dim3(256), 0, stream, a.act, pl.cq, pl.cbad, a.ispp);
     launch_mx_stage_t<1, 2>(pl.g1, stream);
   } else {

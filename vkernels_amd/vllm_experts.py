@@ -249,6 +249,7 @@ def resolve_moe_ws_fn(lib):
 MOE_OVERWRITE_OUT = 1  # VK_HIP_MOE_OVERWRITE_OUT
 MOE_SPLIT2 = 2         # VK_HIP_MOE_SPLIT2
 MOE_W4A4 = 4           # VK_HIP_MOE_W4A4
+MOE_SPLIT3 = 8         # VK_HIP_MOE_SPLIT3
 
 
 def resolve_prepack_fns(lib):
@@ -405,7 +406,7 @@ class FusedExperts:
     def __init__(self, w13, w13_scale, w2, w2_scale, *, b13=None, b2=None, activation="swiglu",
                  swiglu_limit: float = 0.0, beta: float = 4.0, linear_beta: float = 25.0,
                  expert_map=None, local_num_experts=None, scratch: CaptureSafeScratch | None = None,
-                 prepack: bool = False, split_terms: int = 3, w4a4: bool = False):
+                 prepack: bool = False, split_terms: int | None = None, w4a4: bool = False):
         torch = _require_torch()
         self.torch = torch
         self.lib = load_libvkernels_hip()
@@ -444,8 +445,9 @@ class FusedExperts:
         self.scratch = scratch or _scratch
         # a second copy of the weights in the layout of the prefill-sized kernels
         # (load time; batches of more than 512 routed rows then run at the FP4 rate)
-        if split_terms not in (2, 3):
-            raise ValueError("split_terms must be 2 or 3")
+        if split_terms not in (None, 2, 3):
+            raise ValueError("split_terms must be None (three FP6 terms in the first stage, two in the "
+                             "second), 2 or 3 (that many in both)")
         self.split_terms = split_terms
         # W4A4: batches of more than 512 routed rows quantise their activations to MXFP4 as
         # the reference's mxfp4_moe_quant does (needs the prepacked weights)
@@ -582,6 +584,8 @@ class FusedExperts:
                     flags |= MOE_W4A4
                 elif self.split_terms == 2:
                     flags |= MOE_SPLIT2
+                elif self.split_terms == 3:
+                    flags |= MOE_SPLIT3
                 self.moe_prepacked_fn(*args, _ptr(ws), need, flags, _ptr(self.w13_packed),
                                       _ptr(self.w2_packed), self.E, _stream(torch))
             elif self.moe_ex_fn is not None:
