@@ -56,6 +56,7 @@
 #include <stdlib.h>
 
 #include "moe_common.hpp"
+#include "moe_prefill_layout.hpp"
 #include "vk_internal.hpp"
 
 namespace vk {
@@ -68,12 +69,6 @@ typedef __attribute__((ext_vector_type(6))) uint32_t u32x6;
 typedef __attribute__((ext_vector_type(16))) float f32x16;
 typedef __attribute__((ext_vector_type(32))) float f32x32;
 typedef __attribute__((ext_vector_type(32))) __bf16 bf16x32;
-
-constexpr int kMxRows = 128;        // sorted rows per window
-constexpr int kMxUnitRows = 128;    // weight rows per unit
-constexpr int kMxWaves = 4;
-constexpr int kMxRing = 3;          // K steps of split rows in LDS
-constexpr int kMxStepBytes = 8704;  // prepacked bytes of one unit's K step: 8 KiB of codes + 512 of scales
 
 struct MxArgs {
   const uint8_t* Wp;       // prepacked weights of the stage
@@ -115,23 +110,6 @@ int g_mx_trace_stage = 1;
 #define MX_TRACE(slot_) do {} while (0)
 #endif
 
-__host__ __device__ inline int mx_kp(int K) { return (K + 127) & ~127; }
-__host__ __device__ inline int mx_units(int stage, int ncols) {
-  return stage == 0 ? ncols / 64 : (ncols + kMxUnitRows - 1) / kMxUnitRows;
-}
-// Row of W (within an expert) that lane row n of tile t of `unit` multiplies; the
-// caller checks it against the expert's row count (stage 1's last unit may be ragged).
-__host__ __device__ inline int mx_weight_row(int stage, int ncols, int unit, int t, int n) {
-  if (stage == 0) return (t >> 1) * ncols + unit * 64 + (t & 1) * 32 + n;
-  return unit * kMxUnitRows + t * 32 + n;
-}
-__host__ __device__ inline int mx_window_rows(int block_size) {
-  if (kMxRows % block_size == 0) return kMxRows;
-  for (int rows = kMxRows; rows > 16; rows -= 16)
-    if (block_size % rows == 0) return rows;
-  return 16;
-}
-
 // ---------------------------------------------------------------------------
 // Prepacking (load time).
 // ---------------------------------------------------------------------------
@@ -169,7 +147,7 @@ __global__ __launch_bounds__(256) void prepack_kernel(const uint8_t* __restrict_
                                                       int ksteps) {
   const int kstep = blockIdx.x, unit = blockIdx.y, e = blockIdx.z;
   const int groups = K / 32;
-  uint8_t* dst = packed + (((size_t)e * units + unit) * (size_t)ksteps + kstep) * (size_t)kMxStepBytes;
+  uint8_t* dst = packed + mx_unit_offset(e, units, unit, ksteps) + (size_t)kstep * (size_t)kMxStepBytes;
 #pragma unroll
   for (int i = 0; i < 2; ++i) {
     const int pc = threadIdx.x + 256 * i;  // [half][tile][lane]
@@ -597,20 +575,23 @@ __global__ __launch_bounds__(64 * kMxWaves) void tile_mx_kernel(MxArgs p) {
       size_t grow;
       if (STAGE == 0) grow = f >= 0 ? (size_t)(f / p.top_k) : 0;
       else grow = rl < n_rows ? (size_t)(row0 + rl) : (size_t)row0;
-      cp_off[g] = (uint32_t)(grow * (size_t)(TERMS * Kp)) + 16u * (uint32_t)(c ^ r);
+      cp_off[g] = mx_row_copy_lane_offset(grow, TERMS, Kp, lane);
     }
     auto copy_rows = [&](int step, int d) {  // operation d (0 .. 4 TERMS - 1) of the step's row copies
       const int term = d >> 2, g = d & 3;
-      const int k0 = min(step, nsteps - 1) * 128;  // past the end: the last step again
-      const uint32_t dst = lds_base + (uint32_t)((step % R) * kSlotBytes +
-                                                 ((wave * TERMS + term) * 32 + g * 8) * 128);
-      dma16_saddr(cp_off[g] + (uint32_t)(term * Kp + k0), p.Aq, dst);
+      // (past the end: the last step again)
+      dma16_saddr(cp_off[g] + mx_row_copy_step_offset(term, Kp, step, nsteps), p.Aq,
+                  lds_base + mx_row_copy_lds(step, wave, TERMS, term, g));
     };
     // ---- weight loads
-    const uint8_t* wp_unit = p.Wp + ((size_t)e * p.units + unit) * (size_t)nsteps * (size_t)kMxStepBytes;
+    const uint8_t* wp_unit = p.Wp + mx_unit_offset(e, p.units, unit, nsteps);
     const uint32_t voff16 = (uint32_t)lane * 16u, voff8 = (uint32_t)lane * 8u;
     auto load_weights = [&](WeightStep& ws, int step, int j) {  // operation j (0 .. 8)
-      const uint8_t* base = wp_unit + (size_t)min(step, nsteps - 1) * (size_t)kMxStepBytes;
+      const uint8_t* base = wp_unit + mx_step_offset(step, nsteps);
+      // (the immediates and lane offsets below are mx_weight_load_offset(j, lane))
+      static_assert(mx_weight_load_offset(3, 2) == 3072 + 32 && mx_weight_load_offset(6, 0) == 4096 + 2048 &&
+                        mx_weight_load_offset(8, 3) == 8192 + 24,
+                    "weight loads and their layout function disagree");
       switch (j) {
         case 0: load16_nowait<0>(ws.w[0], voff16, base); break;
         case 1: load16_nowait<1024>(ws.w[1], voff16, base); break;
@@ -634,13 +615,8 @@ __global__ __launch_bounds__(64 * kMxWaves) void tile_mx_kernel(MxArgs p) {
     // lane-dependent offsets (half 0 / 1, first / second piece) are added to the slot's
     // base once per K step; row tile and term are immediate offsets of the reads.
     uint32_t rd_off[4];
-    {
-      const uint32_t pos0 = (uint32_t)(((2 * hh) ^ (ln & 7)) * 16);
-      rd_off[0] = (uint32_t)(ln * 128) + pos0;
-      rd_off[1] = (uint32_t)(ln * 128) + (pos0 ^ 16u);
-      rd_off[2] = (uint32_t)(ln * 128) + (pos0 ^ 64u);
-      rd_off[3] = (uint32_t)(ln * 128) + (pos0 ^ 80u);
-    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j) rd_off[j] = mx_operand_lane_offset(j, ln, hh);
     struct SlotBase {
       const uint8_t* b[4];
     };
@@ -648,14 +624,14 @@ __global__ __launch_bounds__(64 * kMxWaves) void tile_mx_kernel(MxArgs p) {
       SlotBase sb;
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
-        uint32_t off = rd_off[j] + (uint32_t)(slot_ * kSlotBytes);
+        uint32_t off = rd_off[j] + mx_operand_tile_offset(slot_, TERMS, 0, 0);
         __asm__ volatile("" : "+v"(off));  // one register per base: nothing to precompute per tile
         sb.b[j] = lds_bytes + off;
       }
       return sb;
     };
     auto read_operand = [&](const SlotBase& sb, int m, int term, int half) {
-      const int tile_off = ((m * TERMS + term) * 32) * 128;
+      const int tile_off = (int)mx_operand_tile_offset(0, TERMS, m, term);
       const u32x4 lo = *reinterpret_cast<const u32x4*>(sb.b[2 * half] + tile_off);
       const u32x4 hi4 = *reinterpret_cast<const u32x4*>(sb.b[2 * half + 1] + tile_off);
       return i32x8{(int)lo[0], (int)lo[1], (int)lo[2], (int)lo[3],
@@ -776,7 +752,7 @@ __global__ __launch_bounds__(64 * kMxWaves) void tile_mx_kernel(MxArgs p) {
     // rows go through a staging area of the wavefront's own in the ring (free after the
     // barrier above) and leave as whole lines: 4 rows x 256 bytes (8 rows x 128 bytes in
     // stage 0) per store instruction ----
-    uint8_t* stage_lds = reinterpret_cast<uint8_t*>(mx_lds) + wave * (R * kSlotBytes / kMxWaves);
+    uint8_t* stage_lds = reinterpret_cast<uint8_t*>(mx_lds) + mx_stage_base(wave, TERMS);
     auto wave_fence = [] {  // LDS operations of a wavefront execute in order; this keeps the compiler's too
       __asm__ volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
     };
@@ -798,7 +774,7 @@ __global__ __launch_bounds__(64 * kMxWaves) void tile_mx_kernel(MxArgs p) {
         exact_unit_mx<STAGE>(p, e, unit, a_row, q_row, lane, tile);
       }
       if (STAGE == 0) {
-        constexpr int kPitch = 144;  // 64 bf16 of a row + 16: rows stay 16-byte aligned
+        constexpr int kPitch = kMxActPitch;
         // 128 activation values per lane and row tile: the plain SwiGLU (no bias, no
         // clamp), which is what serving runs, gets a loop of its own without a branch per
         // value; the same act_value with its parameters known at compile time.
@@ -856,7 +832,7 @@ __global__ __launch_bounds__(64 * kMxWaves) void tile_mx_kernel(MxArgs p) {
         // workgroup's window.  Then rows that are not routed are stored like the others
         // (with a routing weight of zero): nothing reads them (pos never points at them),
         // and a later segment of this window, if they are its rows, overwrites them.
-        constexpr int kPitch = 272;  // 64 floats of a row + 16 bytes
+        constexpr int kPitch = kMxYPitch;
         // (from LDS, put there when the rows were listed: a load from memory still pending
         // when the stores begin makes every later wait for it a wait for those stores)
         const float w = row_w[m * 32 + ln];
@@ -979,8 +955,7 @@ size_t moe_prepack_bytes(int num_experts, int rows, int K, int stage) {
   if (num_experts <= 0 || rows <= 0 || K <= 0) return 0;
   const int ncols = stage == 0 ? rows / 2 : rows;
   const size_t units = (size_t)mx_units(stage, ncols);
-  return align256((size_t)num_experts * units * (size_t)(mx_kp(K) / 128) * kMxStepBytes) +
-         align256((size_t)num_experts * units);
+  return mx_packed_bytes(num_experts, units, mx_kp(K) / 128);
 }
 
 void launch_moe_prepack(const uint8_t* w, const uint8_t* w_scale, int num_experts, int rows, int K,
@@ -988,7 +963,7 @@ void launch_moe_prepack(const uint8_t* w, const uint8_t* w_scale, int num_expert
   const int ncols = stage == 0 ? rows / 2 : rows;
   const int units = mx_units(stage, ncols);
   const int ksteps = mx_kp(K) / 128;
-  uint8_t* flags = packed + align256((size_t)num_experts * units * (size_t)ksteps * kMxStepBytes);
+  uint8_t* flags = packed + mx_packed_body_bytes(num_experts, units, ksteps);
   hipLaunchKernelGGL(prepack_flag_kernel, dim3(units, num_experts), dim3(256), 0, stream, w, w_scale,
                      flags, stage, rows, ncols, K, units);
   hipLaunchKernelGGL(prepack_kernel, dim3(ksteps, units, num_experts), dim3(256), 0, stream, w,
@@ -1070,9 +1045,9 @@ bool mx_plan(const FusedMoeArgs& a, bool need_stage0, MxPlan& pl) {
   const int units0 = mx_units(0, a.ispp), units1 = mx_units(1, a.hidden);
   pl.g0.Wp = a.w13_packed;
   pl.g0.Wflags = a.w13_packed == nullptr ? nullptr :
-      a.w13_packed + align256((size_t)a.num_experts * units0 * (size_t)(mx_kp(a.hidden) / 128) * kMxStepBytes);
+      a.w13_packed + mx_packed_body_bytes(a.num_experts, units0, mx_kp(a.hidden) / 128);
   pl.g1.Wp = a.w2_packed;
-  pl.g1.Wflags = a.w2_packed + align256((size_t)a.num_experts * units1 * (size_t)(mx_kp(a.ispp) / 128) * kMxStepBytes);
+  pl.g1.Wflags = a.w2_packed + mx_packed_body_bytes(a.num_experts, units1, mx_kp(a.ispp) / 128);
   pl.g0.Aq = pl.aq; pl.g0.row_bad = pl.abad;
   pl.g1.Aq = pl.cq; pl.g1.row_bad = pl.cbad;
   pl.g1.y = pl.y; pl.g1.pos = pl.pos;
