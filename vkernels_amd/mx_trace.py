@@ -18,7 +18,8 @@ def main() -> None:
     ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
     ap.add_argument("workload", help="config:T, e.g. c3:16384")
     ap.add_argument("--stage", type=int, default=1, choices=(0, 1))
-    ap.add_argument("--split-terms", type=int, default=3, choices=(2, 3))
+    ap.add_argument("--split-terms", type=int, default=0, choices=(0, 2, 3),
+                    help="0 = the library's default (3 FP6 terms in the first stage, 2 in the second)")
     ap.add_argument("--w4a4", action="store_true")
     args = ap.parse_args()
 
@@ -35,7 +36,7 @@ def main() -> None:
     cfg, T = synth.CONFIGS[name], int(t_str)
     dev = torch.device("cuda", 0)
     w = synth.make_weights(cfg.E, cfg.H, cfg.I, 5, device=dev)
-    fe = ve.FusedExperts(w.w13, w.w13_scale, w.w2, w.w2_scale, prepack=True, split_terms=args.split_terms,
+    fe = ve.FusedExperts(w.w13, w.w13_scale, w.w2, w.w2_scale, prepack=True, split_terms=args.split_terms or None,
                          w4a4=args.w4a4)
     a_bits = synth.make_activations(T, cfg.H, 5)
     A = torch.from_numpy(a_bits.view(np.int16)).view(torch.bfloat16).to(dev)
