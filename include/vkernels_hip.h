@@ -348,10 +348,11 @@ void vk_hip_moe_down_mxfp4_ex(
  * Additive, for tests: bf16 rows [rows, K] -> the split rows the prefill-sized
  * kernels multiply: per row `terms` (2 or 3) planes of Kp = K rounded up to 128
  * bytes; a plane is Kp/32 blocks of 32 bytes: the 32 FP6 (E2M3) codes of the
- * term (code i at bit 6 i), the term's scale byte (e-2-4t for term t, e the
- * block's largest exponent field), 7 zero bytes.  row_flags[r] = 1 when a block
- * of the row is outside the range of the split (inf/NaN, scale byte outside
- * [64 + 4 (terms-1), 190]).  `split` holds rows * terms * Kp bytes.
+ * term (code i at bit 6 i), the term's scale byte (the largest exponent field
+ * of what the terms before it left of the block, less 2, at least 64), 7 zero
+ * bytes.  row_flags[r] = 1 when a block of the row is outside the range of the
+ * split (inf/NaN, first scale byte outside [64 + 4 (terms-1), 190]).  `split`
+ * holds rows * terms * Kp bytes.
  */
 int vk_hip_split_rows_fp6(const uint16_t* x, int32_t rows, int32_t K, int32_t terms, void* split,
                           uint8_t* row_flags, void* stream);

@@ -13,12 +13,15 @@
 // points and their scale bytes decremented once, when the weights are
 // prepacked (mxfp4.hpp: the reference's decode table is half of OCP's).  A
 // bf16 activation is fed as a sum of TERMS FP6 terms per block of 32 along K:
-// with e the largest exponent field of the block and s = 2^(e-2-127),
-//     t0 = Q(a / s) s,  t1 = Q((a - t0) / (s/16)) (s/16),  t2 = Q((a - t0 - t1) / (s/256)) (s/256),
-// Q = round to nearest even on the E2M3 grid; one MFMA per term, the term's
-// scale byte being e-2, e-6, e-10.  Three terms represent a bf16 value exactly
-// unless it lies more than 2^-13 below the largest of its block; two terms
-// (VK_HIP_MOE_SPLIT2) leave an error of at most 2^-10 of the block's largest.
+//     t0 = Q(a / s0) s0,  t1 = Q((a - t0) / s1) s1,  t2 = Q((a - t0 - t1) / s2) s2,
+// Q = round to nearest even on the E2M3 grid, s_i = 2^(e_i - 2 - 127) with e_i the
+// largest exponent field of what the terms before left in the block (e_0: of the
+// block itself); one MFMA per term, the term's scale byte being e_i - 2.  Three
+// terms represent a bf16 value exactly unless it lies more than 2^-13 below the
+// largest of its block; two terms leave an error of at most 2^-10 of the block's
+// largest.  By default the first stage takes three terms and the second two
+// (VK_HIP_MOE_SPLIT3 / VK_HIP_MOE_SPLIT2: three / two in both); TERMS = 1 is the
+// W4A4 mode (MXFP4 activations, FP4 x FP4).
 // Units whose weights hold an inf/NaN code or a scale byte outside
 // [kScaleLo, kScaleHi] (flagged when the weights are prepacked) and segments
 // with a row whose blocks are outside the representable range (flagged when
