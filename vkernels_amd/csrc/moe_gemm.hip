@@ -110,13 +110,15 @@ __host__ __device__ inline int split_row_k(int K) { return (K + 127) & ~127; }
 
 // Stage 0 of a call that was asked to overwrite `out`: every workgroup clears
 // its share (the stage does not use `out`; the next stage starts after this one).
+// THREADS = the workgroup's size, known to every caller at compile time.
+template <int THREADS>
 __device__ __forceinline__ void clear_out_share(const GemmArgs& p) {
   if (p.zero_out == nullptr) return;
   const long long n4 = p.zero_count / 4;
   const long long wg = (long long)blockIdx.y * gridDim.x + blockIdx.x;
   const long long wgs = (long long)gridDim.x * gridDim.y;
   f32x4* out4 = reinterpret_cast<f32x4*>(p.zero_out);
-  for (long long i = wg * blockDim.x + threadIdx.x; i < n4; i += wgs * blockDim.x)
+  for (long long i = wg * THREADS + threadIdx.x; i < n4; i += wgs * THREADS)
     out4[i] = f32x4{0.f, 0.f, 0.f, 0.f};
 }
 
@@ -228,7 +230,7 @@ __device__ __forceinline__ void unit_tiles(const GemmArgs& p, int e, int unit, i
 // Work split.  The launch has as many workgroups as the device has compute
 // units.  Every workgroup lists the runs (consecutive blocks of one expert),
 // flattens (run, weight unit) into one index space and takes a contiguous
-// slice of it (workgroup_slice), so the weight bytes are spread evenly over
+// slice of it (kStagingUnits below), so the weight bytes are spread evenly over
 // the compute units whatever the number of active experts.  For each run its
 // slice touches, and each 16-row pass of that run, the workgroup stages the
 // 16 activation rows, all of K, into LDS as MFMA operands (split as above).
@@ -254,7 +256,10 @@ __device__ __forceinline__ void unit_tiles(const GemmArgs& p, int e, int unit, i
 // masking of the weight side.
 // ---------------------------------------------------------------------------
 constexpr int kMaxRuns = 512;   // runs the resident kernel can list in LDS
-constexpr int kScMax = 4;       // 16-byte scale pieces per lane: NT * K/32 <= 64 * kScMax
+// 16-byte scale pieces of a unit a lane holds: NT * K/32 <= 64 * resident_scale_pieces.
+// Workgroups of 8 wavefronts stage K <= 3072 (resident_batch), 96 groups, and have
+// 256 registers a lane: three pieces and not four keeps the kernel clear of scratch memory.
+__host__ __device__ constexpr int resident_scale_pieces(int waves) { return waves == 4 ? 4 : 3; }
 
 typedef __attribute__((ext_vector_type(8))) int i32x8;
 typedef __attribute__((ext_vector_type(4))) int i32x4;
@@ -288,31 +293,11 @@ __device__ __forceinline__ int slice_begin(int total, int i, int parts) {
 // rows of a run costs about as much as streaming kStagingUnits units.  So when
 // every run can have workgroups of its own, run r gets a share of the grid
 // proportional to its passes (taken as its 16-row tiles, an upper bound that
-// is exact for block size 16) and the slices stop at run boundaries; `aligned` says whether that gives every run
-// a workgroup and does not unbalance the workgroups by more than a second
-// staging would cost.  Otherwise the space is cut evenly and a slice may span
-// runs.
+// is exact for block size 16) and the slices stop at run boundaries, provided
+// that gives every run a workgroup and does not unbalance the workgroups by
+// more than a second staging would cost.  Otherwise the space is cut evenly
+// and a slice may span runs.
 constexpr int kStagingUnits = 4;
-__device__ __forceinline__ void workgroup_slice(int n_runs, int units, int wg, int grid,
-                                                const int* run_end, bool aligned, int& s0,
-                                                int& s1) {
-  if (aligned) {  // run_end[r] = workgroups of the runs up to r
-    int lo = 0, hi = n_runs - 1;  // smallest r with run_end[r] > wg
-    while (lo < hi) {
-      const int mid = (lo + hi) >> 1;
-      if (run_end[mid] > wg) hi = mid;
-      else lo = mid + 1;
-    }
-    const int first = lo == 0 ? 0 : run_end[lo - 1];
-    const int g = run_end[lo] - first;
-    s0 = lo * units + slice_begin(units, wg - first, g);
-    s1 = lo * units + slice_begin(units, wg - first + 1, g);
-    return;
-  }
-  const int total = n_runs * units;
-  s0 = slice_begin(total, wg, grid);
-  s1 = slice_begin(total, wg + 1, grid);
-}
 
 // Reference-exact slow path for one unit: one K step at a time, integer-exact
 // dequantisation, the activation row of this lane's column read from global
@@ -389,11 +374,10 @@ __global__ __launch_bounds__(64 * WAVES) void stream_resident_kernel(GemmArgs p)
   __shared__ int run_block0[kMaxRuns];
   __shared__ int run_block1[kMaxRuns];  // one past the last block of the run
   __shared__ int run_expert[kMaxRuns];
-  __shared__ int run_end[kMaxRuns];     // aligned slicing: workgroups of the runs up to this one
+  __shared__ int run_cum[kMaxRuns];     // blocks of the runs up to and including this one
   __shared__ int slice_sh[2];           // this workgroup's slice of the (run, unit) space
-  __shared__ int first_ids[64];         // sorted ids of the first 64 rows of this workgroup's first run
   __shared__ int pass_slow[2];          // set while staging: this pass takes the exact path
-  if (STAGE == 0) clear_out_share(p);
+  if (STAGE == 0) clear_out_share<64 * WAVES>(p);
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // uniform, and known to be
@@ -412,20 +396,35 @@ __global__ __launch_bounds__(64 * WAVES) void stream_resident_kernel(GemmArgs p)
   const size_t w_unit_stride = unit_stride_rows * (size_t)(K / 2);
   const size_t s_unit_stride = unit_stride_rows * (size_t)groups;
 
+  // While wavefront 0 lists the runs, the others copy the head of sorted_ids to
+  // the start of the operand planes (free until the first pass is staged): the
+  // ids of the workgroup's first rows are then an LDS read behind the barrier,
+  // not one more round trip to memory in front of the row loads.
+  int* const ids_lds = reinterpret_cast<int*>(b_lds);
+  const int ids_cached = min(p.num_blocks * p.block_size, nsteps * 1024);  // 4 KB of planes per K step
+  if (WAVES > 1 && wave != 0) {
+    for (int i = tid - 64; i < ids_cached; i += 64 * (WAVES - 1)) ids_lds[i] = p.sorted_ids[i];
+  }
+
   // ---- list the runs (first and last block of every run, in order) ---------
   if (wave == 0) {
+    const int nb = p.num_blocks;
+    const int grid = (int)gridDim.x, wg = (int)blockIdx.x;
+    const unsigned long long below = (1ull << lane) - 1ull;
     int n = 0, n_last = 0;
-    for (int base = 0; base < p.num_blocks; base += 64) {
+    int listed_blocks = 0;  // blocks with an expert so far = the blocks of the runs so far
+    for (int base = 0; base < nb; base += 64) {
       const int b = base + lane;
-      bool first = false, last = false;
-      int e = -1;
-      if (b < p.num_blocks) {
-        e = p.expert_ids[b];
-        first = e >= 0 && (b == 0 || p.expert_ids[b - 1] != e);
-        last = e >= 0 && (b == p.num_blocks - 1 || p.expert_ids[b + 1] != e);
-      }
-      const unsigned long long mf = __ballot(first), ml = __ballot(last);
-      const unsigned long long below = (1ull << lane) - 1ull;
+      // the block's expert and its two neighbours': three loads without a branch
+      // between them, so one round trip to memory and not three
+      const int bc = min(b, nb - 1);
+      const int e_here = p.expert_ids[bc];
+      const int e_before = p.expert_ids[max(bc - 1, 0)];
+      const int e_after = p.expert_ids[min(bc + 1, nb - 1)];
+      const int e = b < nb ? e_here : -1;
+      const bool first = e >= 0 && (b == 0 || e_before != e);
+      const bool last = e >= 0 && (b == nb - 1 || e_after != e);
+      const unsigned long long mv = __ballot(e >= 0), mf = __ballot(first), ml = __ballot(last);
       if (first) {
         const int idx = n + (int)__popcll(mf & below);
         if (idx < kMaxRuns) {
@@ -435,69 +434,68 @@ __global__ __launch_bounds__(64 * WAVES) void stream_resident_kernel(GemmArgs p)
       }
       if (last) {  // a run's last block is its first one or comes after it
         const int idx = n_last + (int)__popcll(ml & below);
-        if (idx < kMaxRuns) run_block1[idx] = b + 1;
+        if (idx < kMaxRuns) {
+          run_block1[idx] = b + 1;
+          run_cum[idx] = listed_blocks + (int)__popcll(mv & below) + 1;
+        }
       }
       n += (int)__popcll(mf);
       n_last += (int)__popcll(ml);
+      listed_blocks += (int)__popcll(mv);
     }
     n = n < kMaxRuns ? n : kMaxRuns;
     if (lane == 0) {
       pass_slow[0] = 0;
       pass_slow[1] = 0;
     }
-    // ---- weights of the runs and this workgroup's slice ------------------------
-    // weight of a run = its 16-row tiles; run_end[r] = floor(grid * (weights up to
-    // r) / (all weights)).  Two sweeps over the runs, 64 at a time.
+    // ---- this workgroup's slice --------------------------------------------
+    // Weight of a run = its 16-row tiles.  Aligned slicing gives the runs up to
+    // and including r the first floor(grid * (their weight) / (all weight))
+    // workgroups; the tiles per block cancel in that quotient, so it is taken
+    // over blocks (run_cum).  A lane per run, and ballots instead of reductions:
+    // this wavefront is the only one at work until the barrier below.
     const int tiles_per_block = p.block_size / 16;
-    int total_weight = 0;
-    for (int base = 0; base < n; base += 64) {
-      const int r = base + lane;
-      int w = r < n ? (run_block1[r] - run_block0[r]) * tiles_per_block : 0;
-#pragma unroll
-      for (int d = 32; d >= 1; d >>= 1) w += __shfl_xor(w, d);
-      total_weight += w;
-    }
-    bool ok = n > 0 && n <= (int)gridDim.x;
+    const int total_weight = listed_blocks * tiles_per_block;
+    bool ok = n > 0 && n <= grid;
+    int t0 = 0, t1 = 0;
     if (ok) {
-      int carry = 0, worst = 0;  // worst = largest (units per workgroup) x (passes) over the runs
+      // largest (units per workgroup) x (passes) a run may have
+      const int limit = (units * total_weight + grid - 1) / grid + kStagingUnits;
+      int mine = -1, mine_begin = 0, mine_end = 0;  // the first run whose workgroups end past this one
       for (int base = 0; base < n; base += 64) {
         const int r = base + lane;
-        const int w = r < n ? (run_block1[r] - run_block0[r]) * tiles_per_block : 0;
-        int x = w;
-#pragma unroll
-        for (int d = 1; d < 64; d <<= 1) {
-          const int y = __shfl_up(x, d);
-          if (lane >= d) x += y;
+        const bool live = r < n;
+        const int cum = live ? run_cum[r] : 0;  // written by this wavefront; LDS operations stay in order
+        const int len = live ? run_block1[r] - run_block0[r] : 0;
+        const int end = (int)((unsigned)(grid * cum) / (unsigned)listed_blocks);
+        const int begin = (int)((unsigned)(grid * (cum - len)) / (unsigned)listed_blocks);
+        bool bad = false;
+        if (live) {
+          bad = end <= begin;
+          if (!bad) bad = (units + end - begin - 1) / (end - begin) * (len * tiles_per_block) > limit;
         }
-        const int cum = carry + x;
-        const int end = (int)((unsigned)(gridDim.x * cum) / (unsigned)total_weight);
-        const int begin = (int)((unsigned)(gridDim.x * (cum - w)) / (unsigned)total_weight);
-        int cost = 0;
-        if (r < n) {
-          run_end[r] = end;
-          if (end > begin) cost = (units + end - begin - 1) / (end - begin) * w;
+        ok = ok && __ballot(bad) == 0ull;
+        const unsigned long long past = __ballot(live && end > wg);
+        if (mine < 0 && past != 0ull) {  // uniform
+          const int l = __builtin_ctzll(past);
+          mine = base + l;
+          mine_begin = __builtin_amdgcn_readlane(begin, l);
+          mine_end = __builtin_amdgcn_readlane(end, l);
         }
-        ok = ok && __ballot(r < n && end <= begin) == 0ull;
-#pragma unroll
-        for (int d = 32; d >= 1; d >>= 1) cost = max(cost, __shfl_xor(cost, d));
-        worst = max(worst, cost);
-        carry += __shfl(x, 63);
       }
-      ok = ok && worst <= (units * total_weight + (int)gridDim.x - 1) / (int)gridDim.x + kStagingUnits;
+      if (ok) {  // the last run ends at `grid`, so `mine` is set
+        const int g = mine_end - mine_begin;
+        t0 = mine * units + slice_begin(units, wg - mine_begin, g);
+        t1 = mine * units + slice_begin(units, wg - mine_begin + 1, g);
+      }
     }
-    int t0 = 0, t1 = 0;
-    if (n > 0) workgroup_slice(n, units, blockIdx.x, gridDim.x, run_end, ok, t0, t1);
+    if (!ok && n > 0) {  // the (run, unit) space cut evenly; a slice may span runs
+      t0 = slice_begin(n * units, wg, grid);
+      t1 = slice_begin(n * units, wg + 1, grid);
+    }
     if (lane == 0) {
       slice_sh[0] = t0;
       slice_sh[1] = t1;
-    }
-    // The ids of the first rows this workgroup will stage, fetched once here
-    // rather than by every wavefront after the barrier.
-    if (t0 < t1) {
-      const int r0 = t0 / units;
-      const int b0 = run_block0[r0];  // written by this wavefront, LDS operations stay in order
-      const int rows = (run_block1[r0] - b0) * p.block_size;
-      first_ids[lane] = lane < rows ? p.sorted_ids[b0 * p.block_size + lane] : -1;
     }
   }
   __syncthreads();
@@ -509,6 +507,40 @@ __global__ __launch_bounds__(64 * WAVES) void stream_resident_kernel(GemmArgs p)
     u32x4 w[NT];
   };
   int pass_no = 0;
+
+  // Scale bytes of a unit: byte offset of this lane's piece j from the unit's first tile
+  // (tile_row = the first weight row of the piece's tile, counted from the first tile's, as
+  // unit_tiles lays them out; lanes past the end re-read the last piece).
+  constexpr int kHalfTiles = NT >= 2 ? NT / 2 : 1;
+  constexpr int kScMax = resident_scale_pieces(WAVES);
+  int sc_piece[kScMax];
+#pragma unroll
+  for (int j = 0; j < kScMax; ++j) {
+    const int piece = min(lane + 64 * j, NT * groups - 1);
+    int t = 0;
+#pragma unroll
+    for (int t2 = 1; t2 < NT; ++t2)
+      if (piece >= t2 * groups) t = t2;
+    int tile_row = STAGE == 0 ? 0 : t * 16;
+    if (STAGE == 0) {
+#pragma unroll
+      for (int t2 = 1; t2 < NT; ++t2)
+        if (t == t2) tile_row = (t2 / kHalfTiles) * p.ncols + (t2 % kHalfTiles) * 16;
+    }
+    sc_piece[j] = tile_row * groups + (piece - t * groups) * 16;
+  }
+
+  // Staging: a wavefront takes the groups wave, wave + WAVES, ... (its pieces 0, 1, ...).
+  static_assert(WAVES % 4 == 0, "a wavefront's pieces keep their quarter of a K step");
+  const int my_groups = (groups - wave + WAVES - 1) / WAVES;      // pieces with values of the row
+  const int my_pieces = (nsteps * 4 - wave + WAVES - 1) / WAVES;  // ... and those of the zero padding
+  // where lane (row lane / 4, eighth lane % 4) writes piece 0: the leading plane
+  // (the remainder plane is 2 KB on) and the block scale byte
+  uint8_t* const plane0 =
+      reinterpret_cast<uint8_t*>(b_lds) +
+      (size_t)((((wave >> 2) * 4 + ((wave >> 1) & 1)) * 64 + ((wave & 1) * 2 + ((lane & 3) >> 1)) * 16 +
+                (lane >> 2)) * 16 + (lane & 1) * 8);
+  uint8_t* const bsc0 = bsc_lds + (wave >> 2) * 64 + (wave & 3) * 16 + (lane >> 2);
 
   for (int r = r_first; r <= (s1 - 1) / units; ++r) {
     const int base_slot = r * units;
@@ -555,41 +587,34 @@ __global__ __launch_bounds__(64 * WAVES) void stream_resident_kernel(GemmArgs p)
 
     // ---- scale block of a unit: coalesced loads into registers, parked in
     // the wavefront's LDS region when the unit before it is complete --------
+    // The unit's tiles are read as NT * groups 16-byte pieces, lane + 64 j the pieces of a
+    // lane (sc_piece: where piece j lies from the start of the unit's first tile) and
+    // parked in the same order: tile t starts at piece t * groups, which is where
+    // sc_lds + t * sc_tile_bytes is.
     u32x4 scn[kScMax];
+    const uint8_t* sc_unit = nullptr;  // scale bytes of the first tile of the unit being computed
     auto fetch_scales = [&](size_t ahead) {
 #pragma unroll
-      for (int j = 0; j < kScMax; ++j) {
-        // branch-free: lanes past the end re-read the last piece
-        const int piece = min(lane + 64 * j, NT * groups - 1);
-        const int t = piece / groups, off = (piece - t * groups) * 16;
-        const uint8_t* base = cs[0] - (size_t)ln * groups;
-#pragma unroll
-        for (int t2 = 1; t2 < NT; ++t2)
-          if (t == t2) base = cs[t2] - (size_t)ln * groups;
-        scn[j] = *reinterpret_cast<const u32x4*>(base + ahead + off);
-      }
+      for (int j = 0; j < kScMax; ++j)
+        scn[j] = *reinterpret_cast<const u32x4*>(sc_unit + ahead + sc_piece[j]);
     };
     auto park_scales = [&]() {
 #pragma unroll
       for (int j = 0; j < kScMax; ++j) {
         const int piece = lane + 64 * j;
-        if (piece < NT * groups) {
-          const int t = piece / groups, off = (piece - t * groups) * 16;
-          *reinterpret_cast<u32x4*>(sc_lds + t * sc_tile_bytes + off) = scn[j];
-        }
+        if (piece < NT * groups) *reinterpret_cast<u32x4*>(sc_lds + piece * 16) = scn[j];
       }
     };
 
 
     // Start of a pass's weight stream: pointers of the wavefront's first unit,
-    // its scale block and the first D steps.  Issued before anything else of
-    // the pass (it depends on the run alone, not on the rows), so the loads
-    // are under way while the rows are fetched, split and written; a
-    // wavefront without units loads the slice's first unit and drops it.
+    // its scale block and the first D steps.  Issued right behind the row loads
+    // of the pass, so the weights are under way while the rows are split and
+    // written; a wavefront without units loads the slice's first unit and drops it.
     Stage st[D];
-    bool primed = false;
     auto prime = [&]() {
       unit_tiles<STAGE, NT>(p, e, n_my > 0 ? first : u0, ln, cw, cs, col0);
+      sc_unit = cs[0] - (size_t)ln * groups;
 #pragma unroll
       for (int t = 0; t < NT; ++t) lrow[t] = cw[t];
       ld_ks = 0;
@@ -597,16 +622,18 @@ __global__ __launch_bounds__(64 * WAVES) void stream_resident_kernel(GemmArgs p)
       fetch_scales(0);
 #pragma unroll
       for (int i = 0; i < D; ++i) issue(st[i]);
-      primed = true;
     };
 
     // Passes of 16 rows, four at a time: one load brings the ids of 64 rows,
     // and a pass none of whose rows is routed is skipped.
     for (int tile0 = 0; tile0 < run_tiles; tile0 += 4) {
-      if (!primed) prime();
       int fl = -1;
-      if (r == r_first && tile0 == 0) fl = first_ids[lane];
-      else if (tile0 * 16 + lane < run_tiles * 16) fl = p.sorted_ids[run_row0 + tile0 * 16 + lane];
+      if (tile0 * 16 + lane < run_tiles * 16) {
+        const int at = run_row0 + tile0 * 16 + lane;
+        // uniform: the first rows a workgroup stages come from the copy in LDS
+        if (pass_no == 0 && run_row0 + tile0 * 16 + 64 <= ids_cached) fl = ids_lds[at];
+        else fl = p.sorted_ids[at];
+      }
       if (fl < 0 || fl >= p.n_flat) fl = -1;
       const unsigned long long routed = __ballot(fl >= 0);
       for (int tt = 0; tt < 4; ++tt) {
@@ -617,8 +644,6 @@ __global__ __launch_bounds__(64 * WAVES) void stream_resident_kernel(GemmArgs p)
         const int srow = run_row0 + tile * 16 + ln;
         const int flag = pass_no & 1;
         ++pass_no;
-        if (!primed) prime();
-        primed = false;  // this pass consumes the stream
 
         // ---- stage the 16 rows, all of K, as MFMA operands --------------------
         // Lane (j, d) = (lane / 4, lane % 4) takes the 8 values k = 32 g + 8 d ..
@@ -638,13 +663,14 @@ __global__ __launch_bounds__(64 * WAVES) void stream_resident_kernel(GemmArgs p)
                                                       : run_row0 + tile * 16 + sj)
                                         : 0) * (size_t)p.a_stride;
         u32x4 v[kBatch];
+        const uint16_t* piece0 = src + (st_flat >= 0 && my_groups > 0 ? wave * 32 + sd * 8 : 0);
+        const int piece_stride = st_flat >= 0 ? WAVES * 32 : 0;
 #pragma unroll
         for (int it = 0; it < kBatch; ++it) {
-          const int pq = wave + it * WAVES;
-          // branch-free: an invalid piece reads the row's first bytes instead
-          const bool valid = pq < groups && st_flat >= 0;
-          v[it] = *reinterpret_cast<const u32x4*>(src + (valid ? pq * 32 + sd * 8 : 0));
+          // branch-free: an invalid piece reads the first piece (the row's first bytes) instead
+          v[it] = *reinterpret_cast<const u32x4*>(piece0 + (it < my_groups ? it * piece_stride : 0));
         }
+        prime();
         // Block scale byte of piece `it` (0 = outside the fast path's range).
         auto block_scale = [&](int it) -> uint32_t {
           uint32_t emax = bf16x8_max_exponent(v[it]);
@@ -661,19 +687,17 @@ __global__ __launch_bounds__(64 * WAVES) void stream_resident_kernel(GemmArgs p)
         auto write_rows = [&](int upto) {
 #pragma unroll
           for (int it = 0; it < kBatch; ++it) {
-            const int pq = wave + it * WAVES;
-            if (it >= staged && it < upto && pq < nsteps * 4) {
+            if (it >= staged && it < upto && it < my_pieces) {
               uint32_t sb = block_scale(it);
               if (sb == 0u) sb = 127u;  // the pass takes the exact path; keep the bytes defined
               uint2 hi, lo;
               split_bf16x8(v[it], sb, hi, lo);
-              const int ks = pq >> 2, qq = pq & 3;
-              const int slot = ((qq & 1) * 2 + (sd >> 1)) * 16 + sj;
-              uint8_t* plane = reinterpret_cast<uint8_t*>(b_lds) +
-                               (size_t)(((ks * 2) * 2 + (qq >> 1)) * 64 + slot) * 16 + (sd & 1) * 8;
+              // piece `it` is group wave + it * WAVES: K step (wave / 4) + it * (WAVES / 4),
+              // quarter wave % 4 of it, so its places are those of piece 0 plus constants
+              uint8_t* plane = plane0 + it * (WAVES / 4) * 4096;
               *reinterpret_cast<uint2*>(plane) = hi;
               *reinterpret_cast<uint2*>(plane + 2 * 64 * 16) = lo;
-              if (sd == 0) bsc_lds[ks * 64 + qq * 16 + sj] = (uint8_t)sb;
+              if (sd == 0) bsc0[it * (WAVES / 4) * 64] = (uint8_t)sb;
             }
           }
           staged = upto;
@@ -685,9 +709,8 @@ __global__ __launch_bounds__(64 * WAVES) void stream_resident_kernel(GemmArgs p)
           bool slow = false;
 #pragma unroll
           for (int it = 0; it < kBatch; ++it) {
-            const int pq = wave + it * WAVES;
-            if (!(pq < groups && st_flat >= 0)) v[it] = u32x4{0u, 0u, 0u, 0u};
-            if (pq < nsteps * 4) slow |= block_scale(it) == 0u;
+            if (!(it < my_groups && st_flat >= 0)) v[it] = u32x4{0u, 0u, 0u, 0u};
+            if (it < my_pieces) slow |= block_scale(it) == 0u;
           }
           __syncthreads();  // the previous pass is done with the planes and with its flag
           if (slow) pass_slow[flag] = 1;
@@ -780,6 +803,7 @@ __global__ __launch_bounds__(64 * WAVES) void stream_resident_kernel(GemmArgs p)
                       cs[t] += s_unit_stride;
                       col0[t] += WAVES * (STAGE == 0 ? 8 * NT : 16 * NT);
                     }
+                    sc_unit += s_unit_stride;
                     if (cunit + 1 < n_my) fetch_scales(s_unit_stride);
                   }
                   cks = 0;
@@ -873,7 +897,7 @@ __global__ __launch_bounds__(64 * kTileWaves, 2) void tile_gemm_kernel(GemmArgs 
   __shared__ int row_flat[MT * 16];
   __shared__ int group_slow;
 
-  if (STAGE == 0) clear_out_share(p);
+  if (STAGE == 0) clear_out_share<64 * kTileWaves>(p);
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -1115,7 +1139,7 @@ __global__ __launch_bounds__(64 * kWideWaves) void tile_wide_kernel(GemmArgs p) 
   __shared__ int row_flat[kWideRows];
   __shared__ int wave_valid[2];
 
-  if (STAGE == 0) clear_out_share(p);
+  if (STAGE == 0) clear_out_share<64 * kWideWaves>(p);
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -1608,7 +1632,7 @@ StagePlan plan_stage(const GemmArgs& g) {
   pl.resident_lds = (size_t)nsteps * (4096 + 64) + (size_t)pl.waves * pl.nt * 16 * groups;
   const int res_units = STAGE == 0 ? g.ncols / (8 * pl.nt) : g.ncols / (16 * pl.nt);
   if (pl.resident_lds > kResidentLdsLimit || g.num_blocks > kMaxRuns ||
-      pl.nt * groups > 64 * kScMax ||
+      pl.nt * groups > 64 * resident_scale_pieces(pl.waves) ||
       (res_units + pl.waves - 1) / pl.waves > 64 ||  // one bit per unit in a wavefront's redo mask
       nsteps * 4 > resident_batch(pl.waves) * pl.waves)  // the rows are staged in one batch
     pl.variant = kMoeVariantLds;
