@@ -241,13 +241,25 @@ __device__ __forceinline__ void unit_tiles(const GemmArgs& p, int e, int unit, i
 // per tile) are fetched with a few coalesced loads while the previous unit
 // streams and parked in a per-wavefront LDS region.
 //
+// Start-up.  Until the stream runs, a workgroup is a chain of dependent steps
+// on an otherwise idle compute unit, where every instruction and every round
+// trip to memory is paid in full (about 10 us of a 65 us kernel at 2880 x
+// 2880 x 32 experts, 64 tokens).  So: wavefront 0 lists the runs with one
+// round trip (a block's expert and both neighbours' loaded together) and
+// finds the slice with ballots, a lane per run, no reductions; meanwhile the
+// other wavefronts copy the head of sorted_ids to LDS, so the ids of the first
+// rows are an LDS read; offsets that depend on the piece index alone are
+// compile-time constants (a wavefront's pieces keep their quarter of a K
+// step); the scale pieces of a unit are addressed without divisions.
+//
 // Order within a pass.  The memory pipe of a compute unit returns data in the
-// order of issue, and a pass starts with a burst of loads, so: (1) the first
-// D steps of the weight stream, which depend on the run alone, (2) the row
-// ids, (3) the rows, then the barrier with the previous pass.  The rows are
-// split and written in K order, a few K steps ahead of the first unit's
-// arithmetic with a barrier after each portion, so the stream starts after
-// the first portion and the rest of the splitting overlaps it.
+// order of issue, and the stream cannot start before the rows are staged, so:
+// (1) the row ids, (2) the rows, (3) the first D steps of the weight stream,
+// which then are on their way while the rows are checked, split and written,
+// then the barrier with the previous pass.  The rows are split and written in
+// K order, a few K steps ahead of the first unit's arithmetic with a barrier
+// after each portion, so the stream starts after the first portion and the
+// rest of the splitting overlaps it.
 //
 // LDS operand planes of K step ks: [term hi/lo][half h][64 lanes] x 16 bytes;
 // lane (n, q') of half h holds the 16 values k = 128 ks + 64 h + 16 q' + 0..15
@@ -258,7 +270,7 @@ __device__ __forceinline__ void unit_tiles(const GemmArgs& p, int e, int unit, i
 constexpr int kMaxRuns = 512;   // runs the resident kernel can list in LDS
 // 16-byte scale pieces of a unit a lane holds: NT * K/32 <= 64 * resident_scale_pieces.
 // Workgroups of 8 wavefronts stage K <= 3072 (resident_batch), 96 groups, and have
-// 256 registers a lane: three pieces and not four keeps the kernel clear of scratch memory.
+// 256 registers a lane: three pieces are enough there, and a fourth would cost four registers.
 __host__ __device__ constexpr int resident_scale_pieces(int waves) { return waves == 4 ? 4 : 3; }
 
 typedef __attribute__((ext_vector_type(8))) int i32x8;
@@ -368,6 +380,23 @@ __device__ __forceinline__ void split_bf16x8(u32x4 v, uint32_t sb, uint2& hi, ui
 // register file each, K <= 4096.
 __host__ __device__ constexpr int resident_batch(int waves) { return waves == 4 ? 32 : 96 / waves; }
 
+// Profiling build only (-DVK_DECODE_TRACE, `python -m vkernels_amd.build --define
+// VK_DECODE_TRACE --out DIR`; read by vkernels_amd/decode_trace.py): thread 0 of every
+// workgroup stamps the device's 100 MHz clock at the steps of the kernel's start and at
+// its end, for its first pass.  vk_debug_decode_trace copies the stamps of the last
+// launches of both stages out.  The product build compiles none of this.
+#ifdef VK_DECODE_TRACE
+constexpr int kTraceWorkgroups = 1024, kTraceSlots = 12;
+__device__ unsigned long long g_decode_trace[2][kTraceWorkgroups][kTraceSlots];
+#define DECODE_TRACE(slot_)                                                             \
+  do {                                                                                  \
+    if (threadIdx.x == 0 && blockIdx.x < kTraceWorkgroups)                              \
+      g_decode_trace[STAGE][blockIdx.x][slot_] = wall_clock64();                        \
+  } while (0)
+#else
+#define DECODE_TRACE(slot_) do { } while (0)
+#endif
+
 template <int STAGE, int WAVES, int NT, int D>
 __global__ __launch_bounds__(64 * WAVES) void stream_resident_kernel(GemmArgs p) {
   extern __shared__ u32x4 b_lds[];  // [nsteps][2][2][64] operand planes, block scales, weight scales
@@ -377,6 +406,7 @@ __global__ __launch_bounds__(64 * WAVES) void stream_resident_kernel(GemmArgs p)
   __shared__ int run_cum[kMaxRuns];     // blocks of the runs up to and including this one
   __shared__ int slice_sh[2];           // this workgroup's slice of the (run, unit) space
   __shared__ int pass_slow[2];          // set while staging: this pass takes the exact path
+  DECODE_TRACE(0);  // entry
   if (STAGE == 0) clear_out_share<64 * WAVES>(p);
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -444,6 +474,7 @@ __global__ __launch_bounds__(64 * WAVES) void stream_resident_kernel(GemmArgs p)
       listed_blocks += (int)__popcll(mv);
     }
     n = n < kMaxRuns ? n : kMaxRuns;
+    DECODE_TRACE(5);  // runs listed
     if (lane == 0) {
       pass_slow[0] = 0;
       pass_slow[1] = 0;
@@ -499,6 +530,7 @@ __global__ __launch_bounds__(64 * WAVES) void stream_resident_kernel(GemmArgs p)
     }
   }
   __syncthreads();
+  DECODE_TRACE(1);  // slice known to every wavefront
   const int s0 = slice_sh[0], s1 = slice_sh[1];  // n_runs * units is far below 2^31
   if (s0 >= s1) return;  // uniform over the workgroup
   const int r_first = s0 / units;
@@ -662,6 +694,7 @@ __global__ __launch_bounds__(64 * WAVES) void stream_resident_kernel(GemmArgs p)
             p.A + (size_t)(st_flat >= 0 ? (STAGE == 0 ? st_flat / p.top_k
                                                       : run_row0 + tile * 16 + sj)
                                         : 0) * (size_t)p.a_stride;
+        if (pass_no == 1) DECODE_TRACE(6);  // set-up of the loops done
         u32x4 v[kBatch];
         const uint16_t* piece0 = src + (st_flat >= 0 && my_groups > 0 ? wave * 32 + sd * 8 : 0);
         const int piece_stride = st_flat >= 0 ? WAVES * 32 : 0;
@@ -671,6 +704,7 @@ __global__ __launch_bounds__(64 * WAVES) void stream_resident_kernel(GemmArgs p)
           v[it] = *reinterpret_cast<const u32x4*>(piece0 + (it < my_groups ? it * piece_stride : 0));
         }
         prime();
+        if (pass_no == 1) DECODE_TRACE(7);  // rows and first weight steps asked for
         // Block scale byte of piece `it` (0 = outside the fast path's range).
         auto block_scale = [&](int it) -> uint32_t {
           uint32_t emax = bf16x8_max_exponent(v[it]);
@@ -712,18 +746,23 @@ __global__ __launch_bounds__(64 * WAVES) void stream_resident_kernel(GemmArgs p)
             if (!(it < my_groups && st_flat >= 0)) v[it] = u32x4{0u, 0u, 0u, 0u};
             if (it < my_pieces) slow |= block_scale(it) == 0u;
           }
+          if (pass_no == 1) DECODE_TRACE(2);  // this wavefront's rows are in and checked
           __syncthreads();  // the previous pass is done with the planes and with its flag
           if (slow) pass_slow[flag] = 1;
         }
+        if (pass_no == 1) DECODE_TRACE(8);  // every wavefront's are
         // The rows are staged in K order, a few K steps ahead of the first unit's
         // arithmetic, with a barrier after each portion: the weight stream starts
         // after the first portion and the rest of the splitting overlaps it.
         write_rows(pieces_for(min(nsteps, D)));
+        if (pass_no == 1) DECODE_TRACE(9);  // first K steps split and written
         if (n_my > 0) {
           park_scales();
           if (n_my > 1) fetch_scales(s_unit_stride);
         }
+        if (pass_no == 1) DECODE_TRACE(10);  // scales parked
         __syncthreads();
+        if (pass_no == 1) DECODE_TRACE(3);  // the stream starts
         if (tid == 0) pass_slow[flag ^ 1] = 0;  // for the next pass; its last reader is behind us
         const bool slow_pass = pass_slow[flag] != 0;
         if (n_my == 0 || slow_pass) {
@@ -833,6 +872,7 @@ __global__ __launch_bounds__(64 * WAVES) void stream_resident_kernel(GemmArgs p)
       }
     }
   }
+  DECODE_TRACE(4);  // end
 }
 
 // Stage 0 with a workspace: 32 consecutive act columns (two 16-column tiles, first
@@ -1375,7 +1415,8 @@ __global__ __launch_bounds__(64 * kWideWaves) void tile_wide_kernel(GemmArgs p) 
           // operations before the barrier: two per row tile but the last (all at once
           // where the step has a single tile, or does no arithmetic)
           constexpr int kBefore = 13;
-          constexpr int kPer = LIVE > 1 ? (kBefore + 2 * (LIVE - 1) - 1) / (2 * (LIVE - 1)) : kBefore;
+          constexpr int kSlots = LIVE > 1 ? 2 * (LIVE - 1) : 1;  // places between the tiles' halves
+          constexpr int kPer = (kBefore + kSlots - 1) / kSlots;
           auto before = [&](int first) {
 #pragma unroll
             for (int k = first; k < first + kPer; ++k)
@@ -1930,3 +1971,11 @@ void launch_fused_moe(const FusedMoeArgs& a, hipStream_t stream) {
 }
 
 }  // namespace vk
+
+#ifdef VK_DECODE_TRACE
+// Copies the stamps of the last decode launches to host memory:
+// [2 stages][1024 workgroups][12 stamps] of 64 bits.  Synchronous.
+extern "C" int vk_debug_decode_trace(void* host_buffer) {
+  return (int)hipMemcpyFromSymbol(host_buffer, HIP_SYMBOL(vk::g_decode_trace), sizeof(vk::g_decode_trace));
+}
+#endif
