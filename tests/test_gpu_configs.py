@@ -253,6 +253,20 @@ def test_block_sizes(bs):
     _check(cfg, T, w, A, lg, block_size=bs)
 
 
+def test_decode_with_more_sorted_rows_than_the_kernel_copies_to_lds():
+    """Many experts and a short K.  The decode kernel copies the head of sorted_ids to LDS
+    (1024 ids per K step of its operand planes: 2048 here) and reads the ids of the runs
+    behind that from memory; both ways are taken here, in both stages, and with more than
+    64 blocks the run listing takes several rounds."""
+    cfg = synth.MoEConfig("c9", 256, 256, 256, 8, (40,), "uniform")
+    T, seed = 40, 9040
+    w = _weights(cfg, 9000)
+    A, lg = _inputs(cfg, T, seed)
+    g, _ = _check(cfg, T, w, A, lg)
+    assert g["bs"] == 16 and T * cfg.top_k <= 512, "not a decode-sized call"
+    assert g["EM"] > 2048 + 64, "every run's ids fit the copy in LDS"
+
+
 @pytest.mark.parametrize("use_workspace", [True, False])
 @pytest.mark.parametrize("bs", [16, 48, 80, 128])
 def test_tile_kernels_block_sizes(bs, use_workspace):
