@@ -62,6 +62,9 @@ def parse_args():
     ap.add_argument("--no-modes", action="store_true",
                     help="skip the prefill record's other arithmetic modes (2 <-> 3 terms, W4A4)")
     ap.add_argument("--w4a4", action="store_true", help="top-level record in the W4A4 mode (prefill sizes)")
+    ap.add_argument("--epilogue", default="plain", choices=("plain", "bias_limit", "situ_bias"),
+                    help="what the first stage's epilogue applies besides the activation: nothing; both "
+                         "biases and swiglu_limit 7.0; the SiTU activation (beta 3, linear_beta 20) and both biases")
     ap.add_argument("--weight-sets", type=int, default=0, help="0 = enough to exceed 1 GiB")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--block-size", type=int, default=0)
@@ -162,10 +165,18 @@ def run_workload(args, workload, steps, warmup, prepack, split_terms=None, w4a4=
     if per_set > (1 << 30):
         n_sets = 1  # one set is already several times the Infinity Cache
     experts = []
+    epi = {}
+    if args.epilogue != "plain":
+        epi.update(b13=torch.from_numpy((synth.rand_normal((cfg.E, 2 * I), seed, 21) * 0.5).astype(np.float32)).to(dev),
+                   b2=torch.from_numpy((synth.rand_normal((cfg.E, H), seed, 22) * 0.5).astype(np.float32)).to(dev))
+        if args.epilogue == "bias_limit":
+            epi.update(swiglu_limit=7.0)
+        else:
+            epi.update(activation="situ", beta=3.0, linear_beta=20.0)
     for s in range(n_sets):
         w = synth.make_weights(cfg.E, H, I, seed + 7919 * s, device=dev)
         experts.append(ve.FusedExperts(w.w13, w.w13_scale, w.w2, w.w2_scale, prepack=prepack,
-                                       split_terms=terms or None, w4a4=w4a4 and prepack))
+                                       split_terms=terms or None, w4a4=w4a4 and prepack, **epi))
         if args.no_workspace:
             experts[-1].use_workspace = False
     A_bits = synth.make_activations(T, H, seed)
@@ -202,12 +213,12 @@ def run_workload(args, workload, steps, warmup, prepack, split_terms=None, w4a4=
         e0.record()
         lib.vk_hip_moe_gateup_mxfp4(
             ve._ptr(A), ve._ptr(fe.w13), ve._ptr(fe.w13_scale), ve._ptr(act), T, H, I,
-            k, ve._ptr(sids), ve._ptr(eids), max_em, ve._F(0.0), 0, ve._F(4.0),
-            ve._F(25.0), None, bs, st)
+            k, ve._ptr(sids), ve._ptr(eids), max_em, ve._F(float(fe.swiglu_limit)), fe.activation,
+            ve._F(float(fe.beta)), ve._F(float(fe.linear_beta)), ve._ptr(fe.b13), bs, st)
         e1.record()
         lib.vk_hip_moe_down_mxfp4(
             ve._ptr(act), ve._ptr(fe.w2), ve._ptr(fe.w2_scale), ve._ptr(w), ve._ptr(out), T,
-            H, I, k, ve._ptr(sids), ve._ptr(eids), max_em, None, bs, st)
+            H, I, k, ve._ptr(sids), ve._ptr(eids), max_em, ve._ptr(fe.b2), bs, st)
         e2.record()
 
     for i in range(warmup):
@@ -284,6 +295,7 @@ def run_workload(args, workload, steps, warmup, prepack, split_terms=None, w4a4=
                         f"top-{k}, MXFP4 weights, bf16 activations, {cfg.logits} routing",
             "block_size": bs, "active_experts": active, "weight_sets": n_sets,
             "weights": "prepacked at load time (+ raw)" if prepack else "raw",
+            "epilogue": args.epilogue,
         },
         "roofline": roofline,
         "layer": {

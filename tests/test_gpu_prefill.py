@@ -332,8 +332,11 @@ def test_config4_prepacked(T):
     _check_prefill(cfg, T, w, A, lg, contract_only=True)
 
 
-@pytest.mark.parametrize("variant", ["bias", "limit", "situ_bias"])
+@pytest.mark.parametrize("variant", ["bias", "limit", "bias_limit", "situ", "situ_bias"])
 def test_epilogue_variants_prepacked(variant):
+    """The first stage's epilogue is compiled per combination of bias, clamp and activation
+    (a clamp that is off runs as a clamp at infinity next to a bias, SiTU without biases
+    adds zeros): every combination that takes a different loop."""
     cfg = synth.CONFIGS["c1"]
     T, seed = 200, 1500
     w = cfgs._weights(cfg, seed)
@@ -344,7 +347,7 @@ def test_epilogue_variants_prepacked(variant):
     if "bias" in variant:
         gpu_kw.update(b13=to_dev(b13), b2=to_dev(b2))
         cpu_kw.update(b13=b13, b2=b2)
-    if variant == "limit":
+    if "limit" in variant:
         gpu_kw.update(swiglu_limit=1.5)
         cpu_kw.update(swiglu_limit=1.5)
     if "situ" in variant:

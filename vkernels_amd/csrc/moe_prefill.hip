@@ -759,6 +759,28 @@ __global__ __launch_bounds__(64 * kMxWaves) void tile_mx_kernel(MxArgs p) {
     auto wave_fence = [] {  // LDS operations of a wavefront execute in order; this keeps the compiler's too
       __asm__ volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
     };
+    // The biases of the columns this lane holds (the same for every row tile), tile by
+    // tile as the accumulators are laid out: asked for here, all at once, not value by
+    // value inside the loops below.
+    const bool has_bias = p.bias != nullptr;  // uniform
+    f32x4 bias_v[4][4];  // [tile][row group]
+    if (has_bias) {
+      // stage 0: tiles 0, 1 = gate columns, 2, 3 = the same columns of up
+      // stage 1: the last unit may be ragged (ncols is a multiple of 64); its columns past
+      // the end are not stored, so the first tiles' biases stand in
+      const float* b = p.bias + (STAGE == 0 ? (size_t)e * (size_t)(2 * p.ncols) + unit * 64
+                                            : (size_t)e * (size_t)p.ncols + unit * kMxUnitRows) + hh * 4;
+#pragma unroll
+      for (int t = 0; t < 4; ++t) {
+        const int c = STAGE == 0 ? (t >> 1) * p.ncols + (t & 1) * 32
+                                 : (unit * kMxUnitRows + (t >> 1) * 64 < p.ncols ? t * 32 : 0);
+#pragma unroll
+        for (int rg = 0; rg < 4; ++rg) bias_v[t][rg] = *reinterpret_cast<const f32x4*>(b + c + rg * 8);
+      }
+    } else if (STAGE == 0 && p.activation == 1) {  // the one loop that adds them without a bias
+#pragma unroll
+      for (int i = 0; i < 16; ++i) bias_v[i >> 2][i & 3] = f32x4{0.f, 0.f, 0.f, 0.f};
+    }
 #pragma unroll
     for (int m = 0; m < 4; ++m) {
       if (m >= n_live) break;
@@ -778,31 +800,44 @@ __global__ __launch_bounds__(64 * kMxWaves) void tile_mx_kernel(MxArgs p) {
       }
       if (STAGE == 0) {
         constexpr int kPitch = kMxActPitch;
-        // 128 activation values per lane and row tile: the plain SwiGLU (no bias, no
-        // clamp), which is what serving runs, gets a loop of its own without a branch per
-        // value; the same act_value with its parameters known at compile time.
-        auto act_rows = [&](auto plain_c) {
-          constexpr bool kPlain = decltype(plain_c)::value != 0;
-          const float* bias = p.bias != nullptr ? p.bias + (size_t)e * (size_t)(2 * p.ncols) : nullptr;
+        // 128 activation values per lane and row tile.  A wavefront runs alone on its SIMD,
+        // so a branch per value (bias or not, clamp or not, which activation) is paid in
+        // full: the loop is compiled once per combination of what is uniform, act_value's
+        // formulas with their parameters known at compile time.
+        auto act_rows = [&](auto bias_c, auto limit_c, auto situ_c) {
+          constexpr bool kBias = decltype(bias_c)::value != 0, kLimit = decltype(limit_c)::value != 0,
+                         kSitu = decltype(situ_c)::value != 0;
+          float limit = 0.0f, beta = 0.0f, linear_beta = 0.0f, inv_beta = 0.0f, inv_linear_beta = 0.0f;
+          if constexpr (kLimit) limit = p.swiglu_limit > 0.0f ? p.swiglu_limit : __builtin_inff();
+          if constexpr (kSitu) {
+            beta = p.beta;
+            linear_beta = p.linear_beta;
+            inv_beta = __builtin_amdgcn_rcpf(beta);
+            inv_linear_beta = linear_beta > 0.0f ? __builtin_amdgcn_rcpf(linear_beta) : 0.0f;
+          }
 #pragma unroll
           for (int tp = 0; tp < 2; ++tp)
 #pragma unroll
             for (int rg = 0; rg < 4; ++rg) {
               const int cl = tp * 32 + rg * 8 + hh * 4;  // column within the unit's 64
-              const int col = unit * 64 + cl;
               uint32_t packed[2];
 #pragma unroll
               for (int i = 0; i < 4; ++i) {
                 float g = tile[tp][rg * 4 + i], u = tile[tp + 2][rg * 4 + i];
+                if constexpr (kBias) {
+                  g += bias_v[tp][rg][i];
+                  u += bias_v[tp + 2][rg][i];
+                }
                 float a;
-                if constexpr (kPlain) {
-                  a = act_value(0, g, u, 0.0f, 0.0f, 0.0f);
+                if constexpr (kSitu) {
+                  a = situ_value(g, u, beta, inv_beta, linear_beta, inv_linear_beta);
                 } else {
-                  if (bias != nullptr) {
-                    g += bias[col + i];
-                    u += bias[p.ncols + col + i];
+                  if constexpr (kLimit) {
+                    g = g > limit ? limit : g;  // (a NaN stays one, as in act_value)
+                    u = u > limit ? limit : u;
+                    u = u < -limit ? -limit : u;
                   }
-                  a = act_value(p.activation, g, u, p.swiglu_limit, p.beta, p.linear_beta);
+                  a = act_value(0, g, u, 0.0f, 0.0f, 0.0f);
                 }
                 const uint32_t v = f32_to_bf16_bits(a);
                 if (i & 1) packed[i >> 1] |= v << 16;
@@ -812,8 +847,13 @@ __global__ __launch_bounds__(64 * kMxWaves) void tile_mx_kernel(MxArgs p) {
             }
         };
         if (flat >= 0) {
-          if (p.activation == 0 && !(p.swiglu_limit > 0.0f) && p.bias == nullptr) act_rows(IntC<1>{});
-          else act_rows(IntC<0>{});
+          // (uniform conditions.  Four loops, not eight: a clamp that is off is a clamp at
+          // infinity, and SiTU without biases adds zeros)
+          const bool clamp = p.swiglu_limit > 0.0f;
+          if (p.activation == 1) act_rows(IntC<1>{}, IntC<0>{}, IntC<1>{});
+          else if (has_bias) act_rows(IntC<1>{}, IntC<1>{}, IntC<0>{});
+          else if (clamp) act_rows(IntC<0>{}, IntC<1>{}, IntC<0>{});
+          else act_rows(IntC<0>{}, IntC<0>{}, IntC<0>{});
         }
         wave_fence();
         u32x4 v[4];  // all the reads, one wait, then the stores: 8 rows x 128 bytes per instruction
@@ -852,8 +892,7 @@ __global__ __launch_bounds__(64 * kMxWaves) void tile_mx_kernel(MxArgs p) {
                 const int t = 2 * tp + tl;
                 const int cl = tl * 32 + rg * 8 + hh * 4;
                 f32x4 v = {tile[t][rg * 4], tile[t][rg * 4 + 1], tile[t][rg * 4 + 2], tile[t][rg * 4 + 3]};
-                if constexpr (kBias)
-                  v += *reinterpret_cast<const f32x4*>(p.bias + (size_t)e * (size_t)p.ncols + col0 + cl);
+                if constexpr (kBias) v += bias_v[t][rg];
                 *reinterpret_cast<f32x4*>(stage_lds + ln * kPitch + cl * 4) = v * w;
               }
             wave_fence();
@@ -875,7 +914,7 @@ __global__ __launch_bounds__(64 * kMxWaves) void tile_mx_kernel(MxArgs p) {
           }
         };
         const bool inside = row0 + m * 32 + 32 <= win_end;  // uniform
-        if (p.bias == nullptr) {
+        if (!has_bias) {
           if (inside) store_rows(IntC<0>{}, IntC<0>{});
           else store_rows(IntC<0>{}, IntC<1>{});
         } else {

@@ -21,6 +21,8 @@ def main() -> None:
     ap.add_argument("--split-terms", type=int, default=0, choices=(0, 2, 3),
                     help="0 = the library's default (3 FP6 terms in the first stage, 2 in the second)")
     ap.add_argument("--w4a4", action="store_true")
+    ap.add_argument("--epilogue", default="plain", choices=("plain", "bias_limit", "situ_bias"),
+                    help="as bench.py's: both biases and swiglu_limit 7.0, or SiTU (beta 3, linear_beta 20) and both biases")
     args = ap.parse_args()
 
     import torch
@@ -36,8 +38,16 @@ def main() -> None:
     cfg, T = synth.CONFIGS[name], int(t_str)
     dev = torch.device("cuda", 0)
     w = synth.make_weights(cfg.E, cfg.H, cfg.I, 5, device=dev)
+    epi = {}
+    if args.epilogue != "plain":
+        epi.update(b13=torch.from_numpy((synth.rand_normal((cfg.E, 2 * cfg.I), 5, 21) * 0.5).astype(np.float32)).to(dev),
+                   b2=torch.from_numpy((synth.rand_normal((cfg.E, cfg.H), 5, 22) * 0.5).astype(np.float32)).to(dev))
+        if args.epilogue == "bias_limit":
+            epi.update(swiglu_limit=7.0)
+        else:
+            epi.update(activation="situ", beta=3.0, linear_beta=20.0)
     fe = ve.FusedExperts(w.w13, w.w13_scale, w.w2, w.w2_scale, prepack=True, split_terms=args.split_terms or None,
-                         w4a4=args.w4a4)
+                         w4a4=args.w4a4, **epi)
     a_bits = synth.make_activations(T, cfg.H, 5)
     A = torch.from_numpy(a_bits.view(np.int16)).view(torch.bfloat16).to(dev)
     logits = torch.from_numpy(synth.make_logits(cfg.logits, T, cfg.E, 5, a_bits, cfg.H)).to(dev)
