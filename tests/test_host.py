@@ -268,6 +268,11 @@ def test_entry_points_reject_contract_violations_without_a_device(lib):
         16, None)                                                             # hidden not /64
     assert lib.vk_last_error_code() != 0 and b"vk_hip_fused_moe_mxfp4" in lib.vk_last_error()
     lib.vk_set_last_error(0, b"")
+    odd = P(ctypes.addressof(buf) + 4)
+    moe(p, p, p, p, p, p, p, p, p, 4, 128, 128, 2, p, p, 64, F(0), 0, F(4), F(25), odd, None,
+        16, None)                                                             # bias not 16-byte aligned
+    assert lib.vk_last_error_code() != 0 and b"aligned" in lib.vk_last_error()
+    lib.vk_set_last_error(0, b"")
     moe(p, p, p, p, p, p, p, p, p, 0, 128, 128, 2, p, p, 64, F(0), 0, F(4), F(25), None, None,
         16, None)                                                             # nothing routed: no-op
     assert lib.vk_last_error_code() == 0

@@ -5,6 +5,7 @@
 
 #include <hip/hip_runtime.h>
 
+#include <cstdint>
 #include <cstring>
 #include <string>
 
@@ -69,6 +70,8 @@ bool layer_args_ok(const char* who, bool need13, bool need2, const vk::FusedMoeA
     why = "top_k must be positive";
   else if (a.block_size <= 0 || a.block_size % 16 != 0 || a.EM % a.block_size != 0)
     why = "block_size must be a multiple of 16 and divide EM";
+  else if (((reinterpret_cast<uintptr_t>(a.b13) | reinterpret_cast<uintptr_t>(a.b2)) & 15u) != 0)
+    why = "b13 and b2 must be 16-byte aligned (the kernels load four columns at a time)";
   if (why == nullptr) return true;
   vk_set_last_error(VK_ERROR_INVALID_ARGUMENT, (std::string(who) + ": " + why).c_str());
   return false;
@@ -372,6 +375,9 @@ int vk_hip_moe_combine(const float* partial, const float* b2, const float* topk_
   if (partial == nullptr || topk_w_sorted == nullptr || sorted_ids == nullptr || expert_ids == nullptr ||
       out == nullptr)
     return fail(VK_ERROR_INVALID_ARGUMENT, "vk_hip_moe_combine: buffers must not be null");
+  if (((reinterpret_cast<uintptr_t>(partial) | reinterpret_cast<uintptr_t>(b2) |
+        reinterpret_cast<uintptr_t>(out)) & 15u) != 0)
+    return fail(VK_ERROR_INVALID_ARGUMENT, "vk_hip_moe_combine: partial, b2 and out must be 16-byte aligned");
   if (workspace == nullptr || workspace_bytes < sizeof(int32_t) * (size_t)M * (size_t)top_k ||
       (reinterpret_cast<uintptr_t>(workspace) & 3) != 0)
     return fail(VK_ERROR_INVALID_ARGUMENT, "vk_hip_moe_combine: workspace must hold M * top_k int32 values");

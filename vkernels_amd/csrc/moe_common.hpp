@@ -12,15 +12,38 @@ namespace vk {
 // and rows outside go to the exact path.
 constexpr uint32_t kScaleLo = 64u, kScaleHi = 190u;
 
+// tanh for the SiTU epilogue: 1 - 2 / (1 + e^2x) with the
+// hardware's exponential and reciprocal (+-1 at the infinities, NaN for NaN), and the
+// series x - x^3/3 + 2 x^5/15 below |x| = 0.1, where the first form cancels (its error
+// there is below 1e-8 relative).  A few ulp, far inside the bf16 rounding that follows.
+__device__ __forceinline__ float tanh_fast(float x) {
+  const float big = 1.0f - 2.0f * __builtin_amdgcn_rcpf(1.0f + __expf(2.0f * x));
+  const float x2 = x * x;
+  const float small = x * (1.0f - x2 * (0.33333334f - x2 * 0.13333334f));
+  return fabsf(x) < 0.1f ? small : big;
+}
+
+// The SiTU activation (activation 1 of act_value; the reference's
+// beta * tanh(g / beta) * sigmoid(g) * linear_beta * tanh(u / linear_beta), the second
+// tanh left out when linear_beta <= 0) with those: inv_beta = 1 / beta,
+// inv_linear_beta = 1 / linear_beta (unused when linear_beta <= 0).
+__device__ __forceinline__ float situ_value(float g, float u, float beta, float inv_beta,
+                                            float linear_beta, float inv_linear_beta) {
+  // (below g = -87 the sigmoid is subnormal, which v_rcp_f32 flushes to zero: the
+  // reciprocal is taken of the denominator scaled by 2^-64 and scaled back by a multiply)
+  const float s = g < -87.0f ? 0x1p-64f : 1.0f;
+  const float sig = __builtin_amdgcn_rcpf((1.0f + __expf(-g)) * s) * s;
+  const float gate_out = beta * tanh_fast(g * inv_beta) * sig;
+  const float up_out = linear_beta > 0.0f ? linear_beta * tanh_fast(u * inv_linear_beta) : u;
+  return gate_out * up_out;
+}
+
 __device__ __forceinline__ float act_value(int activation, float g, float u,
                                            float limit, float beta,
                                            float linear_beta) {
-  if (activation == 1) {
-    const float sig = 1.0f / (1.0f + expf(-g));
-    const float gate_out = beta * tanhf(g / beta) * sig;
-    const float up_out = linear_beta > 0.0f ? linear_beta * tanhf(u / linear_beta) : u;
-    return gate_out * up_out;
-  }
+  if (activation == 1)
+    return situ_value(g, u, beta, __builtin_amdgcn_rcpf(beta), linear_beta,
+                      linear_beta > 0.0f ? __builtin_amdgcn_rcpf(linear_beta) : 0.0f);
   if (limit > 0.0f) {
     if (g > limit) g = limit;
     if (u > limit) u = limit;
@@ -32,27 +55,6 @@ __device__ __forceinline__ float act_value(int activation, float g, float u,
   // reciprocal is taken of the denominator scaled by 2^-64 and scaled back by a multiply.
   const float s = g < -87.0f ? 0x1p-64f : 1.0f;
   return (g * (__builtin_amdgcn_rcpf((1.0f + __expf(-g)) * s) * s)) * u;
-}
-
-// tanh for the SiTU epilogue of the prefill kernels: 1 - 2 / (1 + e^2x) with the
-// hardware's exponential and reciprocal (+-1 at the infinities, NaN for NaN), and the
-// series x - x^3/3 + 2 x^5/15 below |x| = 0.1, where the first form cancels (its error
-// there is below 1e-8 relative).  A few ulp, far inside the bf16 rounding that follows.
-__device__ __forceinline__ float tanh_fast(float x) {
-  const float big = 1.0f - 2.0f * __builtin_amdgcn_rcpf(1.0f + __expf(2.0f * x));
-  const float x2 = x * x;
-  const float small = x * (1.0f - x2 * (0.33333334f - x2 * 0.13333334f));
-  return fabsf(x) < 0.1f ? small : big;
-}
-
-// act_value's SiTU branch (activation 1) with those: inv_beta = 1 / beta,
-// inv_linear_beta = 1 / linear_beta (unused when linear_beta <= 0).
-__device__ __forceinline__ float situ_value(float g, float u, float beta, float inv_beta,
-                                            float linear_beta, float inv_linear_beta) {
-  const float sig = __builtin_amdgcn_rcpf(1.0f + __expf(-g));
-  const float gate_out = beta * tanh_fast(g * inv_beta) * sig;
-  const float up_out = linear_beta > 0.0f ? linear_beta * tanh_fast(u * inv_linear_beta) : u;
-  return gate_out * up_out;
 }
 
 __device__ __forceinline__ bf16x8 as_bf16x8(u32x4 v) {

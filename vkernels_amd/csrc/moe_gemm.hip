@@ -145,16 +145,17 @@ __device__ __forceinline__ void epilogue_tile(const GemmArgs& p, int e, const f3
 #pragma unroll
     for (int t = 0; t < NT / 2; ++t) {
       const int c = col0[t] + 4 * lq;
+      f32x4 gate = acc[t], up = acc[t + NT / 2];
+      if (p.bias != nullptr) {  // uniform; the lane's four columns in one load each
+        const float* b = p.bias + (size_t)e * (size_t)(2 * p.ncols) + c;
+        gate += *reinterpret_cast<const f32x4*>(b);
+        up += *reinterpret_cast<const f32x4*>(b + p.ncols);
+      }
       uint32_t packed[2];
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
-        float g = acc[t][r];
-        float u = acc[t + NT / 2][r];
-        if (p.bias != nullptr) {
-          const float* b = p.bias + (size_t)e * (size_t)(2 * p.ncols);
-          g += b[c + r];
-          u += b[p.ncols + c + r];
-        }
+        const float g = gate[r];
+        const float u = up[r];
         const uint32_t v = f32_to_bf16_bits(
             act_value(p.activation, g, u, p.swiglu_limit, p.beta, p.linear_beta));
         if (r & 1) packed[r >> 1] |= v << 16;
@@ -170,12 +171,11 @@ __device__ __forceinline__ void epilogue_tile(const GemmArgs& p, int e, const f3
 #pragma unroll
     for (int t = 0; t < NT; ++t) {
       const int c = col0[t] + 4 * lq;
+      f32x4 v = acc[t];
+      if (p.bias != nullptr)  // uniform
+        v += *reinterpret_cast<const f32x4*>(p.bias + (size_t)e * (size_t)p.ncols + c);
 #pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        float v = acc[t][r];
-        if (p.bias != nullptr) v += p.bias[(size_t)e * (size_t)p.ncols + c + r];
-        unsafeAtomicAdd(orow + c + r, v * w);
-      }
+      for (int r = 0; r < 4; ++r) unsafeAtomicAdd(orow + c + r, v[r] * w);
     }
   }
 }
