@@ -191,10 +191,12 @@ def run_workload(args, workload, steps, warmup, prepack, split_terms=None, w4a4=
 
     def step(i, events=None):
         fe = experts[i % n_sets]
-        ids, w = fe.route(logits, k, True)
         if events is None:
-            fe.apply(A, ids, w, block_size=bs, out_fp32=out)
+            # router and alignment through the library's one call (one launch at decode sizes)
+            ids, w, sids, eids, _, max_em, _ = fe.route_align(logits, k, True, bs)
+            fe.apply(A, ids, w, block_size=bs, out_fp32=out, aligned=(sids, eids, max_em))
             return
+        ids, w = fe.route(logits, k, True)
         # same launches, with events around the two GEMM stages (decode) or around
         # the fused call (prefill-sized batches, which run with a workspace)
         sids, eids, _, max_em = fe.align(ids, bs)

@@ -487,6 +487,22 @@ int vk_hip_moe_route_topk(const float* logits, int32_t T, int32_t E,
                           int32_t* topk_ids, float* topk_w, void* stream);
 
 /*
+ * Additive: vk_hip_moe_route_topk followed by vk_hip_moe_align_block_size,
+ * with the same arguments, results and errors as the two calls
+ * (num_experts = E).  No counterpart in the reference, whose router is a
+ * Python function (routing.py:59-157) and whose alignment is a call of its
+ * own (hip_capi.hpp:148-153).  For the smallest batches (T <= 16) the two
+ * are ONE launch: every workgroup of the alignment routes the tokens itself,
+ * a wavefront per token, and keeps the table in LDS.  A launch is a few
+ * microseconds, of a step of forty to eighty there.  Larger batches run the
+ * two kernels one after the other.
+ */
+int vk_hip_moe_route_align(const float* logits, int32_t T, int32_t E, int32_t top_k,
+                           int32_t renormalize, const int32_t* expert_map, int32_t block_size,
+                           int32_t local_n, int32_t max_EM, int32_t* topk_ids, float* topk_w,
+                           int32_t* sorted_ids, int32_t* expert_ids, int32_t* out_EM, void* stream);
+
+/*
  * Additive: dequantise an [N, K] tile of packed weights to bf16 with the
  * decode routines of the device library, written transposed as [K][N].
  * Device counterpart of dequant_weight_tile,

@@ -156,3 +156,45 @@ def test_align_matches_oracle_bitwise(hip_lib):
         assert int(out_em.item()) == rem, (M, k, bs, E, kind)
         assert np.array_equal(sids.cpu().numpy(), rs), (M, k, bs, E, kind)
         assert np.array_equal(eids.cpu().numpy(), re), (M, k, bs, E, kind)
+
+
+def test_route_align_in_one_call_matches_oracle_bitwise(hip_lib):
+    """vk_hip_moe_route_align against the oracle's router followed by its alignment: up to
+    16 tokens run as one launch (every workgroup routes the tokens itself), the others as
+    the two kernels in sequence."""
+    fn = ve.resolve_route_align_fn(hip_lib)
+    rng = np.random.default_rng(3)
+    cases = [(1, 32, 4, 16, None), (8, 8, 2, 16, None), (16, 32, 4, 16, None), (13, 256, 8, 16, None),
+             (16, 128, 4, 16, "map"), (7, 64, 6, 128, None), (16, 1000, 32, 16, None),
+             (9, 7, 1, 32, None), (16, 128, 4, 64, "ties"), (12, 384, 16, 16, "map"),
+             (17, 32, 4, 16, None), (64, 32, 4, 16, None), (300, 128, 4, 128, None), (700, 32, 8, 64, "map")]
+    for (T, E, k, bs, kind) in cases:
+        lg = synth.make_logits("uniform", T, E, 11 + T)
+        if kind == "ties":
+            lg[:, 1::2] = lg[:, 0::2]  # exact ties: the lower index must win
+        emap, local_n = None, E
+        if kind == "map":
+            local_n = E // 2
+            emap = np.full(E, -1, dtype=np.int32)
+            emap[rng.permutation(E)[:local_n]] = np.arange(local_n, dtype=np.int32)
+        max_em = ve._align_em_bound(T, k, local_n, bs)
+        d_lg = to_dev(lg)
+        d_map = None if emap is None else to_dev(emap)
+        ids = torch.full((T, k), -7, dtype=torch.int32, device=dev())
+        w = torch.full((T, k), -7.0, dtype=torch.float32, device=dev())
+        sids = torch.full((max_em,), -7, dtype=torch.int32, device=dev())
+        eids = torch.full((max_em // bs,), -7, dtype=torch.int32, device=dev())
+        out_em = torch.full((1,), -7, dtype=torch.int32, device=dev())
+        st = fn(d_lg.data_ptr(), T, E, k, 1, None if d_map is None else d_map.data_ptr(), bs, local_n,
+                max_em, ids.data_ptr(), w.data_ptr(), sids.data_ptr(), eids.data_ptr(),
+                out_em.data_ptr(), None)
+        assert st == 0, (T, E, k, bs, kind, ve.last_error(hip_lib))
+        torch.cuda.synchronize()
+        rid, rw = oracle.route_topk(lg, k, True)
+        assert np.array_equal(ids.cpu().numpy(), rid), (T, E, k, bs, kind)
+        assert np.array_equal(w.cpu().numpy().view(np.uint32), rw.view(np.uint32)), (T, E, k, bs, kind)
+        rs, re, rem = oracle.moe_align_block_size_with_map(rid.ravel(), E, bs, emap, local_n=local_n,
+                                                           max_EM=max_em)
+        assert int(out_em.item()) == rem, (T, E, k, bs, kind)
+        assert np.array_equal(sids.cpu().numpy(), rs), (T, E, k, bs, kind)
+        assert np.array_equal(eids.cpu().numpy(), re), (T, E, k, bs, kind)

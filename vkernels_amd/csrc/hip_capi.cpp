@@ -602,6 +602,28 @@ int vk_hip_moe_route_topk(const float* logits, int32_t T, int32_t E,
   return VK_OK;
 }
 
+int vk_hip_moe_route_align(const float* logits, int32_t T, int32_t E, int32_t top_k,
+                           int32_t renormalize, const int32_t* expert_map, int32_t block_size,
+                           int32_t local_n, int32_t max_EM, int32_t* topk_ids, float* topk_w,
+                           int32_t* sorted_ids, int32_t* expert_ids, int32_t* out_EM, void* stream) {
+  // the shapes one launch does not take (and T = 0, where only the alignment has work:
+  // the sentinels and out_EM) go through the two entry points, which check the rest
+  if (T <= 0 || E <= 0 || top_k <= 0 || top_k > E || E > VK_HIP_ROUTE_MAX_EXPERTS ||
+      top_k > VK_HIP_ROUTE_MAX_TOPK || block_size <= 0 || local_n < 0 || local_n > E ||
+      max_EM <= 0 || max_EM % block_size != 0 || local_n > VK_HIP_ALIGN_MAX_EXPERTS ||
+      logits == nullptr || topk_ids == nullptr || topk_w == nullptr || sorted_ids == nullptr ||
+      expert_ids == nullptr || out_EM == nullptr || !vk::route_align_fits(T, E, top_k, local_n)) {
+    const int rc = vk_hip_moe_route_topk(logits, T, E, top_k, renormalize, topk_ids, topk_w, stream);
+    if (rc != VK_OK) return rc;
+    return vk_hip_moe_align_block_size(topk_ids, expert_map, T, top_k, block_size, E, local_n, max_EM,
+                                       sorted_ids, expert_ids, out_EM, stream);
+  }
+  vk::launch_route_align(logits, T, E, top_k, renormalize, expert_map, block_size, local_n, max_EM,
+                         topk_ids, topk_w, sorted_ids, expert_ids, out_EM,
+                         static_cast<hipStream_t>(stream));
+  return VK_OK;
+}
+
 int vk_hip_dequant_weight_tile(const uint8_t* packed, const uint8_t* scale,
                                uint16_t* out_bf16, int32_t N, int32_t K,
                                int32_t group_size, int32_t stride_packed,

@@ -26,10 +26,21 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include "moe_route.hpp"
 #include "vk_internal.hpp"
+
+// (the router's arithmetic is spelled out operation by operation: no contraction here)
+#pragma clang fp contract(off)
 
 namespace vk {
 namespace {
+
+// What route_align_kernel takes: every workgroup routes all the tokens, a wavefront per
+// token, and keeps the table in LDS.  Up to one token per wavefront (16): with more, a
+// workgroup routes them one after the other (about 4 us each, a chain of cross-lane
+// steps), and the router's own launch, which spreads the tokens over the device, is the
+// faster way (measured at 64 tokens, 32 experts: 132 against 124 us per layer step).
+constexpr int kRouteAlignMaxTokens = 16, kRouteAlignMaxRows = 1024, kRouteAlignMaxExperts = 1024;
 
 constexpr int kAlignThreads = 1024;
 constexpr int kAlignWaves = kAlignThreads / 64;
@@ -54,12 +65,13 @@ __device__ __forceinline__ int block_sum(int v, int* red) {
   return t;
 }
 
-__global__ __launch_bounds__(kAlignThreads) void align_kernel(
-    const int32_t* __restrict__ topk_ids, const int32_t* __restrict__ expert_map,
+// The work of workgroup blockIdx.x (steps 1 to 4 above).  topk_ids: the N flat routing
+// indices, in global memory or in LDS; hist: local_n ints of LDS.
+__device__ __forceinline__ void align_workgroup(
+    const int32_t* topk_ids, const int32_t* __restrict__ expert_map,
     int N, int block_size, int num_experts, int local_n, int max_EM,
     int32_t* __restrict__ sorted_ids, int32_t* __restrict__ expert_ids,
-    int32_t* __restrict__ out_em) {
-  extern __shared__ int32_t hist[];  // [local_n]
+    int32_t* __restrict__ out_em, int32_t* hist) {
   __shared__ int wave_cnt[kAlignWaves];
   __shared__ int red[kAlignWaves];
 
@@ -154,7 +166,74 @@ __global__ __launch_bounds__(kAlignThreads) void align_kernel(
   }
 }
 
+__global__ __launch_bounds__(kAlignThreads) void align_kernel(
+    const int32_t* __restrict__ topk_ids, const int32_t* __restrict__ expert_map,
+    int N, int block_size, int num_experts, int local_n, int max_EM,
+    int32_t* __restrict__ sorted_ids, int32_t* __restrict__ expert_ids,
+    int32_t* __restrict__ out_em) {
+  extern __shared__ int32_t hist[];  // [local_n]
+  align_workgroup(topk_ids, expert_map, N, block_size, num_experts, local_n, max_EM, sorted_ids,
+                  expert_ids, out_em, hist);
+}
+
+// Router and alignment in one launch, for decode-sized batches: every workgroup routes
+// all T tokens itself (a wavefront per token, the same arithmetic as route_topk_kernel,
+// so every workgroup holds the same table), keeps the indices in LDS, and then does its
+// expert's share of the alignment from there; workgroup 0 also writes the routing
+// table out.  One launch less in front of the layer, where a launch is a few
+// microseconds of a step of fifty to a hundred.
+template <int PER>
+__global__ __launch_bounds__(kAlignThreads) void route_align_kernel(
+    const float* __restrict__ logits, int T, int E, int top_k, int renormalize,
+    const int32_t* __restrict__ expert_map, int block_size, int local_n, int max_EM,
+    int32_t* __restrict__ topk_ids, float* __restrict__ topk_w,
+    int32_t* __restrict__ sorted_ids, int32_t* __restrict__ expert_ids,
+    int32_t* __restrict__ out_em) {
+  extern __shared__ int32_t lds[];  // [max(local_n, 1)] histogram, [T * top_k] routing indices
+  int32_t* const ids = lds + (local_n > 0 ? local_n : 1);
+  const int lane = threadIdx.x & 63;
+  for (int token = threadIdx.x >> 6; token < T; token += kAlignWaves) {  // uniform per wavefront
+    int my_id;
+    float my_w;
+    route_token<PER>(logits + (size_t)token * E, E, top_k, renormalize, lane, my_id, my_w);
+    if (lane < top_k) {
+      ids[token * top_k + lane] = my_id;
+      if (blockIdx.x == 0) {
+        topk_ids[(size_t)token * top_k + lane] = my_id;
+        topk_w[(size_t)token * top_k + lane] = my_w;
+      }
+    }
+  }
+  __syncthreads();
+  align_workgroup(ids, expert_map, T * top_k, block_size, E, local_n, max_EM, sorted_ids, expert_ids,
+                  out_em, lds);
+}
+
 }  // namespace
+
+bool route_align_fits(int T, int E, int top_k, int local_n) {
+  (void)E;
+  return T > 0 && T <= kRouteAlignMaxTokens && top_k <= 64 &&
+         (long long)T * top_k <= kRouteAlignMaxRows && local_n <= kRouteAlignMaxExperts;
+}
+
+void launch_route_align(const float* logits, int T, int E, int top_k, int renormalize,
+                        const int32_t* expert_map, int block_size, int local_n, int max_EM,
+                        int32_t* topk_ids, float* topk_w, int32_t* sorted_ids, int32_t* expert_ids,
+                        int32_t* out_em, hipStream_t stream) {
+  const int groups = local_n > 0 ? local_n : 1;
+  const size_t lds = sizeof(int32_t) * ((size_t)groups + (size_t)T * (size_t)top_k);
+#define VK_ROUTE_ALIGN_LAUNCH(PER)                                                                     \
+  hipLaunchKernelGGL((route_align_kernel<PER>), dim3(groups), dim3(kAlignThreads), lds, stream, logits, \
+                     T, E, top_k, renormalize, expert_map, block_size, local_n, max_EM, topk_ids,       \
+                     topk_w, sorted_ids, expert_ids, out_em)
+  if (E <= 64) VK_ROUTE_ALIGN_LAUNCH(1);
+  else if (E <= 128) VK_ROUTE_ALIGN_LAUNCH(2);
+  else if (E <= 256) VK_ROUTE_ALIGN_LAUNCH(4);
+  else if (E <= 512) VK_ROUTE_ALIGN_LAUNCH(8);
+  else VK_ROUTE_ALIGN_LAUNCH(16);
+#undef VK_ROUTE_ALIGN_LAUNCH
+}
 
 void launch_align(const int32_t* topk_ids, const int32_t* expert_map, int N,
                   int block_size, int num_experts, int local_n, int max_EM,

@@ -16,6 +16,14 @@ void launch_align(const int32_t* topk_ids, const int32_t* expert_map, int N,
                   int32_t* sorted_ids, int32_t* expert_ids, int32_t* out_em,
                   hipStream_t stream);
 
+// Router and alignment of a decode-sized batch in one launch (route_align_fits says
+// whether the shape is one it takes).
+bool route_align_fits(int T, int E, int top_k, int local_n);
+void launch_route_align(const float* logits, int T, int E, int top_k, int renormalize,
+                        const int32_t* expert_map, int block_size, int local_n, int max_EM,
+                        int32_t* topk_ids, float* topk_w, int32_t* sorted_ids, int32_t* expert_ids,
+                        int32_t* out_em, hipStream_t stream);
+
 void launch_dequant_tile(const uint8_t* packed, const uint8_t* scale,
                          uint16_t* out_bf16, int N, int K, int stride_packed,
                          int stride_scale_n, int stride_scale_k, int fast,

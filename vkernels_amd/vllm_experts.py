@@ -40,6 +40,7 @@ __all__ = [
     "resolve_align_fn",
     "resolve_moe_fn",
     "resolve_route_fn",
+    "resolve_route_align_fn",
     "resolve_dequant_fn",
     "resolve_prepack_fns",
 ]
@@ -298,6 +299,16 @@ def resolve_route_fn(lib):
     return fn
 
 
+def resolve_route_align_fn(lib):
+    """vk_hip_moe_route_align (router and alignment, one launch for decode-sized batches)."""
+    fn = getattr(lib, "vk_hip_moe_route_align", None)
+    if fn is None:
+        raise RuntimeError("vk_hip_moe_route_align not found in libvkernels_hip.so")
+    fn.restype = _I
+    fn.argtypes = [_P, _I, _I, _I, _I, _P, _I, _I, _I, _P, _P, _P, _P, _P, _P]
+    return fn
+
+
 def resolve_dequant_fn(lib):
     fn = getattr(lib, "vk_hip_dequant_weight_tile", None)
     if fn is None:
@@ -417,6 +428,7 @@ class FusedExperts:
         if self.align_fn is None:
             raise RuntimeError("vk_hip_moe_align_block_size not found in libvkernels_hip.so")
         self.route_fn = resolve_route_fn(self.lib)
+        self.route_align_fn = resolve_route_align_fn(self.lib)
         for name, t in (("w13", w13), ("w13_scale", w13_scale), ("w2", w2), ("w2_scale", w2_scale)):
             if t.dtype != torch.uint8 or not t.is_contiguous() or not t.is_cuda:
                 raise ValueError(f"{name} must be a contiguous uint8 device tensor")
@@ -514,13 +526,42 @@ class FusedExperts:
         _check(self.lib, st, "vk_hip_moe_align_block_size")
         return sids, eids, out_em, max_em
 
+    def route_align(self, logits, top_k: int, renormalize: bool = True, block_size: int | None = None,
+                    max_tokens: int | None = None):
+        """route() and align() through the library's one call (one launch for decode-sized
+        batches).  Returns (topk_ids, topk_w, sorted_ids, expert_ids, out_EM, max_EM,
+        block_size); logits' E columns are the experts the expert map speaks of."""
+        torch = self.torch
+        T, E = logits.shape
+        dev = logits.device
+        block_size = default_block_size(T, top_k) if block_size is None else block_size
+        if block_size <= 0 or block_size % 16 != 0:
+            raise ValueError(f"block_size must be a positive multiple of 16, got {block_size}")
+        logits = logits.contiguous()
+        ids = torch.empty((T, top_k), dtype=torch.int32, device=dev)
+        w = torch.empty((T, top_k), dtype=torch.float32, device=dev)
+        max_em = _align_em_bound(T, top_k, self.local_n, block_size)
+        cap = _align_em_bound(max(T, max_tokens or 0), top_k, self.local_n, block_size)
+        sids = self.scratch.get(("sids", block_size), max_em, dtype=torch.int32, device=dev,
+                                capacity=cap, name="sorted_ids")
+        eids = self.scratch.get(("eids", block_size), max_em // block_size, dtype=torch.int32,
+                                device=dev, capacity=cap // block_size, name="expert_ids")
+        out_em = self.scratch.get("out_em", 1, dtype=torch.int32, device=dev, name="out_em")
+        st = self.route_align_fn(_ptr(logits), T, E, top_k, int(renormalize), _ptr(self.expert_map),
+                                 block_size, self.local_n, max_em, _ptr(ids), _ptr(w), _ptr(sids),
+                                 _ptr(eids), _ptr(out_em), _stream(torch))
+        _check(self.lib, st, "vk_hip_moe_route_align")
+        return ids, w, sids, eids, out_em, max_em, block_size
+
     # -- the layer --------------------------------------------------------------
     def apply(self, hidden_states, topk_ids, topk_weights=None, *, block_size: int | None = None,
-              max_tokens: int | None = None, out_fp32=None, output_dtype=None):
+              max_tokens: int | None = None, out_fp32=None, output_dtype=None, aligned=None):
         """hidden_states [M, H] bf16, topk_ids [M, k] int32, topk_weights [M, k]
         fp32 (None = ones).  Returns the fp32 [M, H] result, or, with output_dtype
         (say torch.bfloat16, what the reference's apply hands back,
-        src/python/vkernels/vllm_experts.py:1092), that result cast."""
+        src/python/vkernels/vllm_experts.py:1092), that result cast.
+        aligned = (sorted_ids, expert_ids, max_EM) of route_align() / align() for this
+        block_size: the alignment is then not made again."""
         torch = self.torch
         M, K = hidden_states.shape
         if K != self.hidden:
@@ -544,7 +585,10 @@ class FusedExperts:
         if not overwrite:
             out_fp32.zero_()
         if M > 0:
-            sids, eids, _, max_em = self.align(topk_ids, block_size, max_tokens=max_tokens)
+            if aligned is None:
+                sids, eids, _, max_em = self.align(topk_ids, block_size, max_tokens=max_tokens)
+            else:
+                sids, eids, max_em = aligned
             self.fused_call(hidden_states, topk_ids, topk_weights, sids, eids, max_em, block_size,
                             out_fp32, max_tokens=max_tokens, overwrite=overwrite)
         return out_fp32 if output_dtype is None else out_fp32.to(output_dtype)
