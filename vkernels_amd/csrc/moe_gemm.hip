@@ -452,8 +452,14 @@ __global__ __launch_bounds__(64 * WAVES) void stream_resident_kernel(GemmArgs p)
       const int e_before = p.expert_ids[max(bc - 1, 0)];
       const int e_after = p.expert_ids[min(bc + 1, nb - 1)];
       const int e = b < nb ? e_here : -1;
-      const bool first = e >= 0 && (b == 0 || e_before != e);
-      const bool last = e >= 0 && (b == nb - 1 || e_after != e);
+      // With blocks of 16 rows every block is a run of its own: an expert's 16-row passes
+      // then go to different workgroups side by side, each staging once, where a run of
+      // several blocks has every workgroup of its share stage pass after pass.  (Larger
+      // blocks stay merged: their tiles may be empty, and a run of its own for an empty
+      // tile would idle its workgroups.)
+      const bool alone = p.block_size == 16;
+      const bool first = e >= 0 && (alone || b == 0 || e_before != e);
+      const bool last = e >= 0 && (alone || b == nb - 1 || e_after != e);
       const unsigned long long mv = __ballot(e >= 0), mf = __ballot(first), ml = __ballot(last);
       if (first) {
         const int idx = n + (int)__popcll(mf & below);
