@@ -10,7 +10,8 @@
 // Three kernels share the arithmetic (scaled FP4 x FP8 MFMA, see the decode
 // kernel's comment) and the work decomposition:
 //
-//   * a run = the consecutive blocks of one expert; padding rows (sorted id
+//   * a run = the consecutive blocks of one expert (in the decode kernel, with
+//     blocks of 16 rows, every block by itself); padding rows (sorted id
 //     >= M*top_k) and blocks with expert id < 0 are skipped;
 //   * a wavefront owns NT weight tiles of 16 rows each (stage 0: NT/2 gate
 //     tiles and the NT/2 up tiles of the same columns, so the activation is
@@ -228,8 +229,10 @@ __device__ __forceinline__ void unit_tiles(const GemmArgs& p, int e, int unit, i
 // memory.
 //
 // Work split.  The launch has as many workgroups as the device has compute
-// units.  Every workgroup lists the runs (consecutive blocks of one expert),
-// flattens (run, weight unit) into one index space and takes a contiguous
+// units.  Every workgroup lists the runs (consecutive blocks of one expert;
+// with blocks of 16 rows every block by itself, so that the 16-row passes over
+// an expert's weights run side by side in different workgroups, each staging
+// its rows once), flattens (run, weight unit) into one index space and takes a contiguous
 // slice of it (kStagingUnits below), so the weight bytes are spread evenly over
 // the compute units whatever the number of active experts.  For each run its
 // slice touches, and each 16-row pass of that run, the workgroup stages the
