@@ -33,6 +33,7 @@ import argparse
 import hashlib
 import json
 import os
+import re
 import sys
 import time
 from pathlib import Path
@@ -75,11 +76,15 @@ def parse_args():
 
 
 def sources_digest() -> str:
-    """Digest of the kernel sources: names the build a profile was taken on."""
+    """Digest of the kernel sources, comments and white space left out: names the code a
+    profile was taken on."""
     h = hashlib.sha256()
     for path in sorted((ROOT / "vkernels_amd" / "csrc").iterdir()):
+        text = path.read_text(errors="replace")
+        text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+        text = re.sub(r"//[^\n]*", "", text)
         h.update(path.name.encode())
-        h.update(path.read_bytes())
+        h.update("".join(text.split()).encode())
     return h.hexdigest()[:16]
 
 

@@ -84,13 +84,13 @@ struct MoeTileRule {
 // tiles (nt = 1) and keeps the bytes in flight per wavefront with a deeper pipeline.
 // Rows (each from the sweep table profiles/moe_decode_tile_sweep.md):
 //  - K <= 1024: a unit is a few steps long, and steps in flight past its end are
-//    wasted loads: the shallowest pipelines (256x512x8x2 at T = 64: 13.8 against 15.2 us);
+//    wasted loads: the shallowest pipelines (256x512x8x2 at T = 64: 10.7 against 11.6 us);
 //  - 3072 < K <= 4096 (4096x1536x64x6 gate/up): the rows of a pass fit LDS and registers
-//    only with 4 wavefronts per workgroup (35 against 67 us at T = 1, 100 against 175 us
+//    only with 4 wavefronts per workgroup (34 against 69 us at T = 1, 98 against 185 us
 //    at T = 32 for the tile kernel, which is what runs beyond K = 4096);
-//  - otherwise (8, 2, 4) / (8, 1, 8), within 4 % of the best of every other point swept:
+//  - otherwise (8, 2, 4) / (8, 1, 8), within 5 % of the best of every other point swept:
 //    with 128 experts and 32 tokens or more, uniformly routed, the 4-wavefront shapes
-//    are 3 to 4 % faster for gate/up; the number of runs that makes it so is not known
+//    are 3 to 5 % faster for gate/up; the number of runs that makes it so is not known
 //    here, and with skewed routing (27 active experts of 128) the same shape is much
 //    slower, so that choice is left to the tuning store.
 inline MoeTile pick_moe_tile(int n_flat, int K, int ncols, int stage) {
