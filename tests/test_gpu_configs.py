@@ -267,6 +267,19 @@ def test_decode_with_more_sorted_rows_than_the_kernel_copies_to_lds():
     assert g["EM"] > 2048 + 64, "every run's ids fit the copy in LDS"
 
 
+def test_decode_with_more_runs_than_workgroups():
+    """512 experts, 480 routed rows: more than 256 blocks of 16 rows, each a run of its own,
+    so the runs cannot have workgroups of their own and the (run, unit) space is cut
+    evenly, a workgroup's slice spanning several runs."""
+    cfg = synth.MoEConfig("c8", 256, 256, 512, 8, (60,), "uniform")
+    T, seed = 60, 8060
+    w = _weights(cfg, 8000)
+    A, lg = _inputs(cfg, T, seed)
+    g, _ = _check(cfg, T, w, A, lg)
+    assert g["bs"] == 16 and T * cfg.top_k <= 512, "not a decode-sized call"
+    assert g["EM"] // 16 > 256, "fewer runs than the device has compute units"
+
+
 @pytest.mark.parametrize("use_workspace", [True, False])
 @pytest.mark.parametrize("bs", [16, 48, 80, 128])
 def test_tile_kernels_block_sizes(bs, use_workspace):

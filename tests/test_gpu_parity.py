@@ -164,7 +164,7 @@ def test_route_align_in_one_call_matches_oracle_bitwise(hip_lib):
     the two kernels in sequence."""
     fn = ve.resolve_route_align_fn(hip_lib)
     rng = np.random.default_rng(3)
-    cases = [(1, 32, 4, 16, None), (8, 8, 2, 16, None), (16, 32, 4, 16, None), (13, 256, 8, 16, None),
+    cases = [(0, 8, 2, 16, None), (1, 32, 4, 16, None), (8, 8, 2, 16, None), (16, 32, 4, 16, None), (13, 256, 8, 16, None),
              (16, 128, 4, 16, "map"), (7, 64, 6, 128, None), (16, 1000, 32, 16, None),
              (9, 7, 1, 32, None), (16, 128, 4, 64, "ties"), (12, 384, 16, 16, "map"),
              (17, 32, 4, 16, None), (64, 32, 4, 16, None), (300, 128, 4, 128, None), (700, 32, 8, 64, "map")]
