@@ -194,8 +194,10 @@ void vk_hip_fused_moe_mxfp4_ex(
  * each term with a block scale of its own: three terms (exact unless an element
  * lies more than 2^-13 below its block's largest) in the first stage, whose
  * error passes through the activation function and the second GEMM, and two
- * terms (error at most 2^-10 of the block's largest per element) in the second:
- * 5e-4 relative L2 of the layer against the reference's bf16 arithmetic.
+ * terms (error at most 2^-10 of the block's largest per element) in the second
+ * (three there too when ispp < 1024: short sums average less, and such layers
+ * are small): 5e-4 relative L2 of the layer against the reference's bf16
+ * arithmetic.
  * VK_HIP_MOE_SPLIT3 selects three terms in both stages (7e-5; 12 % more
  * matrix-core work), VK_HIP_MOE_SPLIT2 two in both (1.4e-3, worst element 1e-2
  * of the RMS: inside the reference's tolerance of 5e-3 / 2e-2, with less margin;

@@ -270,7 +270,8 @@ def _check_prefill(cfg, T, w, A_bits, logits, terms=None, sample=128, wn=None, g
     wn = w.numpy() if wn is None else wn
     c = cpu_layer(A_bits[rows], wn, ids[rows], tw[rows], threads=16, **(cpu_kw or {}))
     max_rel, rel_l2, nf = error_metrics(g["out"][rows], c["out"])
-    oracle.set_act_model(3 + 16 * 2 if terms is None else terms)
+    # the default: 3 terms in the first stage, 2 in the second (3 where its sums are short)
+    oracle.set_act_model(3 + 16 * (3 if cfg.I < 1024 else 2) if terms is None else terms)
     try:
         cm = cpu_layer(A_bits[rows], wn, ids[rows], tw[rows], threads=16, **(cpu_kw or {}))
     finally:

@@ -1044,6 +1044,8 @@ bool prepare_mx_kernels() {
 
 namespace {
 
+constexpr int kMxShortK = 1024;  // second-stage sums shorter than this take three terms by default
+
 struct MxPlan {
   MxArgs g0, g1;
   uint8_t *aq, *cq, *abad, *cbad;
@@ -1065,11 +1067,15 @@ bool mx_plan(const FusedMoeArgs& a, bool need_stage0, MxPlan& pl) {
       (unsigned long long)a.M * 3ull * mx_kp(a.hidden) >= (1ull << 32))
     return false;
   // VK_HIP_MOE_W4A4; _SPLIT2; _SPLIT3; default: three terms where the error passes through
-  // the activation function and the second GEMM, two in the second stage
+  // the activation function and the second GEMM, two in the second stage -- but three
+  // there as well when its sums are short (ispp < kMxShortK): the worst element's error
+  // grows as the sums get shorter (1.7e-2 of the RMS at ispp = 64, 6.7e-3 at 256,
+  // 4.6e-3 at 1024 and beyond with two terms; 2.5e-4 at 64 with three), and such
+  // layers are small enough that the third term costs microseconds
   if ((a.flags & 4u) != 0u) pl.terms0 = pl.terms1 = 1;
   else if ((a.flags & 2u) != 0u) pl.terms0 = pl.terms1 = 2;
   else if ((a.flags & 8u) != 0u) pl.terms0 = pl.terms1 = 3;
-  else { pl.terms0 = 3; pl.terms1 = 2; }
+  else { pl.terms0 = 3; pl.terms1 = a.ispp < kMxShortK ? 3 : 2; }
   const bool ready0 = !need_stage0 || (pl.terms0 == 1 ? mx_kernel_ready<0, 1>()
                                        : pl.terms0 == 2 ? mx_kernel_ready<0, 2>() : mx_kernel_ready<0, 3>());
   const bool ready1 = pl.terms1 == 1 ? mx_kernel_ready<1, 1>()
