@@ -190,17 +190,35 @@ __global__ __launch_bounds__(256) void prepack_kernel(const uint8_t* __restrict_
 // term's scale byte, 7 zero bytes.  Blocks between K and Kp are zero with a
 // neutral scale.  row_bad[r] = 1 when a block of the row is outside the range
 // (inf/NaN, or a scale byte the scaled MFMA path does not take).
-// One workgroup per row, one lane per block of 32.
+// One lane per block of 32; a workgroup takes as many whole rows as its 256 lanes hold
+// (split_rows_per_group: 4 rows of 2048, 1 of 7168), so that short rows do not leave
+// three of its four wavefronts idle.
 // ---------------------------------------------------------------------------
+__host__ __device__ constexpr int split_rows_per_group(int kp) { return kp / 32 >= 256 ? 1 : 256 / (kp / 32); }
+
+// Workgroups of split_rows_fp6_kernel for `rows` rows of K values.
+static inline dim3 split_grid(int rows, int K) {
+  const int rpg = split_rows_per_group(mx_kp(K));
+  return dim3((unsigned)((rows + rpg - 1) / rpg));
+}
+
 template <int TERMS>
 __global__ __launch_bounds__(256) void split_rows_fp6_kernel(const uint16_t* __restrict__ x,
                                                              uint8_t* __restrict__ xq,
-                                                             uint8_t* __restrict__ row_bad, int K) {
+                                                             uint8_t* __restrict__ row_bad, int K,
+                                                             int rows) {
+  __shared__ int bad_rows[256];  // per row of the workgroup
   const int kp = mx_kp(K);
-  const size_t row = blockIdx.x;
+  const int bpr = kp / 32;                       // blocks of a row
+  const int rpg = split_rows_per_group(kp);      // rows of a workgroup
+  const int sub = rpg > 1 ? (int)threadIdx.x / bpr : 0;  // this lane's row within the workgroup
+  const size_t row = (size_t)blockIdx.x * rpg + sub;
+  const bool live = sub < rpg && row < (size_t)rows;
+  if (threadIdx.x < rpg) bad_rows[threadIdx.x] = 0;
+  __syncthreads();
   uint8_t* qrow = xq + row * (size_t)(TERMS * kp);
   int bad = 0;
-  for (int b = threadIdx.x; b < kp / 32; b += 256) {
+  for (int b = rpg > 1 ? (int)threadIdx.x - sub * bpr : (int)threadIdx.x; live && b < bpr; b += 256) {
     union { u32x4 q[4]; bf16x32 v; uint32_t d[16]; } in;
 #pragma unroll
     for (int i = 0; i < 4; ++i) in.q[i] = u32x4{0u, 0u, 0u, 0u};
@@ -247,8 +265,10 @@ __global__ __launch_bounds__(256) void split_rows_fp6_kernel(const uint16_t* __r
       *reinterpret_cast<u32x4*>(blk + 16) = u32x4{codes[4], codes[5], st, 0u};
     }
   }
-  bad = __syncthreads_or(bad);
-  if (threadIdx.x == 0) row_bad[row] = (uint8_t)(bad != 0);
+  if (bad != 0 && live) atomicOr(&bad_rows[sub], 1);
+  __syncthreads();
+  if (threadIdx.x < rpg && (size_t)blockIdx.x * rpg + threadIdx.x < (size_t)rows)
+    row_bad[(size_t)blockIdx.x * rpg + threadIdx.x] = (uint8_t)(bad_rows[threadIdx.x] != 0);
 }
 
 // ---------------------------------------------------------------------------
@@ -1107,10 +1127,10 @@ void mx_stage0(const FusedMoeArgs& a, const MxPlan& pl, hipStream_t stream) {
     hipLaunchKernelGGL(quant_rows_w4_kernel, dim3(a.M), dim3(256), 0, stream, a.A, pl.aq, pl.abad, a.hidden);
     launch_mx_stage_t<0, 1>(pl.g0, stream);
   } else if (pl.terms0 == 2) {
-    hipLaunchKernelGGL(split_rows_fp6_kernel<2>, dim3(a.M), dim3(256), 0, stream, a.A, pl.aq, pl.abad, a.hidden);
+    hipLaunchKernelGGL(split_rows_fp6_kernel<2>, split_grid(a.M, a.hidden), dim3(256), 0, stream, a.A, pl.aq, pl.abad, a.hidden, a.M);
     launch_mx_stage_t<0, 2>(pl.g0, stream);
   } else {
-    hipLaunchKernelGGL(split_rows_fp6_kernel<3>, dim3(a.M), dim3(256), 0, stream, a.A, pl.aq, pl.abad, a.hidden);
+    hipLaunchKernelGGL(split_rows_fp6_kernel<3>, split_grid(a.M, a.hidden), dim3(256), 0, stream, a.A, pl.aq, pl.abad, a.hidden, a.M);
     launch_mx_stage_t<0, 3>(pl.g0, stream);
   }
 }
@@ -1123,10 +1143,10 @@ void mx_stage1(const FusedMoeArgs& a, const MxPlan& pl, hipStream_t stream) {
     hipLaunchKernelGGL(quant_rows_w4_kernel, dim3(a.EM), dim3(256), 0, stream, a.act, pl.cq, pl.cbad, a.ispp);
     launch_mx_stage_t<1, 1>(pl.g1, stream);
   } else if (pl.terms1 == 2) {
-    hipLaunchKernelGGL(split_rows_fp6_kernel<2>, dim3(a.EM), dim3(256), 0, stream, a.act, pl.cq, pl.cbad, a.ispp);
+    hipLaunchKernelGGL(split_rows_fp6_kernel<2>, split_grid(a.EM, a.ispp), dim3(256), 0, stream, a.act, pl.cq, pl.cbad, a.ispp, a.EM);
     launch_mx_stage_t<1, 2>(pl.g1, stream);
   } else {
-    hipLaunchKernelGGL(split_rows_fp6_kernel<3>, dim3(a.EM), dim3(256), 0, stream, a.act, pl.cq, pl.cbad, a.ispp);
+    hipLaunchKernelGGL(split_rows_fp6_kernel<3>, split_grid(a.EM, a.ispp), dim3(256), 0, stream, a.act, pl.cq, pl.cbad, a.ispp, a.EM);
     launch_mx_stage_t<1, 3>(pl.g1, stream);
   }
   launch_combine(pl.y, pl.pos, a.out, a.M, a.top_k, a.hidden, (a.flags & 1u) != 0u, stream);
@@ -1157,9 +1177,9 @@ void launch_split_rows_fp6(const uint16_t* x, int rows, int K, int terms, uint8_
                            hipStream_t stream) {
   if (rows <= 0) return;
   if (terms == 2)
-    hipLaunchKernelGGL(split_rows_fp6_kernel<2>, dim3(rows), dim3(256), 0, stream, x, xq, row_bad, K);
+    hipLaunchKernelGGL(split_rows_fp6_kernel<2>, split_grid(rows, K), dim3(256), 0, stream, x, xq, row_bad, K, rows);
   else
-    hipLaunchKernelGGL(split_rows_fp6_kernel<3>, dim3(rows), dim3(256), 0, stream, x, xq, row_bad, K);
+    hipLaunchKernelGGL(split_rows_fp6_kernel<3>, split_grid(rows, K), dim3(256), 0, stream, x, xq, row_bad, K, rows);
 }
 
 // ---- MXFP4 orchestration ops (device counterparts of moe_aux.cpp) -----------------
