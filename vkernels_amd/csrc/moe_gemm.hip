@@ -10,9 +10,9 @@
 // Three kernels share the arithmetic (scaled FP4 x FP8 MFMA, see the decode
 // kernel's comment) and the work decomposition:
 //
-//   * a run = the consecutive blocks of one expert (in the decode kernel, with
-//     blocks of 16 rows, every block by itself); padding rows (sorted id
-//     >= M*top_k) and blocks with expert id < 0 are skipped;
+//   * a run = the consecutive blocks of one expert (in the decode kernel every
+//     block by itself); padding rows (sorted id >= M*top_k) and blocks with
+//     expert id < 0 are skipped;
 //   * a wavefront owns NT weight tiles of 16 rows each (stage 0: NT/2 gate
 //     tiles and the NT/2 up tiles of the same columns, so the activation is
 //     fused; stage 1: NT consecutive tiles) and walks the whole K dimension;
@@ -229,10 +229,10 @@ __device__ __forceinline__ void unit_tiles(const GemmArgs& p, int e, int unit, i
 // memory.
 //
 // Work split.  The launch has as many workgroups as the device has compute
-// units.  Every workgroup lists the runs (consecutive blocks of one expert;
-// with blocks of 16 rows every block by itself, so that the 16-row passes over
-// an expert's weights run side by side in different workgroups, each staging
-// its rows once), flattens (run, weight unit) into one index space and takes a contiguous
+// units.  Every workgroup lists the runs (every block with an expert by
+// itself, so that with blocks of 16 rows the 16-row passes over an expert's
+// weights run side by side in different workgroups, each staging its rows
+// once), flattens (run, weight unit) into one index space and takes a contiguous
 // slice of it (kStagingUnits below), so the weight bytes are spread evenly over
 // the compute units whatever the number of active experts.  For each run its
 // slice touches, and each 16-row pass of that run, the workgroup stages the
@@ -404,7 +404,6 @@ template <int STAGE, int WAVES, int NT, int D>
 __global__ __launch_bounds__(64 * WAVES) void stream_resident_kernel(GemmArgs p) {
   extern __shared__ u32x4 b_lds[];  // [nsteps][2][2][64] operand planes, block scales, weight scales
   __shared__ int run_block0[kMaxRuns];
-  __shared__ int run_block1[kMaxRuns];  // one past the last block of the run
   __shared__ int run_expert[kMaxRuns];
   __shared__ int run_cum[kMaxRuns];     // blocks of the runs up to and including this one
   __shared__ int slice_sh[2];           // this workgroup's slice of the (run, unit) space
@@ -444,43 +443,53 @@ __global__ __launch_bounds__(64 * WAVES) void stream_resident_kernel(GemmArgs p)
     const int nb = p.num_blocks;
     const int grid = (int)gridDim.x, wg = (int)blockIdx.x;
     const unsigned long long below = (1ull << lane) - 1ull;
-    int n = 0, n_last = 0;
-    int listed_blocks = 0;  // blocks with an expert so far = the blocks of the runs so far
+    // Every block with an expert is a run of its own: the blocks of an expert then go to
+    // different workgroups side by side, each staging once, where a run of several blocks
+    // would have every workgroup of its share stage pass after pass.  Weight of a run =
+    // its 16-row tiles that hold routed rows: 1 for blocks of 16; for larger blocks the
+    // tiles whose first row is routed (the rows of an expert are packed at the front of its
+    // blocks; where they are not, only the balance of the split suffers: which tiles are
+    // passes is decided below from all their rows).
+    const int tpb = p.block_size / 16;
+    int n = 0;
+    int listed_weight = 0;  // weight of the runs so far
     for (int base = 0; base < nb; base += 64) {
       const int b = base + lane;
-      // the block's expert and its two neighbours': three loads without a branch
-      // between them, so one round trip to memory and not three
       const int bc = min(b, nb - 1);
       const int e_here = p.expert_ids[bc];
-      const int e_before = p.expert_ids[max(bc - 1, 0)];
-      const int e_after = p.expert_ids[min(bc + 1, nb - 1)];
+      int w = tpb;  // (more than 8 tiles a block: all of them)
+      if (tpb > 1 && tpb <= 8) {  // uniform; loads without a branch between them: one round trip
+        w = 0;
+#pragma unroll
+        for (int jt = 0; jt < 8; ++jt) {
+          const int id = p.sorted_ids[(size_t)(bc * tpb + min(jt, tpb - 1)) * 16];
+          w += (jt < tpb && id >= 0 && id < p.n_flat) ? 1 : 0;
+        }
+        w = max(w, 1);
+      }
       const int e = b < nb ? e_here : -1;
-      // With blocks of 16 rows every block is a run of its own: an expert's 16-row passes
-      // then go to different workgroups side by side, each staging once, where a run of
-      // several blocks has every workgroup of its share stage pass after pass.  (Larger
-      // blocks stay merged: their tiles may be empty, and a run of its own for an empty
-      // tile would idle its workgroups.)
-      const bool alone = p.block_size == 16;
-      const bool first = e >= 0 && (alone || b == 0 || e_before != e);
-      const bool last = e >= 0 && (alone || b == nb - 1 || e_after != e);
-      const unsigned long long mv = __ballot(e >= 0), mf = __ballot(first), ml = __ballot(last);
-      if (first) {
-        const int idx = n + (int)__popcll(mf & below);
+      const bool run = e >= 0;
+      const unsigned long long mr = __ballot(run);
+      int cum = run ? w : 0;  // inclusive prefix of the weights over the lanes
+      if (tpb > 1) {
+#pragma unroll
+        for (int d = 1; d < 64; d <<= 1) {
+          const int y = __shfl_up(cum, d);
+          if (lane >= d) cum += y;
+        }
+      } else {
+        cum = (int)__popcll(mr & below) + (run ? 1 : 0);
+      }
+      if (run) {
+        const int idx = n + (int)__popcll(mr & below);
         if (idx < kMaxRuns) {
           run_block0[idx] = b;
           run_expert[idx] = e;
+          run_cum[idx] = listed_weight + cum;
         }
       }
-      if (last) {  // a run's last block is its first one or comes after it
-        const int idx = n_last + (int)__popcll(ml & below);
-        if (idx < kMaxRuns) {
-          run_block1[idx] = b + 1;
-          run_cum[idx] = listed_blocks + (int)__popcll(mv & below) + 1;
-        }
-      }
-      n += (int)__popcll(mf);
-      n_last += (int)__popcll(ml);
-      listed_blocks += (int)__popcll(mv);
+      n += (int)__popcll(mr);
+      listed_weight += tpb > 1 ? __shfl(cum, 63) : (int)__popcll(mr);
     }
     n = n < kMaxRuns ? n : kMaxRuns;
     DECODE_TRACE(5);  // runs listed
@@ -489,13 +498,11 @@ __global__ __launch_bounds__(64 * WAVES) void stream_resident_kernel(GemmArgs p)
       pass_slow[1] = 0;
     }
     // ---- this workgroup's slice --------------------------------------------
-    // Weight of a run = its 16-row tiles.  Aligned slicing gives the runs up to
-    // and including r the first floor(grid * (their weight) / (all weight))
-    // workgroups; the tiles per block cancel in that quotient, so it is taken
-    // over blocks (run_cum).  A lane per run, and ballots instead of reductions:
-    // this wavefront is the only one at work until the barrier below.
-    const int tiles_per_block = p.block_size / 16;
-    const int total_weight = listed_blocks * tiles_per_block;
+    // Aligned slicing gives the runs up to and including r the first
+    // floor(grid * (their weight) / (all weight)) workgroups (run_cum = the weights
+    // summed).  A lane per run, and ballots instead of reductions: this wavefront is the
+    // only one at work until the barrier below.
+    const int total_weight = listed_weight;
     bool ok = n > 0 && n <= grid;
     int t0 = 0, t1 = 0;
     if (ok) {
@@ -506,13 +513,13 @@ __global__ __launch_bounds__(64 * WAVES) void stream_resident_kernel(GemmArgs p)
         const int r = base + lane;
         const bool live = r < n;
         const int cum = live ? run_cum[r] : 0;  // written by this wavefront; LDS operations stay in order
-        const int len = live ? run_block1[r] - run_block0[r] : 0;
-        const int end = (int)((unsigned)(grid * cum) / (unsigned)listed_blocks);
-        const int begin = (int)((unsigned)(grid * (cum - len)) / (unsigned)listed_blocks);
+        const int len = cum - (live && r > 0 ? run_cum[r - 1] : 0);  // the run's weight
+        const int end = (int)((unsigned)(grid * cum) / (unsigned)total_weight);
+        const int begin = (int)((unsigned)(grid * (cum - len)) / (unsigned)total_weight);
         bool bad = false;
         if (live) {
           bad = end <= begin;
-          if (!bad) bad = (units + end - begin - 1) / (end - begin) * (len * tiles_per_block) > limit;
+          if (!bad) bad = (units + end - begin - 1) / (end - begin) * len > limit;
         }
         ok = ok && __ballot(bad) == 0ull;
         const unsigned long long past = __ballot(live && end > wg);
@@ -588,7 +595,7 @@ __global__ __launch_bounds__(64 * WAVES) void stream_resident_kernel(GemmArgs p)
     const int u0 = max(s0, base_slot) - base_slot;
     const int u1 = min(s1, base_slot + units) - base_slot;
     const int b0 = run_block0[r];
-    const int run_blocks = run_block1[r] - b0;
+    const int run_blocks = 1;  // every block is a run of its own
     const int e = run_expert[r];
     const int run_row0 = b0 * p.block_size;
     const int run_tiles = run_blocks * (p.block_size / 16);
