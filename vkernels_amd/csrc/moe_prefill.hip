@@ -192,7 +192,10 @@ __global__ __launch_bounds__(256) void prepack_kernel(const uint8_t* __restrict_
 // (inf/NaN, or a scale byte the scaled MFMA path does not take).
 // One lane per block of 32; a workgroup takes as many whole rows as its 256 lanes hold
 // (split_rows_per_group: 4 rows of 2048, 1 of 7168), so that short rows do not leave
-// three of its four wavefronts idle.
+// three of its four wavefronts idle.  With sorted_ids, x is in sorted order and only
+// its routed rows (0 <= sorted_ids[r] < n_flat) are split: the padding rows of xq and
+// row_bad keep what they held, and no consumer looks at them (a padding row of the
+// alignment is most of the rows when experts are many and rows few).
 // ---------------------------------------------------------------------------
 __host__ __device__ constexpr int split_rows_per_group(int kp) { return kp / 32 >= 256 ? 1 : 256 / (kp / 32); }
 
@@ -206,14 +209,20 @@ template <int TERMS>
 __global__ __launch_bounds__(256) void split_rows_fp6_kernel(const uint16_t* __restrict__ x,
                                                              uint8_t* __restrict__ xq,
                                                              uint8_t* __restrict__ row_bad, int K,
-                                                             int rows) {
+                                                             int rows,
+                                                             const int32_t* __restrict__ sorted_ids,
+                                                             int n_flat) {
   __shared__ int bad_rows[256];  // per row of the workgroup
   const int kp = mx_kp(K);
   const int bpr = kp / 32;                       // blocks of a row
   const int rpg = split_rows_per_group(kp);      // rows of a workgroup
   const int sub = rpg > 1 ? (int)threadIdx.x / bpr : 0;  // this lane's row within the workgroup
   const size_t row = (size_t)blockIdx.x * rpg + sub;
-  const bool live = sub < rpg && row < (size_t)rows;
+  bool live = sub < rpg && row < (size_t)rows;
+  if (live && sorted_ids != nullptr) {  // rows of a sorted order: only the routed ones are read
+    const int f = sorted_ids[row];
+    live = f >= 0 && f < n_flat;
+  }
   if (threadIdx.x < rpg) bad_rows[threadIdx.x] = 0;
   __syncthreads();
   uint8_t* qrow = xq + row * (size_t)(TERMS * kp);
@@ -363,9 +372,15 @@ __global__ __launch_bounds__(256) void mxfp4_quant_kernel(const uint16_t* __rest
 // byte is outside the range the scaled MFMA path takes.
 __global__ __launch_bounds__(256) void quant_rows_w4_kernel(const uint16_t* __restrict__ x,
                                                             uint8_t* __restrict__ xq,
-                                                            uint8_t* __restrict__ row_bad, int K) {
+                                                            uint8_t* __restrict__ row_bad, int K,
+                                                            const int32_t* __restrict__ sorted_ids,
+                                                            int n_flat) {
   const int kp = mx_kp(K);
   const size_t row = blockIdx.x;
+  if (sorted_ids != nullptr) {  // as split_rows_fp6_kernel: routed rows only (uniform per workgroup)
+    const int f = sorted_ids[row];
+    if (f < 0 || f >= n_flat) return;
+  }
   uint8_t* qrow = xq + row * (size_t)kp;
   int bad = 0;
   for (int b = threadIdx.x; b < kp / 32; b += 256) {
@@ -1124,29 +1139,28 @@ bool mx_plan(const FusedMoeArgs& a, bool need_stage0, MxPlan& pl) {
 
 void mx_stage0(const FusedMoeArgs& a, const MxPlan& pl, hipStream_t stream) {
   if (pl.terms0 == 1) {
-    hipLaunchKernelGGL(quant_rows_w4_kernel, dim3(a.M), dim3(256), 0, stream, a.A, pl.aq, pl.abad, a.hidden);
+    hipLaunchKernelGGL(quant_rows_w4_kernel, dim3(a.M), dim3(256), 0, stream, a.A, pl.aq, pl.abad, a.hidden, nullptr, 0);
     launch_mx_stage_t<0, 1>(pl.g0, stream);
   } else if (pl.terms0 == 2) {
-    hipLaunchKernelGGL(split_rows_fp6_kernel<2>, split_grid(a.M, a.hidden), dim3(256), 0, stream, a.A, pl.aq, pl.abad, a.hidden, a.M);
+    hipLaunchKernelGGL(split_rows_fp6_kernel<2>, split_grid(a.M, a.hidden), dim3(256), 0, stream, a.A, pl.aq, pl.abad, a.hidden, a.M, nullptr, 0);
     launch_mx_stage_t<0, 2>(pl.g0, stream);
   } else {
-    hipLaunchKernelGGL(split_rows_fp6_kernel<3>, split_grid(a.M, a.hidden), dim3(256), 0, stream, a.A, pl.aq, pl.abad, a.hidden, a.M);
+    hipLaunchKernelGGL(split_rows_fp6_kernel<3>, split_grid(a.M, a.hidden), dim3(256), 0, stream, a.A, pl.aq, pl.abad, a.hidden, a.M, nullptr, 0);
     launch_mx_stage_t<0, 3>(pl.g0, stream);
   }
 }
 
-// split act (every sorted row; padding rows hold old data and are never routed) ->
-// second stage -> per-token sum
+// split act (the routed rows of the sorted order) -> second stage -> per-token sum
 void mx_stage1(const FusedMoeArgs& a, const MxPlan& pl, hipStream_t stream) {
   launch_fill_i32(pl.pos, -1, a.M * a.top_k, stream);
   if (pl.terms1 == 1) {
-    hipLaunchKernelGGL(quant_rows_w4_kernel, dim3(a.EM), dim3(256), 0, stream, a.act, pl.cq, pl.cbad, a.ispp);
+    hipLaunchKernelGGL(quant_rows_w4_kernel, dim3(a.EM), dim3(256), 0, stream, a.act, pl.cq, pl.cbad, a.ispp, a.sorted_ids, a.M * a.top_k);
     launch_mx_stage_t<1, 1>(pl.g1, stream);
   } else if (pl.terms1 == 2) {
-    hipLaunchKernelGGL(split_rows_fp6_kernel<2>, split_grid(a.EM, a.ispp), dim3(256), 0, stream, a.act, pl.cq, pl.cbad, a.ispp, a.EM);
+    hipLaunchKernelGGL(split_rows_fp6_kernel<2>, split_grid(a.EM, a.ispp), dim3(256), 0, stream, a.act, pl.cq, pl.cbad, a.ispp, a.EM, a.sorted_ids, a.M * a.top_k);
     launch_mx_stage_t<1, 2>(pl.g1, stream);
   } else {
-    hipLaunchKernelGGL(split_rows_fp6_kernel<3>, split_grid(a.EM, a.ispp), dim3(256), 0, stream, a.act, pl.cq, pl.cbad, a.ispp, a.EM);
+    hipLaunchKernelGGL(split_rows_fp6_kernel<3>, split_grid(a.EM, a.ispp), dim3(256), 0, stream, a.act, pl.cq, pl.cbad, a.ispp, a.EM, a.sorted_ids, a.M * a.top_k);
     launch_mx_stage_t<1, 3>(pl.g1, stream);
   }
   launch_combine(pl.y, pl.pos, a.out, a.M, a.top_k, a.hidden, (a.flags & 1u) != 0u, stream);
@@ -1177,9 +1191,9 @@ void launch_split_rows_fp6(const uint16_t* x, int rows, int K, int terms, uint8_
                            hipStream_t stream) {
   if (rows <= 0) return;
   if (terms == 2)
-    hipLaunchKernelGGL(split_rows_fp6_kernel<2>, split_grid(rows, K), dim3(256), 0, stream, x, xq, row_bad, K, rows);
+    hipLaunchKernelGGL(split_rows_fp6_kernel<2>, split_grid(rows, K), dim3(256), 0, stream, x, xq, row_bad, K, rows, nullptr, 0);
   else
-    hipLaunchKernelGGL(split_rows_fp6_kernel<3>, split_grid(rows, K), dim3(256), 0, stream, x, xq, row_bad, K, rows);
+    hipLaunchKernelGGL(split_rows_fp6_kernel<3>, split_grid(rows, K), dim3(256), 0, stream, x, xq, row_bad, K, rows, nullptr, 0);
 }
 
 // ---- MXFP4 orchestration ops (device counterparts of moe_aux.cpp) -----------------
