@@ -1583,7 +1583,11 @@ __global__ __launch_bounds__(256) void fill_i32_kernel(int32_t* dst, int32_t val
 }
 
 // out[t, :] (+)= the sum over the token's selections s, in order, of y[pos[t * top_k + s], :]
-// (selections whose expert is not local have pos < 0).  One thread per 4 columns.
+// (selections whose expert is not local have pos < 0).  One thread per 4 columns.  TOPK > 0:
+// top_k known at compile time, so that a thread asks for all of a token's rows before it
+// adds the first (one load in flight per thread leaves a quarter of the bandwidth unused);
+// a selection that is not local adds zeros, which changes no bit of a sum that starts at +0.
+template <int TOPK>
 __global__ __launch_bounds__(256) void combine_kernel(const float* __restrict__ y,
                                                       const int32_t* __restrict__ pos,
                                                       float* __restrict__ out, int M, int top_k,
@@ -1592,9 +1596,23 @@ __global__ __launch_bounds__(256) void combine_kernel(const float* __restrict__ 
   if (c >= ncols) return;
   for (int t = blockIdx.y; t < M; t += gridDim.y) {  // grid.y is capped at 65535
     f32x4 sum = {0.f, 0.f, 0.f, 0.f};
-    for (int s = 0; s < top_k; ++s) {
-      const int r = pos[t * top_k + s];  // uniform
-      if (r >= 0) sum += *reinterpret_cast<const f32x4*>(y + (size_t)r * (size_t)ncols + c);
+    if constexpr (TOPK > 0) {
+      int r[TOPK];
+      f32x4 v[TOPK];
+#pragma unroll
+      for (int s = 0; s < TOPK; ++s) r[s] = pos[t * TOPK + s];  // uniform
+#pragma unroll
+      for (int s = 0; s < TOPK; ++s) {
+        v[s] = f32x4{0.f, 0.f, 0.f, 0.f};
+        if (r[s] >= 0) v[s] = *reinterpret_cast<const f32x4*>(y + (size_t)r[s] * (size_t)ncols + c);
+      }
+#pragma unroll
+      for (int s = 0; s < TOPK; ++s) sum += v[s];
+    } else {
+      for (int s = 0; s < top_k; ++s) {
+        const int r = pos[t * top_k + s];  // uniform
+        if (r >= 0) sum += *reinterpret_cast<const f32x4*>(y + (size_t)r * (size_t)ncols + c);
+      }
     }
     f32x4* o = reinterpret_cast<f32x4*>(out + (size_t)t * (size_t)ncols + c);
     *o = overwrite ? sum : *o + sum;
@@ -1847,8 +1865,17 @@ void launch_fill_i32(int32_t* dst, int32_t value, int n, hipStream_t stream) {
 void launch_combine(const float* y, const int32_t* pos, float* out, int M, int top_k, int hidden,
                     bool overwrite, hipStream_t stream) {
   const dim3 grid((unsigned)((hidden / 4 + 255) / 256), (unsigned)(M < 65535 ? M : 65535));
-  hipLaunchKernelGGL(combine_kernel, grid, dim3(256), 0, stream, y, pos, out, M, top_k, hidden,
-                     overwrite ? 1 : 0);
+  const int ow = overwrite ? 1 : 0;
+  switch (top_k) {
+#define VK_COMBINE(K_)                                                                              \
+  case K_:                                                                                          \
+    hipLaunchKernelGGL(combine_kernel<K_>, grid, dim3(256), 0, stream, y, pos, out, M, top_k, hidden, ow); \
+    break;
+    VK_COMBINE(2) VK_COMBINE(4) VK_COMBINE(6) VK_COMBINE(8)
+#undef VK_COMBINE
+    default:
+      hipLaunchKernelGGL(combine_kernel<0>, grid, dim3(256), 0, stream, y, pos, out, M, top_k, hidden, ow);
+  }
 }
 
 bool prepare_moe_kernels() {
