@@ -280,6 +280,38 @@ def test_decode_with_more_runs_than_workgroups():
     assert g["EM"] // 16 > 256, "fewer runs than the device has compute units"
 
 
+@pytest.mark.parametrize("T", [1, 2, 9, 40])
+def test_decode_with_k_shared_between_wavefronts(T):
+    """Every K-split shape of the decode kernel, put in the tuning store for the call's size:
+    one token (a unit per 2 to 8 wavefronts, what the compiled-in rule chooses it for), and
+    sizes where a workgroup has more units than half its wavefronts and takes them a few at
+    a time.  Weight scales outside the fast range make some units leave the fast path in
+    one part of K only."""
+    cfg = synth.MoEConfig("c9", 1536, 1024, 8, 2, (T,), "uniform")
+    w = _weights(cfg, 9001 if T == 9 else 9000)
+    if T == 9 and not getattr(w, "tiny_scales_set", False):
+        for t in (w.w13_scale, w.w2_scale):  # (tiny ones: nothing overflows)
+            special = torch.tensor([0, 1, 63], dtype=torch.uint8, device=dev())
+            pick = (synth.rand_u63(t.numel(), 91, 31, dev()).reshape(t.shape) >> 12) % 2048
+            mask = pick < 3
+            t[mask] = special[pick[mask]]
+        w.tiny_scales_set = True
+    A, lg = _inputs(cfg, T, 9100 + T)
+    n_flat = T * cfg.top_k
+    split = [(st, c) for st in (0, 1) for c in ve.moe_tile_candidates(st) if c[0] == 3]
+    assert {st for st, _ in split} == {0, 1}, "no K-split shape among the candidates"
+    for st0, c0 in [x for x in split if x[0] == 0]:
+        for st1, c1 in [x for x in split if x[0] == 1]:
+            ve.moe_tile_set(0, cfg.H, cfg.I, n_flat, c0)
+            ve.moe_tile_set(1, cfg.I, cfg.H, n_flat, c1)
+            try:
+                assert ve.moe_tile_query(0, cfg.H, cfg.I, n_flat) == (c0, True)
+                _check(cfg, T, w, A, lg, tight=True)
+            finally:
+                ve.moe_tile_set(0, cfg.H, cfg.I, n_flat, None)
+                ve.moe_tile_set(1, cfg.I, cfg.H, n_flat, None)
+
+
 @pytest.mark.parametrize("use_workspace", [True, False])
 @pytest.mark.parametrize("bs", [16, 48, 80, 128])
 def test_tile_kernels_block_sizes(bs, use_workspace):

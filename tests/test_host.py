@@ -300,16 +300,22 @@ def test_synth_is_deterministic_and_prefix_stable():
 def test_tile_candidates_and_compiled_in_rules():
     for stage in (0, 1):
         cands = ve.moe_tile_candidates(stage)
-        assert len(cands) == 6 and len(set(cands)) == 6
+        assert len(cands) == 8 and len(set(cands)) == 8
+        plain = {c[1:] for c in cands if c[0] == 2}
+        assert all(c[1:] in plain for c in cands if c[0] == 3)   # a K-split shape has its plain form to fall back to
         assert (0, 4, 4, 0) in cands                      # the tile kernels
         for n_flat, K, ncols in [(1, 2880, 2880), (256, 2880, 2880), (512, 7168, 2048), (513, 2880, 2880),
                                  (131072, 7168, 2048), (64, 256, 512)]:
             shape, stored = ve.moe_tile_query(stage, K, ncols, n_flat)
             assert not stored and shape in cands, (stage, n_flat, shape)   # selectors return table entries only
             # the decode kernels up to 512 routed rows, where a pass's rows fit LDS and registers
-            assert (shape[0] == 2) == (n_flat <= 512 and K <= (4096 if stage == 0 else 3072))
+            assert (shape[0] in (2, 3)) == (n_flat <= 512 and K <= (4096 if stage == 0 else 3072))
     assert ve.moe_tile_query(0, 2880, 2880, 128)[0] == (2, 8, 2, 4)
     assert ve.moe_tile_query(0, 4096, 1536, 6)[0] == (2, 4, 2, 8)                   # rows of K = 4096
+    # one token: fewer units than half the device's wavefronts, K shared between them
+    assert ve.moe_tile_query(0, 2880, 2880, 4)[0] == (3, 8, 2, 4) and ve.moe_tile_query(1, 2880, 2880, 4)[0] == (3, 8, 1, 8)
+    assert ve.moe_tile_query(1, 1536, 4096, 6)[0] == (3, 8, 2, 4)                   # ... with two tiles a unit
+    assert ve.moe_tile_query(0, 2880, 2880, 8)[0] == (2, 8, 2, 4) and ve.moe_tile_query(0, 512, 2880, 4)[0] == (2, 8, 2, 2)
     assert ve.moe_tile_query(0, 256, 512, 32)[0] == (2, 8, 2, 2) and ve.moe_tile_query(1, 512, 256, 32)[0] == (2, 8, 1, 4)
     assert ve.default_block_size(0, 4) == 16 and ve.default_block_size(1 << 20, 32) == 128
 

@@ -400,7 +400,7 @@ __device__ unsigned long long g_decode_trace[2][kTraceWorkgroups][kTraceSlots];
 #define DECODE_TRACE(slot_) do { } while (0)
 #endif
 
-template <int STAGE, int WAVES, int NT, int D>
+template <int STAGE, int WAVES, int NT, int D, bool KSPLIT = false>
 __global__ __launch_bounds__(64 * WAVES) void stream_resident_kernel(GemmArgs p) {
   extern __shared__ u32x4 b_lds[];  // [nsteps][2][2][64] operand planes, block scales, weight scales
   __shared__ int run_block0[kMaxRuns];
@@ -408,6 +408,7 @@ __global__ __launch_bounds__(64 * WAVES) void stream_resident_kernel(GemmArgs p)
   __shared__ int run_cum[kMaxRuns];     // blocks of the runs up to and including this one
   __shared__ int slice_sh[2];           // this workgroup's slice of the (run, unit) space
   __shared__ int pass_slow[2];          // set while staging: this pass takes the exact path
+  __shared__ int ks_bad[KSPLIT ? WAVES : 1];  // K split: a wavefront's part of its unit left the fast path
   DECODE_TRACE(0);  // entry
   if (STAGE == 0) clear_out_share<64 * WAVES>(p);
   const int tid = threadIdx.x;
@@ -549,7 +550,6 @@ __global__ __launch_bounds__(64 * WAVES) void stream_resident_kernel(GemmArgs p)
   DECODE_TRACE(1);  // slice known to every wavefront
   const int s0 = slice_sh[0], s1 = slice_sh[1];  // n_runs * units is far below 2^31
   if (s0 >= s1) return;  // uniform over the workgroup
-  const int r_first = s0 / units;
 
   struct Stage {
     u32x4 w[NT];
@@ -590,18 +590,38 @@ __global__ __launch_bounds__(64 * WAVES) void stream_resident_kernel(GemmArgs p)
                 (lane >> 2)) * 16 + (lane & 1) * 8);
   uint8_t* const bsc0 = bsc_lds + (wave >> 2) * 64 + (wave & 3) * 16 + (lane >> 2);
 
-  for (int r = r_first; r <= (s1 - 1) / units; ++r) {
+  // Segments of the slice: the units [u0, u1) of run r.  K split: at most WAVES / 2 units
+  // at a time, each shared by WAVES / (u1 - u0) wavefronts (ks_n of them, wavefront
+  // my_u + c * n_seg the c-th part of K: steps [k_begin, k_end)), summed through LDS.
+  for (int sl = s0; sl < s1;) {
+    const int r = sl / units;
     const int base_slot = r * units;
-    const int u0 = max(s0, base_slot) - base_slot;
-    const int u1 = min(s1, base_slot + units) - base_slot;
+    const int u0 = sl - base_slot;
+    int u1_ = min(s1, base_slot + units) - base_slot;
+    if constexpr (KSPLIT) u1_ = min(u1_, u0 + WAVES / 2);
+    const int u1 = u1_;
+    sl = base_slot + u1;
     const int b0 = run_block0[r];
     const int run_blocks = 1;  // every block is a run of its own
     const int e = run_expert[r];
     const int run_row0 = b0 * p.block_size;
     const int run_tiles = run_blocks * (p.block_size / 16);
     // units of this wavefront in the segment: first, first + WAVES, ...
-    const int first = u0 + wave;
-    const int n_my = first < u1 ? (u1 - first + WAVES - 1) / WAVES : 0;
+    int first_ = u0 + wave;
+    int n_my_ = first_ < u1 ? (u1 - first_ + WAVES - 1) / WAVES : 0;
+    int n_seg = 1, ks_n = 1, my_c = 0, k_begin_ = 0, k_end_ = nsteps;
+    if constexpr (KSPLIT) {
+      n_seg = u1 - u0;                      // 1 .. WAVES / 2
+      ks_n = min(WAVES / n_seg, nsteps);    // parts of K, every one with a step
+      my_c = wave / n_seg;
+      first_ = u0 + (wave - my_c * n_seg);
+      n_my_ = my_c < ks_n ? 1 : 0;
+      if (n_my_ > 0) {
+        k_begin_ = my_c * nsteps / ks_n;
+        k_end_ = (my_c + 1) * nsteps / ks_n;
+      }
+    }
+    const int first = first_, n_my = n_my_, k_begin = k_begin_, k_end = k_end_;
 
     // compute-side pointers of the current unit (start: the first one)
     const uint8_t* cw[NT];
@@ -621,7 +641,9 @@ __global__ __launch_bounds__(64 * WAVES) void stream_resident_kernel(GemmArgs p)
 #pragma unroll
       for (int t = 0; t < NT; ++t)
         st.w[t] = *reinterpret_cast<const u32x4*>(lrow[t] + (size_t)g * 16);
-      if (++ld_ks == nsteps) {  // uniform, no memory operation inside
+      if constexpr (KSPLIT) {
+        if (++ld_ks == k_end) ld_ks = k_end - 1;  // past this wavefront's part: stay on its last step
+      } else if (++ld_ks == nsteps) {  // uniform, no memory operation inside
         if (ld_units > 1) {
           --ld_units;
           ld_ks = 0;
@@ -665,7 +687,7 @@ __global__ __launch_bounds__(64 * WAVES) void stream_resident_kernel(GemmArgs p)
       sc_unit = cs[0] - (size_t)ln * groups;
 #pragma unroll
       for (int t = 0; t < NT; ++t) lrow[t] = cw[t];
-      ld_ks = 0;
+      ld_ks = KSPLIT ? k_begin : 0;
       ld_units = max(n_my, 1);
       fetch_scales(0);
 #pragma unroll
@@ -770,7 +792,7 @@ __global__ __launch_bounds__(64 * WAVES) void stream_resident_kernel(GemmArgs p)
         // The rows are staged in K order, a few K steps ahead of the first unit's
         // arithmetic, with a barrier after each portion: the weight stream starts
         // after the first portion and the rest of the splitting overlaps it.
-        write_rows(pieces_for(min(nsteps, D)));
+        write_rows(KSPLIT ? n_pieces : pieces_for(min(nsteps, D)));  // (K split: every part starts at once)
         if (pass_no == 1) DECODE_TRACE(9);  // first K steps split and written
         if (n_my > 0) {
           park_scales();
@@ -781,19 +803,22 @@ __global__ __launch_bounds__(64 * WAVES) void stream_resident_kernel(GemmArgs p)
         if (pass_no == 1) DECODE_TRACE(3);  // the stream starts
         if (tid == 0) pass_slow[flag ^ 1] = 0;  // for the next pass; its last reader is behind us
         const bool slow_pass = pass_slow[flag] != 0;
-        if (n_my == 0 || slow_pass) {
-          // no fast stream here: finish the staging in step with the other wavefronts
-          for (int f0 = D; staged < n_pieces; f0 += D) {
-            write_rows(pieces_for(min(nsteps, f0 + D)));
-            __syncthreads();
+        if constexpr (!KSPLIT) {
+          if (n_my == 0 || slow_pass) {
+            // no fast stream here: finish the staging in step with the other wavefronts
+            for (int f0 = D; staged < n_pieces; f0 += D) {
+              write_rows(pieces_for(min(nsteps, f0 + D)));
+              __syncthreads();
+            }
+            if (n_my == 0) continue;
           }
-          if (n_my == 0) continue;
         }
 
         f32x4 acc[NT];
         unsigned long long redo = 0ull;  // units (bit = index among this wavefront's) to redo
         if (slow_pass) {
           redo = n_my >= 64 ? ~0ull : (1ull << n_my) - 1ull;
+          if (KSPLIT && my_c > 0) redo = 0ull;  // the unit's first wavefront redoes all of it
         } else {
 #pragma unroll
           for (int t = 0; t < NT; ++t) acc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
@@ -830,6 +855,39 @@ __global__ __launch_bounds__(64 * WAVES) void stream_resident_kernel(GemmArgs p)
                                                                         sa[t], 0, sbl);
           };
 
+          if constexpr (KSPLIT) {
+            // this wavefront's part of K (none: a wavefront left over), then the parts of
+            // a unit summed in order by its first wavefront; every wavefront keeps the barriers
+            const int my_steps = n_my > 0 ? k_end - k_begin : 0;
+            for (int f0 = 0; f0 < my_steps; f0 += D) {
+#pragma unroll
+              for (int i = 0; i < D; ++i) {
+                if (f0 + i < my_steps) compute(st[i], k_begin + f0 + i);  // uniform
+                issue(st[i]);
+              }
+            }
+            __syncthreads();  // every wavefront is done with the operand planes: they hold the sums now
+            f32x4* const part = reinterpret_cast<f32x4*>(b_lds);
+            bool any_bad = __ballot(bad != 0u) != 0ull;
+            if (n_my > 0 && my_c > 0) {
+#pragma unroll
+              for (int t = 0; t < NT; ++t) part[(wave * NT + t) * 64 + lane] = acc[t];
+              if (lane == 0) ks_bad[wave] = any_bad ? 1 : 0;
+            }
+            __syncthreads();
+            if (n_my > 0 && my_c == 0) {
+              for (int c = 1; c < ks_n; ++c) {
+                const int w2 = wave + c * n_seg;
+#pragma unroll
+                for (int t = 0; t < NT; ++t) acc[t] += part[(w2 * NT + t) * 64 + lane];
+                any_bad |= ks_bad[w2] != 0;
+              }
+              if (any_bad)
+                redo = 1ull;
+              else if (my_flat >= 0)
+                epilogue_tile<STAGE, NT>(p, e, acc, col0, my_flat, srow, lq);
+            }
+          } else {
           const int total_steps = n_my * nsteps;
           int cks = 0;    // K step of the unit being computed
           int cunit = 0;  // its index among this wavefront's units
@@ -870,6 +928,7 @@ __global__ __launch_bounds__(64 * WAVES) void stream_resident_kernel(GemmArgs p)
               issue(st[i]);
             }
           }
+          }  // (not K split)
         }
 
         // ---- reference-exact pass over the units the fast path could not take
@@ -1664,11 +1723,11 @@ constexpr size_t kResidentLdsLimit = 150 * 1024;  // dynamic LDS the resident ke
 
 // True when the device grants the kernel its dynamic LDS (asked once per kernel;
 // a refusal makes the caller take the other variant).
-template <int STAGE, int WAVES, int NT, int D>
+template <int STAGE, int WAVES, int NT, int D, bool KSPLIT = false>
 bool resident_kernel_ready() {
   static const bool configured = [] {
     const hipError_t err = hipFuncSetAttribute(
-        reinterpret_cast<const void*>(stream_resident_kernel<STAGE, WAVES, NT, D>),
+        reinterpret_cast<const void*>(stream_resident_kernel<STAGE, WAVES, NT, D, KSPLIT>),
         hipFuncAttributeMaxDynamicSharedMemorySize, (int)kResidentLdsLimit);
     if (err != hipSuccess) (void)hipGetLastError();  // not left for the next caller to find
     return err == hipSuccess;
@@ -1676,10 +1735,10 @@ bool resident_kernel_ready() {
   return configured;
 }
 
-template <int STAGE, int WAVES, int NT, int D>
+template <int STAGE, int WAVES, int NT, int D, bool KSPLIT = false>
 bool launch_resident(const GemmArgs& g, size_t lds, hipStream_t stream) {
-  if (!resident_kernel_ready<STAGE, WAVES, NT, D>()) return false;
-  hipLaunchKernelGGL((stream_resident_kernel<STAGE, WAVES, NT, D>), dim3(num_compute_units()),
+  if (!resident_kernel_ready<STAGE, WAVES, NT, D, KSPLIT>()) return false;
+  hipLaunchKernelGGL((stream_resident_kernel<STAGE, WAVES, NT, D, KSPLIT>), dim3(num_compute_units()),
                      dim3(64 * WAVES), lds, stream, g);
   return true;
 }
@@ -1687,6 +1746,7 @@ bool launch_resident(const GemmArgs& g, size_t lds, hipStream_t stream) {
 // Launch shape of one stage.  variant kMoeVariantLds = the tile kernel.
 struct StagePlan {
   int variant, waves, nt, depth;
+  bool ksplit;  // the resident kernel with K shared between the wavefronts of a unit
   size_t resident_lds;
 };
 
@@ -1697,7 +1757,8 @@ StagePlan plan_stage(const GemmArgs& g) {
   if (!moe_tuning_find(STAGE, g.K, g.ncols, g.n_flat, &tile))
     tile = pick_moe_tile(g.n_flat, g.K, g.ncols, STAGE);
   StagePlan pl;
-  pl.variant = tile.variant;
+  pl.ksplit = tile.variant == kMoeVariantResidentKSplit;
+  pl.variant = pl.ksplit ? (int)kMoeVariantResident : tile.variant;
   pl.nt = tile.nt;
   pl.depth = tile.depth;
   pl.waves = tile.waves;
@@ -1705,6 +1766,8 @@ StagePlan plan_stage(const GemmArgs& g) {
   const int nsteps = (groups + 3) / 4;
   // operand planes + block scales + one weight-scale region per wavefront
   pl.resident_lds = (size_t)nsteps * (4096 + 64) + (size_t)pl.waves * pl.nt * 16 * groups;
+  // (K split: the partial sums of the wavefronts, 1 KB a tile, lie over the operand planes)
+  if (pl.ksplit && (size_t)nsteps * 4096 < (size_t)pl.waves * pl.nt * 1024) pl.ksplit = false;
   const int res_units = STAGE == 0 ? g.ncols / (8 * pl.nt) : g.ncols / (16 * pl.nt);
   if (pl.resident_lds > kResidentLdsLimit || g.num_blocks > kMaxRuns ||
       pl.nt * groups > 64 * resident_scale_pieces(pl.waves) ||
@@ -1735,6 +1798,14 @@ bool wide_kernel_applies(const GemmArgs& g) { return g.Aq != nullptr; }
 template <int STAGE>
 void launch_stage(const GemmArgs& g, const StagePlan& pl, hipStream_t stream) {
   if (pl.variant == kMoeVariantResident) {
+#define VK_RESIDENT(S_, W_, NT_, D_) \
+  if constexpr (STAGE == S_) { \
+    if (pl.ksplit && pl.waves == W_ && pl.nt == NT_ && pl.depth == D_ && \
+        launch_resident<S_, W_, NT_, D_, true>(g, pl.resident_lds, stream)) \
+      return; \
+  }
+    VK_KSPLIT_VARIANTS(VK_RESIDENT)
+#undef VK_RESIDENT
 #define VK_RESIDENT(S_, W_, NT_, D_) \
   if constexpr (STAGE == S_) { \
     if (pl.waves == W_ && pl.nt == NT_ && pl.depth == D_ && \
@@ -1882,6 +1953,9 @@ bool prepare_moe_kernels() {
   bool ok = wide_kernel_ready<0>() && wide_kernel_ready<1>() && prepare_mx_kernels();
 #define VK_READY(S_, W_, NT_, D_) ok = resident_kernel_ready<S_, W_, NT_, D_>() && ok;
   VK_RESIDENT_VARIANTS(VK_READY)
+#undef VK_READY
+#define VK_READY(S_, W_, NT_, D_) ok = resident_kernel_ready<S_, W_, NT_, D_, true>() && ok;
+  VK_KSPLIT_VARIANTS(VK_READY)
 #undef VK_READY
   MoeTile unused;
   (void)moe_tuning_find(0, 64, 64, 1, &unused);  // reads the tuning store now rather than on the first launch

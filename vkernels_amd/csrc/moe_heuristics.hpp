@@ -11,11 +11,13 @@
 
 namespace vk {
 
-enum { kMoeVariantLds = 0, kMoeVariantResident = 2 };
+enum { kMoeVariantLds = 0, kMoeVariantResident = 2, kMoeVariantResidentKSplit = 3 };
 
 struct MoeTile {
   int variant;  // kMoeVariantResident: one workgroup per compute unit, the
                 // activation rows of a run resident in LDS (decode);
+                // kMoeVariantResidentKSplit: the same, the K steps of a unit shared between
+                // the wavefronts that would otherwise have none (a handful of rows);
                 // kMoeVariantLds: the tile kernels (rows staged through LDS)
   int waves;    // wavefronts per workgroup
   int nt;       // 16-row weight tiles per wavefront
@@ -33,6 +35,9 @@ inline bool operator==(const MoeTile& a, const MoeTile& b) {
 #define VK_RESIDENT_VARIANTS(X) \
   X(0, 8, 2, 2) X(0, 8, 2, 4) X(0, 8, 2, 6) X(0, 4, 2, 4) X(0, 4, 2, 8) \
   X(1, 8, 2, 4) X(1, 8, 1, 4) X(1, 8, 1, 6) X(1, 8, 1, 8) X(1, 8, 1, 12)
+// ... and of its K-split form (every one is also in the list above: a plan that cannot
+// split K falls back to the same shape there).
+#define VK_KSPLIT_VARIANTS(X) X(0, 8, 2, 4) X(0, 8, 2, 6) X(1, 8, 1, 8) X(1, 8, 2, 4)
 
 struct MoeTileCandidate {
   int stage;
@@ -43,6 +48,9 @@ inline const MoeTileCandidate* moe_tile_candidates(size_t* count) {
   static const MoeTileCandidate table[] = {
 #define VK_CANDIDATE(S_, W_, NT_, D_) {S_, {kMoeVariantResident, W_, NT_, D_}},
       VK_RESIDENT_VARIANTS(VK_CANDIDATE)
+#undef VK_CANDIDATE
+#define VK_CANDIDATE(S_, W_, NT_, D_) {S_, {kMoeVariantResidentKSplit, W_, NT_, D_}},
+      VK_KSPLIT_VARIANTS(VK_CANDIDATE)
 #undef VK_CANDIDATE
       {0, {kMoeVariantLds, 4, 4, 0}},
       {1, {kMoeVariantLds, 4, 4, 0}},
@@ -93,8 +101,23 @@ struct MoeTileRule {
 //    are 3 to 5 % faster for gate/up; the number of runs that makes it so is not known
 //    here, and with skewed routing (27 active experts of 128) the same shape is much
 //    slower, so that choice is left to the tuning store.
+//
+// A single token or two: when the units of all rows (at most n_flat runs) are fewer than
+// half the wavefronts of the device, a wavefront has one unit or none, and a unit is a chain
+// of K / 128 dependent steps, a few in flight.  The K-split form gives the idle wavefronts a
+// part of K each.  Only the shapes whose rows of K values need 8 wavefronts to stage have it.
+constexpr int kMoeComputeUnits = 256;  // of the device the rules were swept on
+
 inline MoeTile pick_moe_tile(int n_flat, int K, int ncols, int stage) {
-  (void)ncols;  // no swept point separates on it: the units per wavefront follow from it, not the shape
+  if (n_flat <= kMoeDecodeMaxRows && K >= 1024 && K <= 3072) {
+    const long long spare = (long long)kMoeComputeUnits * 4;  // half of 8 wavefronts per compute unit
+    if (stage == 0 && (long long)n_flat * (ncols / 16) <= spare)
+      return MoeTile{kMoeVariantResidentKSplit, 8, 2, 4};
+    if (stage == 1 && (long long)n_flat * (ncols / 16) <= spare)
+      return MoeTile{kMoeVariantResidentKSplit, 8, 1, 8};
+    if (stage == 1 && (long long)n_flat * (ncols / 32) <= spare)
+      return MoeTile{kMoeVariantResidentKSplit, 8, 2, 4};
+  }
   static const MoeTileRule rules[] = {
       {0, kMoeDecodeMaxRows, 1024, {kMoeVariantResident, 8, 2, 2}},
       {0, kMoeDecodeMaxRows, 3072, {kMoeVariantResident, 8, 2, 4}},
