@@ -400,6 +400,13 @@ __device__ unsigned long long g_decode_trace[2][kTraceWorkgroups][kTraceSlots];
 #define DECODE_TRACE(slot_) do { } while (0)
 #endif
 
+// KSPLIT: the form for a handful of rows (one token), where a workgroup's slice is fewer
+// units than half its wavefronts and a unit, a chain of K / 128 dependent steps with D in
+// flight, is all a wavefront would do while most have nothing.  The slice is taken at most
+// WAVES / 2 units at a time; the WAVES / units wavefronts of a unit take a part of its K
+// steps each, all rows are staged before any of them starts, and the unit's first wavefront
+// adds the others' sums (through LDS, over the operand planes, in a fixed order) and runs
+// the epilogue, or the exact path if any part met a value outside the fast path's domain.
 template <int STAGE, int WAVES, int NT, int D, bool KSPLIT = false>
 __global__ __launch_bounds__(64 * WAVES) void stream_resident_kernel(GemmArgs p) {
   extern __shared__ u32x4 b_lds[];  // [nsteps][2][2][64] operand planes, block scales, weight scales

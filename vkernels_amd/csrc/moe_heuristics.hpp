@@ -92,9 +92,9 @@ struct MoeTileRule {
 // tiles (nt = 1) and keeps the bytes in flight per wavefront with a deeper pipeline.
 // Rows (each from the sweep table profiles/moe_decode_tile_sweep.md):
 //  - K <= 1024: a unit is a few steps long, and steps in flight past its end are
-//    wasted loads: the shallowest pipelines (256x512x8x2 at T = 64: 10.7 against 11.6 us);
+//    wasted loads: the shallowest pipelines (256x512x8x2 at T = 64: 10.7 against 11.4 us);
 //  - 3072 < K <= 4096 (4096x1536x64x6 gate/up): the rows of a pass fit LDS and registers
-//    only with 4 wavefronts per workgroup (34 against 69 us at T = 1, 98 against 185 us
+//    only with 4 wavefronts per workgroup (34 against 69 us at T = 1, 97 against 185 us
 //    at T = 32 for the tile kernel, which is what runs beyond K = 4096);
 //  - otherwise (8, 2, 4) / (8, 1, 8), within 5 % of the best of every other point swept:
 //    with 128 experts and 32 tokens or more, uniformly routed, the 4-wavefront shapes
