@@ -256,7 +256,11 @@ int vk_hip_init(void);
  * M tokens routed to top_k experts each (what to pass to
  * vk_hip_moe_align_block_size and on to the layer).  Any multiple of 16 works.
  *
- * A launch shape is four ints {variant, wavefronts, tiles, depth}.
+ * A launch shape is four ints {variant, wavefronts, tiles, depth}: variant 2 =
+ * the decode kernel (one workgroup per compute unit, a run's rows resident in
+ * LDS), 3 = the same with the K steps of a unit shared between wavefronts (a
+ * single token), 0 = the tile kernels; wavefronts per workgroup; 16-row weight
+ * tiles per wavefront; K steps in flight per wavefront.
  * vk_hip_moe_tile_candidates writes up to `capacity` shapes that stage 0
  * (gate/up) or 1 (down) can be launched at and returns how many there are.
  * vk_hip_moe_tile_query writes the shape a call of this problem size would be
