@@ -169,7 +169,7 @@ def test_sentinel_inside_a_block_keeps_the_rows_behind_it(hip_lib, prepack):
         assert nf and l2 <= 1e-4, (use_ws, m, l2)
 
 
-@pytest.mark.parametrize("T,prepack", [(16, False), (300, False), (300, True)])
+@pytest.mark.parametrize("T,prepack", [(1, False), (16, False), (300, False), (300, True)])
 def test_call_sequence_under_graph_capture(hip_lib, T, prepack):
     """route -> align -> fused layer (out overwritten) captured in a HIP graph after an
     eager warm-up, replayed with new inputs written into the same buffers, with eager

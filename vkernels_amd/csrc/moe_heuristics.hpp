@@ -96,6 +96,9 @@ struct MoeTileRule {
 //  - 3072 < K <= 4096 (4096x1536x64x6 gate/up): the rows of a pass fit LDS and registers
 //    only with 4 wavefronts per workgroup (34 against 69 us at T = 1, 97 against 185 us
 //    at T = 32 for the tile kernel, which is what runs beyond K = 4096);
+//  - down stage, up to 24 rows (2 to 4 tokens): units of two tiles, 4 to 5 % faster than
+//    single tiles there (2880x2880x32x4 at T = 4: 23.5 against 24.6 us; 4096x1536x64x6 at
+//    T = 2: 17.7 against 18.6 us), level or behind from 32 rows on;
 //  - otherwise (8, 2, 4) / (8, 1, 8), within 5 % of the best of every other point swept:
 //    with 128 experts and 32 tokens or more, uniformly routed, the 4-wavefront shapes
 //    are 3 to 5 % faster for gate/up; the number of runs that makes it so is not known
@@ -123,6 +126,7 @@ inline MoeTile pick_moe_tile(int n_flat, int K, int ncols, int stage) {
       {0, kMoeDecodeMaxRows, 3072, {kMoeVariantResident, 8, 2, 4}},
       {0, kMoeDecodeMaxRows, 4096, {kMoeVariantResident, 4, 2, 8}},
       {1, kMoeDecodeMaxRows, 1024, {kMoeVariantResident, 8, 1, 4}},
+      {1, 24, 3072, {kMoeVariantResident, 8, 2, 4}},
       {1, kMoeDecodeMaxRows, 3072, {kMoeVariantResident, 8, 1, 8}},
   };
   for (const MoeTileRule& r : rules)
