@@ -70,7 +70,8 @@ def _rms_metrics(g, c):
     return float(np.abs(d).max() / rms), float(np.linalg.norm(d) / np.linalg.norm(c.astype(np.float64)))
 
 
-@pytest.mark.parametrize("name,T,bs", [("c1", 16, 16), ("c1", 64, 16), ("c4", 33, 16), ("c1", 300, 64), ("c0", 16, 16)])
+@pytest.mark.parametrize("name,T,bs", [("c1", 1, 16), ("c1", 16, 16), ("c1", 64, 16), ("c4", 33, 16), ("c1", 300, 64),
+                                       ("c0", 16, 16)])
 def test_each_stage_against_the_oracle(hip_lib, name, T, bs):
     lib = _fns(hip_lib)
     cfg = synth.CONFIGS[name]
@@ -152,7 +153,8 @@ def test_each_stage_against_the_oracle(hip_lib, name, T, bs):
         assert np.array_equal(out.cpu().numpy().view(np.uint32), c_out.view(np.uint32)), bias is None
 
 
-@pytest.mark.parametrize("name,T,bs,tp", [("c1", 32, 16, 2), ("c4", 7, 16, 2), ("c1", 200, 64, 3), ("c0", 16, 16, 2)])
+@pytest.mark.parametrize("name,T,bs,tp", [("c1", 1, 16, 2), ("c1", 32, 16, 2), ("c4", 7, 16, 2), ("c1", 200, 64, 3),
+                                          ("c0", 16, 16, 2)])
 def test_tensor_parallel_composition(hip_lib, name, T, bs, tp):
     """Every rank's K slice through the GEMM stages, the slices summed where the caller's
     all-reduce goes, the epilogues once: the fused oracle's layer."""
