@@ -211,8 +211,11 @@ __global__ __launch_bounds__(256) void split_rows_fp6_kernel(const uint16_t* __r
                                                              uint8_t* __restrict__ row_bad, int K,
                                                              int rows,
                                                              const int32_t* __restrict__ sorted_ids,
-                                                             int n_flat) {
+                                                             int n_flat, int32_t* __restrict__ fill,
+                                                             int fill_n) {
   __shared__ int bad_rows[256];  // per row of the workgroup
+  // (the second stage's table of sorted positions, set to "none" on the way: one launch less)
+  for (int i = (int)(blockIdx.x * 256 + threadIdx.x); i < fill_n; i += (int)(gridDim.x * 256)) fill[i] = -1;
   const int kp = mx_kp(K);
   const int bpr = kp / 32;                       // blocks of a row
   const int rpg = split_rows_per_group(kp);      // rows of a workgroup
@@ -374,7 +377,9 @@ __global__ __launch_bounds__(256) void quant_rows_w4_kernel(const uint16_t* __re
                                                             uint8_t* __restrict__ xq,
                                                             uint8_t* __restrict__ row_bad, int K,
                                                             const int32_t* __restrict__ sorted_ids,
-                                                            int n_flat) {
+                                                            int n_flat, int32_t* __restrict__ fill,
+                                                            int fill_n) {
+  for (int i = (int)(blockIdx.x * 256 + threadIdx.x); i < fill_n; i += (int)(gridDim.x * 256)) fill[i] = -1;
   const int kp = mx_kp(K);
   const size_t row = blockIdx.x;
   if (sorted_ids != nullptr) {  // as split_rows_fp6_kernel: routed rows only (uniform per workgroup)
@@ -1139,28 +1144,28 @@ bool mx_plan(const FusedMoeArgs& a, bool need_stage0, MxPlan& pl) {
 
 void mx_stage0(const FusedMoeArgs& a, const MxPlan& pl, hipStream_t stream) {
   if (pl.terms0 == 1) {
-    hipLaunchKernelGGL(quant_rows_w4_kernel, dim3(a.M), dim3(256), 0, stream, a.A, pl.aq, pl.abad, a.hidden, nullptr, 0);
+    hipLaunchKernelGGL(quant_rows_w4_kernel, dim3(a.M), dim3(256), 0, stream, a.A, pl.aq, pl.abad, a.hidden, nullptr, 0, nullptr, 0);
     launch_mx_stage_t<0, 1>(pl.g0, stream);
   } else if (pl.terms0 == 2) {
-    hipLaunchKernelGGL(split_rows_fp6_kernel<2>, split_grid(a.M, a.hidden), dim3(256), 0, stream, a.A, pl.aq, pl.abad, a.hidden, a.M, nullptr, 0);
+    hipLaunchKernelGGL(split_rows_fp6_kernel<2>, split_grid(a.M, a.hidden), dim3(256), 0, stream, a.A, pl.aq, pl.abad, a.hidden, a.M, nullptr, 0, nullptr, 0);
     launch_mx_stage_t<0, 2>(pl.g0, stream);
   } else {
-    hipLaunchKernelGGL(split_rows_fp6_kernel<3>, split_grid(a.M, a.hidden), dim3(256), 0, stream, a.A, pl.aq, pl.abad, a.hidden, a.M, nullptr, 0);
+    hipLaunchKernelGGL(split_rows_fp6_kernel<3>, split_grid(a.M, a.hidden), dim3(256), 0, stream, a.A, pl.aq, pl.abad, a.hidden, a.M, nullptr, 0, nullptr, 0);
     launch_mx_stage_t<0, 3>(pl.g0, stream);
   }
 }
 
-// split act (the routed rows of the sorted order) -> second stage -> per-token sum
+// split act (the routed rows of the sorted order; the same kernel clears the table of
+// sorted positions) -> second stage -> per-token sum
 void mx_stage1(const FusedMoeArgs& a, const MxPlan& pl, hipStream_t stream) {
-  launch_fill_i32(pl.pos, -1, a.M * a.top_k, stream);
   if (pl.terms1 == 1) {
-    hipLaunchKernelGGL(quant_rows_w4_kernel, dim3(a.EM), dim3(256), 0, stream, a.act, pl.cq, pl.cbad, a.ispp, a.sorted_ids, a.M * a.top_k);
+    hipLaunchKernelGGL(quant_rows_w4_kernel, dim3(a.EM), dim3(256), 0, stream, a.act, pl.cq, pl.cbad, a.ispp, a.sorted_ids, a.M * a.top_k, pl.pos, a.M * a.top_k);
     launch_mx_stage_t<1, 1>(pl.g1, stream);
   } else if (pl.terms1 == 2) {
-    hipLaunchKernelGGL(split_rows_fp6_kernel<2>, split_grid(a.EM, a.ispp), dim3(256), 0, stream, a.act, pl.cq, pl.cbad, a.ispp, a.EM, a.sorted_ids, a.M * a.top_k);
+    hipLaunchKernelGGL(split_rows_fp6_kernel<2>, split_grid(a.EM, a.ispp), dim3(256), 0, stream, a.act, pl.cq, pl.cbad, a.ispp, a.EM, a.sorted_ids, a.M * a.top_k, pl.pos, a.M * a.top_k);
     launch_mx_stage_t<1, 2>(pl.g1, stream);
   } else {
-    hipLaunchKernelGGL(split_rows_fp6_kernel<3>, split_grid(a.EM, a.ispp), dim3(256), 0, stream, a.act, pl.cq, pl.cbad, a.ispp, a.EM, a.sorted_ids, a.M * a.top_k);
+    hipLaunchKernelGGL(split_rows_fp6_kernel<3>, split_grid(a.EM, a.ispp), dim3(256), 0, stream, a.act, pl.cq, pl.cbad, a.ispp, a.EM, a.sorted_ids, a.M * a.top_k, pl.pos, a.M * a.top_k);
     launch_mx_stage_t<1, 3>(pl.g1, stream);
   }
   launch_combine(pl.y, pl.pos, a.out, a.M, a.top_k, a.hidden, (a.flags & 1u) != 0u, stream);
@@ -1191,9 +1196,9 @@ void launch_split_rows_fp6(const uint16_t* x, int rows, int K, int terms, uint8_
                            hipStream_t stream) {
   if (rows <= 0) return;
   if (terms == 2)
-    hipLaunchKernelGGL(split_rows_fp6_kernel<2>, split_grid(rows, K), dim3(256), 0, stream, x, xq, row_bad, K, rows, nullptr, 0);
+    hipLaunchKernelGGL(split_rows_fp6_kernel<2>, split_grid(rows, K), dim3(256), 0, stream, x, xq, row_bad, K, rows, nullptr, 0, nullptr, 0);
   else
-    hipLaunchKernelGGL(split_rows_fp6_kernel<3>, split_grid(rows, K), dim3(256), 0, stream, x, xq, row_bad, K, rows, nullptr, 0);
+    hipLaunchKernelGGL(split_rows_fp6_kernel<3>, split_grid(rows, K), dim3(256), 0, stream, x, xq, row_bad, K, rows, nullptr, 0, nullptr, 0);
 }
 
 // ---- MXFP4 orchestration ops (device counterparts of moe_aux.cpp) -----------------
