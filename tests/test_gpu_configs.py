@@ -312,6 +312,25 @@ def test_decode_with_k_shared_between_wavefronts(T):
                 ve.moe_tile_set(1, cfg.I, cfg.H, n_flat, None)
 
 
+def test_k_shared_between_wavefronts_with_rows_outside_the_fast_range():
+    """Two tokens, the compiled-in rule's K-split shapes: one row of tiny activations (block
+    exponents below the fast path's range) makes its pass take the exact path, which the
+    first wavefront of every unit runs over all of K."""
+    cfg = synth.MoEConfig("c9", 1536, 1024, 8, 2, (2,), "uniform")
+    assert ve.moe_tile_query(0, cfg.H, cfg.I, 4)[0][0] == 3 and ve.moe_tile_query(1, cfg.I, cfg.H, 4)[0][0] == 3
+    w = _weights(cfg, 9000)
+    A, lg = _inputs(cfg, 2, 9300)
+    A = A.copy()
+    A[1, :] = synth.f32_to_bf16_bits(synth.bf16_bits_to_f32(A[1, :]) * np.float32(2.0 ** -60))
+    g = _run_gpu(cfg, w, A, lg)
+    ids, tw = oracle.route_topk(lg, cfg.top_k, True)
+    c = cpu_layer(A, w.numpy(), ids, tw)
+    for t in range(2):  # row by row: the rows differ by many orders of magnitude (relative L2 is what binds)
+        max_rel, rel_l2, nf = error_metrics(g["out"][t], c["out"][t])
+        assert nf and max_rel <= MAX_ABS_TOL and rel_l2 <= REL_L2_TOL, (t, max_rel, rel_l2)
+    assert np.any(c["out"][1] != 0)
+
+
 @pytest.mark.parametrize("use_workspace", [True, False])
 @pytest.mark.parametrize("bs", [16, 48, 80, 128])
 def test_tile_kernels_block_sizes(bs, use_workspace):
