@@ -68,6 +68,8 @@ def parse_args():
                          "biases and swiglu_limit 7.0; the SiTU activation (beta 3, linear_beta 20) and both biases")
     ap.add_argument("--weight-sets", type=int, default=0, help="0 = enough to exceed 1 GiB")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    ap.add_argument("--no-graph", action="store_true",
+                    help="skip the HIP-graph replay of the decode step (`graph_ms_per_step`)")
     ap.add_argument("--block-size", type=int, default=0)
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a 512 MiB device copy three times, so that a profiler's "
@@ -237,6 +239,32 @@ def run_workload(args, workload, steps, warmup, prepack, split_terms=None, w4a4=
     torch.cuda.synchronize()
     ms_per_step = (time.perf_counter() - t0) / steps * 1e3
 
+    # The same steps as captured HIP graphs, one per weight set, replayed in rotation: how a
+    # serving loop runs decode (the reference's caller captures the layer,
+    # src/python/vkernels/vllm_experts.py:142-246).  Decode-sized batches only: beyond, a
+    # step is milliseconds and its launches do not matter.
+    graph_ms_per_step = None
+    if not prefill and not args.no_graph:
+        graphs = []
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            for s in range(n_sets):
+                g = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(g, stream=side):
+                    step(s)
+                graphs.append(g)
+        torch.cuda.current_stream().wait_stream(side)
+        for i in range(min(warmup, 5)):
+            graphs[i % n_sets].replay()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for i in range(steps):
+            graphs[i % n_sets].replay()
+        torch.cuda.synchronize()
+        graph_ms_per_step = (time.perf_counter() - t0) / steps * 1e3
+        del graphs
+
     # Second loop: the same steps with events around each GEMM stage.
     ev = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(steps)]
     for i in range(min(warmup, 5)):
@@ -277,7 +305,8 @@ def run_workload(args, workload, steps, warmup, prepack, split_terms=None, w4a4=
         roofline = {
             "bound": "mfma", "kernel": kernel,
             "achieved": fused_tflops, "peak": FP4_PEAK_TFLOPS, "unit": "TFLOP/s",
-            "frac": fused_tflops / FP4_PEAK_TFLOPS, "traffic": None,
+            "frac": fused_tflops / FP4_PEAK_TFLOPS,
+            "traffic": measured_traffic(workload) if prepack and not w4a4 and not terms else None,
             "matrix_rate_frac": issued * fused_tflops / FP4_PEAK_TFLOPS,
             "flops_per_launch": flops, "avg_launch_us": down_avg * 1e3,
             "median_launch_us": down_ms[len(down_ms) // 2] * 1e3,
@@ -297,6 +326,7 @@ def run_workload(args, workload, steps, warmup, prepack, split_terms=None, w4a4=
         "steps": steps,
         "warmup": warmup,
         "ms_per_step": ms_per_step,
+        "graph_ms_per_step": graph_ms_per_step,
         "config": {
             "workload": f"{cfg.name} T={T}: hidden {H}, intermediate {I}, {cfg.E} experts, "
                         f"top-{k}, MXFP4 weights, bf16 activations, {cfg.logits} routing",
@@ -344,6 +374,7 @@ def main():
         "steps": args.steps,
         "warmup": args.warmup,
         "ms_per_step": rec["ms_per_step"],
+        "graph_ms_per_step": rec["graph_ms_per_step"],
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,

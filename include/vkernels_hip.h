@@ -98,9 +98,8 @@ size_t vk_moe_align_block_size_max_em(int32_t M, int32_t top_k,
  *   block_size  the alignment sorted_ids/expert_ids were built with; any
  *               positive multiple of 16
  *   hidden, ispp multiples of 64
- *   b13         [E, 2*ispp] fp32 or null; b2 [E, hidden] fp32 or null; 16-byte
- *               aligned (the kernels read four columns at a time; a pointer
- *               that is not is refused with VK_ERROR_INVALID_ARGUMENT)
+ *   b13         [E, 2*ispp] fp32 or null; b2 [E, hidden] fp32 or null; aligned
+ *               like any float array (4 bytes), as in the reference
  *   activation  0 = SwiGLU (g, u clamped by swiglu_limit when it is > 0),
  *               1 = SiTU with beta, linear_beta
  */

@@ -247,3 +247,42 @@ def test_apply_hands_back_bf16_on_request(hip_lib):
     assert half.dtype == torch.bfloat16 and torch.equal(half, full.to(torch.bfloat16))
     none = fe.apply(A[:0], ids[:0], tw[:0], output_dtype=torch.bfloat16)
     assert none.dtype == torch.bfloat16 and tuple(none.shape) == (0, cfg.H)
+
+
+@pytest.mark.parametrize("T,prepack,use_workspace", [(32, False, True), (300, False, False), (300, False, True),
+                                                     (300, True, True)])
+def test_biases_need_only_the_alignment_of_floats(hip_lib, T, prepack, use_workspace):
+    """b13 / b2 that start 4 bytes into an allocation (a view inside a larger buffer), as
+    the reference accepts them: the act rows are the same bits as with the 16-byte
+    aligned copies, on the decode kernels, both raw-weight tile kernels and the prepacked
+    path, and `out` is the same up to the spread of the atomic adds."""
+    cfg = synth.CONFIGS["c1"]
+    w = cfgs._weights(cfg, 1500)
+    A_bits, lg = cfgs._inputs(cfg, T, 5300 + T)
+    b13 = (synth.rand_normal((cfg.E, 2 * cfg.I), 5300, 21) * 0.5).astype(np.float32)
+    b2 = (synth.rand_normal((cfg.E, cfg.H), 5300, 22) * 0.5).astype(np.float32)
+    res = []
+    for shift in (0, 1):
+        h13 = torch.zeros(b13.size + 1, dtype=torch.float32, device=dev())
+        h2 = torch.zeros(b2.size + 1, dtype=torch.float32, device=dev())
+        v13 = h13[shift:shift + b13.size].view(b13.shape)
+        v2 = h2[shift:shift + b2.size].view(b2.shape)
+        v13.copy_(to_dev(b13))
+        v2.copy_(to_dev(b2))
+        assert v13.data_ptr() % 16 == 4 * shift and v2.data_ptr() % 16 == 4 * shift
+        fe = ve.FusedExperts(w.w13, w.w13_scale, w.w2, w.w2_scale, b13=v13, b2=v2,
+                             scratch=ve.CaptureSafeScratch(), prepack=prepack)
+        fe.use_workspace = use_workspace
+        A = to_dev(A_bits, torch.bfloat16)
+        ids, tw = fe.route(to_dev(lg), cfg.top_k, True)
+        bs = ve.default_block_size(T, cfg.top_k)
+        sids, eids, _, max_em = fe.align(ids, bs)
+        out = fe.apply(A, ids, tw, block_size=bs)
+        torch.cuda.synchronize()
+        act = fe.scratch.get(("act", fe.ispp), max_em * fe.ispp, dtype=torch.bfloat16, device=dev())
+        real = np.nonzero(sids.cpu().numpy() < T * cfg.top_k)[0]
+        res.append((out.cpu().numpy(), act.view(torch.int16).cpu().numpy().reshape(max_em, cfg.I)[real].copy()))
+    assert np.array_equal(res[0][1], res[1][1]), "act differs with a bias that is only 4-byte aligned"
+    f, o = res[0][0].astype(np.float64), res[1][0].astype(np.float64)
+    rms = float(np.sqrt(np.mean(f ** 2)))
+    assert float(np.max(np.abs(f - o))) <= 1e-3 * rms

@@ -247,6 +247,126 @@ def test_onehot_rows_read_back_the_dequantised_weights(hip_lib, path):
     assert np.isnan(exp[I:, 5]).all() and np.isfinite(exp[I:, 6]).all()
 
 
+def _bf16_order(bits):
+    """bf16 bit patterns -> integers that order like the values, +0 and -0 both 0."""
+    b = bits.astype(np.int64)
+    return np.where(b & 0x8000, -(b & 0x7FFF), b & 0x7FFF)
+
+
+@pytest.mark.parametrize("path", ["packed", "packed3", "packed2", "workspace", "plain", "resident"])
+def test_onehot_rows_through_the_first_stage(hip_lib, path):
+    """A rows with a single 1.0 at column k: the gate and up sums of sorted row r are single
+    exact products, W13[e, c, k] and W13[e, I + c, k], so act[r, c] = bf16(silu(g) u) pins
+    the values the first stage multiplies by (its prepack row map and its template
+    instantiations differ from the second stage's).  Expert 0: the 12 finite codes; gate
+    rows take scale bytes 64, 65, 127, 189, 190 and the up row of the same column the
+    mirrored byte (254 - s), so every product is of order one: a tiny g gives g / 2 * u and
+    a huge positive one g * u exactly, in the oracle and in the kernels' hardware
+    exponential and reciprocal alike.  Expert 1: all 16 codes in two rows, scale bytes 0,
+    1, 63, 191, 200, 255 (flagged units: the exact path).  act must be within one bf16 unit
+    in the last place of the oracle's everywhere, and bit-equal in at least 99 % of the
+    values."""
+    E, I = 2, 192
+    H = 256 if path == "resident" else 576
+    M = E * H
+    rng = np.random.default_rng(23)
+    fin = np.array(synth.FINITE_CODES, dtype=np.uint8)
+    w13 = np.zeros((E, 2 * I, H // 2), dtype=np.uint8)
+    w13[0] = fin[rng.integers(0, 12, (2 * I, H // 2))] | (fin[rng.integers(0, 12, (2 * I, H // 2))] << 4)
+    w13[1] = rng.integers(0, 256, (2 * I, H // 2)).astype(np.uint8)
+    keep = np.ones(2 * I, dtype=bool)
+    keep[[5, I + 70]] = False                                       # rows that keep their inf/NaN codes
+    lo, hi = w13[1] & 15, w13[1] >> 4
+    lo[keep] = fin[lo[keep] % 12]
+    hi[keep] = fin[hi[keep] % 12]
+    w13[1] = lo | (hi << 4)
+    w13s = np.zeros((E, 2 * I, H // 32), dtype=np.uint8)
+    w13s[0, :I] = np.array([64, 65, 127, 189, 190], dtype=np.uint8)[rng.integers(0, 5, (I, H // 32))]
+    w13s[0, I:] = 254 - w13s[0, :I]
+    w13s[1] = np.array([0, 1, 63, 191, 200, 255], dtype=np.uint8)[rng.integers(0, 6, (2 * I, H // 32))]
+    w2 = (fin[rng.integers(0, 12, (E, H, I // 2))] | (fin[rng.integers(0, 12, (E, H, I // 2))] << 4)).astype(np.uint8)
+    w2s = np.full((E, H, I // 32), 127, dtype=np.uint8)
+    ids = (np.arange(M) // H).astype(np.int32).reshape(M, 1)
+    A = np.zeros((M, H), dtype=np.uint16)
+    A[np.arange(M), np.arange(M) % H] = 0x3F80                        # 1.0
+    kw = dict(prepack=path.startswith("packed"))
+    if path in ("packed2", "packed3"):
+        kw["split_terms"] = int(path[-1])
+    fe = ve.FusedExperts(to_dev(w13), to_dev(w13s), to_dev(w2), to_dev(w2s), scratch=ve.CaptureSafeScratch(), **kw)
+    fe.use_workspace = path not in ("plain", "resident")
+    bs = 16 if path == "resident" else 128
+    d_ids = to_dev(ids)
+    sids, eids, out_em, max_em = fe.align(d_ids, bs)
+    fe.apply(to_dev(A, torch.bfloat16), d_ids, None, block_size=bs)
+    torch.cuda.synchronize()
+    act = fe.scratch.get(("act", I), max_em * I, dtype=torch.bfloat16, device=dev())
+    got = act.view(torch.int16).cpu().numpy().view(np.uint16).reshape(max_em, I)
+    s_np = sids.cpu().numpy()
+    # expected: the oracle's first stage on the same rows, in the same sorted order
+    eids16 = np.repeat(eids.cpu().numpy(), bs // 16).astype(np.int32)
+    gate_up = oracle.moe_gateup(A, w13, w13s, s_np, eids16, M, H, 0, H, I, 1, max_em)
+    exp = oracle.moe_act_epilogue(gate_up, None, s_np, eids16, M, 1, max_em, I)
+    real = np.nonzero(s_np < M)[0]
+    first = real[s_np[real] < H]                                     # expert 0's rows: the scaled-MFMA path
+    # ... where the expectation is the products themselves for the tiny and the huge gates
+    g = synth.bf16_bits_to_f32(oracle.dequant_weight_tile(w13[0], w13s[0], 2 * I, H)).astype(np.float64)  # [H, 2I]
+    k_of = s_np[first] % H
+    gg, uu = g[k_of, :I], g[k_of, I:]
+    gsc = np.repeat(w13s[0, :I].T, 32, axis=0)[k_of]                 # the gate's scale byte per (row, column)
+    want = np.where(gsc <= 65, gg / 2 * uu, np.where(gg > 0, gg * uu, 0.0))
+    closed = gsc != 127
+    assert np.array_equal(synth.bf16_bits_to_f32(exp[first])[closed].astype(np.float64), want[closed])
+    for name, rows in (("scaled MFMA path", first), ("exact path", real[s_np[real] >= H])):
+        a, b = got[rows], exp[rows]
+        nan_a, nan_b = (a & 0x7FFF) > 0x7F80, (b & 0x7FFF) > 0x7F80
+        assert np.array_equal(nan_a, nan_b), f"{path}, {name}: NaN patterns differ"
+        ok = ~nan_a
+        dist = np.abs(_bf16_order(a) - _bf16_order(b))[ok]
+        equal = np.mean(dist == 0)
+        print(f"{path}, {name}: {rows.size} rows, bit-equal {equal:.5f}, worst distance {dist.max()} ulp")
+        assert dist.max() <= 1, f"{path}, {name}: act is {dist.max()} bf16 ulps from the oracle's"
+        assert equal >= 0.99
+
+
+def _run_layer_rows(cfg, w, A_bits, logits, **kw):
+    fe = ve.FusedExperts(w.w13, w.w13_scale, w.w2, w.w2_scale, scratch=ve.CaptureSafeScratch(), **kw)
+    A = to_dev(A_bits, torch.bfloat16)
+    ids, tw = fe.route(to_dev(logits), cfg.top_k, True)
+    out = fe.apply(A, ids, tw)
+    torch.cuda.synchronize()
+    return out
+
+
+@pytest.mark.parametrize("name,T", [("c2", 4096), ("c3", 16384)])
+def test_all_rows_agree_between_the_two_kernel_families(name, T):
+    """Full size, every token: the prepacked call (FP4-rate kernels, three FP6 terms in both
+    stages) against the raw-weight call with a workspace (FP8-rate kernels, exact two-term
+    split) on the same inputs.  Two kernel families with different tilings, layouts and
+    row maps: a localised error of either (a tile, a window edge, an expert's last rows)
+    shows as a row that disagrees, which the oracle's sample of rows may miss.  The
+    sampled rows' own distance to the oracle is measured in the tests above; here every
+    row must stay inside the same bound."""
+    cfg = synth.CONFIGS[name]
+    w = cfgs._weights(cfg)
+    A, lg = cfgs._inputs(cfg, T, 2000 if name == "c2" else 3000)
+    a = _run_layer_rows(cfg, w, A, lg, prepack=True, split_terms=3).double()
+    b = _run_layer_rows(cfg, w, A, lg).double()
+    assert bool(torch.isfinite(a).all()) and bool(torch.isfinite(b).all())
+    row_l2 = ((a - b).norm(dim=1) / b.norm(dim=1).clamp_min(1e-30)).cpu().numpy()
+    rms = float(b.pow(2).mean().sqrt())
+    worst_el = float(((a - b).abs() / b.abs().clamp_min(max(rms, 1.0))).max())
+    print(f"{name} T={T}: per-row relative L2 between the families: median {np.median(row_l2):.3e}, "
+          f"worst {row_l2.max():.3e} (row {int(row_l2.argmax())}); worst element / rms {worst_el:.3e}")
+    assert row_l2.max() <= 2e-3
+    assert worst_el <= EXACT_SPLIT_MAX_ABS_TOL
+    # the default arithmetic (three terms, then two) on every row as well
+    c = _run_layer_rows(cfg, w, A, lg, prepack=True).double()
+    row_l2 = ((c - b).norm(dim=1) / b.norm(dim=1).clamp_min(1e-30)).cpu().numpy()
+    print(f"{name} T={T}: default terms against the raw-weight call: median {np.median(row_l2):.3e}, "
+          f"worst {row_l2.max():.3e}")
+    assert row_l2.max() <= 2e-3
+
+
 # ---- the layer -------------------------------------------------------------------------
 
 # The default arithmetic of the prepacked path (three FP6 terms in the first stage, two in

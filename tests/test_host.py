@@ -268,9 +268,9 @@ def test_entry_points_reject_contract_violations_without_a_device(lib):
         16, None)                                                             # hidden not /64
     assert lib.vk_last_error_code() != 0 and b"vk_hip_fused_moe_mxfp4" in lib.vk_last_error()
     lib.vk_set_last_error(0, b"")
-    odd = P(ctypes.addressof(buf) + 4)
+    odd = P(ctypes.addressof(buf) + 2)
     moe(p, p, p, p, p, p, p, p, p, 4, 128, 128, 2, p, p, 64, F(0), 0, F(4), F(25), odd, None,
-        16, None)                                                             # bias not 16-byte aligned
+        16, None)                                                             # bias not aligned like a float
     assert lib.vk_last_error_code() != 0 and b"aligned" in lib.vk_last_error()
     lib.vk_set_last_error(0, b"")
     moe(p, p, p, p, p, p, p, p, p, 0, 128, 128, 2, p, p, 64, F(0), 0, F(4), F(25), None, None,
@@ -350,6 +350,16 @@ def test_tuning_store_round_trip(tmp_path):
         assert ve.moe_tile_query(*key) == (other, True)                    # a record set by hand survives a load
         assert ve.moe_tuning_load(str(tmp_path / "nowhere")) == 0          # no file: the file's records go
         assert ve.moe_tile_query(1, 1536, 4096, 17)[1] is False
+        # a body without the format's first line, or swept on another architecture, is no
+        # store of this library's: its records are not taken (and the last load's go)
+        good = (tmp_path / "moe_fused.gfx950.tune").read_text()
+        assert ve.moe_tuning_load(str(tmp_path)) == 2
+        (tmp_path / "moe_fused.gfx950.tune").write_text(good.split("\n", 1)[1])
+        assert ve.moe_tuning_load(str(tmp_path)) == 0 and ve.moe_tile_query(1, 1536, 4096, 17)[1] is False
+        (tmp_path / "moe_fused.gfx950.tune").write_text(good.replace("arch=gfx950", "arch=gfx942"))
+        assert ve.moe_tuning_load(str(tmp_path)) == 0 and ve.moe_tile_query(1, 1536, 4096, 17)[1] is False
+        (tmp_path / "moe_fused.gfx950.tune").write_text(good.replace("# arch=gfx950", "# swept"))
+        assert ve.moe_tuning_load(str(tmp_path)) == 2                      # no arch named: the file name's
     finally:
         ve.moe_tile_set(*key, None)
         ve.moe_tuning_load(str(tmp_path / "nowhere"))

@@ -70,8 +70,8 @@ bool layer_args_ok(const char* who, bool need13, bool need2, const vk::FusedMoeA
     why = "top_k must be positive";
   else if (a.block_size <= 0 || a.block_size % 16 != 0 || a.EM % a.block_size != 0)
     why = "block_size must be a multiple of 16 and divide EM";
-  else if (((reinterpret_cast<uintptr_t>(a.b13) | reinterpret_cast<uintptr_t>(a.b2)) & 15u) != 0)
-    why = "b13 and b2 must be 16-byte aligned (the kernels load four columns at a time)";
+  else if (((reinterpret_cast<uintptr_t>(a.b13) | reinterpret_cast<uintptr_t>(a.b2)) & 3u) != 0)
+    why = "b13 and b2 must be aligned like the floats they hold";
   if (why == nullptr) return true;
   vk_set_last_error(VK_ERROR_INVALID_ARGUMENT, (std::string(who) + ": " + why).c_str());
   return false;
@@ -117,14 +117,17 @@ void vk_hip_fused_moe_mxfp4_ws(
 
 namespace {
 
-// After the launches of a void entry point: a launch the runtime refused is
-// recorded for vk_last_error() (peeked, so hipGetLastError() still reports it
-// to the caller as the conventions promise).
-void note_launch_error(const char* who) {
+// After the launches of an entry point: a launch the runtime refused is recorded for
+// vk_last_error() (peeked, so hipGetLastError() still reports it to the caller as the
+// conventions promise).  `before` is the runtime's error state peeked ahead of the
+// launches: an error that an earlier, unrelated call left there stays that call's and is
+// not reported as this one's.  True when this call's launches failed.
+bool note_launch_error(const char* who, hipError_t before) {
   const hipError_t err = hipPeekAtLastError();
-  if (err != hipSuccess)
-    vk_set_last_error(VK_ERROR_INTERNAL,
-                      (std::string(who) + ": launch failed: " + hipGetErrorString(err)).c_str());
+  if (err == hipSuccess || before != hipSuccess) return false;
+  vk_set_last_error(VK_ERROR_INTERNAL,
+                    (std::string(who) + ": launch failed: " + hipGetErrorString(err)).c_str());
+  return true;
 }
 
 vk::FusedMoeArgs fused_args(
@@ -165,8 +168,9 @@ void vk_hip_fused_moe_mxfp4_ex(
                  top_k, sorted_ids, expert_ids, EM, swiglu_limit, activation, beta, linear_beta,
                  b13, b2, block_size, workspace, workspace_bytes, flags);
   if (!layer_args_ok("vk_hip_fused_moe_mxfp4", true, true, a)) return;
+  const hipError_t before = hipPeekAtLastError();
   vk::launch_fused_moe(a, static_cast<hipStream_t>(stream));
-  note_launch_error("vk_hip_fused_moe_mxfp4");
+  note_launch_error("vk_hip_fused_moe_mxfp4", before);
 }
 
 void vk_hip_fused_moe_mxfp4_prepacked(
@@ -197,8 +201,9 @@ void vk_hip_fused_moe_mxfp4_prepacked(
   a.w13_packed = static_cast<const uint8_t*>(w13_packed);
   a.w2_packed = static_cast<const uint8_t*>(w2_packed);
   a.num_experts = num_experts;
+  const hipError_t before = hipPeekAtLastError();
   vk::launch_fused_moe(a, static_cast<hipStream_t>(stream));
-  note_launch_error("vk_hip_fused_moe_mxfp4_prepacked");
+  note_launch_error("vk_hip_fused_moe_mxfp4_prepacked", before);
 }
 
 void vk_hip_moe_down_mxfp4_ex(
@@ -223,8 +228,9 @@ void vk_hip_moe_down_mxfp4_ex(
                       "vk_hip_moe_down_mxfp4_ex: num_experts must be positive with packed weights");
     return;
   }
+  const hipError_t before = hipPeekAtLastError();
   vk::launch_moe_down(a, static_cast<hipStream_t>(stream));
-  note_launch_error("vk_hip_moe_down_mxfp4_ex");
+  note_launch_error("vk_hip_moe_down_mxfp4_ex", before);
 }
 
 int vk_hip_split_rows_fp6(const uint16_t* x, int32_t rows, int32_t K, int32_t terms, void* split,
@@ -278,6 +284,8 @@ int vk_hip_mxfp4_moe_scatter_reduce(const float* partial, const float* topk_w,
   if (M == 0 || width == 0 || EM == 0) return VK_OK;
   if (partial == nullptr || topk_w == nullptr || sorted_ids == nullptr || out == nullptr)
     return fail(VK_ERROR_INVALID_ARGUMENT, "partial/topk_w/sorted_ids/out must not be null");
+  if (((reinterpret_cast<uintptr_t>(partial) | reinterpret_cast<uintptr_t>(out)) & 3u) != 0)
+    return fail(VK_ERROR_INVALID_ARGUMENT, "partial and out must be aligned like floats");
   if (workspace == nullptr || workspace_bytes < sizeof(int32_t) * (size_t)M * (size_t)top_k ||
       (reinterpret_cast<uintptr_t>(workspace) & 3) != 0)
     return fail(VK_ERROR_INVALID_ARGUMENT, "workspace must hold M * top_k int32 values");
@@ -302,9 +310,8 @@ const char* stage_shape_error(int M, int width_a, int ncols, int top_k, int EM, 
   return nullptr;
 }
 
-int stage_launch_status(const char* who) {
-  note_launch_error(who);
-  return vk_last_error_code() == VK_OK ? VK_OK : VK_ERROR_INTERNAL;
+int stage_launch_status(const char* who, hipError_t before) {
+  return note_launch_error(who, before) ? VK_ERROR_INTERNAL : VK_OK;
 }
 
 }  // namespace
@@ -320,9 +327,10 @@ int vk_hip_moe_gateup_preact(const uint16_t* A, const uint8_t* w13, const uint8_
       expert_ids == nullptr || gate_up == nullptr)
     return fail(VK_ERROR_INVALID_ARGUMENT, "vk_hip_moe_gateup_preact: buffers must not be null");
   vk_set_last_error(VK_OK, "");
+  const hipError_t before = hipPeekAtLastError();
   vk::launch_moe_preact(0, A, w13, w13_scale, sorted_ids, expert_ids, gate_up, M, hidden, ispp, top_k, EM,
                         k_base, hidden_k, block_size, static_cast<hipStream_t>(stream));
-  return stage_launch_status("vk_hip_moe_gateup_preact");
+  return stage_launch_status("vk_hip_moe_gateup_preact", before);
 }
 
 int vk_hip_moe_act_epilogue(const float* gate_up, const float* b13, uint16_t* act,
@@ -340,10 +348,11 @@ int vk_hip_moe_act_epilogue(const float* gate_up, const float* b13, uint16_t* ac
   if (gate_up == nullptr || act == nullptr || sorted_ids == nullptr || expert_ids == nullptr)
     return fail(VK_ERROR_INVALID_ARGUMENT, "vk_hip_moe_act_epilogue: buffers must not be null");
   vk_set_last_error(VK_OK, "");
+  const hipError_t before = hipPeekAtLastError();
   vk::launch_moe_act_epilogue(gate_up, b13, act, sorted_ids, expert_ids, M, top_k, EM, ispp, block_size,
                               swiglu_limit, activation, beta, linear_beta,
                               static_cast<hipStream_t>(stream));
-  return stage_launch_status("vk_hip_moe_act_epilogue");
+  return stage_launch_status("vk_hip_moe_act_epilogue", before);
 }
 
 int vk_hip_moe_down_preact(const uint16_t* act, const uint8_t* w2, const uint8_t* w2_scale,
@@ -357,9 +366,10 @@ int vk_hip_moe_down_preact(const uint16_t* act, const uint8_t* w2, const uint8_t
       expert_ids == nullptr || partial == nullptr)
     return fail(VK_ERROR_INVALID_ARGUMENT, "vk_hip_moe_down_preact: buffers must not be null");
   vk_set_last_error(VK_OK, "");
+  const hipError_t before = hipPeekAtLastError();
   vk::launch_moe_preact(1, act, w2, w2_scale, sorted_ids, expert_ids, partial, M, ispp, hidden, top_k, EM,
                         k_base, ispp_k, block_size, static_cast<hipStream_t>(stream));
-  return stage_launch_status("vk_hip_moe_down_preact");
+  return stage_launch_status("vk_hip_moe_down_preact", before);
 }
 
 int vk_hip_moe_combine(const float* partial, const float* b2, const float* topk_w_sorted,
@@ -376,16 +386,17 @@ int vk_hip_moe_combine(const float* partial, const float* b2, const float* topk_
       out == nullptr)
     return fail(VK_ERROR_INVALID_ARGUMENT, "vk_hip_moe_combine: buffers must not be null");
   if (((reinterpret_cast<uintptr_t>(partial) | reinterpret_cast<uintptr_t>(b2) |
-        reinterpret_cast<uintptr_t>(out)) & 15u) != 0)
-    return fail(VK_ERROR_INVALID_ARGUMENT, "vk_hip_moe_combine: partial, b2 and out must be 16-byte aligned");
+        reinterpret_cast<uintptr_t>(out)) & 3u) != 0)
+    return fail(VK_ERROR_INVALID_ARGUMENT, "vk_hip_moe_combine: partial, b2 and out must be aligned like floats");
   if (workspace == nullptr || workspace_bytes < sizeof(int32_t) * (size_t)M * (size_t)top_k ||
       (reinterpret_cast<uintptr_t>(workspace) & 3) != 0)
     return fail(VK_ERROR_INVALID_ARGUMENT, "vk_hip_moe_combine: workspace must hold M * top_k int32 values");
   vk_set_last_error(VK_OK, "");
+  const hipError_t before = hipPeekAtLastError();
   vk::launch_moe_combine_sorted(partial, b2, topk_w_sorted, sorted_ids, expert_ids, out, M, hidden, top_k,
                                 EM, block_size, static_cast<int32_t*>(workspace),
                                 static_cast<hipStream_t>(stream));
-  return stage_launch_status("vk_hip_moe_combine");
+  return stage_launch_status("vk_hip_moe_combine", before);
 }
 
 size_t vk_hip_moe_prepack_bytes(int32_t num_experts, int32_t rows, int32_t K, int32_t stage) {
@@ -512,13 +523,9 @@ int vk_hip_fused_moe_mxfp4_static(
                 (std::string("vk_hip_fused_moe_mxfp4_static: the library's scratch array has no "
                              "device address: ") + hipGetErrorString(err)).c_str());
   a.workspace_bytes = vk::static_scratch_bytes();
+  const hipError_t before = hipPeekAtLastError();
   vk::launch_fused_moe(a, static_cast<hipStream_t>(stream));
-  const hipError_t launched = hipPeekAtLastError();
-  if (launched != hipSuccess)
-    return fail(VK_ERROR_INTERNAL,
-                (std::string("vk_hip_fused_moe_mxfp4_static: launch failed: ") +
-                 hipGetErrorString(launched)).c_str());
-  return VK_OK;
+  return note_launch_error("vk_hip_fused_moe_mxfp4_static", before) ? VK_ERROR_INTERNAL : VK_OK;
 }
 
 void vk_hip_moe_gateup_mxfp4(
@@ -535,8 +542,9 @@ void vk_hip_moe_gateup_mxfp4(
   a.block_size = block_size; a.swiglu_limit = swiglu_limit; a.beta = beta;
   a.linear_beta = linear_beta; a.activation = activation;
   if (!layer_args_ok("vk_hip_moe_gateup_mxfp4", true, false, a)) return;
+  const hipError_t before = hipPeekAtLastError();
   vk::launch_moe_gateup(a, static_cast<hipStream_t>(stream));
-  note_launch_error("vk_hip_moe_gateup_mxfp4");
+  note_launch_error("vk_hip_moe_gateup_mxfp4", before);
 }
 
 void vk_hip_moe_down_mxfp4(
@@ -552,8 +560,9 @@ void vk_hip_moe_down_mxfp4(
   a.M = M; a.hidden = hidden; a.ispp = ispp; a.top_k = top_k; a.EM = EM;
   a.block_size = block_size;
   if (!layer_args_ok("vk_hip_moe_down_mxfp4", false, true, a)) return;
+  const hipError_t before = hipPeekAtLastError();
   vk::launch_moe_down(a, static_cast<hipStream_t>(stream));
-  note_launch_error("vk_hip_moe_down_mxfp4");
+  note_launch_error("vk_hip_moe_down_mxfp4", before);
 }
 
 int vk_hip_moe_align_block_size(

@@ -149,8 +149,8 @@ __device__ __forceinline__ void epilogue_tile(const GemmArgs& p, int e, const f3
       f32x4 gate = acc[t], up = acc[t + NT / 2];
       if (p.bias != nullptr) {  // uniform; the lane's four columns in one load each
         const float* b = p.bias + (size_t)e * (size_t)(2 * p.ncols) + c;
-        gate += *reinterpret_cast<const f32x4*>(b);
-        up += *reinterpret_cast<const f32x4*>(b + p.ncols);
+        gate += *reinterpret_cast<const f32x4u*>(b);
+        up += *reinterpret_cast<const f32x4u*>(b + p.ncols);
       }
       uint32_t packed[2];
 #pragma unroll
@@ -174,7 +174,7 @@ __device__ __forceinline__ void epilogue_tile(const GemmArgs& p, int e, const f3
       const int c = col0[t] + 4 * lq;
       f32x4 v = acc[t];
       if (p.bias != nullptr)  // uniform
-        v += *reinterpret_cast<const f32x4*>(p.bias + (size_t)e * (size_t)p.ncols + c);
+        v += *reinterpret_cast<const f32x4u*>(p.bias + (size_t)e * (size_t)p.ncols + c);
 #pragma unroll
       for (int r = 0; r < 4; ++r) unsafeAtomicAdd(orow + c + r, v[r] * w);
     }
@@ -1603,7 +1603,7 @@ __global__ __launch_bounds__(64 * kWideWaves) void tile_wide_kernel(GemmArgs p) 
             const int c = col0[t] + 4 * lq;
             f32x4 v = acc[m][t];
             if (p.bias != nullptr)
-              v += *reinterpret_cast<const f32x4*>(p.bias + (size_t)e * (size_t)p.ncols + c);
+              v += *reinterpret_cast<const f32x4u*>(p.bias + (size_t)e * (size_t)p.ncols + c);
             *reinterpret_cast<f32x4*>(yrow + c) = v * w;
           }
         }

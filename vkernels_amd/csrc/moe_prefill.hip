@@ -815,7 +815,7 @@ __global__ __launch_bounds__(64 * kMxWaves) void tile_mx_kernel(MxArgs p) {
         const int c = STAGE == 0 ? (t >> 1) * p.ncols + (t & 1) * 32
                                  : (unit * kMxUnitRows + (t >> 1) * 64 < p.ncols ? t * 32 : 0);
 #pragma unroll
-        for (int rg = 0; rg < 4; ++rg) bias_v[t][rg] = *reinterpret_cast<const f32x4*>(b + c + rg * 8);
+        for (int rg = 0; rg < 4; ++rg) bias_v[t][rg] = *reinterpret_cast<const f32x4u*>(b + c + rg * 8);
       }
     } else if (STAGE == 0 && p.activation == 1) {  // the one loop that adds them without a bias
 #pragma unroll

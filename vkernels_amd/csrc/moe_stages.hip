@@ -34,8 +34,8 @@ __global__ __launch_bounds__(256) void act_epilogue_kernel(
     f32x4 u = *reinterpret_cast<const f32x4*>(row + ispp + c);
     if (b13 != nullptr) {
       const float* b = b13 + (size_t)e * (size_t)(2 * ispp);
-      g += *reinterpret_cast<const f32x4*>(b + c);
-      u += *reinterpret_cast<const f32x4*>(b + ispp + c);
+      g += *reinterpret_cast<const f32x4u*>(b + c);
+      u += *reinterpret_cast<const f32x4u*>(b + ispp + c);
     }
     uint32_t v[4];
 #pragma unroll
@@ -70,7 +70,7 @@ __global__ __launch_bounds__(256) void combine_rows_kernel(
   const int c = (blockIdx.x * blockDim.x + threadIdx.x) * 4;
   if (c >= width) return;
   for (int t = blockIdx.y; t < M; t += gridDim.y) {
-    f32x4* o = reinterpret_cast<f32x4*>(out + (size_t)t * (size_t)width + c);
+    f32x4u* o = reinterpret_cast<f32x4u*>(out + (size_t)t * (size_t)width + c);
     f32x4 sum = *o;
     int last = -1;
     for (int s = 0; s < top_k; ++s) {   // the next larger sorted row of this token (top_k is small)
@@ -84,8 +84,8 @@ __global__ __launch_bounds__(256) void combine_rows_kernel(
       int e = 0;
       if (expert_ids != nullptr) e = expert_ids[r / block_size];
       if (e < 0) continue;
-      f32x4 p = *reinterpret_cast<const f32x4*>(partial + (size_t)r * (size_t)width + c);
-      if (bias != nullptr) p += *reinterpret_cast<const f32x4*>(bias + (size_t)e * (size_t)width + c);
+      f32x4 p = *reinterpret_cast<const f32x4u*>(partial + (size_t)r * (size_t)width + c);
+      if (bias != nullptr) p += *reinterpret_cast<const f32x4u*>(bias + (size_t)e * (size_t)width + c);
       const float w = w_sorted[r];
 #pragma unroll
       for (int i = 0; i < 4; ++i) {

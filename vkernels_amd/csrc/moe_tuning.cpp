@@ -23,6 +23,7 @@ struct Record {
 std::mutex g_lock;
 std::map<Key, Record> g_table;
 std::atomic<int> g_records{0};  // launches skip the lock while the table is empty
+std::atomic<unsigned> g_version{0};  // bumped by every change of the table (under the lock)
 std::once_flag g_default_loaded;
 
 Key make_key(int stage, int K, int ncols, int n_flat) {
@@ -90,6 +91,7 @@ int parse_locked(const std::string& text) {
     }
   }
   commit(open, key, val, seen, &taken);
+  g_version.fetch_add(1u, std::memory_order_relaxed);
   g_records.store((int)g_table.size(), std::memory_order_release);
   return taken;
 }
@@ -116,6 +118,29 @@ int moe_tuning_parse(const std::string& text) {
   return parse_locked(text);
 }
 
+// True for a body this library may take records from: it starts with the format's header
+// line, as the reference requires of a store file (src/c/vkernels/core/tuning.cpp:195), and
+// the architecture it names in its `# arch=` comment, if it names one, is the one this
+// library is compiled for (the reference keys its stores by that token,
+// core/tuning.cpp:137-150; records swept on another device say nothing about this one).
+bool moe_tuning_body_ok(const std::string& body) {
+  static const char kHeader[] = "# vk-native-tuning/2";
+  if (body.rfind(kHeader, 0) != 0) return false;
+  std::istringstream in(body);
+  std::string line;
+  while (std::getline(in, line)) {
+    const size_t first = line.find_first_not_of(" \t\r");
+    if (first == std::string::npos) continue;
+    if (line[first] != '#') break;  // the header comments are over
+    const size_t at = line.find("arch=", first);
+    if (at == std::string::npos) continue;
+    std::string arch = line.substr(at + 5);
+    arch = arch.substr(0, arch.find_first_of(" \t\r"));
+    return arch == kMoeTuningArch;
+  }
+  return true;
+}
+
 int moe_tuning_load(const char* dir) {
   const std::string root = dir != nullptr ? std::string(dir) : moe_tuning_dir();
   std::string body;
@@ -127,16 +152,38 @@ int moe_tuning_load(const char* dir) {
       body = all.str();
     }
   }
+  // a file of another format or another device is as good as no file
+  if (!moe_tuning_body_ok(body)) body.clear();
   return moe_tuning_parse(body);
 }
 
 bool moe_tuning_find(int stage, int K, int ncols, int n_flat, MoeTile* tile) {
   std::call_once(g_default_loaded, [] { (void)moe_tuning_load(nullptr); });
   if (g_records.load(std::memory_order_acquire) == 0) return false;
-  std::lock_guard<std::mutex> hold(g_lock);
-  const auto it = g_table.find(make_key(stage, K, ncols, n_flat));
-  if (it == g_table.end()) return false;
-  *tile = it->second.tile;
+  // A serving loop asks for the same few problems call after call: each thread keeps
+  // its last answer per stage and takes the lock only when the problem or the table
+  // has changed since.
+  struct Last {
+    unsigned version;
+    Key key;
+    bool valid, found;
+    MoeTile tile;
+  };
+  thread_local Last last[2] = {};
+  const Key key = make_key(stage, K, ncols, n_flat);
+  Last& l = last[stage & 1];
+  const unsigned version = g_version.load(std::memory_order_acquire);
+  if (!(l.valid && l.version == version && l.key == key)) {
+    std::lock_guard<std::mutex> hold(g_lock);
+    const auto it = g_table.find(key);
+    l.version = g_version.load(std::memory_order_relaxed);
+    l.key = key;
+    l.valid = true;
+    l.found = it != g_table.end();
+    if (l.found) l.tile = it->second.tile;
+  }
+  if (!l.found) return false;
+  *tile = l.tile;
   return true;
 }
 
@@ -148,6 +195,7 @@ bool moe_tuning_set(int stage, int K, int ncols, int n_flat, const MoeTile* tile
   const Key k = make_key(stage, K, ncols, n_flat);
   if (tile != nullptr) g_table[k] = Record{*tile, false};
   else g_table.erase(k);
+  g_version.fetch_add(1u, std::memory_order_relaxed);
   g_records.store((int)g_table.size(), std::memory_order_release);
   return true;
 }
@@ -155,7 +203,7 @@ bool moe_tuning_set(int stage, int K, int ncols, int n_flat, const MoeTile* tile
 std::string moe_tuning_dump(const char* written_by) {
   std::lock_guard<std::mutex> hold(g_lock);
   std::ostringstream out;
-  out << "# vk-native-tuning/2\n# arch=gfx950 written_by=" << (written_by != nullptr ? written_by : "unknown") << "\n";
+  out << "# vk-native-tuning/2\n# arch=" << kMoeTuningArch << " written_by=" << (written_by != nullptr ? written_by : "unknown") << "\n";
   for (const auto& kv : g_table) {
     const Key& k = kv.first;
     const MoeTile& t = kv.second.tile;

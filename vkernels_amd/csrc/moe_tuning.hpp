@@ -18,6 +18,7 @@
 namespace vk {
 
 constexpr const char* kMoeTuningFile = "moe_fused.gfx950.tune";
+constexpr const char* kMoeTuningArch = "gfx950";  // the one architecture this library is compiled for
 
 // Bucket of the routed rows a record is kept under: the power of two at or above
 // n_flat up to the decode limit, one bucket beyond it.
@@ -28,7 +29,9 @@ std::string moe_tuning_dir();
 
 // Reads `dir`/moe_fused.gfx950.tune (null: the store directory) into the process's
 // table, replacing what a file put there before; records set by moe_tuning_set stay.
-// Returns the number of records taken, 0 when there is no file.
+// Returns the number of records taken, 0 when there is no file.  A file whose first line
+// is not `# vk-native-tuning/2`, or whose `# arch=` comment names another architecture,
+// counts as no file.
 int moe_tuning_load(const char* dir);
 
 // Parses a .tune body into the table (what moe_tuning_load does with the file).

@@ -26,6 +26,9 @@ namespace vk {
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
 typedef __attribute__((ext_vector_type(4))) float f32x4;
+// The same four floats at an address that is only 4-byte aligned (a caller's bias row, a
+// view into a larger buffer): global memory takes multi-dword accesses at dword alignment.
+typedef float f32x4u __attribute__((ext_vector_type(4), aligned(4)));
 typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
 
 // One code with one scale byte -> bf16 bits, every case of the reference's

@@ -4,6 +4,9 @@
     python -m vkernels_amd.traffic_record --workload c1:64 --kernel "stream_resident_kernel<0" \
         --fetch <FETCH_SIZE counter_collection.csv> --write <WRITE_SIZE counter_collection.csv>
 
+--kernel may be repeated for a record that covers a whole call (the prefill record: the
+split, the two GEMM kernels and the combine): the kernels' means are then summed.
+
 Both counters are in KiB per dispatch.  Each is scaled by what it reads for the
 calibration copy (a kernel that reads and writes a known number of bytes): on this
 device FETCH_SIZE counts half of what a copy reads.  The record names the digest of the
@@ -46,7 +49,9 @@ def copy_scale(path: str, counter: str) -> tuple[float, float]:
 def main() -> None:
     ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
     ap.add_argument("--workload", required=True)
-    ap.add_argument("--kernel", required=True, help="substring of the dominant kernel's name")
+    ap.add_argument("--kernel", required=True, action="append",
+                    help="substring of the dominant kernel's name; given several times, the kernels of "
+                         "one call (each launched once per call): their per-dispatch means are summed")
     ap.add_argument("--fetch", required=True)
     ap.add_argument("--write", required=True)
     ap.add_argument("--out", default=str(ROOT / "profiles" / "traffic.json"))
@@ -56,21 +61,25 @@ def main() -> None:
 
     f_scale, f_copy = copy_scale(args.fetch, "FETCH_SIZE")
     w_scale, w_copy = copy_scale(args.write, "WRITE_SIZE")
-    fetch = counter_values(args.fetch, "FETCH_SIZE", args.kernel)
-    write = counter_values(args.write, "WRITE_SIZE", args.kernel)
-    if not fetch or not write:
-        raise SystemExit(f"no dispatch of a kernel named *{args.kernel}* in the counter files")
-    read_bytes = statistics.mean(fetch) * 1024.0 * f_scale
-    write_bytes = statistics.mean(write) * 1024.0 * w_scale
+    fetch_kib = write_kib = 0.0
+    for name in args.kernel:
+        fetch = counter_values(args.fetch, "FETCH_SIZE", name)
+        write = counter_values(args.write, "WRITE_SIZE", name)
+        if not fetch or not write:
+            raise SystemExit(f"no dispatch of a kernel named *{name}* in the counter files")
+        fetch_kib += statistics.mean(fetch)
+        write_kib += statistics.mean(write)
+    read_bytes = fetch_kib * 1024.0 * f_scale
+    write_bytes = write_kib * 1024.0 * w_scale
     out = Path(args.out)
     table = json.loads(out.read_text()) if out.is_file() else {}
     table[args.workload] = {
-        "kernel": args.kernel,
+        "kernel": args.kernel[0] if len(args.kernel) == 1 else args.kernel,
         "traffic_bytes": round(read_bytes + write_bytes),
         "read_bytes": round(read_bytes),
         "write_bytes": round(write_bytes),
-        "fetch_size_kib_raw": round(statistics.mean(fetch), 1),
-        "write_size_kib_raw": round(statistics.mean(write), 1),
+        "fetch_size_kib_raw": round(fetch_kib, 1),
+        "write_size_kib_raw": round(write_kib, 1),
         "fetch_scale": round(f_scale, 4),
         "write_scale": round(w_scale, 4),
         "copy_fetch_kib_raw": round(f_copy, 1),
