@@ -31,7 +31,10 @@
 extern "C" {
 #endif
 
-/* Status codes.  Replaces src/c/vkernels/capi/capi.hpp:41-47. */
+/* Status codes.  Replaces src/c/vkernels/capi/capi.hpp:41-47.  (vkernels_cpu.h declares
+ * the same codes under the same guard.) */
+#ifndef VKERNELS_STATUS_CODES_
+#define VKERNELS_STATUS_CODES_
 enum {
   VK_OK = 0,
   VK_ERROR_INVALID_ARGUMENT = 1,
@@ -39,6 +42,7 @@ enum {
   VK_ERROR_UNSUPPORTED = 3,
   VK_ERROR_INTERNAL = 4
 };
+#endif
 
 /* Activation tags.  Replaces MoEActivation,
  * src/c/vkernels/kernels/moe_fused.hpp:47-50. */
@@ -384,8 +388,28 @@ int vk_hip_split_rows_fp6(const uint16_t* x, int32_t rows, int32_t K, int32_t te
  *   vk_hip_mxfp4_moe_scatter_reduce out[token, :] += partial[r, :] * topk_w[r] for
  *                                  every routed sorted row r, in ascending r (gather
  *                                  form: no atomics; workspace: M*top_k int32)
+ *   vk_hip_mxfp4_moe_sort          A_sorted[r, :] = A[sorted_ids[r] / top_k, :], bf16 rows
+ *                                  of `hidden` values, a padding row zeroed
+ *                                  (moe_aux.hpp:75, moe_aux.cpp:209-234)
+ *   vk_hip_mxfp4_moe_sort_scales   the same for rows of n_groups ue8m0 bytes
+ *                                  (moe_aux.hpp:90, moe_aux.cpp:236-260)
+ *   vk_hip_mxfp4_moe_scatter_reduce_q  the routed combine of a quantised partial:
+ *                                  partial_q [EM, width/2] E2M1 codes, partial_s
+ *                                  [EM, width/32] ue8m0 (0xFF = zero), dequantised
+ *                                  inline; the same order and roundings as the
+ *                                  reference (moe_aux.hpp:174, moe_aux.cpp:288-321);
+ *                                  out accumulates; workspace: M*top_k int32
  * group_size must be 32.  Return VK_OK or a VK_ERROR_* code.
  */
+int vk_hip_mxfp4_moe_sort(const uint16_t* A, const int32_t* sorted_ids, uint16_t* A_sorted, int32_t M,
+                          int32_t hidden, int32_t top_k, int32_t EM, void* stream);
+int vk_hip_mxfp4_moe_sort_scales(const uint8_t* scales, const int32_t* sorted_ids, uint8_t* scales_sorted,
+                                 int32_t M, int32_t n_groups, int32_t top_k, int32_t EM, void* stream);
+int vk_hip_mxfp4_moe_scatter_reduce_q(const uint8_t* partial_q, const uint8_t* partial_s,
+                                      const float* topk_w, const int32_t* sorted_ids, float* out,
+                                      int32_t M, int32_t width, int32_t top_k, int32_t EM,
+                                      int32_t group_size, void* workspace, size_t workspace_bytes,
+                                      void* stream);
 int vk_hip_mxfp4_moe_quant(const uint16_t* A, uint8_t* packed, uint8_t* scales, int32_t M,
                            int32_t hidden, int32_t group_size, void* stream);
 int vk_hip_mxfp4_moe_sorted_quant(const uint16_t* A, const int32_t* sorted_ids, uint8_t* packed,

@@ -101,6 +101,80 @@ def test_sorted_quant_and_scatter_reduce_bitwise(hip_lib):
     assert sr(None, None, None, None, M, width, top_k, em, None, 0, None) == ve.VK_ERROR_INVALID_ARGUMENT
 
 
+@pytest.mark.parametrize("hidden", [512, 2880, 76])
+def test_sort_and_sort_scales_bitwise(hip_lib, hidden):
+    """mxfp4_moe_sort / mxfp4_moe_sort_scales on the device: rows gathered into sorted
+    order, padding rows (ids at or beyond M * top_k, negative ids) zeroed; byte for byte
+    the oracle's.  hidden = 76: rows that are no multiple of 16 bytes (the byte-wise
+    kernel), scale rows of 2 bytes."""
+    st = hip_lib.vk_hip_mxfp4_moe_sort
+    st.restype = _I
+    st.argtypes = [_P, _P, _P, _I, _I, _I, _I, _P]
+    ss = hip_lib.vk_hip_mxfp4_moe_sort_scales
+    ss.restype = _I
+    ss.argtypes = [_P, _P, _P, _I, _I, _I, _I, _P]
+    rng = np.random.default_rng(hidden)
+    M, top_k, E = 70, 4, 16
+    A = rng.integers(0, 65536, (M, hidden)).astype(np.uint16)
+    n_groups = max(hidden // 32, 1)
+    scales = rng.integers(0, 256, (M, n_groups)).astype(np.uint8)
+    ids = rng.integers(0, E, (M, top_k)).astype(np.int32)
+    sids, _, em = oracle.moe_align_block_size(ids, 16, E)
+    sids = sids[:em].copy()
+    sids[3] = -1
+    d_A, d_s, d_sids = to_dev(A), to_dev(scales), to_dev(sids)
+    a_sorted = torch.full((em, hidden), 0x1234, dtype=torch.int16, device=dev())
+    s_sorted = torch.full((em, n_groups), 9, dtype=torch.uint8, device=dev())
+    assert st(d_A.data_ptr(), d_sids.data_ptr(), a_sorted.data_ptr(), M, hidden, top_k, em, None) == 0
+    assert ss(d_s.data_ptr(), d_sids.data_ptr(), s_sorted.data_ptr(), M, n_groups, top_k, em, None) == 0
+    torch.cuda.synchronize()
+    assert np.array_equal(a_sorted.cpu().numpy().view(np.uint16), oracle.mxfp4_moe_sort(A, sids, top_k))
+    assert np.array_equal(s_sorted.cpu().numpy(), oracle.mxfp4_moe_sort_scales(scales, sids, top_k))
+    assert st(None, None, None, M, hidden, 0, em, None) == ve.VK_ERROR_INVALID_ARGUMENT
+    assert ss(None, None, None, M, n_groups, top_k, em, None) == ve.VK_ERROR_INVALID_ARGUMENT
+    assert st(None, None, None, M, hidden, top_k, 0, None) == 0              # nothing to do
+
+
+def test_scatter_reduce_q_bitwise(hip_lib):
+    """mxfp4_moe_scatter_reduce_q on the device: the routed combine of a quantised partial,
+    dequantised inline; the same bits as the oracle (each product and each sum rounded on
+    its own, rows in ascending order), with every code (inf and NaN included), scale bytes
+    0, 1, 254 and 0xFF, and an `out` that already holds values."""
+    fn = hip_lib.vk_hip_mxfp4_moe_scatter_reduce_q
+    fn.restype = _I
+    fn.argtypes = [_P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _P, ctypes.c_size_t, _P]
+    rng = np.random.default_rng(77)
+    M, width, top_k, E = 70, 2880, 4, 16
+    ids = rng.integers(0, E, (M, top_k)).astype(np.int32)
+    sids, _, em = oracle.moe_align_block_size(ids, 16, E)
+    sids = sids[:em].copy()
+    sids[7] = -2
+    pq = rng.integers(0, 256, (em, width // 2)).astype(np.uint8)
+    fin = np.array(synth.FINITE_CODES, dtype=np.uint8)
+    finite_rows = np.arange(em) % 4 != 0                               # three rows in four: finite codes only
+    pq[finite_rows] = fin[pq[finite_rows] % 12 & 15] | (fin[(pq[finite_rows] >> 4) % 12] << 4)
+    ps = rng.integers(110, 140, (em, width // 32)).astype(np.uint8)
+    ps[:, 0] = 0
+    ps[:, 1] = 1
+    ps[:, 2] = 254
+    ps[:, 3] = 255
+    tws = rng.random(em).astype(np.float32)
+    base = rng.standard_normal((M, width)).astype(np.float32)
+    out = to_dev(base.copy())
+    ws = torch.zeros(M * top_k, dtype=torch.int32, device=dev())
+    d_pq, d_ps, d_tws, d_sids = to_dev(pq), to_dev(ps), to_dev(tws), to_dev(sids)
+    assert fn(d_pq.data_ptr(), d_ps.data_ptr(), d_tws.data_ptr(), d_sids.data_ptr(), out.data_ptr(), M, width,
+              top_k, em, 32, ws.data_ptr(), ws.numel() * 4, None) == 0, ve.last_error(hip_lib)
+    torch.cuda.synchronize()
+    ref = oracle.mxfp4_moe_scatter_reduce_q(pq, ps, tws, sids, M, top_k, out=base.copy())
+    got = out.cpu().numpy()
+    nan_g, nan_r = np.isnan(got), np.isnan(ref)
+    assert np.array_equal(nan_g, nan_r) and nan_r.any() and not nan_r.all()
+    assert np.array_equal(got.view(np.uint32)[~nan_r], ref.view(np.uint32)[~nan_r])
+    assert fn(None, None, None, None, None, M, width, top_k, em, 32, None, 0, None) == ve.VK_ERROR_INVALID_ARGUMENT
+    assert fn(None, None, None, None, None, M, width, top_k, em, 16, None, 0, None) == ve.VK_ERROR_UNSUPPORTED
+
+
 def _check_w4a4(cfg, T, w, A_bits, logits, sample=128, wn=None):
     g = cfgs._run_gpu(cfg, w, A_bits, logits, None, True, prepack=True, w4a4=True)
     ids, tw = oracle.route_topk(logits, cfg.top_k, True)

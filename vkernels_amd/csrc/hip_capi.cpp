@@ -274,6 +274,53 @@ int vk_hip_mxfp4_moe_sorted_quant(const uint16_t* A, const int32_t* sorted_ids, 
   return VK_OK;
 }
 
+int vk_hip_mxfp4_moe_sort(const uint16_t* A, const int32_t* sorted_ids, uint16_t* A_sorted, int32_t M,
+                          int32_t hidden, int32_t top_k, int32_t EM, void* stream) {
+  if (M < 0 || hidden < 0 || top_k <= 0 || EM < 0)
+    return fail(VK_ERROR_INVALID_ARGUMENT, "M, hidden, top_k, EM must be valid");
+  if (EM == 0 || hidden == 0) return VK_OK;
+  if (A == nullptr || sorted_ids == nullptr || A_sorted == nullptr)
+    return fail(VK_ERROR_INVALID_ARGUMENT, "A/sorted_ids/A_sorted must not be null");
+  vk::launch_mxfp4_gather_rows(A, sorted_ids, A_sorted, sizeof(uint16_t) * (size_t)hidden, top_k, M * top_k,
+                               EM, static_cast<hipStream_t>(stream));
+  return VK_OK;
+}
+
+int vk_hip_mxfp4_moe_sort_scales(const uint8_t* scales, const int32_t* sorted_ids, uint8_t* scales_sorted,
+                                 int32_t M, int32_t n_groups, int32_t top_k, int32_t EM, void* stream) {
+  if (M < 0 || n_groups < 0 || top_k <= 0 || EM < 0)
+    return fail(VK_ERROR_INVALID_ARGUMENT, "M, n_groups, top_k, EM must be valid");
+  if (EM == 0 || n_groups == 0) return VK_OK;
+  if (scales == nullptr || sorted_ids == nullptr || scales_sorted == nullptr)
+    return fail(VK_ERROR_INVALID_ARGUMENT, "scales/sorted_ids/scales_sorted must not be null");
+  vk::launch_mxfp4_gather_rows(scales, sorted_ids, scales_sorted, (size_t)n_groups, top_k, M * top_k, EM,
+                               static_cast<hipStream_t>(stream));
+  return VK_OK;
+}
+
+int vk_hip_mxfp4_moe_scatter_reduce_q(const uint8_t* partial_q, const uint8_t* partial_s,
+                                      const float* topk_w, const int32_t* sorted_ids, float* out,
+                                      int32_t M, int32_t width, int32_t top_k, int32_t EM,
+                                      int32_t group_size, void* workspace, size_t workspace_bytes,
+                                      void* stream) {
+  if (group_size != 32) return fail(VK_ERROR_UNSUPPORTED, "group_size must be 32");
+  if (M < 0 || width < 0 || EM < 0 || top_k <= 0 || width % 32 != 0)
+    return fail(VK_ERROR_INVALID_ARGUMENT,
+                "M, width, EM must be non-negative, top_k positive, width a multiple of group_size");
+  if (M == 0 || width == 0 || EM == 0) return VK_OK;
+  if (partial_q == nullptr || partial_s == nullptr || topk_w == nullptr || sorted_ids == nullptr ||
+      out == nullptr)
+    return fail(VK_ERROR_INVALID_ARGUMENT, "partial_q/partial_s/topk_w/sorted_ids/out must not be null");
+  if ((reinterpret_cast<uintptr_t>(partial_q) & 3u) != 0 || (reinterpret_cast<uintptr_t>(out) & 3u) != 0)
+    return fail(VK_ERROR_INVALID_ARGUMENT, "partial_q and out must be 4-byte aligned");
+  if (workspace == nullptr || workspace_bytes < sizeof(int32_t) * (size_t)M * (size_t)top_k ||
+      (reinterpret_cast<uintptr_t>(workspace) & 3) != 0)
+    return fail(VK_ERROR_INVALID_ARGUMENT, "workspace must hold M * top_k int32 values");
+  vk::launch_mxfp4_scatter_reduce_q(partial_q, partial_s, topk_w, sorted_ids, out, M, width, top_k, EM,
+                                    static_cast<int32_t*>(workspace), static_cast<hipStream_t>(stream));
+  return VK_OK;
+}
+
 int vk_hip_mxfp4_moe_scatter_reduce(const float* partial, const float* topk_w,
                                     const int32_t* sorted_ids, float* out, int32_t M, int32_t width,
                                     int32_t top_k, int32_t EM, void* workspace,

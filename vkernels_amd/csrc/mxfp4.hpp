@@ -31,6 +31,16 @@ typedef __attribute__((ext_vector_type(4))) float f32x4;
 typedef float f32x4u __attribute__((ext_vector_type(4), aligned(4)));
 typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
 
+// One code -> the fp32 bits of the reference's decode table
+// (src/c/vkernels/kernels/moe_fused.cpp:24-39): +-{0, .25, 1, 1.5, 2, 3, inf}, NaN.
+__device__ __forceinline__ uint32_t fp4nib_to_f32bits(uint32_t nib) {
+  const uint32_t sign = (nib & 8u) << 28;
+  const uint32_t e = (nib >> 1) & 3u, m = nib & 1u;
+  if (e == 0u) return m ? (sign | 0x3E800000u) : sign;
+  if (e == 3u) return m ? 0x7FC00000u : (sign | 0x7F800000u);
+  return sign | ((126u + e) << 23) | (m << 22);
+}
+
 // One code with one scale byte -> bf16 bits, every case of the reference's
 // fp32 multiply-then-round reproduced with integers.
 __device__ __forceinline__ uint32_t dequant1_exact(uint32_t nib, uint32_t s) {

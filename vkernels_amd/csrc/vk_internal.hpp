@@ -99,6 +99,14 @@ void launch_mxfp4_scatter_reduce(const float* partial, const float* topk_w, cons
                                  float* out, int M, int width, int top_k, int EM, int32_t* pos,
                                  hipStream_t stream);
 
+// Rows gathered into sorted order (mxfp4_moe_sort / _sort_scales: rows of row_bytes bytes,
+// padding rows zeroed) and the routed combine of a quantised partial (pos: M * top_k ints).
+void launch_mxfp4_gather_rows(const void* src, const int32_t* sorted_ids, void* dst, size_t row_bytes,
+                              int top_k, int n_flat, int EM, hipStream_t stream);
+void launch_mxfp4_scatter_reduce_q(const uint8_t* partial_q, const uint8_t* partial_s, const float* topk_w,
+                                   const int32_t* sorted_ids, float* out, int M, int width, int top_k,
+                                   int EM, int32_t* pos, hipStream_t stream);
+
 // Per-kernel set-up that the launchers otherwise do on their first call (the
 // dynamic-LDS limits of the GEMM kernels), for callers that want it done before
 // a graph capture.  False when the device refuses a limit.
