@@ -436,14 +436,57 @@ __global__ __launch_bounds__(64 * WAVES) void stream_resident_kernel(GemmArgs p)
   const size_t w_unit_stride = unit_stride_rows * (size_t)(K / 2);
   const size_t s_unit_stride = unit_stride_rows * (size_t)groups;
 
-  // While wavefront 0 lists the runs, the others copy the head of sorted_ids to
-  // the start of the operand planes (free until the first pass is staged): the
-  // ids of the workgroup's first rows are then an LDS read behind the barrier,
-  // not one more round trip to memory in front of the row loads.
+  // Order of the start: what memory must bring is asked for first (wavefront 0: the experts
+  // of the first 64 blocks, for the run list; the others: the head of sorted_ids, which
+  // they copy to the start of the operand planes, free until the first pass is staged, so
+  // that the ids of the workgroup's first rows are an LDS read behind the barrier), then
+  // every wavefront does the set-up that does not depend on its slice while those loads
+  // are under way, then the run list and the slice.
   int* const ids_lds = reinterpret_cast<int*>(b_lds);
   const int ids_cached = min(p.num_blocks * p.block_size, nsteps * 1024);  // 4 KB of planes per K step
+  constexpr int kIdsAhead = 2;  // loads of the copy a lane asks for before the set-up
+  int e_first = -1;             // wavefront 0: the expert of block `lane`
+  int ids_ahead[kIdsAhead];
+  if (wave == 0) {
+    e_first = p.expert_ids[min(lane, p.num_blocks - 1)];
+  } else {
+#pragma unroll
+    for (int j = 0; j < kIdsAhead; ++j)
+      ids_ahead[j] = p.sorted_ids[min(tid - 64 + j * 64 * (WAVES - 1), ids_cached - 1)];
+  }
+
+  // Scale bytes of a unit: byte offset of this lane's piece j from the unit's first tile
+  // (tile_row = the first weight row of the piece's tile, counted from the first tile's, as
+  // unit_tiles lays them out; lanes past the end re-read the last piece).
+  constexpr int kHalfTiles = NT >= 2 ? NT / 2 : 1;
+  constexpr int kScMax = resident_scale_pieces(WAVES);
+  int sc_piece[kScMax];
+#pragma unroll
+  for (int j = 0; j < kScMax; ++j) {
+    const int piece = min(lane + 64 * j, NT * groups - 1);
+    int t = 0;
+#pragma unroll
+    for (int t2 = 1; t2 < NT; ++t2)
+      if (piece >= t2 * groups) t = t2;
+    int tile_row = STAGE == 0 ? 0 : t * 16;
+    if (STAGE == 0) {
+#pragma unroll
+      for (int t2 = 1; t2 < NT; ++t2)
+        if (t == t2) tile_row = (t2 / kHalfTiles) * p.ncols + (t2 % kHalfTiles) * 16;
+    }
+    sc_piece[j] = tile_row * groups + (piece - t * groups) * 16;
+  }
+
+  static_assert(WAVES % 4 == 0, "a wavefront's pieces keep their quarter of a K step");
+
   if (WAVES > 1 && wave != 0) {
-    for (int i = tid - 64; i < ids_cached; i += 64 * (WAVES - 1)) ids_lds[i] = p.sorted_ids[i];
+#pragma unroll
+    for (int j = 0; j < kIdsAhead; ++j) {
+      const int i = tid - 64 + j * 64 * (WAVES - 1);
+      if (i < ids_cached) ids_lds[i] = ids_ahead[j];
+    }
+    for (int i = tid - 64 + kIdsAhead * 64 * (WAVES - 1); i < ids_cached; i += 64 * (WAVES - 1))
+      ids_lds[i] = p.sorted_ids[i];
   }
 
   // ---- list the runs (first and last block of every run, in order) ---------
@@ -464,7 +507,7 @@ __global__ __launch_bounds__(64 * WAVES) void stream_resident_kernel(GemmArgs p)
     for (int base = 0; base < nb; base += 64) {
       const int b = base + lane;
       const int bc = min(b, nb - 1);
-      const int e_here = p.expert_ids[bc];
+      const int e_here = base == 0 ? e_first : p.expert_ids[bc];
       int w = tpb;  // (more than 8 tiles a block: all of them)
       if (tpb > 1 && tpb <= 8) {  // uniform; loads without a branch between them: one round trip
         w = 0;
@@ -562,40 +605,6 @@ __global__ __launch_bounds__(64 * WAVES) void stream_resident_kernel(GemmArgs p)
     u32x4 w[NT];
   };
   int pass_no = 0;
-
-  // Scale bytes of a unit: byte offset of this lane's piece j from the unit's first tile
-  // (tile_row = the first weight row of the piece's tile, counted from the first tile's, as
-  // unit_tiles lays them out; lanes past the end re-read the last piece).
-  constexpr int kHalfTiles = NT >= 2 ? NT / 2 : 1;
-  constexpr int kScMax = resident_scale_pieces(WAVES);
-  int sc_piece[kScMax];
-#pragma unroll
-  for (int j = 0; j < kScMax; ++j) {
-    const int piece = min(lane + 64 * j, NT * groups - 1);
-    int t = 0;
-#pragma unroll
-    for (int t2 = 1; t2 < NT; ++t2)
-      if (piece >= t2 * groups) t = t2;
-    int tile_row = STAGE == 0 ? 0 : t * 16;
-    if (STAGE == 0) {
-#pragma unroll
-      for (int t2 = 1; t2 < NT; ++t2)
-        if (t == t2) tile_row = (t2 / kHalfTiles) * p.ncols + (t2 % kHalfTiles) * 16;
-    }
-    sc_piece[j] = tile_row * groups + (piece - t * groups) * 16;
-  }
-
-  // Staging: a wavefront takes the groups wave, wave + WAVES, ... (its pieces 0, 1, ...).
-  static_assert(WAVES % 4 == 0, "a wavefront's pieces keep their quarter of a K step");
-  const int my_groups = (groups - wave + WAVES - 1) / WAVES;      // pieces with values of the row
-  const int my_pieces = (nsteps * 4 - wave + WAVES - 1) / WAVES;  // ... and those of the zero padding
-  // where lane (row lane / 4, eighth lane % 4) writes piece 0: the leading plane
-  // (the remainder plane is 2 KB on) and the block scale byte
-  uint8_t* const plane0 =
-      reinterpret_cast<uint8_t*>(b_lds) +
-      (size_t)((((wave >> 2) * 4 + ((wave >> 1) & 1)) * 64 + ((wave & 1) * 2 + ((lane & 3) >> 1)) * 16 +
-                (lane >> 2)) * 16 + (lane & 1) * 8);
-  uint8_t* const bsc0 = bsc_lds + (wave >> 2) * 64 + (wave & 3) * 16 + (lane >> 2);
 
   // Segments of the slice: the units [u0, u1) of run r.  K split: at most WAVES / 2 units
   // at a time, each shared by WAVES / (u1 - u0) wavefronts (ks_n of them, wavefront
@@ -726,33 +735,78 @@ __global__ __launch_bounds__(64 * WAVES) void stream_resident_kernel(GemmArgs p)
         // Lane (j, d) = (lane / 4, lane % 4) takes the 8 values k = 32 g + 8 d ..
         // of row j for group g = pq; the four lanes of a group share the block
         // scale.  All the loads of a lane (up to kBatch) are in flight together.
-        // Order of issue: the row loads, then the first D steps of the weight
-        // stream (every wavefront, with or without units: no branch between
-        // the loads, so that the wait below counts only the row loads), then
-        // the wait for the slowest wavefront of the previous pass.  The weight
-        // loads so stay in flight while the rows are split and written.
+        // Order of issue: the row pieces that the first D K steps need, then the
+        // first D steps of the weight stream (every wavefront, with or without
+        // units: no branch between the loads, so that the waits below count them
+        // exactly), then the rest of the rows.  The weights are so asked for as early
+        // as the order of the data allows, and both they and the later row pieces
+        // stay in flight while the first pieces are split and written.
         constexpr int kBatch = resident_batch(WAVES);  // pieces per lane, all of K in one batch
+        // pieces of a lane that K steps [0, D) need (K split: all, every part starts at once)
+        constexpr int kFirst = KSPLIT ? kBatch : ((D * 4 + WAVES - 1) / WAVES < kBatch ? (D * 4 + WAVES - 1) / WAVES : kBatch);
         const int n_pieces = (nsteps * 4 + WAVES - 1) / WAVES;  // the launcher keeps it <= kBatch
-        const int sd = lane & 3;
-        const int sj = lane >> 2;
-        const uint16_t* src =
-            p.A + (size_t)(st_flat >= 0 ? (STAGE == 0 ? st_flat / p.top_k
-                                                      : run_row0 + tile * 16 + sj)
-                                        : 0) * (size_t)p.a_stride;
+        // What depends on the wavefront and the lane alone is formed here, from values the
+        // compiler cannot see through, and not once in front of the loops over segments and
+        // passes: hoisted there, the dozens of piece predicates, plane addresses and row
+        // addresses would live through the whole kernel, beyond what the register file
+        // holds, and their reloads from the spill area would each wait for every load in
+        // flight.
+        int wave_l = wave;
+        __asm__ volatile("" : "+s"(wave_l));
+        int lane_l = lane;
+        __asm__ volatile("" : "+v"(lane_l));
+        // Staging: a wavefront takes the groups wave, wave + WAVES, ... (its pieces 0, 1, ...).
+        const int my_groups = (groups - wave_l + WAVES - 1) / WAVES;      // pieces with values of the row
+        const int my_pieces = (nsteps * 4 - wave_l + WAVES - 1) / WAVES;  // ... and those of the zero padding
+        // where lane (row lane / 4, eighth lane % 4) writes piece 0: the leading plane
+        // (the remainder plane is 2 KB on) and the block scale byte
+        uint8_t* const plane0 =
+            reinterpret_cast<uint8_t*>(b_lds) +
+            (size_t)((((wave_l >> 2) * 4 + ((wave_l >> 1) & 1)) * 64 + ((wave_l & 1) * 2 + ((lane_l & 3) >> 1)) * 16 +
+                      (lane_l >> 2)) * 16 + (lane_l & 1) * 8);
+        uint8_t* const bsc0 = bsc_lds + (wave_l >> 2) * 64 + (wave_l & 3) * 16 + (lane_l >> 2);
+        const int sd = lane_l & 3;
+        const int sj = lane_l >> 2;
+        // The row pieces of a lane: one 32-bit offset per lane from the uniform base (the row,
+        // the wavefront's group and the lane's eighth of it) and a uniform offset per piece,
+        // so that the dozen loads share one address register.  A lane without a row, or a
+        // wavefront without a group, reads the first bytes of the first row instead.
+        const bool has_row = st_flat >= 0 && my_groups > 0;
+        const uint32_t row_off =
+            has_row ? ((uint32_t)(STAGE == 0 ? st_flat / p.top_k : run_row0 + tile * 16 + sj) * (uint32_t)p.a_stride +
+                       (uint32_t)(wave_l * 32 + sd * 8)) * 2u
+                    : 0u;
+        const char* const a_base = reinterpret_cast<const char*>(p.A);
+        auto load_piece = [&](int it) {
+          // branch-free: an invalid piece reads piece 0 again
+          const uint32_t piece_off = it < my_groups ? (uint32_t)(it * WAVES * 64) : 0u;  // uniform
+          return *reinterpret_cast<const u32x4*>(a_base + piece_off + row_off);
+        };
         if (pass_no == 1) DECODE_TRACE(6);  // set-up of the loops done
         u32x4 v[kBatch];
-        const uint16_t* piece0 = src + (st_flat >= 0 && my_groups > 0 ? wave * 32 + sd * 8 : 0);
-        const int piece_stride = st_flat >= 0 ? WAVES * 32 : 0;
+#ifndef VK_EXP_ORDER
+#define VK_EXP_ORDER 1
+#endif
+#if VK_EXP_ORDER == 0
 #pragma unroll
-        for (int it = 0; it < kBatch; ++it) {
-          // branch-free: an invalid piece reads the first piece (the row's first bytes) instead
-          v[it] = *reinterpret_cast<const u32x4*>(piece0 + (it < my_groups ? it * piece_stride : 0));
-        }
+        for (int it = 0; it < kBatch; ++it) v[it] = load_piece(it);
+        __builtin_amdgcn_sched_barrier(0);
         prime();
+        __builtin_amdgcn_sched_barrier(0);
+#else
+#pragma unroll
+        for (int it = 0; it < kFirst; ++it) v[it] = load_piece(it);
+        __builtin_amdgcn_sched_barrier(0);  // (the order of issue is the point)
+        prime();
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int it = kFirst; it < kBatch; ++it) v[it] = load_piece(it);
+        __builtin_amdgcn_sched_barrier(0);
+#endif
         if (pass_no == 1) DECODE_TRACE(7);  // rows and first weight steps asked for
-        // Block scale byte of piece `it` (0 = outside the fast path's range).
-        auto block_scale = [&](int it) -> uint32_t {
-          uint32_t emax = bf16x8_max_exponent(v[it]);
+        // Block scale byte of a piece (0 = outside the fast path's range).
+        auto block_scale = [&](const u32x4& x) -> uint32_t {
+          uint32_t emax = bf16x8_max_exponent(x);
           emax = max(emax, (uint32_t)__builtin_amdgcn_mov_dpp((int)emax, 0xB1, 0xF, 0xF, true));
           emax = max(emax, (uint32_t)__builtin_amdgcn_mov_dpp((int)emax, 0x4E, 0xF, 0xF, true));
           if (emax == 0u) return 127u;  // a block of zeros (or bf16 subnormals, taken as zero)
@@ -761,16 +815,26 @@ __global__ __launch_bounds__(64 * WAVES) void stream_resident_kernel(GemmArgs p)
         };
         // Split and write the pieces [staged, upto) of this lane.  Piece `it` of
         // wavefront w is group w + it * WAVES, so once every wavefront has
-        // written `n` pieces the K steps below n * WAVES / 4 are complete.
+        // written `n` pieces the K steps below n * WAVES / 4 are complete.  A block
+        // outside the fast path's range (checked here, as the pieces arrive) marks the
+        // pass for the exact path: the mark is complete once every piece is written, which
+        // is before the first unit of any wavefront is (its last K step needs the last
+        // pieces), so nothing of a marked pass is stored by the fast path.
         int staged = 0;
         auto write_rows = [&](int upto) {
+          bool slow = false;
 #pragma unroll
           for (int it = 0; it < kBatch; ++it) {
             if (it >= staged && it < upto && it < my_pieces) {
-              uint32_t sb = block_scale(it);
-              if (sb == 0u) sb = 127u;  // the pass takes the exact path; keep the bytes defined
+              u32x4 x = v[it];
+              if (!(it < my_groups && st_flat >= 0)) x = u32x4{0u, 0u, 0u, 0u};
+              uint32_t sb = block_scale(x);
+              if (sb == 0u) {  // the pass takes the exact path; keep the bytes defined
+                slow = true;
+                sb = 127u;
+              }
               uint2 hi, lo;
-              split_bf16x8(v[it], sb, hi, lo);
+              split_bf16x8(x, sb, hi, lo);
               // piece `it` is group wave + it * WAVES: K step (wave / 4) + it * (WAVES / 4),
               // quarter wave % 4 of it, so its places are those of piece 0 plus constants
               uint8_t* plane = plane0 + it * (WAVES / 4) * 4096;
@@ -779,27 +843,21 @@ __global__ __launch_bounds__(64 * WAVES) void stream_resident_kernel(GemmArgs p)
               if (sd == 0) bsc0[it * (WAVES / 4) * 64] = (uint8_t)sb;
             }
           }
+          if (slow) pass_slow[flag] = 1;
           staged = upto;
         };
         // pieces every wavefront must have written before K steps [0, steps) can run
         auto pieces_for = [&](int steps) { return min(n_pieces, (steps * 4 + WAVES - 1) / WAVES); };
 
-        {
-          bool slow = false;
-#pragma unroll
-          for (int it = 0; it < kBatch; ++it) {
-            if (!(it < my_groups && st_flat >= 0)) v[it] = u32x4{0u, 0u, 0u, 0u};
-            if (it < my_pieces) slow |= block_scale(it) == 0u;
-          }
-          if (pass_no == 1) DECODE_TRACE(2);  // this wavefront's rows are in and checked
-          __syncthreads();  // the previous pass is done with the planes and with its flag
-          if (slow) pass_slow[flag] = 1;
-        }
-        if (pass_no == 1) DECODE_TRACE(8);  // every wavefront's are
+        __syncthreads();  // the previous pass is done with the planes and with its flag
+        if (pass_no == 1) DECODE_TRACE(8);
         // The rows are staged in K order, a few K steps ahead of the first unit's
         // arithmetic, with a barrier after each portion: the weight stream starts
         // after the first portion and the rest of the splitting overlaps it.
-        write_rows(KSPLIT ? n_pieces : pieces_for(min(nsteps, D)));  // (K split: every part starts at once)
+#ifndef VK_EXP_STAGE_ALL
+#define VK_EXP_STAGE_ALL 0
+#endif
+        write_rows((KSPLIT || VK_EXP_STAGE_ALL) ? n_pieces : pieces_for(min(nsteps, D)));  // (K split: every part starts at once)
         if (pass_no == 1) DECODE_TRACE(9);  // first K steps split and written
         if (n_my > 0) {
           park_scales();
@@ -809,60 +867,51 @@ __global__ __launch_bounds__(64 * WAVES) void stream_resident_kernel(GemmArgs p)
         __syncthreads();
         if (pass_no == 1) DECODE_TRACE(3);  // the stream starts
         if (tid == 0) pass_slow[flag ^ 1] = 0;  // for the next pass; its last reader is behind us
-        const bool slow_pass = pass_slow[flag] != 0;
-        if constexpr (!KSPLIT) {
-          if (n_my == 0 || slow_pass) {
-            // no fast stream here: finish the staging in step with the other wavefronts
-            for (int f0 = D; staged < n_pieces; f0 += D) {
-              write_rows(pieces_for(min(nsteps, f0 + D)));
-              __syncthreads();
-            }
-            if (n_my == 0) continue;
-          }
-        }
 
         f32x4 acc[NT];
         unsigned long long redo = 0ull;  // units (bit = index among this wavefront's) to redo
-        if (slow_pass) {
-          redo = n_my >= 64 ? ~0ull : (1ull << n_my) - 1ull;
-          if (KSPLIT && my_c > 0) redo = 0ull;  // the unit's first wavefront redoes all of it
-        } else {
 #pragma unroll
-          for (int t = 0; t < NT; ++t) acc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
-          uint32_t bad = 0u;
+        for (int t = 0; t < NT; ++t) acc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+        uint32_t bad = 0u;
 
-          auto compute = [&](const Stage& sg, int ks) {
-            const int g = min(ks * 4 + lq, groups - 1);
-            int sa[NT];
+        auto compute = [&](const Stage& sg, int ks) {
+          const int g = min(ks * 4 + lq, groups - 1);
+          int sa[NT];
 #pragma unroll
-            for (int t = 0; t < NT; ++t) {
-              const uint32_t sb = sc_lds[t * sc_tile_bytes + ln * groups + g];
-              bad |= (uint32_t)((sb - kScaleLo) > (kScaleHi - kScaleLo));
-              bad |= fp4x8_nonfinite(sg.w[t][0]) | fp4x8_nonfinite(sg.w[t][1]) |
-                     fp4x8_nonfinite(sg.w[t][2]) | fp4x8_nonfinite(sg.w[t][3]);
-              sa[t] = (int)sb - 1;
-            }
-            const int sbh = bsc_lds[ks * 64 + lane];
-            const int sbl = sbh - 4;
-            const u32x4 h0 = b_lds[(ks * 4 + 0) * 64 + lane], h1 = b_lds[(ks * 4 + 1) * 64 + lane];
-            const u32x4 l0 = b_lds[(ks * 4 + 2) * 64 + lane], l1 = b_lds[(ks * 4 + 3) * 64 + lane];
-            const i32x8 bh = fp8_operand(h0, h1);
-            const i32x8 bl = fp8_operand(l0, l1);
-            i32x8 wa[NT];
+          for (int t = 0; t < NT; ++t) {
+            const uint32_t sb = sc_lds[t * sc_tile_bytes + ln * groups + g];
+            bad |= (uint32_t)((sb - kScaleLo) > (kScaleHi - kScaleLo));
+            bad |= fp4x8_nonfinite(sg.w[t][0]) | fp4x8_nonfinite(sg.w[t][1]) |
+                   fp4x8_nonfinite(sg.w[t][2]) | fp4x8_nonfinite(sg.w[t][3]);
+            sa[t] = (int)sb - 1;
+          }
+          const int sbh = bsc_lds[ks * 64 + lane];
+          const int sbl = sbh - 4;
+          const u32x4 h0 = b_lds[(ks * 4 + 0) * 64 + lane], h1 = b_lds[(ks * 4 + 1) * 64 + lane];
+          const u32x4 l0 = b_lds[(ks * 4 + 2) * 64 + lane], l1 = b_lds[(ks * 4 + 3) * 64 + lane];
+          const i32x8 bh = fp8_operand(h0, h1);
+          const i32x8 bl = fp8_operand(l0, l1);
+          i32x8 wa[NT];
 #pragma unroll
-            for (int t = 0; t < NT; ++t) wa[t] = fp4_operand(sg.w[t]);
-            // the two MFMAs of an accumulator are kept NT instructions apart
+          for (int t = 0; t < NT; ++t) wa[t] = fp4_operand(sg.w[t]);
+          // the two MFMAs of an accumulator are kept NT instructions apart
 #pragma unroll
-            for (int t = 0; t < NT; ++t)
-              acc[t] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wa[t], bh, acc[t], 4, 0, 0,
-                                                                        sa[t], 0, sbh);
+          for (int t = 0; t < NT; ++t)
+            acc[t] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wa[t], bh, acc[t], 4, 0, 0,
+                                                                      sa[t], 0, sbh);
 #pragma unroll
-            for (int t = 0; t < NT; ++t)
-              acc[t] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wa[t], bl, acc[t], 4, 0, 0,
-                                                                        sa[t], 0, sbl);
-          };
+          for (int t = 0; t < NT; ++t)
+            acc[t] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wa[t], bl, acc[t], 4, 0, 0,
+                                                                      sa[t], 0, sbl);
+        };
 
-          if constexpr (KSPLIT) {
+        if constexpr (KSPLIT) {
+          // All the rows were written before the barrier above, so the mark is complete.
+          const bool slow_pass = pass_slow[flag] != 0;
+          if (slow_pass) {
+            redo = n_my >= 64 ? ~0ull : (1ull << n_my) - 1ull;
+            if (my_c > 0) redo = 0ull;  // the unit's first wavefront redoes all of it
+          } else {
             // this wavefront's part of K (none: a wavefront left over), then the parts of
             // a unit summed in order by its first wavefront; every wavefront keeps the barriers
             const int my_steps = n_my > 0 ? k_end - k_begin : 0;
@@ -894,7 +943,16 @@ __global__ __launch_bounds__(64 * WAVES) void stream_resident_kernel(GemmArgs p)
               else if (my_flat >= 0)
                 epilogue_tile<STAGE, NT>(p, e, acc, col0, my_flat, srow, lq);
             }
-          } else {
+          }
+        } else {
+          if (n_my == 0) {
+            // no stream here: finish the staging in step with the other wavefronts
+            for (int f0 = D; staged < n_pieces; f0 += D) {
+              write_rows(pieces_for(min(nsteps, f0 + D)));
+              __syncthreads();
+            }
+            continue;
+          }
           const int total_steps = n_my * nsteps;
           int cks = 0;    // K step of the unit being computed
           int cunit = 0;  // its index among this wavefront's units
@@ -909,9 +967,11 @@ __global__ __launch_bounds__(64 * WAVES) void stream_resident_kernel(GemmArgs p)
                 compute(st[i], cks);
                 if (++cks == nsteps) {
                   // ---- the unit is complete ---------------------------------
-                  // a unit that met a code or scale outside the fast path's
-                  // domain is redone after the stream, so the hot loop stays small
-                  if (__ballot(bad != 0u) != 0ull)
+                  // (every piece of the rows was written, and its barrier passed, before this
+                  // unit's last K step could run: the pass's mark is complete.)  A unit of a
+                  // marked pass, or one that met a code or scale outside the fast path's
+                  // domain, is redone after the stream, so the hot loop stays small
+                  if (__ballot(bad != 0u) != 0ull || pass_slow[flag] != 0)
                     redo |= 1ull << cunit;
                   else if (my_flat >= 0)
                     epilogue_tile<STAGE, NT>(p, e, acc, col0, my_flat, srow, lq);
@@ -935,7 +995,6 @@ __global__ __launch_bounds__(64 * WAVES) void stream_resident_kernel(GemmArgs p)
               issue(st[i]);
             }
           }
-          }  // (not K split)
         }
 
         // ---- reference-exact pass over the units the fast path could not take

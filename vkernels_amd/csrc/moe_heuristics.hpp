@@ -33,8 +33,8 @@ inline bool operator==(const MoeTile& a, const MoeTile& b) {
 // the tile kernels as one more entry.  The sweep (vkernels_amd/tune_moe.py) times each
 // of these for a stage and a problem size.
 #define VK_RESIDENT_VARIANTS(X) \
-  X(0, 8, 2, 2) X(0, 8, 2, 4) X(0, 8, 2, 6) X(0, 4, 2, 4) X(0, 4, 2, 8) \
-  X(1, 8, 2, 4) X(1, 8, 1, 4) X(1, 8, 1, 6) X(1, 8, 1, 8) X(1, 8, 1, 12)
+  X(0, 8, 2, 2) X(0, 8, 2, 3) X(0, 8, 2, 4) X(0, 8, 2, 6) X(0, 4, 2, 4) X(0, 4, 2, 8) \
+  X(1, 8, 2, 4) X(1, 8, 2, 2) X(1, 8, 1, 4) X(1, 8, 1, 5) X(1, 8, 1, 6) X(1, 8, 1, 8) X(1, 8, 1, 12)
 // ... and of its K-split form (every one is also in the list above: a plan that cannot
 // split K falls back to the same shape there).
 #define VK_KSPLIT_VARIANTS(X) X(0, 8, 2, 4) X(0, 8, 2, 6) X(1, 8, 1, 8) X(1, 8, 2, 4)
@@ -122,12 +122,11 @@ inline MoeTile pick_moe_tile(int n_flat, int K, int ncols, int stage) {
       return MoeTile{kMoeVariantResidentKSplit, 8, 2, 4};
   }
   static const MoeTileRule rules[] = {
-      {0, kMoeDecodeMaxRows, 1024, {kMoeVariantResident, 8, 2, 2}},
-      {0, kMoeDecodeMaxRows, 3072, {kMoeVariantResident, 8, 2, 4}},
+      {0, kMoeDecodeMaxRows, 3072, {kMoeVariantResident, 8, 2, 2}},
       {0, kMoeDecodeMaxRows, 4096, {kMoeVariantResident, 4, 2, 8}},
       {1, kMoeDecodeMaxRows, 1024, {kMoeVariantResident, 8, 1, 4}},
       {1, 24, 3072, {kMoeVariantResident, 8, 2, 4}},
-      {1, kMoeDecodeMaxRows, 3072, {kMoeVariantResident, 8, 1, 8}},
+      {1, kMoeDecodeMaxRows, 3072, {kMoeVariantResident, 8, 1, 6}},
   };
   for (const MoeTileRule& r : rules)
     if (r.stage == stage && n_flat <= r.max_rows && K <= r.max_k) return r.tile;

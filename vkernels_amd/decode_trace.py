@@ -21,9 +21,8 @@ PHASES = (
     ("-> slice known, barrier", 5, 1),
     ("-> set-up of the loops done", 1, 6),
     ("-> rows and first weight steps asked for", 6, 7),
-    ("-> this wavefront's rows in and checked", 7, 2),
-    ("-> every wavefront's (barrier)", 2, 8),
-    ("-> first K steps split and written", 8, 9),
+    ("-> barrier with the previous pass", 7, 8),
+    ("-> first rows in, split and written", 8, 9),
     ("-> scales parked", 9, 10),
     ("-> barrier: the stream starts", 10, 3),
     ("stream", 3, 4),
