@@ -8,7 +8,22 @@
 //   - the 32 bytes a lane reads as its operand are K block (2 half + hh) of row ln of its
 //     row tile and term: the copy's XOR rotation and the read's undo each other;
 //   - the epilogue's staging area lies inside the wavefront's quarter of the ring.
+// and, for every number of live row tiles, the K loop's schedule of one wavefront (the
+// kernel's loop structure restated with the schedule functions of the same header): every
+// vector-memory operation in program order against the counted waits, the LDS reads
+// against the waits for them, the barriers, and the ring slots and weight register sets
+// they touch:
+//   - when an MFMA uses a step's weights, a wait has forced that step's loads to land;
+//   - when an operand is read from a ring slot, every wavefront's copies of that step have
+//     landed (each wavefront waited for its own, then a barrier);
+//   - when a copy is issued into a ring slot, every read of the step it overwrites has
+//     completed in every wavefront (a wait for the LDS reads, then a barrier);
+//   - when a load is issued into a weight register set, the MFMAs of the step it
+//     overwrites are behind it;
+//   - before the epilogue writes its staging area over the ring, nothing is in flight.
 // Usage: prefill_layout_check stage terms K ncols num_experts rows ; exit status 0 = all hold.
+// Built with -DVK_LAYOUT_BREAK_WAIT the model's wait lets one operation too many stay
+// outstanding, which the walk must notice (the test of the test).
 #include <cstdio>
 #include <cstdlib>
 #include <vector>
@@ -26,6 +41,138 @@ using namespace vk;
       return 1;                                           \
     }                                                     \
   } while (0)
+
+// ---- the schedule of one wavefront ----------------------------------------------------------
+namespace {
+
+struct Event {
+  enum Kind { kCopy, kLoad, kWait, kLdsWait, kBarrier, kRead, kUse, kStaging } kind;
+  int step;  // K step the operation belongs to (copies, loads, reads, uses)
+  int n;     // kWait: operations that may stay outstanding
+};
+
+// Program order of the K loop and what follows it, as tile_mx_kernel issues it.
+std::vector<Event> schedule(int terms, int live, int nsteps) {
+  const int ops = mx_step_ops(terms), rows = mx_row_ops(terms);
+  const int Q = mx_step_groups(live, terms), per = mx_ops_per_group(live, terms);
+  std::vector<Event> ev;
+  auto issue = [&](int step, int k) { ev.push_back({k < rows ? Event::kCopy : Event::kLoad, step, 0}); };
+  // prologue: the operations of steps 0 and 1, a wait that leaves step 1's outstanding, a barrier,
+  // the reads of the first two groups
+  for (int k = 0; k < ops; ++k) issue(0, k);
+  for (int k = 0; k < ops; ++k) issue(1, k);
+#ifdef VK_LAYOUT_BREAK_WAIT
+  ev.push_back({Event::kWait, 0, ops + 1});
+#else
+  ev.push_back({Event::kWait, 0, ops});
+#endif
+  ev.push_back({Event::kBarrier, 0, 0});
+  ev.push_back({Event::kRead, 0, 0});
+  ev.push_back({Event::kRead, 0, 0});
+  for (int c = 0; c < nsteps; ++c) {
+    int issued = 0;
+    for (int q = 0; q < Q; ++q) {
+      ev.push_back({Event::kUse, c, 0});                                     // the group's MFMAs
+      ev.push_back({Event::kRead, q + 2 < Q ? c : c + 1, 0});                // the operand of group q + 2
+      if (q < Q - 2) {
+        for (int k = 0; k < per; ++k)
+          if (issued + k < ops) issue(c + 2, issued + k);
+        issued += per;
+      }
+      if (q == mx_wait_group(live, terms)) {
+        ev.push_back({Event::kWait, c, ops});
+        ev.push_back({Event::kLdsWait, c, 0});
+        ev.push_back({Event::kBarrier, c, 0});
+      }
+    }
+  }
+  ev.push_back({Event::kWait, nsteps, 0});   // the loads issued past the last step land
+  ev.push_back({Event::kBarrier, nsteps, 0});
+  ev.push_back({Event::kStaging, nsteps, 0});
+  return ev;
+}
+
+// Walks the schedule; 0 = every rule of the header comment holds.
+int check_schedule(int terms, int live, int nsteps) {
+  const std::vector<Event> ev = schedule(terms, live, nsteps);
+  const int ops = mx_step_ops(terms);
+  std::vector<int> vm;          // issue positions (indices into ev) of the vector-memory operations, in order
+  size_t landed = 0;            // operations known to have landed (a wait forced them)
+  // per K step: operations issued, operations landed, landed-and-behind-a-barrier (every wavefront's),
+  // reads issued, reads completed, completed-and-behind-a-barrier, MFMA groups issued
+  const int S = nsteps + 4;
+  std::vector<int> issued(S, 0), done(S, 0), done_all(S, 0), reads(S, 0), reads_done(S, 0), reads_done_all(S, 0), uses(S, 0);
+  std::vector<int> step_of;     // step of each vector-memory operation
+  for (size_t i = 0; i < ev.size(); ++i) {
+    const Event& e = ev[i];
+    switch (e.kind) {
+      case Event::kCopy: {
+        // the slot held step e.step - kMxRing: all its reads complete everywhere
+        const int old = e.step - kMxRing;
+        if (old >= 0) {
+          CHECK(reads_done_all[old] == reads[old], "terms %d live %d nsteps %d: a copy of step %d is issued while "
+                "reads of step %d may be under way", terms, live, nsteps, e.step, old);
+          CHECK(uses[old] > 0 || old >= nsteps, "copy before the step it overwrites was used");
+        }
+        CHECK(mx_ring_slot(e.step) == mx_ring_slot(e.step + kMxRing), "ring");
+        vm.push_back((int)i);
+        step_of.push_back(e.step);
+        ++issued[e.step];
+        break;
+      }
+      case Event::kLoad: {
+        const int old = e.step - 3;  // the register set's previous step: its MFMAs are all issued
+        if (old >= 0 && old < nsteps)
+          CHECK(uses[old] == mx_step_groups(live, terms), "terms %d live %d nsteps %d: a weight load of step %d is "
+                "issued before the MFMAs of step %d", terms, live, nsteps, e.step, old);
+        CHECK(mx_weight_set(e.step) == mx_weight_set(e.step + 3), "sets");
+        vm.push_back((int)i);
+        step_of.push_back(e.step);
+        ++issued[e.step];
+        break;
+      }
+      case Event::kWait: {
+        const size_t must = vm.size() > (size_t)e.n ? vm.size() - (size_t)e.n : 0;
+        for (; landed < must; ++landed) ++done[step_of[landed]];
+        break;
+      }
+      case Event::kLdsWait:
+        for (int s = 0; s < S; ++s) reads_done[s] = reads[s];
+        break;
+      case Event::kBarrier:
+        for (int s = 0; s < S; ++s) {
+          if (done[s] == issued[s]) done_all[s] = done[s];
+          reads_done_all[s] = reads_done[s];
+        }
+        break;
+      case Event::kRead:
+        // (a read of the step after the last only fetches an operand nobody multiplies, but
+        // it still reads the ring: the same rule)
+        CHECK(issued[e.step] == ops && done_all[e.step] == ops, "terms %d live %d nsteps %d: an operand of step %d "
+              "is read before every wavefront's copies of it have landed", terms, live, nsteps, e.step);
+        ++reads[e.step];
+        break;
+      case Event::kUse:
+        CHECK(issued[e.step] == ops && done[e.step] == ops, "terms %d live %d nsteps %d: step %d's weights are used "
+              "before a wait has let them land", terms, live, nsteps, e.step);
+        ++uses[e.step];
+        break;
+      case Event::kStaging:
+        CHECK(landed == vm.size(), "terms %d live %d nsteps %d: operations in flight when the epilogue starts",
+              terms, live, nsteps);
+        for (int s = 0; s < S; ++s)
+          CHECK(reads_done_all[s] == reads[s] || reads[s] == 0 || s >= nsteps,
+                "reads of step %d outstanding at the epilogue", s);
+        break;
+    }
+  }
+  // every K step was multiplied, with all its groups, and every step's operations were issued once
+  for (int c = 0; c < nsteps; ++c) CHECK(uses[c] == mx_step_groups(live, terms) && issued[c] == ops, "step %d", c);
+  CHECK(mx_ops_per_group(live, terms) * (mx_step_groups(live, terms) - 2) >= ops, "a step's operations do not fit its groups");
+  return 0;
+}
+
+}  // namespace
 
 int main(int argc, char** argv) {
   if (argc != 7) return 2;
@@ -126,5 +273,12 @@ int main(int argc, char** argv) {
     CHECK(lo % 16 == 0 && lo + need <= hi, "staging area of wavefront %d: %d bytes in [%d, %d)", wave, need, lo, hi);
   }
   CHECK(kMxActPitch % 16 == 0 && kMxYPitch % 16 == 0, "pitch");
+  // ---- the K loop's schedule: every number of live row tiles the kernel compiles, the
+  // problem's own K steps and the shortest loops ----
+  for (int live = 1; live <= 4; ++live) {
+    if (live == 1 && terms == 1) continue;  // (one plane per row: the kernel runs two live tiles then)
+    for (int steps : {1, 2, 3, 4, 5, 7, nsteps})
+      if (check_schedule(terms, live, steps) != 0) return 1;
+  }
   return 0;
 }

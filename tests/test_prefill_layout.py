@@ -3,7 +3,12 @@ offset through the functions of vkernels_amd/csrc/moe_prefill_layout.hpp, and
 tests/prefill_layout_check.cpp (compiled here with g++) walks all lanes, K steps and tiles of
 a problem with the same functions: loads inside the prepacked weights and the split rows,
 copies inside their ring slot without overlap, operand reads hitting exactly the bytes of
-their row, term and K block, staging areas inside the ring.  Shapes: every configuration of
+their row, term and K block, staging areas inside the ring.  The same program also walks the
+K loop's schedule of a wavefront (prologue, every group of every step, the step's one wait
+and barrier, the tail, loops of one and two steps, one to four live row tiles, one to three
+terms) built from the schedule functions the kernel's counted waits are built from: issued
+against waited vector-memory operations, ring slots written against slots still read,
+weight register sets loaded against sets still multiplied.  Shapes: every configuration of
 the benchmark list, both stages, every term count, and ragged ones."""
 from __future__ import annotations
 
@@ -57,3 +62,13 @@ def test_the_checker_notices_a_wrong_layout(checker, tmp_path):
                     "-o", str(exe)], check=True)
     res = subprocess.run([str(exe), "0", "3", "2880", "2880", "4", "64"], capture_output=True, text=True)
     assert res.returncode == 1 and "FAILED" in res.stderr
+
+
+def test_the_checker_notices_a_wait_that_counts_wrong(tmp_path):
+    """The schedule walk is not vacuous either: with the prologue's wait letting one more
+    operation stay outstanding than the kernel's does, the first operand read is flagged."""
+    exe = tmp_path / "broken_wait"
+    subprocess.run(["g++", "-O2", "-std=c++17", "-DVK_LAYOUT_BREAK_WAIT", f"-I{ROOT / 'vkernels_amd' / 'csrc'}",
+                    str(ROOT / "tests" / "prefill_layout_check.cpp"), "-o", str(exe)], check=True)
+    res = subprocess.run([str(exe), "1", "2", "2048", "7168", "4", "640"], capture_output=True, text=True)
+    assert res.returncode == 1 and "before every wavefront's copies of it have landed" in res.stderr

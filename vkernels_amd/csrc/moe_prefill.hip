@@ -567,8 +567,8 @@ __global__ __launch_bounds__(64 * kMxWaves) void tile_mx_kernel(MxArgs p) {
 
   // Vector-memory operations of a wavefront per K step (for step c + 2): 4 TERMS row
   // copies, 8 weight loads, 1 scale load.
-  constexpr int kRowOps = 4 * TERMS;
-  constexpr int kOps = kRowOps + 9;
+  constexpr int kRowOps = mx_row_ops(TERMS);
+  constexpr int kOps = mx_step_ops(TERMS);
 
   // the rows of this workgroup's window
   const int total_rows = p.num_blocks * p.block_size;
@@ -700,8 +700,9 @@ __global__ __launch_bounds__(64 * kMxWaves) void tile_mx_kernel(MxArgs p) {
     // barrier step c + 1 can be read and the slot of step c can take step c + 3.
     auto k_loop = [&](auto live_c) {
       constexpr int LIVE = decltype(live_c)::value;
-      constexpr int Q = 2 * LIVE * TERMS;                  // groups (operand reads) per step
-      constexpr int kPer = (kOps + Q - 3) / (Q - 2);       // memory operations per issuing group
+      constexpr int Q = mx_step_groups(LIVE, TERMS);       // groups (operand reads) per step
+      constexpr int kPer = mx_ops_per_group(LIVE, TERMS);  // memory operations per issuing group
+      static_assert(Q >= 4 && kPer * (Q - 2) >= kOps, "a step's loads are all issued before its wait");
       auto group_operand = [&](const SlotBase& sb, int q) {
         return read_operand(sb, (q / TERMS) % LIVE, q % TERMS, q / (LIVE * TERMS));
       };
@@ -723,7 +724,7 @@ __global__ __launch_bounds__(64 * kMxWaves) void tile_mx_kernel(MxArgs p) {
       auto step = [&](auto i_c, const int c) {
         constexpr int i = decltype(i_c)::value;
         constexpr int in1 = (i + 1) % 3, in2 = (i + 2) % 3;
-        int slot_next = (c + 1) % R;
+        int slot_next = mx_ring_slot(c + 1);
         __asm__ volatile("" : "+s"(slot_next));
         const SlotBase sbn = slot_base(slot_next);
         int issued = 0;
@@ -752,7 +753,7 @@ __global__ __launch_bounds__(64 * kMxWaves) void tile_mx_kernel(MxArgs p) {
           __builtin_amdgcn_sched_barrier(0);
           acc[m][3] = mfma_fp4_act<3, TERMS == 1>(ws[i].w[half * 4 + 3], cur, acc[m][3], wsc);
           __builtin_amdgcn_sched_barrier(0);
-          if (q == Q - 3) {
+          if (q == mx_wait_group(LIVE, TERMS)) {
             wait_loads_and_reads<kOps>(ws[in1]);
             __builtin_amdgcn_s_barrier();
             __asm__ volatile("" ::: "memory");

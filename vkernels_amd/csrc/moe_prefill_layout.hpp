@@ -23,6 +23,10 @@ constexpr int kMxWaves = 4;
 constexpr int kMxRing = 3;          // K steps of split rows in LDS
 constexpr int kMxStepBytes = 8704;  // prepacked bytes of one unit's K step: 8 KiB of codes + 512 of scales
 
+// ring slot that holds the rows of K step `step`, register set that holds its weights
+__host__ __device__ constexpr inline int mx_ring_slot(int step) { return step % kMxRing; }
+__host__ __device__ constexpr inline int mx_weight_set(int step) { return step % 3; }
+
 __host__ __device__ constexpr inline int mx_kp(int K) { return (K + 127) & ~127; }
 __host__ __device__ constexpr inline int mx_units(int stage, int ncols) {
   return stage == 0 ? ncols / 64 : (ncols + kMxUnitRows - 1) / kMxUnitRows;
@@ -79,7 +83,7 @@ __host__ __device__ constexpr inline uint32_t mx_row_copy_step_offset(int term, 
 // LDS destination of lane 0 of that copy (lane l lands 16 l bytes further)
 __host__ __device__ constexpr inline int mx_slot_bytes(int terms) { return kMxRows * terms * 128; }
 __host__ __device__ constexpr inline uint32_t mx_row_copy_lds(int step, int wave, int terms, int term, int g) {
-  return (uint32_t)((step % kMxRing) * mx_slot_bytes(terms) + ((wave * terms + term) * 32 + g * 8) * 128);
+  return (uint32_t)(mx_ring_slot(step) * mx_slot_bytes(terms) + ((wave * terms + term) * 32 + g * 8) * 128);
 }
 // ---- operand reads: lane (ln, hh) = (lane % 32, lane / 32) takes K block 2 half + hh of
 // row ln of row tile m: 16-byte pieces 2 blk and 2 blk + 1, at positions (2 blk) ^ (ln & 7)
@@ -92,6 +96,22 @@ __host__ __device__ constexpr inline uint32_t mx_operand_lane_offset(int which, 
 __host__ __device__ constexpr inline uint32_t mx_operand_tile_offset(int slot, int terms, int m, int term) {
   return (uint32_t)(slot * mx_slot_bytes(terms) + ((m * terms + term) * 32) * 128);
 }
+// ---- the K loop's schedule, as numbers: the kernel's counted waits and the host-side
+// model of them (tests/prefill_layout_check.cpp) are built from these ----
+// vector-memory operations a wavefront issues per K step: 4 row copies per term (8 rows
+// x 128 bytes each, its row tile's 32 rows), 8 weight loads, 1 scale load
+__host__ __device__ constexpr inline int mx_row_ops(int terms) { return 4 * terms; }
+__host__ __device__ constexpr inline int mx_step_ops(int terms) { return mx_row_ops(terms) + 9; }
+// groups of 4 MFMAs (one operand read each) per K step with `live` row tiles
+__host__ __device__ constexpr inline int mx_step_groups(int live, int terms) { return 2 * live * terms; }
+// The operations of step c + 2 are issued in groups 0 .. Q - 3 of step c, this many per
+// group; the step's one wait (at most mx_step_ops outstanding: step c + 1 has landed, step
+// c + 2 may be on its way) and barrier come at the end of group Q - 3.
+__host__ __device__ constexpr inline int mx_ops_per_group(int live, int terms) {
+  return (mx_step_ops(terms) + mx_step_groups(live, terms) - 3) / (mx_step_groups(live, terms) - 2);
+}
+__host__ __device__ constexpr inline int mx_wait_group(int live, int terms) { return mx_step_groups(live, terms) - 3; }
+
 // ---- epilogue staging: a wavefront's own quarter of the ring ----
 __host__ __device__ constexpr inline uint32_t mx_stage_base(int wave, int terms) {
   return (uint32_t)(wave * (kMxRing * mx_slot_bytes(terms) / kMxWaves));
