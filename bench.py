@@ -199,6 +199,10 @@ def run_workload(args, workload, steps, warmup, prepack, split_terms=None, w4a4=
     def step(i, events=None):
         fe = experts[i % n_sets]
         if events is None:
+            if not args.no_workspace:
+                # router, alignment and the layer through the library's one call
+                fe.route_layer(A, logits, k, block_size=bs, out_fp32=out)
+                return
             # router and alignment through the library's one call (one launch at decode sizes)
             ids, w, sids, eids, _, max_em, _ = fe.route_align(logits, k, True, bs)
             fe.apply(A, ids, w, block_size=bs, out_fp32=out, aligned=(sids, eids, max_em))

@@ -536,6 +536,30 @@ int vk_hip_moe_route_align(const float* logits, int32_t T, int32_t E, int32_t to
                            int32_t* sorted_ids, int32_t* expert_ids, int32_t* out_EM, void* stream);
 
 /*
+ * Additive: router, alignment and the layer behind one call -- what a serving loop
+ * runs per MoE layer and step.  The arguments are those of vk_hip_moe_route_align
+ * (logits [M, num_experts] in; topk_ids, topk_w, sorted_ids [max_EM], expert_ids
+ * [max_EM / block_size], out_EM out, written as that call writes them) and of
+ * vk_hip_fused_moe_mxfp4_prepacked (the layer's buffers, workspace, flags, optional
+ * prepacked weights of num_local_experts experts).  For a handful of tokens (M <= 16,
+ * M * top_k <= 128, num_experts <= 256, block_size 16, shapes the decode kernels take)
+ * the first stage's kernel routes and aligns for itself and the step is two launches;
+ * every other call runs vk_hip_moe_route_align and then the layer, so the results are
+ * the same either way: the routing tables bit for bit, `out` as the layer computes it.
+ * M = 0 writes the alignment's sentinels and EM and leaves `out` as it is.  Returns
+ * VK_OK or a VK_ERROR_* code; asynchronous on `stream`, no allocation.
+ */
+int vk_hip_moe_route_layer_mxfp4(
+    const uint16_t* A, const float* logits, const uint8_t* w13, const uint8_t* w13_scale,
+    const uint8_t* w2, const uint8_t* w2_scale, int32_t* topk_ids, float* topk_w,
+    uint16_t* act_scratch, float* out, int M, int num_experts, int hidden, int ispp, int top_k,
+    int renormalize, const int32_t* expert_map, int local_n, int block_size, int max_EM,
+    int32_t* sorted_ids, int32_t* expert_ids, int32_t* out_EM, float swiglu_limit, int activation,
+    float beta, float linear_beta, const float* b13, const float* b2, void* workspace,
+    size_t workspace_bytes, unsigned flags, const void* w13_packed, const void* w2_packed,
+    int num_local_experts, void* stream);
+
+/*
  * Additive: dequantise an [N, K] tile of packed weights to bf16 with the
  * decode routines of the device library, written transposed as [K][N].
  * Device counterpart of dequant_weight_tile,

@@ -310,12 +310,12 @@ def test_tile_candidates_and_compiled_in_rules():
             assert not stored and shape in cands, (stage, n_flat, shape)   # selectors return table entries only
             # the decode kernels up to 512 routed rows, where a pass's rows fit LDS and registers
             assert (shape[0] in (2, 3)) == (n_flat <= 512 and K <= (4096 if stage == 0 else 3072))
-    assert ve.moe_tile_query(0, 2880, 2880, 128)[0] == (2, 8, 2, 4)
+    assert ve.moe_tile_query(0, 2880, 2880, 128)[0] == (2, 8, 2, 2) and ve.moe_tile_query(1, 2880, 2880, 128)[0] == (2, 8, 1, 6)
     assert ve.moe_tile_query(0, 4096, 1536, 6)[0] == (2, 4, 2, 8)                   # rows of K = 4096
     # one token: fewer units than half the device's wavefronts, K shared between them
     assert ve.moe_tile_query(0, 2880, 2880, 4)[0] == (3, 8, 2, 4) and ve.moe_tile_query(1, 2880, 2880, 4)[0] == (3, 8, 1, 8)
     assert ve.moe_tile_query(1, 1536, 4096, 6)[0] == (3, 8, 2, 4)                   # ... with two tiles a unit
-    assert ve.moe_tile_query(0, 2880, 2880, 8)[0] == (2, 8, 2, 4) and ve.moe_tile_query(0, 512, 2880, 4)[0] == (2, 8, 2, 2)
+    assert ve.moe_tile_query(0, 2880, 2880, 8)[0] == (2, 8, 2, 2) and ve.moe_tile_query(0, 512, 2880, 4)[0] == (2, 8, 2, 2)
     assert ve.moe_tile_query(0, 256, 512, 32)[0] == (2, 8, 2, 2) and ve.moe_tile_query(1, 512, 256, 32)[0] == (2, 8, 1, 4)
     assert ve.default_block_size(0, 4) == 16 and ve.default_block_size(1 << 20, 32) == 128
 
@@ -324,7 +324,8 @@ def test_tuning_store_round_trip(tmp_path):
     lib = ve.load_libvkernels_hip()
     key = (0, 2880, 2880, 200)
     before, _ = ve.moe_tile_query(*key)
-    other = next(c for c in ve.moe_tile_candidates(0) if c != before and c[0] == 2)
+    other = next(c for c in ve.moe_tile_candidates(0)
+                 if c != before and c[0] == 2 and c not in ve.moe_tile_candidates(1))   # a stage-0 shape only
     try:
         ve.moe_tile_set(*key, other)
         assert ve.moe_tile_query(*key) == (other, True)

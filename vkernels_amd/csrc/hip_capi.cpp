@@ -680,6 +680,55 @@ int vk_hip_moe_route_align(const float* logits, int32_t T, int32_t E, int32_t to
   return VK_OK;
 }
 
+int vk_hip_moe_route_layer_mxfp4(
+    const uint16_t* A, const float* logits, const uint8_t* w13, const uint8_t* w13_scale,
+    const uint8_t* w2, const uint8_t* w2_scale, int32_t* topk_ids, float* topk_w,
+    uint16_t* act_scratch, float* out, int M, int num_experts, int hidden, int ispp, int top_k,
+    int renormalize, const int32_t* expert_map, int local_n, int block_size, int max_EM,
+    int32_t* sorted_ids, int32_t* expert_ids, int32_t* out_EM, float swiglu_limit, int activation,
+    float beta, float linear_beta, const float* b13, const float* b2, void* workspace,
+    size_t workspace_bytes, unsigned flags, const void* w13_packed, const void* w2_packed,
+    int num_local_experts, void* stream) {
+  if (M <= 0) {  // nothing routed: the alignment still writes its sentinels and EM
+    if (M < 0) return fail(VK_ERROR_INVALID_ARGUMENT, "vk_hip_moe_route_layer_mxfp4: M must be non-negative");
+    return vk_hip_moe_align_block_size(topk_ids, expert_map, 0, top_k, block_size, num_experts, local_n,
+                                       max_EM, sorted_ids, expert_ids, out_EM, stream);
+  }
+  vk::FusedMoeArgs a =
+      fused_args(A, w13, w13_scale, w2, w2_scale, topk_w, act_scratch, out, M, hidden, ispp, top_k,
+                 sorted_ids, expert_ids, max_EM, swiglu_limit, activation, beta, linear_beta, b13, b2,
+                 block_size, workspace, workspace_bytes, flags);
+  if (max_EM <= 0 || block_size <= 0 || max_EM % block_size != 0)
+    return fail(VK_ERROR_INVALID_ARGUMENT, "vk_hip_moe_route_layer_mxfp4: block_size must divide max_EM");
+  if (!layer_args_ok("vk_hip_moe_route_layer_mxfp4", true, true, a)) return VK_ERROR_INVALID_ARGUMENT;
+  if (logits == nullptr || topk_ids == nullptr || out_EM == nullptr)
+    return fail(VK_ERROR_INVALID_ARGUMENT, "vk_hip_moe_route_layer_mxfp4: logits/topk_ids/out_EM must not be null");
+  if ((w13_packed == nullptr) != (w2_packed == nullptr) || (w13_packed != nullptr && num_local_experts <= 0))
+    return fail(VK_ERROR_INVALID_ARGUMENT,
+                "vk_hip_moe_route_layer_mxfp4: both packed buffers (or neither) and a positive "
+                "num_local_experts are required");
+  a.w13_packed = static_cast<const uint8_t*>(w13_packed);
+  a.w2_packed = static_cast<const uint8_t*>(w2_packed);
+  a.num_experts = num_local_experts;
+  if (num_experts > 0 && top_k <= num_experts && local_n >= 0 && local_n <= num_experts) {
+    vk::RoutedArgs r{};
+    r.logits = logits; r.expert_map = expert_map; r.topk_ids = topk_ids; r.topk_w = topk_w;
+    r.sorted_ids = sorted_ids; r.expert_ids = expert_ids; r.out_EM = out_EM;
+    r.num_experts = num_experts; r.local_n = local_n; r.renormalize = renormalize; r.max_EM = max_EM;
+    const hipError_t before = hipPeekAtLastError();
+    if (vk::launch_routed_moe(a, r, static_cast<hipStream_t>(stream)))
+      return note_launch_error("vk_hip_moe_route_layer_mxfp4", before) ? VK_ERROR_INTERNAL : VK_OK;
+  }
+  // every other shape: router and alignment (one launch or two), then the layer
+  const int rc = vk_hip_moe_route_align(logits, M, num_experts, top_k, renormalize, expert_map, block_size,
+                                        local_n, max_EM, topk_ids, topk_w, sorted_ids, expert_ids, out_EM,
+                                        stream);
+  if (rc != VK_OK) return rc;
+  const hipError_t before = hipPeekAtLastError();
+  vk::launch_fused_moe(a, static_cast<hipStream_t>(stream));
+  return note_launch_error("vk_hip_moe_route_layer_mxfp4", before) ? VK_ERROR_INTERNAL : VK_OK;
+}
+
 int vk_hip_dequant_weight_tile(const uint8_t* packed, const uint8_t* scale,
                                uint16_t* out_bf16, int32_t N, int32_t K,
                                int32_t group_size, int32_t stride_packed,

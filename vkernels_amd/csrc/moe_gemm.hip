@@ -43,6 +43,7 @@
 
 #include "moe_common.hpp"
 #include "moe_heuristics.hpp"
+#include "moe_route.hpp"
 #include "moe_tuning.hpp"
 #include "mxfp4.hpp"
 #include "vk_internal.hpp"
@@ -92,6 +93,18 @@ struct GemmArgs {
   int block_size;
   float swiglu_limit, beta, linear_beta;
   int activation;
+  // The routed form of the decode kernel's first stage (a handful of tokens): router and
+  // alignment are done by every workgroup for itself, in LDS, from the logits; workgroup 0
+  // writes the tables out for the second stage and the caller.  sorted_ids / expert_ids
+  // above are not read then.
+  const float* rt_logits;        // [M, rt_experts]
+  const int32_t* rt_expert_map;  // or null
+  int32_t* rt_topk_ids;          // [M, top_k] out
+  float* rt_topk_w;              // [M, top_k] out
+  int32_t* rt_sorted_ids;        // [rt_max_em] out
+  int32_t* rt_expert_ids;        // [rt_max_em / 16] out
+  int32_t* rt_out_em;            // out
+  int rt_experts, rt_local_n, rt_renormalize, rt_max_em;
 };
 
 // Rows a tile-kernel workgroup takes at a time: the largest multiple of 16 that
@@ -407,12 +420,29 @@ __device__ unsigned long long g_decode_trace[2][kTraceWorkgroups][kTraceSlots];
 // steps each, all rows are staged before any of them starts, and the unit's first wavefront
 // adds the others' sums (through LDS, over the operand planes, in a fixed order) and runs
 // the epilogue, or the exact path if any part met a value outside the fast path's domain.
-template <int STAGE, int WAVES, int NT, int D, bool KSPLIT = false>
+// ROUTE (first stage, blocks of 16 rows, at most kRouteMaxRows routed rows): the router and
+// the alignment run inside the kernel, so that a decode step of a handful of tokens is two
+// launches and not three.  Every workgroup routes all the tokens itself (a wavefront per
+// token, the arithmetic of route_topk_kernel), counts the rows of every local expert,
+// gives every expert with rows its blocks in ascending order -- these are the runs -- and
+// ranks every routed row inside its expert's blocks, all in LDS, which is what
+// route_align_kernel does per workgroup as well; workgroup 0 also writes topk_ids, topk_w,
+// sorted_ids, expert_ids and EM out, exactly as vk_hip_moe_route_align leaves them.
+constexpr int kRouteMaxRows = 128, kRouteMaxExperts = 256, kRoutePer = kRouteMaxExperts / 64;
+
+template <int STAGE, int WAVES, int NT, int D, bool KSPLIT = false, bool ROUTE = false>
 __global__ __launch_bounds__(64 * WAVES) void stream_resident_kernel(GemmArgs p) {
+  static_assert(!ROUTE || STAGE == 0, "the routed form is the first stage's");
   extern __shared__ u32x4 b_lds[];  // [nsteps][2][2][64] operand planes, block scales, weight scales
   __shared__ int run_block0[kMaxRuns];
   __shared__ int run_expert[kMaxRuns];
   __shared__ int run_cum[kMaxRuns];     // blocks of the runs up to and including this one
+  // routed form: local expert of every routed row, rows per local expert (then the first
+  // block of the expert), the 16 flat indices of every run (0xFF = padding), the run count
+  __shared__ short rt_le[ROUTE ? kRouteMaxRows : 1];
+  __shared__ int rt_hist[ROUTE ? kRouteMaxExperts : 1];
+  __shared__ unsigned char run_ids[ROUTE ? kRouteMaxRows * 16 : 1];
+  __shared__ int rt_runs;
   __shared__ int slice_sh[2];           // this workgroup's slice of the (run, unit) space
   __shared__ int pass_slow[2];          // set while staging: this pass takes the exact path
   __shared__ int ks_bad[KSPLIT ? WAVES : 1];  // K split: a wavefront's part of its unit left the fast path
@@ -447,7 +477,89 @@ __global__ __launch_bounds__(64 * WAVES) void stream_resident_kernel(GemmArgs p)
   constexpr int kIdsAhead = 2;  // loads of the copy a lane asks for before the set-up
   int e_first = -1;             // wavefront 0: the expert of block `lane`
   int ids_ahead[kIdsAhead];
-  if (wave == 0) {
+  if constexpr (ROUTE) {
+    // ---- router: a wavefront per token; the table of local experts stays in LDS ----
+    const int n_flat = p.n_flat, top_k = p.top_k, T = n_flat / top_k;
+    for (int i = tid; i < kRouteMaxExperts; i += 64 * WAVES) rt_hist[i] = 0;
+    for (int i = tid; i < kRouteMaxRows * 16; i += 64 * WAVES) run_ids[i] = 0xFF;
+    for (int token = wave; token < T; token += WAVES) {  // uniform per wavefront
+      int my_id;
+      float my_w;
+      route_token<kRoutePer>(p.rt_logits + (size_t)token * p.rt_experts, p.rt_experts, top_k,
+                             p.rt_renormalize, lane, my_id, my_w);
+      if (lane < top_k) {
+        int le = -1;
+        if (my_id >= 0 && my_id < p.rt_experts) {
+          le = p.rt_expert_map != nullptr ? p.rt_expert_map[my_id] : my_id;
+          if (le < 0 || le >= p.rt_local_n) le = -1;
+        }
+        rt_le[token * top_k + lane] = (short)le;
+        if (blockIdx.x == 0) {
+          p.rt_topk_ids[(size_t)token * top_k + lane] = my_id;
+          p.rt_topk_w[(size_t)token * top_k + lane] = my_w;
+        }
+      }
+    }
+    __syncthreads();
+    // ---- rows per local expert ----
+    for (int i = tid; i < n_flat; i += 64 * WAVES) {
+      const int le = rt_le[i];
+      if (le >= 0) atomicAdd(&rt_hist[le], 1);
+    }
+    __syncthreads();
+    // ---- first block of every expert (wavefront 0: a scan of the blocks, 64 experts a trip) ----
+    if (wave == 0) {
+      int blocks = 0;
+      for (int base = 0; base < p.rt_local_n; base += 64) {
+        const int e = base + lane;
+        const int c = e < p.rt_local_n ? rt_hist[e] : 0;
+        const int nb_e = (c + 15) >> 4;
+        int incl = nb_e;
+#pragma unroll
+        for (int d = 1; d < 64; d <<= 1) {
+          const int y = __shfl_up(incl, d);
+          if (lane >= d) incl += y;
+        }
+        if (e < p.rt_local_n) rt_hist[e] = blocks + incl - nb_e;  // the expert's first block
+        // the runs: every block with rows, in order
+        for (int b = 0; b < nb_e; ++b) {
+          const int r = blocks + incl - nb_e + b;
+          run_block0[r] = r;
+          run_expert[r] = e;
+          run_cum[r] = r + 1;
+        }
+        blocks += __shfl(incl, 63);
+      }
+      if (lane == 0) {
+        rt_runs = blocks;
+        pass_slow[0] = 0;
+        pass_slow[1] = 0;
+      }
+    }
+    __syncthreads();
+    // ---- place of every routed row: its rank among the rows of its expert ----
+    const int n_runs = rt_runs;
+    for (int i = tid; i < n_flat; i += 64 * WAVES) {
+      const int le = rt_le[i];
+      if (le >= 0) {
+        int rank = 0;
+        for (int j = 0; j < i; ++j) rank += rt_le[j] == le ? 1 : 0;
+        run_ids[rt_hist[le] * 16 + rank] = (unsigned char)i;
+      }
+    }
+    __syncthreads();
+    // ---- workgroup 0: the tables for the second stage and the caller ----
+    if (blockIdx.x == 0) {
+      const int em = min(n_runs > 0 ? n_runs * 16 : 16, p.rt_max_em);
+      if (tid == 0) *p.rt_out_em = em;
+      for (int r = tid; r < p.rt_max_em; r += 64 * WAVES) {
+        int id = n_flat;
+        if (r < n_runs * 16 && run_ids[r] != 0xFF) id = run_ids[r];
+        p.rt_sorted_ids[r] = id;
+      }
+      for (int b = tid; b < p.rt_max_em / 16; b += 64 * WAVES) p.rt_expert_ids[b] = b < n_runs ? run_expert[b] : -1;
+    }
+  } else if (wave == 0) {
     e_first = p.expert_ids[min(lane, p.num_blocks - 1)];
   } else {
 #pragma unroll
@@ -479,7 +591,7 @@ __global__ __launch_bounds__(64 * WAVES) void stream_resident_kernel(GemmArgs p)
 
   static_assert(WAVES % 4 == 0, "a wavefront's pieces keep their quarter of a K step");
 
-  if (WAVES > 1 && wave != 0) {
+  if (!ROUTE && WAVES > 1 && wave != 0) {
 #pragma unroll
     for (int j = 0; j < kIdsAhead; ++j) {
       const int i = tid - 64 + j * 64 * (WAVES - 1);
@@ -504,7 +616,11 @@ __global__ __launch_bounds__(64 * WAVES) void stream_resident_kernel(GemmArgs p)
     const int tpb = p.block_size / 16;
     int n = 0;
     int listed_weight = 0;  // weight of the runs so far
-    for (int base = 0; base < nb; base += 64) {
+    if constexpr (ROUTE) {  // the runs are listed already: every block with rows, weight 1 each
+      n = rt_runs;
+      listed_weight = n;
+    }
+    for (int base = 0; !ROUTE && base < nb; base += 64) {
       const int b = base + lane;
       const int bc = min(b, nb - 1);
       const int e_here = base == 0 ? e_first : p.expert_ids[bc];
@@ -717,8 +833,14 @@ __global__ __launch_bounds__(64 * WAVES) void stream_resident_kernel(GemmArgs p)
       if (tile0 * 16 + lane < run_tiles * 16) {
         const int at = run_row0 + tile0 * 16 + lane;
         // uniform: the first rows a workgroup stages come from the copy in LDS
-        if (pass_no == 0 && run_row0 + tile0 * 16 + 64 <= ids_cached) fl = ids_lds[at];
-        else fl = p.sorted_ids[at];
+        if constexpr (ROUTE) {
+          const int x = run_ids[at];  // (a run is a block of 16 rows: index = the sorted row)
+          fl = x == 0xFF ? -1 : x;
+        } else if (pass_no == 0 && run_row0 + tile0 * 16 + 64 <= ids_cached) {
+          fl = ids_lds[at];
+        } else {
+          fl = p.sorted_ids[at];
+        }
       }
       if (fl < 0 || fl >= p.n_flat) fl = -1;
       const unsigned long long routed = __ballot(fl >= 0);
@@ -1789,11 +1911,11 @@ constexpr size_t kResidentLdsLimit = 150 * 1024;  // dynamic LDS the resident ke
 
 // True when the device grants the kernel its dynamic LDS (asked once per kernel;
 // a refusal makes the caller take the other variant).
-template <int STAGE, int WAVES, int NT, int D, bool KSPLIT = false>
+template <int STAGE, int WAVES, int NT, int D, bool KSPLIT = false, bool ROUTE = false>
 bool resident_kernel_ready() {
   static const bool configured = [] {
     const hipError_t err = hipFuncSetAttribute(
-        reinterpret_cast<const void*>(stream_resident_kernel<STAGE, WAVES, NT, D, KSPLIT>),
+        reinterpret_cast<const void*>(stream_resident_kernel<STAGE, WAVES, NT, D, KSPLIT, ROUTE>),
         hipFuncAttributeMaxDynamicSharedMemorySize, (int)kResidentLdsLimit);
     if (err != hipSuccess) (void)hipGetLastError();  // not left for the next caller to find
     return err == hipSuccess;
@@ -1801,10 +1923,10 @@ bool resident_kernel_ready() {
   return configured;
 }
 
-template <int STAGE, int WAVES, int NT, int D, bool KSPLIT = false>
+template <int STAGE, int WAVES, int NT, int D, bool KSPLIT = false, bool ROUTE = false>
 bool launch_resident(const GemmArgs& g, size_t lds, hipStream_t stream) {
-  if (!resident_kernel_ready<STAGE, WAVES, NT, D, KSPLIT>()) return false;
-  hipLaunchKernelGGL((stream_resident_kernel<STAGE, WAVES, NT, D, KSPLIT>), dim3(num_compute_units()),
+  if (!resident_kernel_ready<STAGE, WAVES, NT, D, KSPLIT, ROUTE>()) return false;
+  hipLaunchKernelGGL((stream_resident_kernel<STAGE, WAVES, NT, D, KSPLIT, ROUTE>), dim3(num_compute_units()),
                      dim3(64 * WAVES), lds, stream, g);
   return true;
 }
@@ -2023,9 +2145,58 @@ bool prepare_moe_kernels() {
 #define VK_READY(S_, W_, NT_, D_) ok = resident_kernel_ready<S_, W_, NT_, D_, true>() && ok;
   VK_KSPLIT_VARIANTS(VK_READY)
 #undef VK_READY
+  ok = resident_kernel_ready<0, 8, 2, 4, true, true>() && resident_kernel_ready<0, 8, 2, 2, false, true>() && ok;
   MoeTile unused;
   (void)moe_tuning_find(0, 64, 64, 1, &unused);  // reads the tuning store now rather than on the first launch
   return ok;
+}
+
+// Router, alignment and the layer for a handful of tokens in two launches: the first
+// stage's decode kernel routes and aligns for itself (its routed form) and workgroup 0
+// writes the tables out, the second stage reads them.  False (nothing enqueued) when the
+// call is not one the routed form takes: more than 16 tokens or kRouteMaxRows routed rows,
+// more than kRouteMaxExperts experts, a block size other than 16, a first stage whose
+// launch shape has no routed form, or LDS that does not hold its tables as well.
+bool launch_routed_moe(const FusedMoeArgs& a, const RoutedArgs& r, hipStream_t stream) {
+  if (a.M <= 0 || a.M > 16 || a.M * a.top_k > kRouteMaxRows || r.num_experts > kRouteMaxExperts ||
+      r.num_experts <= 0 || a.top_k > 64 || a.top_k > r.num_experts || a.block_size != 16 ||
+      r.max_EM < 16 || r.max_EM % 16 != 0 || r.max_EM / 16 > kMaxRuns)
+    return false;
+  FusedMoeArgs b = a;
+  b.EM = r.max_EM;
+  GemmArgs g0 = gateup_args(b);
+  GemmArgs g1 = down_args(b);
+  const StagePlan p0 = plan_stage<0>(g0), p1 = plan_stage<1>(g1);
+  if (p0.variant != kMoeVariantResident || p1.variant != kMoeVariantResident) return false;
+  constexpr size_t kRoutedStaticLds = 6 * 1024;  // the routed form's tables, over the plain form's
+  if (p0.resident_lds + kRoutedStaticLds + 8 * 1024 > 160 * 1024) return false;
+  g0.rt_logits = r.logits;
+  g0.rt_expert_map = r.expert_map;
+  g0.rt_topk_ids = r.topk_ids;
+  g0.rt_topk_w = r.topk_w;
+  g0.rt_sorted_ids = r.sorted_ids;
+  g0.rt_expert_ids = r.expert_ids;
+  g0.rt_out_em = r.out_EM;
+  g0.rt_experts = r.num_experts;
+  g0.rt_local_n = r.local_n;
+  g0.rt_renormalize = r.renormalize;
+  g0.rt_max_em = r.max_EM;
+  g0.sorted_ids = nullptr;
+  g0.expert_ids = nullptr;
+  const bool overwrite = (a.flags & 1u) != 0u;  // VK_HIP_MOE_OVERWRITE_OUT
+  if (overwrite) {
+    g0.zero_out = a.out;
+    g0.zero_count = (long long)a.M * a.hidden;
+  }
+  bool launched = false;
+  if (p0.ksplit && p0.waves == 8 && p0.nt == 2 && p0.depth == 4)
+    launched = launch_resident<0, 8, 2, 4, true, true>(g0, p0.resident_lds, stream);
+  else if (!p0.ksplit && p0.waves == 8 && p0.nt == 2 && p0.depth == 2)
+    launched = launch_resident<0, 8, 2, 2, false, true>(g0, p0.resident_lds, stream);
+  if (!launched) return false;
+  g1.topk_w = r.topk_w;
+  launch_stage<1>(g1, p1, stream);
+  return true;
 }
 
 void launch_moe_gateup(const FusedMoeArgs& a, hipStream_t stream) {

@@ -33,8 +33,8 @@ inline bool operator==(const MoeTile& a, const MoeTile& b) {
 // the tile kernels as one more entry.  The sweep (vkernels_amd/tune_moe.py) times each
 // of these for a stage and a problem size.
 #define VK_RESIDENT_VARIANTS(X) \
-  X(0, 8, 2, 2) X(0, 8, 2, 3) X(0, 8, 2, 4) X(0, 8, 2, 6) X(0, 4, 2, 4) X(0, 4, 2, 8) \
-  X(1, 8, 2, 4) X(1, 8, 2, 2) X(1, 8, 1, 4) X(1, 8, 1, 5) X(1, 8, 1, 6) X(1, 8, 1, 8) X(1, 8, 1, 12)
+  X(0, 8, 2, 2) X(0, 8, 2, 4) X(0, 8, 2, 6) X(0, 4, 2, 4) X(0, 4, 2, 8) \
+  X(1, 8, 2, 4) X(1, 8, 1, 4) X(1, 8, 1, 6) X(1, 8, 1, 8) X(1, 8, 1, 12)
 // ... and of its K-split form (every one is also in the list above: a plan that cannot
 // split K falls back to the same shape there).
 #define VK_KSPLIT_VARIANTS(X) X(0, 8, 2, 4) X(0, 8, 2, 6) X(1, 8, 1, 8) X(1, 8, 2, 4)

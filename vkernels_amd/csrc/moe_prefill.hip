@@ -529,6 +529,7 @@ __global__ __launch_bounds__(64 * kMxWaves) void tile_mx_kernel(MxArgs p) {
   constexpr int kSlotBytes = kMxRows * TERMS * 128;
   typedef __attribute__((address_space(3))) void* lds_ptr;
   extern __shared__ u32x4 mx_lds[];
+  __shared__ int win_flat[kMxRows];  // sorted_ids of the window's rows, asked for before its experts are known
   __shared__ int row_flat[kMxRows];
   __shared__ float row_w[kMxRows];  // stage 1: the routing weight of every row (0 where none is routed)
   __shared__ int seg_hi[2];   // highest routed row index among rows 0..63 / 64..127 (or -1)
@@ -580,31 +581,33 @@ __global__ __launch_bounds__(64 * kMxWaves) void tile_mx_kernel(MxArgs p) {
     const int row0 = __builtin_amdgcn_readfirstlane(row0_);
     const int n_rows = __builtin_amdgcn_readfirstlane(n_rows_);
     const int e = __builtin_amdgcn_readfirstlane(e_);
-    __syncthreads();  // the previous segment is done with row_flat and the ring
+    __syncthreads();  // the previous segment is done with row_flat and the ring (and win_flat is written)
+    // The ids of the segment's rows come from the window's, already in LDS.  What hangs on an
+    // id -- the row's flag of the split and, in the second stage, its routing weight -- is
+    // asked for here and looked at behind the K loop: only the epilogue needs it, and a
+    // round trip to memory in front of the first row copy is a microsecond of every workgroup.
+    int bad_v = 0;
+    float w_v = 0.f;
     if (tid < kMxRows) {
       int f = -1;
       if (tid < n_rows) {
-        f = p.sorted_ids[row0 + tid];
+        f = win_flat[row0 - window * win + tid];
         if (f < 0 || f >= p.n_flat) f = -1;
       }
       row_flat[tid] = f;
-      int bad = 0;
-      if (f >= 0) bad = p.row_bad[STAGE == 0 ? f / p.top_k : row0 + tid];
-      if (STAGE == 1) row_w[tid] = f >= 0 ? p.topk_w[f] : 0.f;  // (in flight together with the flag)
+      if (f >= 0) bad_v = p.row_bad[STAGE == 0 ? f / p.top_k : row0 + tid];
+      if (STAGE == 1 && f >= 0) w_v = p.topk_w[f];
       const unsigned long long routed = __ballot(f >= 0);
-      const unsigned long long any_bad = __ballot(bad != 0);
-      if (lane == 0) {
-        seg_hi[wave] = routed != 0ull ? 63 - (int)__builtin_clzll(routed) : -1;
-        seg_bad[wave] = any_bad != 0ull;
-      }
+      if (lane == 0) seg_hi[wave] = routed != 0ull ? 63 - (int)__builtin_clzll(routed) : -1;
     }
-    __syncthreads();
+    // A barrier for LDS alone: __syncthreads() would also wait for the two loads just
+    // asked for (a workgroup-wide fence makes every memory operation of the wavefront land).
+    __asm__ volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
     const int hi = seg_hi[1] >= 0 ? 64 + seg_hi[1] : seg_hi[0];
     const int n_live = (hi + 32) >> 5;  // row tiles of 32 up to the last routed row
     if (n_live == 0) return;            // uniform
     MX_TRACE(1);
-    const bool slow = (seg_bad[0] | seg_bad[1]) != 0 ||
-                      (has_unit && p.Wflags[(size_t)e * p.units + unit] != 0);  // uniform per wavefront
+    const bool w_slow = has_unit && p.Wflags[(size_t)e * p.units + unit] != 0;  // uniform per wavefront
 
     // ---- row copies: one instruction moves 8 rows x 128 bytes of one term.  Lane
     // (r, c) = (lane / 8, lane % 8) copies piece c ^ r of its row, so LDS position c of
@@ -784,8 +787,14 @@ __global__ __launch_bounds__(64 * kMxWaves) void tile_mx_kernel(MxArgs p) {
     else if (n_live == 2 || TERMS == 1) k_loop(IntC<2>{});
     else if constexpr (TERMS > 1) k_loop(IntC<1>{});
     MX_TRACE(2);
+    if (tid < kMxRows) {  // (wavefronts 0 and 1: whole wavefronts)
+      if (STAGE == 1) row_w[tid] = w_v;
+      const unsigned long long any_bad = __ballot(bad_v != 0);
+      if (lane == 0) seg_bad[wave] = any_bad != 0ull;
+    }
     __syncthreads();
     MX_TRACE(3);
+    const bool slow = (seg_bad[0] | seg_bad[1]) != 0 || w_slow;
 
     if (STAGE == 1 && colg == 0 && tid < n_rows && row_flat[tid] >= 0) p.pos[row_flat[tid]] = row0 + tid;
     if (!has_unit) return;
@@ -968,6 +977,12 @@ __global__ __launch_bounds__(64 * kMxWaves) void tile_mx_kernel(MxArgs p) {
     MX_TRACE(4);
   };
 
+  // The ids of the window's rows, asked for together with its first expert: neither
+  // waits for the other.
+  if (tid < kMxRows) {
+    const int r = window * win + tid;
+    win_flat[tid] = (tid < win && r < win_end) ? p.sorted_ids[r] : -1;
+  }
   int row = window * win;
   while (row < win_end) {  // uniform
     const int e = p.expert_ids[row / p.block_size];

@@ -58,6 +58,22 @@ struct FusedMoeArgs {
 size_t fused_moe_workspace_bytes(int M, int hidden, int ispp, int top_k, int EM);
 
 void launch_fused_moe(const FusedMoeArgs& a, hipStream_t stream);
+
+// Router + alignment + layer in one call (vk_hip_moe_route_layer_mxfp4): what the router
+// and the alignment read and write besides the layer's own arguments.
+struct RoutedArgs {
+  const float* logits;        // [M, num_experts]
+  const int32_t* expert_map;  // or null
+  int32_t* topk_ids;          // [M, top_k] out
+  float* topk_w;              // [M, top_k] out
+  int32_t* sorted_ids;        // [max_EM] out
+  int32_t* expert_ids;        // [max_EM / block_size] out
+  int32_t* out_EM;            // out
+  int num_experts, local_n, renormalize, max_EM;
+};
+// The two-launch form for a handful of tokens; false (nothing enqueued) when the call
+// is not one it takes.
+bool launch_routed_moe(const FusedMoeArgs& a, const RoutedArgs& r, hipStream_t stream);
 void launch_moe_gateup(const FusedMoeArgs& a, hipStream_t stream);
 void launch_moe_down(const FusedMoeArgs& a, hipStream_t stream);
 

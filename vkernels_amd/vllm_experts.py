@@ -309,6 +309,18 @@ def resolve_route_align_fn(lib):
     return fn
 
 
+def resolve_route_layer_fn(lib):
+    """vk_hip_moe_route_layer_mxfp4: router, alignment and the layer behind one call."""
+    try:
+        fn = lib.vk_hip_moe_route_layer_mxfp4
+    except AttributeError:
+        return None
+    fn.restype = _I
+    fn.argtypes = ([_P] * 10 + [_I] * 6 + [_P, _I, _I, _I, _P, _P, _P, _F, _I, _F, _F, _P, _P, _P,
+                                           ctypes.c_size_t, ctypes.c_uint, _P, _P, _I, _P])
+    return fn
+
+
 def resolve_dequant_fn(lib):
     fn = getattr(lib, "vk_hip_dequant_weight_tile", None)
     if fn is None:
@@ -429,6 +441,7 @@ class FusedExperts:
             raise RuntimeError("vk_hip_moe_align_block_size not found in libvkernels_hip.so")
         self.route_fn = resolve_route_fn(self.lib)
         self.route_align_fn = resolve_route_align_fn(self.lib)
+        self.route_layer_fn = resolve_route_layer_fn(self.lib)
         for name, t in (("w13", w13), ("w13_scale", w13_scale), ("w2", w2), ("w2_scale", w2_scale)):
             if t.dtype != torch.uint8 or not t.is_contiguous() or not t.is_cuda:
                 raise ValueError(f"{name} must be a contiguous uint8 device tensor")
@@ -645,7 +658,60 @@ class FusedExperts:
         if int(self.lib.vk_last_error_code()) != VK_OK:
             raise RuntimeError(f"fused MoE call refused: {last_error(self.lib)}")
 
+    def route_layer(self, hidden_states, router_logits, top_k: int, *, renormalize: bool = True,
+                    block_size: int | None = None, max_tokens: int | None = None, out_fp32=None):
+        """Router, alignment and the layer through the library's one call
+        (vk_hip_moe_route_layer_mxfp4: two launches for a handful of tokens, the router's,
+        the alignment's and the layer's otherwise).  Returns (out fp32 [M, H], topk_ids,
+        topk_w, sorted_ids, expert_ids, out_EM, max_EM); `out` is written whatever it held."""
+        torch = self.torch
+        if self.route_layer_fn is None:
+            raise RuntimeError("vk_hip_moe_route_layer_mxfp4 not found in libvkernels_hip.so")
+        M, K = hidden_states.shape
+        if K != self.hidden:
+            raise ValueError(f"hidden size {K} does not match the weights ({self.hidden})")
+        E = router_logits.shape[1]
+        dev = hidden_states.device
+        block_size = default_block_size(M, top_k) if block_size is None else block_size
+        if block_size <= 0 or block_size % 16 != 0:
+            raise ValueError(f"block_size must be a positive multiple of 16, got {block_size}")
+        hidden_states = hidden_states.contiguous()
+        logits = router_logits.contiguous()
+        ids = torch.empty((M, top_k), dtype=torch.int32, device=dev)
+        w = torch.empty((M, top_k), dtype=torch.float32, device=dev)
+        max_em = _align_em_bound(M, top_k, self.local_n, block_size)
+        cap = _align_em_bound(max(M, max_tokens or 0), top_k, self.local_n, block_size)
+        sids = self.scratch.get(("sids", block_size), max_em, dtype=torch.int32, device=dev,
+                                capacity=cap, name="sorted_ids")
+        eids = self.scratch.get(("eids", block_size), max_em // block_size, dtype=torch.int32,
+                                device=dev, capacity=cap // block_size, name="expert_ids")
+        out_em = self.scratch.get("out_em", 1, dtype=torch.int32, device=dev, name="out_em")
+        act = self.scratch.get(("act", self.ispp), max_em * self.ispp, dtype=torch.bfloat16,
+                               device=dev, capacity=cap * self.ispp, name="act_scratch")
+        need = int(self.ws_bytes_fn(M, K, self.ispp, top_k, max_em))
+        cap_bytes = int(self.ws_bytes_fn(max(M, max_tokens or 0), K, self.ispp, top_k, cap))
+        ws = self.scratch.get(("ws", K, self.ispp), need, dtype=torch.uint8, device=dev,
+                              capacity=cap_bytes, name="workspace")
+        if out_fp32 is None:
+            out_fp32 = torch.empty((M, K), dtype=torch.float32, device=dev)
+        flags = MOE_OVERWRITE_OUT
+        if self.w13_packed is not None:
+            flags |= MOE_W4A4 if self.w4a4 else MOE_SPLIT2 if self.split_terms == 2 else \
+                MOE_SPLIT3 if self.split_terms == 3 else 0
+        st = self.route_layer_fn(
+            _ptr(hidden_states), _ptr(logits), _ptr(self.w13), _ptr(self.w13_scale), _ptr(self.w2),
+            _ptr(self.w2_scale), _ptr(ids), _ptr(w), _ptr(act), _ptr(out_fp32), M, E, K, self.ispp, top_k,
+            int(renormalize), _ptr(self.expert_map), self.local_n, block_size, max_em, _ptr(sids), _ptr(eids),
+            _ptr(out_em), float(self.swiglu_limit), self.activation, float(self.beta), float(self.linear_beta),
+            _ptr(self.b13), _ptr(self.b2), _ptr(ws), need, flags, _ptr(self.w13_packed), _ptr(self.w2_packed),
+            self.E, _stream(torch))
+        _check(self.lib, st, "vk_hip_moe_route_layer_mxfp4")
+        return out_fp32, ids, w, sids, eids, out_em, max_em
+
     def forward(self, hidden_states, router_logits, top_k: int, **kw):
         """Router + layer: returns (out fp32 [M, H], topk_ids, topk_w)."""
+        if self.route_layer_fn is not None and self.use_workspace and not kw:
+            out, ids, w = self.route_layer(hidden_states, router_logits, top_k)[:3]
+            return out, ids, w
         ids, w = self.route(router_logits, top_k, True)
         return self.apply(hidden_states, ids, w, **kw), ids, w
