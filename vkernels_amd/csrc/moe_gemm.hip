@@ -396,23 +396,6 @@ __device__ __forceinline__ void split_bf16x8(u32x4 v, uint32_t sb, uint2& hi, ui
 // register file each, K <= 4096.
 __host__ __device__ constexpr int resident_batch(int waves) { return waves == 4 ? 32 : 96 / waves; }
 
-// Profiling build only (-DVK_DECODE_TRACE, `python -m vkernels_amd.build --define
-// VK_DECODE_TRACE --out DIR`; read by vkernels_amd/decode_trace.py): thread 0 of every
-// workgroup stamps the device's 100 MHz clock at the steps of the kernel's start and at
-// its end, for its first pass.  vk_debug_decode_trace copies the stamps of the last
-// launches of both stages out.  The product build compiles none of this.
-#ifdef VK_DECODE_TRACE
-constexpr int kTraceWorkgroups = 1024, kTraceSlots = 12;
-__device__ unsigned long long g_decode_trace[2][kTraceWorkgroups][kTraceSlots];
-#define DECODE_TRACE(slot_)                                                             \
-  do {                                                                                  \
-    if (threadIdx.x == 0 && blockIdx.x < kTraceWorkgroups)                              \
-      g_decode_trace[STAGE][blockIdx.x][slot_] = wall_clock64();                        \
-  } while (0)
-#else
-#define DECODE_TRACE(slot_) do { } while (0)
-#endif
-
 // KSPLIT: the form for a handful of rows (one token), where a workgroup's slice is fewer
 // units than half its wavefronts and a unit, a chain of K / 128 dependent steps with D in
 // flight, is all a wavefront would do while most have nothing.  The slice is taken at most
@@ -446,7 +429,6 @@ __global__ __launch_bounds__(64 * WAVES) void stream_resident_kernel(GemmArgs p)
   __shared__ int slice_sh[2];           // this workgroup's slice of the (run, unit) space
   __shared__ int pass_slow[2];          // set while staging: this pass takes the exact path
   __shared__ int ks_bad[KSPLIT ? WAVES : 1];  // K split: a wavefront's part of its unit left the fast path
-  DECODE_TRACE(0);  // entry
   if (STAGE == 0) clear_out_share<64 * WAVES>(p);
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -659,7 +641,6 @@ __global__ __launch_bounds__(64 * WAVES) void stream_resident_kernel(GemmArgs p)
       listed_weight += tpb > 1 ? __shfl(cum, 63) : (int)__popcll(mr);
     }
     n = n < kMaxRuns ? n : kMaxRuns;
-    DECODE_TRACE(5);  // runs listed
     if (lane == 0) {
       pass_slow[0] = 0;
       pass_slow[1] = 0;
@@ -713,7 +694,6 @@ __global__ __launch_bounds__(64 * WAVES) void stream_resident_kernel(GemmArgs p)
     }
   }
   __syncthreads();
-  DECODE_TRACE(1);  // slice known to every wavefront
   const int s0 = slice_sh[0], s1 = slice_sh[1];  // n_runs * units is far below 2^31
   if (s0 >= s1) return;  // uniform over the workgroup
 
@@ -904,18 +884,7 @@ __global__ __launch_bounds__(64 * WAVES) void stream_resident_kernel(GemmArgs p)
           const uint32_t piece_off = it < my_groups ? (uint32_t)(it * WAVES * 64) : 0u;  // uniform
           return *reinterpret_cast<const u32x4*>(a_base + piece_off + row_off);
         };
-        if (pass_no == 1) DECODE_TRACE(6);  // set-up of the loops done
         u32x4 v[kBatch];
-#ifndef VK_EXP_ORDER
-#define VK_EXP_ORDER 1
-#endif
-#if VK_EXP_ORDER == 0
-#pragma unroll
-        for (int it = 0; it < kBatch; ++it) v[it] = load_piece(it);
-        __builtin_amdgcn_sched_barrier(0);
-        prime();
-        __builtin_amdgcn_sched_barrier(0);
-#else
 #pragma unroll
         for (int it = 0; it < kFirst; ++it) v[it] = load_piece(it);
         __builtin_amdgcn_sched_barrier(0);  // (the order of issue is the point)
@@ -924,8 +893,6 @@ __global__ __launch_bounds__(64 * WAVES) void stream_resident_kernel(GemmArgs p)
 #pragma unroll
         for (int it = kFirst; it < kBatch; ++it) v[it] = load_piece(it);
         __builtin_amdgcn_sched_barrier(0);
-#endif
-        if (pass_no == 1) DECODE_TRACE(7);  // rows and first weight steps asked for
         // Block scale byte of a piece (0 = outside the fast path's range).
         auto block_scale = [&](const u32x4& x) -> uint32_t {
           uint32_t emax = bf16x8_max_exponent(x);
@@ -972,22 +939,15 @@ __global__ __launch_bounds__(64 * WAVES) void stream_resident_kernel(GemmArgs p)
         auto pieces_for = [&](int steps) { return min(n_pieces, (steps * 4 + WAVES - 1) / WAVES); };
 
         __syncthreads();  // the previous pass is done with the planes and with its flag
-        if (pass_no == 1) DECODE_TRACE(8);
         // The rows are staged in K order, a few K steps ahead of the first unit's
         // arithmetic, with a barrier after each portion: the weight stream starts
         // after the first portion and the rest of the splitting overlaps it.
-#ifndef VK_EXP_STAGE_ALL
-#define VK_EXP_STAGE_ALL 0
-#endif
-        write_rows((KSPLIT || VK_EXP_STAGE_ALL) ? n_pieces : pieces_for(min(nsteps, D)));  // (K split: every part starts at once)
-        if (pass_no == 1) DECODE_TRACE(9);  // first K steps split and written
+        write_rows(KSPLIT ? n_pieces : pieces_for(min(nsteps, D)));  // (K split: every part starts at once)
         if (n_my > 0) {
           park_scales();
           if (n_my > 1) fetch_scales(s_unit_stride);
         }
-        if (pass_no == 1) DECODE_TRACE(10);  // scales parked
         __syncthreads();
-        if (pass_no == 1) DECODE_TRACE(3);  // the stream starts
         if (tid == 0) pass_slow[flag ^ 1] = 0;  // for the next pass; its last reader is behind us
 
         f32x4 acc[NT];
@@ -1135,7 +1095,6 @@ __global__ __launch_bounds__(64 * WAVES) void stream_resident_kernel(GemmArgs p)
       }
     }
   }
-  DECODE_TRACE(4);  // end
 }
 
 // Stage 0 with a workspace: 32 consecutive act columns (two 16-column tiles, first
@@ -2325,11 +2284,3 @@ void launch_fused_moe(const FusedMoeArgs& a, hipStream_t stream) {
 }
 
 }  // namespace vk
-
-#ifdef VK_DECODE_TRACE
-// Copies the stamps of the last decode launches to host memory:
-// [2 stages][1024 workgroups][12 stamps] of 64 bits.  Synchronous.
-extern "C" int vk_debug_decode_trace(void* host_buffer) {
-  return (int)hipMemcpyFromSymbol(host_buffer, HIP_SYMBOL(vk::g_decode_trace), sizeof(vk::g_decode_trace));
-}
-#endif

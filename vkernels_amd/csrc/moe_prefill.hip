@@ -92,26 +92,7 @@ struct MxArgs {
   float swiglu_limit, beta, linear_beta;
   int activation;
   int units, col_groups, windows;
-#ifdef VK_MX_TRACE
-  unsigned long long* trace;  // 8 values per workgroup (see MX_TRACE)
-#endif
 };
-
-// Profiling build only (-DVK_MX_TRACE, `python -m vkernels_amd.build --define VK_MX_TRACE
-// --out DIR`): thread 0 of every workgroup stores the 100 MHz clock at a few points of the
-// kernel (0 entry, 1 rows listed, 2 K loop done, 3 barrier passed, 5 first row tile stored,
-// 4 epilogue done; 6, 7 = the hardware ids of its compute unit) into a buffer the caller
-// hands to vk_debug_mx_trace(buffer, stage), 8 values per workgroup;
-// vkernels_amd/mx_trace.py runs a workload on such a build and prints the phases.  Not
-// compiled into the library.
-#ifdef VK_MX_TRACE
-unsigned long long* g_mx_trace = nullptr;
-int g_mx_trace_stage = 1;
-#define MX_TRACE(slot_) \
-  do { if (p.trace != nullptr && threadIdx.x == 0) p.trace[(size_t)blockIdx.x * 8 + (slot_)] = wall_clock64(); } while (0)
-#else
-#define MX_TRACE(slot_) do {} while (0)
-#endif
 
 // ---------------------------------------------------------------------------
 // Prepacking (load time).
@@ -547,13 +528,6 @@ __global__ __launch_bounds__(64 * kMxWaves) void tile_mx_kernel(MxArgs p) {
   const int slot = blockIdx.x >> 3;
   const int logical = ((slot >> 5) * 8 + (blockIdx.x & 7)) * 32 + (slot & 31);
   if (logical >= total) return;
-  MX_TRACE(0);
-#ifdef VK_MX_TRACE
-  if (p.trace != nullptr && threadIdx.x == 0) {
-    p.trace[(size_t)blockIdx.x * 8 + 6] = __builtin_amdgcn_s_getreg((4 << 0) | (0 << 6) | (31 << 11));  // HW_ID
-    p.trace[(size_t)blockIdx.x * 8 + 7] = __builtin_amdgcn_s_getreg((20 << 0) | (0 << 6) | (31 << 11)); // XCC_ID
-  }
-#endif
   const int window = logical / p.col_groups;
   const int colg = logical - window * p.col_groups;
 
@@ -606,7 +580,6 @@ __global__ __launch_bounds__(64 * kMxWaves) void tile_mx_kernel(MxArgs p) {
     const int hi = seg_hi[1] >= 0 ? 64 + seg_hi[1] : seg_hi[0];
     const int n_live = (hi + 32) >> 5;  // row tiles of 32 up to the last routed row
     if (n_live == 0) return;            // uniform
-    MX_TRACE(1);
     const bool w_slow = has_unit && p.Wflags[(size_t)e * p.units + unit] != 0;  // uniform per wavefront
 
     // ---- row copies: one instruction moves 8 rows x 128 bytes of one term.  Lane
@@ -786,14 +759,12 @@ __global__ __launch_bounds__(64 * kMxWaves) void tile_mx_kernel(MxArgs p) {
     else if (n_live == 3) k_loop(IntC<3>{});
     else if (n_live == 2 || TERMS == 1) k_loop(IntC<2>{});
     else if constexpr (TERMS > 1) k_loop(IntC<1>{});
-    MX_TRACE(2);
     if (tid < kMxRows) {  // (wavefronts 0 and 1: whole wavefronts)
       if (STAGE == 1) row_w[tid] = w_v;
       const unsigned long long any_bad = __ballot(bad_v != 0);
       if (lane == 0) seg_bad[wave] = any_bad != 0ull;
     }
     __syncthreads();
-    MX_TRACE(3);
     const bool slow = (seg_bad[0] | seg_bad[1]) != 0 || w_slow;
 
     if (STAGE == 1 && colg == 0 && tid < n_rows && row_flat[tid] >= 0) p.pos[row_flat[tid]] = row0 + tid;
@@ -972,9 +943,7 @@ __global__ __launch_bounds__(64 * kMxWaves) void tile_mx_kernel(MxArgs p) {
           else store_rows(IntC<1>{}, IntC<1>{});
         }
       }
-      if (m == 0) MX_TRACE(5);
     }
-    MX_TRACE(4);
   };
 
   // The ids of the window's rows, asked for together with its first expert: neither
@@ -1014,9 +983,6 @@ void launch_mx_stage_t(MxArgs g, hipStream_t stream) {
   g.windows = (g.num_blocks * g.block_size + win - 1) / win;
   const long long total = (long long)g.col_groups * g.windows;
   const unsigned grid = (unsigned)((total + 255) / 256 * 256);  // whole chunks of 32 tiles for each of 8 XCDs
-#ifdef VK_MX_TRACE
-  g.trace = STAGE == g_mx_trace_stage ? g_mx_trace : nullptr;
-#endif
   hipLaunchKernelGGL((tile_mx_kernel<STAGE, TERMS>), dim3(grid), dim3(64 * kMxWaves),
                      kMxRing * kMxRows * TERMS * 128, stream, g);
 }
@@ -1225,12 +1191,5 @@ void launch_mxfp4_quant(const uint16_t* A, const int32_t* sorted_ids, uint8_t* p
   hipLaunchKernelGGL(mxfp4_quant_kernel, dim3(rows), dim3(256), 0, stream, A, sorted_ids, packed, scales,
                      hidden, top_k, n_flat);
 }
-
-#ifdef VK_MX_TRACE
-extern "C" void vk_debug_mx_trace(void* buffer, int stage) {
-  g_mx_trace = static_cast<unsigned long long*>(buffer);
-  g_mx_trace_stage = stage;
-}
-#endif
 
 }  // namespace vk
