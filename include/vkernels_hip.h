@@ -473,6 +473,31 @@ int vk_hip_moe_combine(const float* partial, const float* b2, const float* topk_
                        size_t workspace_bytes, void* stream);
 
 /*
+ * Additive: the two GEMM stages of the split above on prepacked weights, so that a
+ * tensor-parallel caller at prefill sizes runs the FP4-rate kernels as the fused call
+ * does.  w13_packed / w2_packed: vk_hip_moe_prepack_weights of the rank's shard
+ * (K = hidden_k / ispp_k) of num_experts experts; the raw shard is still read where a
+ * unit or a row leaves the fast path's range.  workspace:
+ * vk_hip_moe_preact_workspace_bytes(stage, M, EM, k_dim) bytes, 16-byte aligned (the
+ * split rows of the K slice).  flags: VK_HIP_MOE_SPLIT2 / _SPLIT3 as for the layer
+ * (default: three FP6 terms per activation in the first stage, two in the second).
+ * Calls of up to 512 routed rows, or without packed weights or workspace, run as
+ * vk_hip_moe_gateup_preact / vk_hip_moe_down_preact do.  Same outputs, same rules:
+ * routed rows only are written.
+ */
+size_t vk_hip_moe_preact_workspace_bytes(int stage, int M, int EM, int k_dim);
+int vk_hip_moe_gateup_preact_prepacked(const uint16_t* A, const uint8_t* w13, const uint8_t* w13_scale,
+                                       const void* w13_packed, int num_experts, const int32_t* sorted_ids,
+                                       const int32_t* expert_ids, float* gate_up, int M, int hidden, int ispp,
+                                       int top_k, int EM, int k_base, int hidden_k, int block_size,
+                                       void* workspace, size_t workspace_bytes, unsigned flags, void* stream);
+int vk_hip_moe_down_preact_prepacked(const uint16_t* act, const uint8_t* w2, const uint8_t* w2_scale,
+                                     const void* w2_packed, int num_experts, const int32_t* sorted_ids,
+                                     const int32_t* expert_ids, float* partial, int M, int ispp, int hidden,
+                                     int top_k, int EM, int k_base, int ispp_k, int block_size, void* workspace,
+                                     size_t workspace_bytes, unsigned flags, void* stream);
+
+/*
  * On-device alignment of the routing table: stable bucket of the flat indices
  * by (local) expert, each expert padded to a multiple of block_size.
  * Replaces vk_hip_moe_align_block_size,

@@ -212,3 +212,127 @@ def test_tensor_parallel_composition(hip_lib, name, T, bs, tp):
     max_rel, rel_l2, nf = error_metrics(out.cpu().numpy(), c_out)
     print(f"{name} T={T} tp={tp}: max_abs/rms={max_rel:.3e} rel_l2={rel_l2:.3e}")
     assert nf and max_rel <= EXACT_SPLIT_MAX_ABS_TOL and rel_l2 <= EXACT_SPLIT_REL_L2_TOL
+
+
+# ---- the same GEMM stages on prepacked weights (prefill-sized calls) -------------------------
+
+def _prepacked_fns(lib):
+    _fns(lib)
+    lib.vk_hip_moe_preact_workspace_bytes.restype = ctypes.c_size_t
+    lib.vk_hip_moe_preact_workspace_bytes.argtypes = [_I] * 4
+    for name in ("vk_hip_moe_gateup_preact_prepacked", "vk_hip_moe_down_preact_prepacked"):
+        fn = getattr(lib, name)
+        fn.restype = _I
+        fn.argtypes = [_P] * 4 + [_I] + [_P] * 3 + [_I] * 8 + [_P, ctypes.c_size_t, ctypes.c_uint, _P]
+    return lib
+
+
+def _prepack(lib, w, ws, stage):
+    size_fn, pack_fn, _ = ve.resolve_prepack_fns(lib)
+    E, rows, kb = w.shape
+    n = int(size_fn(E, rows, kb * 2, stage))
+    buf = torch.empty(n, dtype=torch.uint8, device=dev())
+    assert pack_fn(w.data_ptr(), ws.data_ptr(), E, rows, kb * 2, stage, buf.data_ptr(), n, None) == 0
+    return buf
+
+
+# three FP6 terms represent a bf16 activation to 2^-13 of its block's largest: the sums then
+# differ from the oracle's like the exact-split paths'; two terms (the second stage's
+# default) leave 2^-10 of the block's largest per element
+PREPACKED3_MAX_TOL, PREPACKED3_L2_TOL = 2e-3, 2e-4
+PREPACKED2_MAX_TOL, PREPACKED2_L2_TOL = 2e-2, 2e-3
+
+
+@pytest.mark.parametrize("name,T,bs,tp", [("c1", 300, 128, 1), ("c1", 600, 128, 2), ("c4", 255, 64, 3)])
+def test_prepacked_stages_against_the_oracle_and_in_composition(hip_lib, name, T, bs, tp):
+    """vk_hip_moe_gateup_preact_prepacked / _down_preact_prepacked: every rank's K slice of the
+    weights prepacked as its own shard, the A / act slice addressed inside the full rows; each
+    stage against the oracle's function of the same name on the same slice (rows that are not
+    routed left as they were), and the composition (slices summed, epilogues once) against
+    the fused oracle."""
+    lib = _prepacked_fns(hip_lib)
+    cfg = synth.CONFIGS[name]
+    H, I, k = cfg.H, cfg.I, cfg.top_k
+    w, A, ids, tw, (s16, e16, em16), (sids, eids, em) = _case(cfg, T, 7500 + T, bs)
+    wn = w.numpy()
+    n_flat = T * k
+    p16, p = _rows_map(s16, sids, n_flat)
+    pad = np.setdiff1d(np.arange(em), p)
+    rng = np.random.default_rng(T + 2)
+    b13 = (rng.standard_normal((cfg.E, 2 * I)) * 0.5).astype(np.float32)
+    b2 = (rng.standard_normal((cfg.E, H)) * 0.5).astype(np.float32)
+
+    def slices(width):
+        units = width // 64
+        cuts = [64 * (units * r // tp) for r in range(tp + 1)]
+        return [(cuts[r], cuts[r + 1] - cuts[r]) for r in range(tp) if cuts[r + 1] > cuts[r]]
+
+    d_A, d_sids, d_eids = to_dev(A), to_dev(sids), to_dev(eids)
+    gu = torch.zeros((em, 2 * I), dtype=torch.float32, device=dev())
+    for k_base, k_dim in slices(H):
+        d_w = to_dev(np.ascontiguousarray(wn[0][:, :, k_base // 2:(k_base + k_dim) // 2]))
+        d_s = to_dev(np.ascontiguousarray(wn[1][:, :, k_base // 32:(k_base + k_dim) // 32]))
+        packed = _prepack(lib, d_w, d_s, 0)
+        need = int(lib.vk_hip_moe_preact_workspace_bytes(0, T, em, k_dim))
+        ws = torch.empty(need, dtype=torch.uint8, device=dev())
+        part = torch.full((em, 2 * I), 7.0, dtype=torch.float32, device=dev())
+        assert lib.vk_hip_moe_gateup_preact_prepacked(
+            d_A.data_ptr(), d_w.data_ptr(), d_s.data_ptr(), packed.data_ptr(), cfg.E, d_sids.data_ptr(),
+            d_eids.data_ptr(), part.data_ptr(), T, H, I, k, em, k_base, k_dim, bs, ws.data_ptr(), need, 0,
+            None) == 0, ve.last_error(lib)
+        torch.cuda.synchronize()
+        c_part = oracle.moe_gateup(A, wn[0][:, :, k_base // 2:(k_base + k_dim) // 2],
+                                   wn[1][:, :, k_base // 32:(k_base + k_dim) // 32], s16, e16, T, H, k_base, k_dim,
+                                   I, k, em16)
+        g_part = part.cpu().numpy()
+        m, l2 = _rms_metrics(g_part[p], c_part[p16])
+        print(f"{name} T={T} slice {k_base}+{k_dim}: gate_up max/rms {m:.2e} rel_l2 {l2:.2e}")
+        assert m <= PREPACKED3_MAX_TOL and l2 <= PREPACKED3_L2_TOL
+        assert np.all(g_part[pad] == 7.0)                      # rows that are not routed are left alone
+        part[to_dev(pad.astype(np.int64))] = 0.0
+        gu += part                                              # the caller's all-reduce
+    d_b13, d_b2 = to_dev(b13), to_dev(b2)
+    act = torch.zeros((em, I), dtype=torch.int16, device=dev())
+    assert lib.vk_hip_moe_act_epilogue(gu.data_ptr(), d_b13.data_ptr(), act.data_ptr(), d_sids.data_ptr(),
+                                       d_eids.data_ptr(), T, k, em, I, 0.0, 0, 4.0, 25.0, bs, None) == 0
+    torch.cuda.synchronize()
+    act_np = act.cpu().numpy().view(np.uint16)
+    act16 = np.zeros((em16, I), np.uint16)
+    act16[p16] = act_np[p]
+    partial = torch.zeros((em, H), dtype=torch.float32, device=dev())
+    for k_base, k_dim in slices(I):
+        d_w = to_dev(np.ascontiguousarray(wn[2][:, :, k_base // 2:(k_base + k_dim) // 2]))
+        d_s = to_dev(np.ascontiguousarray(wn[3][:, :, k_base // 32:(k_base + k_dim) // 32]))
+        packed = _prepack(lib, d_w, d_s, 1)
+        need = int(lib.vk_hip_moe_preact_workspace_bytes(1, T, em, k_dim))
+        ws = torch.empty(need, dtype=torch.uint8, device=dev())
+        for flags, (mtol, ltol) in ((ve.MOE_SPLIT3, (PREPACKED3_MAX_TOL, PREPACKED3_L2_TOL)),
+                                    (0, (PREPACKED2_MAX_TOL, PREPACKED2_L2_TOL))):
+            part = torch.full((em, H), -3.0, dtype=torch.float32, device=dev())
+            assert lib.vk_hip_moe_down_preact_prepacked(
+                act.data_ptr(), d_w.data_ptr(), d_s.data_ptr(), packed.data_ptr(), cfg.E, d_sids.data_ptr(),
+                d_eids.data_ptr(), part.data_ptr(), T, I, H, k, em, k_base, k_dim, bs, ws.data_ptr(), need, flags,
+                None) == 0, ve.last_error(lib)
+            torch.cuda.synchronize()
+            c_part = oracle.moe_down(act16, wn[2][:, :, k_base // 2:(k_base + k_dim) // 2],
+                                     wn[3][:, :, k_base // 32:(k_base + k_dim) // 32], s16, e16, T, I, k_base, k_dim,
+                                     H, k, em16)
+            g_part = part.cpu().numpy()
+            m, l2 = _rms_metrics(g_part[p], c_part[p16])
+            print(f"{name} T={T} slice {k_base}+{k_dim} flags {flags}: partial max/rms {m:.2e} rel_l2 {l2:.2e}")
+            assert m <= mtol and l2 <= ltol
+            assert np.all(g_part[pad] == -3.0)
+        part[to_dev(pad.astype(np.int64))] = 0.0
+        partial += part                                         # (the default arithmetic's)
+    out = torch.zeros((T, H), dtype=torch.float32, device=dev())
+    wsi = torch.zeros(n_flat, dtype=torch.int32, device=dev())
+    d_tws = to_dev(oracle.gather_sorted_weights(tw, sids))
+    assert lib.vk_hip_moe_combine(partial.data_ptr(), d_b2.data_ptr(), d_tws.data_ptr(), d_sids.data_ptr(),
+                                  d_eids.data_ptr(), out.data_ptr(), T, H, k, em, bs, wsi.data_ptr(),
+                                  wsi.numel() * 4, None) == 0
+    torch.cuda.synchronize()
+    tws16 = oracle.gather_sorted_weights(tw, s16)
+    c_out, _ = oracle.fused_moe_mxfp4(A, *wn, s16, tws16, e16, T, H, I, k, em16, b13=b13, b2=b2)
+    max_rel, rel_l2, nf = error_metrics(out.cpu().numpy(), c_out)
+    print(f"{name} T={T} tp={tp} on prepacked shards: max_abs/rms={max_rel:.3e} rel_l2={rel_l2:.3e}")
+    assert nf and max_rel <= 8e-3 and rel_l2 <= 1e-3     # the bounds of the layer's default arithmetic

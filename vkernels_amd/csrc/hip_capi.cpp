@@ -380,6 +380,62 @@ int vk_hip_moe_gateup_preact(const uint16_t* A, const uint8_t* w13, const uint8_
   return stage_launch_status("vk_hip_moe_gateup_preact", before);
 }
 
+size_t vk_hip_moe_preact_workspace_bytes(int stage, int M, int EM, int k_dim) {
+  return vk::mx_preact_workspace_bytes(stage, M, EM, k_dim);
+}
+
+namespace {
+
+// The pre-activation GEMM of a stage, on prepacked weights where the call is one the
+// FP4-rate kernels take (more routed rows than the decode kernels', a workspace), on the
+// raw weights otherwise.
+int preact_any(const char* who, int stage, const uint16_t* a, const uint8_t* w, const uint8_t* w_scale,
+               const void* packed, int num_experts, const int32_t* sorted_ids, const int32_t* expert_ids,
+               float* preact, int M, int width_a, int ncols, int top_k, int EM, int k_base, int k_dim,
+               int block_size, void* workspace, size_t workspace_bytes, unsigned flags, void* stream) {
+  if (const char* why = stage_shape_error(M, width_a, ncols, top_k, EM, k_base, k_dim, block_size))
+    return fail(VK_ERROR_INVALID_ARGUMENT, (std::string(who) + ": " + why).c_str());
+  if (M == 0 || EM == 0) return VK_OK;
+  if (a == nullptr || w == nullptr || w_scale == nullptr || sorted_ids == nullptr || expert_ids == nullptr ||
+      preact == nullptr)
+    return fail(VK_ERROR_INVALID_ARGUMENT, (std::string(who) + ": buffers must not be null").c_str());
+  if (packed != nullptr && num_experts <= 0)
+    return fail(VK_ERROR_INVALID_ARGUMENT, (std::string(who) + ": num_experts must be positive with packed weights").c_str());
+  vk_set_last_error(VK_OK, "");
+  const hipError_t before = hipPeekAtLastError();
+  const bool prefill_sized = (long long)M * top_k > vk::kMoeDecodeMaxRows;
+  if (!(packed != nullptr && prefill_sized &&
+        vk::launch_moe_preact_prepacked(stage, a, static_cast<const uint8_t*>(packed), w, w_scale, sorted_ids,
+                                        expert_ids, preact, M, width_a, ncols, top_k, EM, k_base, k_dim,
+                                        block_size, num_experts, workspace, workspace_bytes, flags,
+                                        static_cast<hipStream_t>(stream))))
+    vk::launch_moe_preact(stage, a, w, w_scale, sorted_ids, expert_ids, preact, M, width_a, ncols, top_k, EM,
+                          k_base, k_dim, block_size, static_cast<hipStream_t>(stream));
+  return stage_launch_status(who, before);
+}
+
+}  // namespace
+
+int vk_hip_moe_gateup_preact_prepacked(const uint16_t* A, const uint8_t* w13, const uint8_t* w13_scale,
+                                       const void* w13_packed, int num_experts, const int32_t* sorted_ids,
+                                       const int32_t* expert_ids, float* gate_up, int M, int hidden, int ispp,
+                                       int top_k, int EM, int k_base, int hidden_k, int block_size,
+                                       void* workspace, size_t workspace_bytes, unsigned flags, void* stream) {
+  return preact_any("vk_hip_moe_gateup_preact_prepacked", 0, A, w13, w13_scale, w13_packed, num_experts,
+                    sorted_ids, expert_ids, gate_up, M, hidden, ispp, top_k, EM, k_base, hidden_k, block_size,
+                    workspace, workspace_bytes, flags, stream);
+}
+
+int vk_hip_moe_down_preact_prepacked(const uint16_t* act, const uint8_t* w2, const uint8_t* w2_scale,
+                                     const void* w2_packed, int num_experts, const int32_t* sorted_ids,
+                                     const int32_t* expert_ids, float* partial, int M, int ispp, int hidden,
+                                     int top_k, int EM, int k_base, int ispp_k, int block_size, void* workspace,
+                                     size_t workspace_bytes, unsigned flags, void* stream) {
+  return preact_any("vk_hip_moe_down_preact_prepacked", 1, act, w2, w2_scale, w2_packed, num_experts, sorted_ids,
+                    expert_ids, partial, M, ispp, hidden, top_k, EM, k_base, ispp_k, block_size, workspace,
+                    workspace_bytes, flags, stream);
+}
+
 int vk_hip_moe_act_epilogue(const float* gate_up, const float* b13, uint16_t* act,
                             const int32_t* sorted_ids, const int32_t* expert_ids, int M, int top_k,
                             int EM, int ispp, float swiglu_limit, int activation, float beta,

@@ -88,6 +88,8 @@ struct MxArgs {
   uint16_t* act;           // stage 0 output [EM, ncols]
   float* y;                // stage 1 output [EM, ncols]
   int32_t* pos;            // stage 1: pos[flat] = sorted row
+  float* preact;           // PREACT: the linear part alone, fp32 rows of 2 ncols (stage 0) / ncols (stage 1)
+  int a_stride;            // elements between the bf16 rows of A (K, or the full width of a K slice)
   int n_flat, top_k, K, ncols, num_blocks, block_size;
   float swiglu_limit, beta, linear_beta;
   int activation;
@@ -190,7 +192,7 @@ template <int TERMS>
 __global__ __launch_bounds__(256) void split_rows_fp6_kernel(const uint16_t* __restrict__ x,
                                                              uint8_t* __restrict__ xq,
                                                              uint8_t* __restrict__ row_bad, int K,
-                                                             int rows,
+                                                             int x_stride, int rows,
                                                              const int32_t* __restrict__ sorted_ids,
                                                              int n_flat, int32_t* __restrict__ fill,
                                                              int fill_n) {
@@ -216,7 +218,7 @@ __global__ __launch_bounds__(256) void split_rows_fp6_kernel(const uint16_t* __r
 #pragma unroll
     for (int i = 0; i < 4; ++i) in.q[i] = u32x4{0u, 0u, 0u, 0u};
     if (b * 32 < K) {
-      const u32x4* src = reinterpret_cast<const u32x4*>(x + row * (size_t)K + (size_t)b * 32);
+      const u32x4* src = reinterpret_cast<const u32x4*>(x + row * (size_t)x_stride + (size_t)b * 32);
 #pragma unroll
       for (int i = 0; i < 4; ++i) in.q[i] = src[i];
     }
@@ -504,7 +506,10 @@ __device__ __forceinline__ f32x16 mfma_fp4_act(u32x4 w, i32x8 b, f32x16 acc, uin
                                                            (int)wscale, 0, b[6]);
 }
 
-template <int STAGE, int TERMS>
+// PREACT: the stage's linear part alone (tensor-parallel callers sum it over their K slices
+// before the epilogue): the accumulators of the routed rows go to p.preact as fp32, no
+// bias, no activation, no routing weight; rows that are not routed are left as they are.
+template <int STAGE, int TERMS, bool PREACT = false>
 __global__ __launch_bounds__(64 * kMxWaves) void tile_mx_kernel(MxArgs p) {
   constexpr int R = kMxRing;
   constexpr int kSlotBytes = kMxRows * TERMS * 128;
@@ -570,7 +575,7 @@ __global__ __launch_bounds__(64 * kMxWaves) void tile_mx_kernel(MxArgs p) {
       }
       row_flat[tid] = f;
       if (f >= 0) bad_v = p.row_bad[STAGE == 0 ? f / p.top_k : row0 + tid];
-      if (STAGE == 1 && f >= 0) w_v = p.topk_w[f];
+      if (STAGE == 1 && !PREACT && f >= 0) w_v = p.topk_w[f];
       const unsigned long long routed = __ballot(f >= 0);
       if (lane == 0) seg_hi[wave] = routed != 0ull ? 63 - (int)__builtin_clzll(routed) : -1;
     }
@@ -760,14 +765,14 @@ __global__ __launch_bounds__(64 * kMxWaves) void tile_mx_kernel(MxArgs p) {
     else if (n_live == 2 || TERMS == 1) k_loop(IntC<2>{});
     else if constexpr (TERMS > 1) k_loop(IntC<1>{});
     if (tid < kMxRows) {  // (wavefronts 0 and 1: whole wavefronts)
-      if (STAGE == 1) row_w[tid] = w_v;
+      if (STAGE == 1 && !PREACT) row_w[tid] = w_v;
       const unsigned long long any_bad = __ballot(bad_v != 0);
       if (lane == 0) seg_bad[wave] = any_bad != 0ull;
     }
     __syncthreads();
     const bool slow = (seg_bad[0] | seg_bad[1]) != 0 || w_slow;
 
-    if (STAGE == 1 && colg == 0 && tid < n_rows && row_flat[tid] >= 0) p.pos[row_flat[tid]] = row0 + tid;
+    if (STAGE == 1 && !PREACT && colg == 0 && tid < n_rows && row_flat[tid] >= 0) p.pos[row_flat[tid]] = row0 + tid;
     if (!has_unit) return;
 
     // ---- epilogue: lane (ln, hh) holds, of activation row 32 m + ln, the weight rows
@@ -783,7 +788,7 @@ __global__ __launch_bounds__(64 * kMxWaves) void tile_mx_kernel(MxArgs p) {
     // The biases of the columns this lane holds (the same for every row tile), tile by
     // tile as the accumulators are laid out: asked for here, all at once, not value by
     // value inside the loops below.
-    const bool has_bias = p.bias != nullptr;  // uniform
+    const bool has_bias = !PREACT && p.bias != nullptr;  // uniform
     f32x4 bias_v[4][4];  // [tile][row group]
     if (has_bias) {
       // stage 0: tiles 0, 1 = gate columns, 2, 3 = the same columns of up
@@ -798,7 +803,7 @@ __global__ __launch_bounds__(64 * kMxWaves) void tile_mx_kernel(MxArgs p) {
 #pragma unroll
         for (int rg = 0; rg < 4; ++rg) bias_v[t][rg] = *reinterpret_cast<const f32x4u*>(b + c + rg * 8);
       }
-    } else if (STAGE == 0 && p.activation == 1) {  // the one loop that adds them without a bias
+    } else if (STAGE == 0 && !PREACT && p.activation == 1) {  // the one loop that adds them without a bias
 #pragma unroll
       for (int i = 0; i < 16; ++i) bias_v[i >> 2][i & 3] = f32x4{0.f, 0.f, 0.f, 0.f};
     }
@@ -815,11 +820,43 @@ __global__ __launch_bounds__(64 * kMxWaves) void tile_mx_kernel(MxArgs p) {
         if (flat >= 0) {
           const size_t grow = (size_t)(STAGE == 0 ? flat / p.top_k : srow);
           if (TERMS == 1) q_row = p.Aq + grow * (size_t)Kp;
-          else a_row = p.A + grow * (size_t)K;
+          else a_row = p.A + grow * (size_t)p.a_stride;
         }
         exact_unit_mx<STAGE>(p, e, unit, a_row, q_row, lane, tile);
       }
-      if (STAGE == 0) {
+      if constexpr (PREACT) {
+        // the accumulators as they are: 64 columns (two tiles) at a time through the
+        // wavefront's staging area, whole lines out, routed rows only
+        constexpr int kPitch = kMxYPitch;
+        const int width = STAGE == 0 ? 2 * p.ncols : p.ncols;
+#pragma unroll
+        for (int tp = 0; tp < 2; ++tp) {
+          // stage 0: tiles 0, 1 = gate columns of the unit, 2, 3 = the same columns of up
+          const int col0 = STAGE == 0 ? tp * p.ncols + unit * 64 : unit * kMxUnitRows + tp * 64;
+          if (STAGE == 1 && col0 >= p.ncols) break;  // uniform: the last unit may be ragged
+#pragma unroll
+          for (int tl = 0; tl < 2; ++tl)
+#pragma unroll
+            for (int rg = 0; rg < 4; ++rg) {
+              const int t = 2 * tp + tl;
+              const int cl = tl * 32 + rg * 8 + hh * 4;
+              *reinterpret_cast<f32x4*>(stage_lds + ln * kPitch + cl * 4) =
+                  f32x4{tile[t][rg * 4], tile[t][rg * 4 + 1], tile[t][rg * 4 + 2], tile[t][rg * 4 + 3]};
+            }
+          wave_fence();
+          f32x4 v[8];
+#pragma unroll
+          for (int pass = 0; pass < 8; ++pass)
+            v[pass] = *reinterpret_cast<const f32x4*>(stage_lds + (pass * 4 + (lane >> 4)) * kPitch + (lane & 15) * 16);
+          wave_fence();
+          float* dst = p.preact + (size_t)(row0 + m * 32 + (lane >> 4)) * (size_t)width + col0 + (lane & 15) * 4;
+#pragma unroll
+          for (int pass = 0; pass < 8; ++pass) {
+            if ((routed >> (pass * 4 + (lane >> 4))) & 1ull) *reinterpret_cast<f32x4*>(dst) = v[pass];
+            dst += 4 * (size_t)width;
+          }
+        }
+      } else if (STAGE == 0) {
         constexpr int kPitch = kMxActPitch;
         // 128 activation values per lane and row tile.  A wavefront runs alone on its SIMD,
         // so a branch per value (bias or not, clamp or not, which activation) is paid in
@@ -963,11 +1000,11 @@ __global__ __launch_bounds__(64 * kMxWaves) void tile_mx_kernel(MxArgs p) {
   }
 }
 
-template <int STAGE, int TERMS>
+template <int STAGE, int TERMS, bool PREACT = false>
 bool mx_kernel_ready() {
   static const bool configured = [] {
     const hipError_t err = hipFuncSetAttribute(
-        reinterpret_cast<const void*>(tile_mx_kernel<STAGE, TERMS>),
+        reinterpret_cast<const void*>(tile_mx_kernel<STAGE, TERMS, PREACT>),
         hipFuncAttributeMaxDynamicSharedMemorySize, kMxRing * kMxRows * TERMS * 128);
     if (err != hipSuccess) (void)hipGetLastError();  // not left for the next caller to find
     return err == hipSuccess;
@@ -975,7 +1012,7 @@ bool mx_kernel_ready() {
   return configured;
 }
 
-template <int STAGE, int TERMS>
+template <int STAGE, int TERMS, bool PREACT = false>
 void launch_mx_stage_t(MxArgs g, hipStream_t stream) {
   const int win = mx_window_rows(g.block_size);
   g.units = mx_units(STAGE, g.ncols);
@@ -983,7 +1020,7 @@ void launch_mx_stage_t(MxArgs g, hipStream_t stream) {
   g.windows = (g.num_blocks * g.block_size + win - 1) / win;
   const long long total = (long long)g.col_groups * g.windows;
   const unsigned grid = (unsigned)((total + 255) / 256 * 256);  // whole chunks of 32 tiles for each of 8 XCDs
-  hipLaunchKernelGGL((tile_mx_kernel<STAGE, TERMS>), dim3(grid), dim3(64 * kMxWaves),
+  hipLaunchKernelGGL((tile_mx_kernel<STAGE, TERMS, PREACT>), dim3(grid), dim3(64 * kMxWaves),
                      kMxRing * kMxRows * TERMS * 128, stream, g);
 }
 
@@ -1006,6 +1043,7 @@ MxArgs mx_args(const FusedMoeArgs& a, int stage) {
   } else {
     g.A = a.act; g.W = a.w2; g.Ws = a.w2_scale; g.bias = a.b2; g.K = a.ispp; g.ncols = a.hidden;
   }
+  g.a_stride = g.K;
   return g;
 }
 
@@ -1061,7 +1099,9 @@ size_t mx_workspace_bytes(int M, int hidden, int ispp, int top_k, int EM) {
 
 bool prepare_mx_kernels() {
   return mx_kernel_ready<0, 1>() && mx_kernel_ready<0, 2>() && mx_kernel_ready<0, 3>() &&
-         mx_kernel_ready<1, 1>() && mx_kernel_ready<1, 2>() && mx_kernel_ready<1, 3>();
+         mx_kernel_ready<1, 1>() && mx_kernel_ready<1, 2>() && mx_kernel_ready<1, 3>() &&
+         mx_kernel_ready<0, 2, true>() && mx_kernel_ready<0, 3, true>() && mx_kernel_ready<1, 2, true>() &&
+         mx_kernel_ready<1, 3, true>();
 }
 
 namespace {
@@ -1129,10 +1169,10 @@ void mx_stage0(const FusedMoeArgs& a, const MxPlan& pl, hipStream_t stream) {
     hipLaunchKernelGGL(quant_rows_w4_kernel, dim3(a.M), dim3(256), 0, stream, a.A, pl.aq, pl.abad, a.hidden, nullptr, 0, nullptr, 0);
     launch_mx_stage_t<0, 1>(pl.g0, stream);
   } else if (pl.terms0 == 2) {
-    hipLaunchKernelGGL(split_rows_fp6_kernel<2>, split_grid(a.M, a.hidden), dim3(256), 0, stream, a.A, pl.aq, pl.abad, a.hidden, a.M, nullptr, 0, nullptr, 0);
+    hipLaunchKernelGGL(split_rows_fp6_kernel<2>, split_grid(a.M, a.hidden), dim3(256), 0, stream, a.A, pl.aq, pl.abad, a.hidden, a.hidden, a.M, nullptr, 0, nullptr, 0);
     launch_mx_stage_t<0, 2>(pl.g0, stream);
   } else {
-    hipLaunchKernelGGL(split_rows_fp6_kernel<3>, split_grid(a.M, a.hidden), dim3(256), 0, stream, a.A, pl.aq, pl.abad, a.hidden, a.M, nullptr, 0, nullptr, 0);
+    hipLaunchKernelGGL(split_rows_fp6_kernel<3>, split_grid(a.M, a.hidden), dim3(256), 0, stream, a.A, pl.aq, pl.abad, a.hidden, a.hidden, a.M, nullptr, 0, nullptr, 0);
     launch_mx_stage_t<0, 3>(pl.g0, stream);
   }
 }
@@ -1144,10 +1184,10 @@ void mx_stage1(const FusedMoeArgs& a, const MxPlan& pl, hipStream_t stream) {
     hipLaunchKernelGGL(quant_rows_w4_kernel, dim3(a.EM), dim3(256), 0, stream, a.act, pl.cq, pl.cbad, a.ispp, a.sorted_ids, a.M * a.top_k, pl.pos, a.M * a.top_k);
     launch_mx_stage_t<1, 1>(pl.g1, stream);
   } else if (pl.terms1 == 2) {
-    hipLaunchKernelGGL(split_rows_fp6_kernel<2>, split_grid(a.EM, a.ispp), dim3(256), 0, stream, a.act, pl.cq, pl.cbad, a.ispp, a.EM, a.sorted_ids, a.M * a.top_k, pl.pos, a.M * a.top_k);
+    hipLaunchKernelGGL(split_rows_fp6_kernel<2>, split_grid(a.EM, a.ispp), dim3(256), 0, stream, a.act, pl.cq, pl.cbad, a.ispp, a.ispp, a.EM, a.sorted_ids, a.M * a.top_k, pl.pos, a.M * a.top_k);
     launch_mx_stage_t<1, 2>(pl.g1, stream);
   } else {
-    hipLaunchKernelGGL(split_rows_fp6_kernel<3>, split_grid(a.EM, a.ispp), dim3(256), 0, stream, a.act, pl.cq, pl.cbad, a.ispp, a.EM, a.sorted_ids, a.M * a.top_k, pl.pos, a.M * a.top_k);
+    hipLaunchKernelGGL(split_rows_fp6_kernel<3>, split_grid(a.EM, a.ispp), dim3(256), 0, stream, a.act, pl.cq, pl.cbad, a.ispp, a.ispp, a.EM, a.sorted_ids, a.M * a.top_k, pl.pos, a.M * a.top_k);
     launch_mx_stage_t<1, 3>(pl.g1, stream);
   }
   launch_combine(pl.y, pl.pos, a.out, a.M, a.top_k, a.hidden, (a.flags & 1u) != 0u, stream);
@@ -1173,14 +1213,83 @@ bool launch_moe_down_prepacked(const FusedMoeArgs& a, hipStream_t stream) {
   return true;
 }
 
+// ---- the linear part of a stage on prepacked weights (tensor-parallel stage split) ----
+// Workspace: split rows of the K slice [rows, 3 Kp(k_dim)] and a flag byte per row;
+// rows = M (stage 0: the rows of A) or EM (stage 1: the sorted rows of act).
+size_t mx_preact_workspace_bytes(int stage, int M, int EM, int k_dim) {
+  if (M <= 0 || EM <= 0 || k_dim <= 0) return 0;
+  const size_t rows = stage == 0 ? (size_t)M : (size_t)EM;
+  return align256(rows * 3 * (size_t)mx_kp(k_dim)) + align256(rows);
+}
+
+// False (nothing enqueued) when the path does not take the call: workspace short or
+// misaligned, split rows beyond 32-bit offsets, LDS refused.
+bool launch_moe_preact_prepacked(int stage, const uint16_t* a, const uint8_t* packed, const uint8_t* w,
+                                 const uint8_t* w_scale, const int32_t* sorted_ids, const int32_t* expert_ids,
+                                 float* preact, int M, int a_stride, int ncols, int top_k, int EM, int k_base,
+                                 int k_dim, int block_size, int num_experts, void* workspace,
+                                 size_t workspace_bytes, unsigned flags, hipStream_t stream) {
+  if (M <= 0 || EM <= 0 || block_size <= 0 || packed == nullptr || workspace == nullptr) return false;
+  if (workspace_bytes < mx_preact_workspace_bytes(stage, M, EM, k_dim) ||
+      (reinterpret_cast<uintptr_t>(workspace) & 15) != 0)
+    return false;
+  const size_t rows = stage == 0 ? (size_t)M : (size_t)EM;
+  if ((unsigned long long)rows * 3ull * mx_kp(k_dim) >= (1ull << 32)) return false;
+  // terms as in the layer: three in the first stage, two in the second unless its sums are
+  // short; VK_HIP_MOE_SPLIT2 / _SPLIT3: that many
+  int terms = stage == 0 ? 3 : (k_dim < kMxShortK ? 3 : 2);
+  if ((flags & 2u) != 0u) terms = 2;
+  else if ((flags & 8u) != 0u) terms = 3;
+  const bool ready = stage == 0 ? (terms == 2 ? mx_kernel_ready<0, 2, true>() : mx_kernel_ready<0, 3, true>())
+                                : (terms == 2 ? mx_kernel_ready<1, 2, true>() : mx_kernel_ready<1, 3, true>());
+  if (!ready) return false;
+  uint8_t* xq = static_cast<uint8_t*>(workspace);
+  uint8_t* xbad = xq + align256(rows * 3 * (size_t)mx_kp(k_dim));
+  MxArgs g{};
+  g.sorted_ids = sorted_ids;
+  g.expert_ids = expert_ids;
+  g.n_flat = M * top_k;
+  g.top_k = top_k;
+  g.num_blocks = EM / block_size;
+  g.block_size = block_size;
+  g.A = a + k_base;
+  g.a_stride = a_stride;
+  g.W = w;
+  g.Ws = w_scale;
+  g.K = k_dim;
+  g.ncols = ncols;
+  g.preact = preact;
+  g.Aq = xq;
+  g.row_bad = xbad;
+  const int units = mx_units(stage, ncols);
+  g.Wp = packed;
+  g.Wflags = packed + mx_packed_body_bytes(num_experts, units, mx_kp(k_dim) / 128);
+  const int32_t* ids = stage == 0 ? nullptr : sorted_ids;  // stage 1: the routed rows of the sorted order only
+  const int n_flat = stage == 0 ? 0 : M * top_k;
+  if (terms == 2)
+    hipLaunchKernelGGL(split_rows_fp6_kernel<2>, split_grid((int)rows, k_dim), dim3(256), 0, stream, a + k_base, xq,
+                       xbad, k_dim, a_stride, (int)rows, ids, n_flat, nullptr, 0);
+  else
+    hipLaunchKernelGGL(split_rows_fp6_kernel<3>, split_grid((int)rows, k_dim), dim3(256), 0, stream, a + k_base, xq,
+                       xbad, k_dim, a_stride, (int)rows, ids, n_flat, nullptr, 0);
+  if (stage == 0) {
+    if (terms == 2) launch_mx_stage_t<0, 2, true>(g, stream);
+    else launch_mx_stage_t<0, 3, true>(g, stream);
+  } else {
+    if (terms == 2) launch_mx_stage_t<1, 2, true>(g, stream);
+    else launch_mx_stage_t<1, 3, true>(g, stream);
+  }
+  return true;
+}
+
 // Test hook: the split rows of bf16 rows [rows, K] as the GEMM kernels read them.
 void launch_split_rows_fp6(const uint16_t* x, int rows, int K, int terms, uint8_t* xq, uint8_t* row_bad,
                            hipStream_t stream) {
   if (rows <= 0) return;
   if (terms == 2)
-    hipLaunchKernelGGL(split_rows_fp6_kernel<2>, split_grid(rows, K), dim3(256), 0, stream, x, xq, row_bad, K, rows, nullptr, 0, nullptr, 0);
+    hipLaunchKernelGGL(split_rows_fp6_kernel<2>, split_grid(rows, K), dim3(256), 0, stream, x, xq, row_bad, K, K, rows, nullptr, 0, nullptr, 0);
   else
-    hipLaunchKernelGGL(split_rows_fp6_kernel<3>, split_grid(rows, K), dim3(256), 0, stream, x, xq, row_bad, K, rows, nullptr, 0, nullptr, 0);
+    hipLaunchKernelGGL(split_rows_fp6_kernel<3>, split_grid(rows, K), dim3(256), 0, stream, x, xq, row_bad, K, K, rows, nullptr, 0, nullptr, 0);
 }
 
 // ---- MXFP4 orchestration ops (device counterparts of moe_aux.cpp) -----------------

@@ -103,6 +103,14 @@ void launch_moe_preact(int stage, const uint16_t* a, const uint8_t* w, const uin
                        const int32_t* sorted_ids, const int32_t* expert_ids, float* preact, int M,
                        int a_stride, int ncols, int top_k, int EM, int k_base, int k_dim, int block_size,
                        hipStream_t stream);
+// The same on prepacked weights (the FP4-rate kernels of moe_prefill.hip; `packed` from
+// launch_moe_prepack for the shard [num_experts, rows, k_dim / 2]); false = nothing enqueued.
+size_t mx_preact_workspace_bytes(int stage, int M, int EM, int k_dim);
+bool launch_moe_preact_prepacked(int stage, const uint16_t* a, const uint8_t* packed, const uint8_t* w,
+                                 const uint8_t* w_scale, const int32_t* sorted_ids, const int32_t* expert_ids,
+                                 float* preact, int M, int a_stride, int ncols, int top_k, int EM, int k_base,
+                                 int k_dim, int block_size, int num_experts, void* workspace,
+                                 size_t workspace_bytes, unsigned flags, hipStream_t stream);
 void launch_moe_act_epilogue(const float* gate_up, const float* b13, uint16_t* act,
                              const int32_t* sorted_ids, const int32_t* expert_ids, int M, int top_k, int EM,
                              int ispp, int block_size, float swiglu_limit, int activation, float beta,
