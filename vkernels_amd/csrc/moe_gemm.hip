@@ -413,6 +413,15 @@ __host__ __device__ constexpr int resident_batch(int waves) { return waves == 4 
 // sorted_ids, expert_ids and EM out, exactly as vk_hip_moe_route_align leaves them.
 constexpr int kRouteMaxRows = 128, kRouteMaxExperts = 256, kRoutePer = kRouteMaxExperts / 64;
 
+// A workgroup barrier for LDS alone.  __syncthreads() is a workgroup-wide fence as well,
+// which makes a wavefront wait for every global load it has in flight (s_waitcnt vmcnt(0)):
+// in the decode kernel that is the weight stream and the rest of the rows, asked for on
+// purpose before the barrier.  Only LDS is shared across these barriers; registers that
+// global loads fill are waited for where they are used.
+__device__ __forceinline__ void lds_barrier() {
+  __asm__ volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+}
+
 template <int STAGE, int WAVES, int NT, int D, bool KSPLIT = false, bool ROUTE = false>
 __global__ __launch_bounds__(64 * WAVES) void stream_resident_kernel(GemmArgs p) {
   static_assert(!ROUTE || STAGE == 0, "the routed form is the first stage's");
@@ -693,7 +702,7 @@ __global__ __launch_bounds__(64 * WAVES) void stream_resident_kernel(GemmArgs p)
       slice_sh[1] = t1;
     }
   }
-  __syncthreads();
+  lds_barrier();
   const int s0 = slice_sh[0], s1 = slice_sh[1];  // n_runs * units is far below 2^31
   if (s0 >= s1) return;  // uniform over the workgroup
 
@@ -938,7 +947,7 @@ __global__ __launch_bounds__(64 * WAVES) void stream_resident_kernel(GemmArgs p)
         // pieces every wavefront must have written before K steps [0, steps) can run
         auto pieces_for = [&](int steps) { return min(n_pieces, (steps * 4 + WAVES - 1) / WAVES); };
 
-        __syncthreads();  // the previous pass is done with the planes and with its flag
+        lds_barrier();  // the previous pass is done with the planes and with its flag
         // The rows are staged in K order, a few K steps ahead of the first unit's
         // arithmetic, with a barrier after each portion: the weight stream starts
         // after the first portion and the rest of the splitting overlaps it.
@@ -947,7 +956,7 @@ __global__ __launch_bounds__(64 * WAVES) void stream_resident_kernel(GemmArgs p)
           park_scales();
           if (n_my > 1) fetch_scales(s_unit_stride);
         }
-        __syncthreads();
+        lds_barrier();
         if (tid == 0) pass_slow[flag ^ 1] = 0;  // for the next pass; its last reader is behind us
 
         f32x4 acc[NT];
@@ -1031,7 +1040,7 @@ __global__ __launch_bounds__(64 * WAVES) void stream_resident_kernel(GemmArgs p)
             // no stream here: finish the staging in step with the other wavefronts
             for (int f0 = D; staged < n_pieces; f0 += D) {
               write_rows(pieces_for(min(nsteps, f0 + D)));
-              __syncthreads();
+              lds_barrier();
             }
             continue;
           }
@@ -1041,7 +1050,7 @@ __global__ __launch_bounds__(64 * WAVES) void stream_resident_kernel(GemmArgs p)
           for (int f0 = 0; f0 < total_steps; f0 += D) {
             if (f0 > 0 && staged < n_pieces) {  // uniform, and the same in every wavefront
               write_rows(pieces_for(min(nsteps, f0 + D)));
-              __syncthreads();
+              lds_barrier();
             }
 #pragma unroll
             for (int i = 0; i < D; ++i) {
