@@ -58,6 +58,10 @@ def parse_args():
                     help="FP6 terms per activation on the prepacked path: 0 = the library's default "
                          "(3 in the first stage, 2 in the second), 2 or 3 = that many in both")
     ap.add_argument("--no-prepack", action="store_true", help="raw weights only, also for prefill sizes")
+    ap.add_argument("--packed-only", action="store_true",
+                    help="one copy of the weights: prepack at every size and let go of the raw tensors "
+                         "(decode sizes then run the decode kernels' packed instantiations; the "
+                         "`roofline` of such a record is over the fused call, both stages)")
     ap.add_argument("--no-workspace", action="store_true",
                     help="call the reference's own symbol (no workspace, raw weights)")
     ap.add_argument("--no-modes", action="store_true",
@@ -163,7 +167,8 @@ def run_workload(args, workload, steps, warmup, prepack, split_terms=None, w4a4=
     dev = torch.device("cuda", 0)
     H, I, k = cfg.H, cfg.I, cfg.top_k
     prefill = T * k > 512  # the library's own split between its decode and tile kernels
-    prepack = prepack and prefill and not args.no_workspace
+    packed_only = args.packed_only and prepack and not args.no_workspace
+    prepack = prepack and (prefill or packed_only) and not args.no_workspace
     terms = args.split_terms if split_terms is None else split_terms   # 0 = the library's default
 
     per_set = synth.algorithmic_bytes(H, I, cfg.E, k, 0, cfg.E)
@@ -183,7 +188,10 @@ def run_workload(args, workload, steps, warmup, prepack, split_terms=None, w4a4=
     for s in range(n_sets):
         w = synth.make_weights(cfg.E, H, I, seed + 7919 * s, device=dev)
         experts.append(ve.FusedExperts(w.w13, w.w13_scale, w.w2, w.w2_scale, prepack=prepack,
-                                       split_terms=terms or None, w4a4=w4a4 and prepack, **epi))
+                                       split_terms=terms or None, w4a4=w4a4 and prepack,
+                                       keep_raw=not packed_only, **epi))
+        if packed_only:
+            del w
         if args.no_workspace:
             experts[-1].use_workspace = False
     A_bits = synth.make_activations(T, H, seed)
@@ -211,7 +219,7 @@ def run_workload(args, workload, steps, warmup, prepack, split_terms=None, w4a4=
         # same launches, with events around the two GEMM stages (decode) or around
         # the fused call (prefill-sized batches, which run with a workspace)
         sids, eids, _, max_em = fe.align(ids, bs)
-        if prefill:
+        if prefill or packed_only:
             events[0].record()
             events[1].record()
             if args.no_workspace:
@@ -315,6 +323,15 @@ def run_workload(args, workload, steps, warmup, prepack, split_terms=None, w4a4=
             "flops_per_launch": flops, "avg_launch_us": down_avg * 1e3,
             "median_launch_us": down_ms[len(down_ms) // 2] * 1e3,
         }
+    elif packed_only:
+        achieved = (gate_bytes + down_bytes) / (down_avg * 1e-3) / 1e9
+        roofline = {
+            "bound": "hbm", "kernel": "vk_hip_fused_moe_mxfp4_prepacked without raw weights (stream_resident_kernel<0, "
+                                      "..., PACKED> + stream_resident_kernel<1, ..., PACKED>)",
+            "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
+            "traffic": None, "bytes_per_launch": gate_bytes + down_bytes, "avg_launch_us": down_avg * 1e3,
+            "median_launch_us": down_ms[len(down_ms) // 2] * 1e3,
+        }
     else:
         achieved = gate_bytes / (gate_avg * 1e-3) / 1e9
         roofline = {
@@ -335,7 +352,8 @@ def run_workload(args, workload, steps, warmup, prepack, split_terms=None, w4a4=
             "workload": f"{cfg.name} T={T}: hidden {H}, intermediate {I}, {cfg.E} experts, "
                         f"top-{k}, MXFP4 weights, bf16 activations, {cfg.logits} routing",
             "block_size": bs, "active_experts": active, "weight_sets": n_sets,
-            "weights": "prepacked at load time (+ raw)" if prepack else "raw",
+            "weights": "prepacked at load time, raw tensors let go of" if packed_only
+                       else "prepacked at load time (+ raw)" if prepack else "raw",
             "epilogue": args.epilogue,
         },
         "roofline": roofline,
@@ -343,8 +361,8 @@ def run_workload(args, workload, steps, warmup, prepack, split_terms=None, w4a4=
             "algorithmic_bytes": layer_bytes, "algorithmic_flops": flops,
             "hbm_frac_whole_step": layer_bytes / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS,
             "fp4_mfma_frac_whole_step": flops / (ms_per_step * 1e-3) / 1e12 / FP4_PEAK_TFLOPS,
-            "down_kernel_avg_us": None if prefill else down_avg * 1e3,
-            "down_kernel_gbs": None if prefill else down_bytes / (down_avg * 1e-3) / 1e9,
+            "down_kernel_avg_us": None if prefill or packed_only else down_avg * 1e3,
+            "down_kernel_gbs": None if prefill or packed_only else down_bytes / (down_avg * 1e-3) / 1e9,
         },
     }
     if prepack:

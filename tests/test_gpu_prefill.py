@@ -37,7 +37,9 @@ MODEL_MAX_ABS_TOL = 5e-3
 # ---- the prepacked layout ---------------------------------------------------------
 
 def _prepack_reference(w, ws, stage):
-    """numpy restatement of the packed layout documented in include/vkernels_hip.h."""
+    """numpy restatement of the packed layout documented in include/vkernels_hip.h: a flagged
+    unit holds the codes and scale bytes as they are, any other the codes on the OCP points
+    and the scale bytes less one."""
     E, rows, kb = w.shape
     K = kb * 2
     ncols = rows // 2 if stage == 0 else rows
@@ -48,8 +50,12 @@ def _prepack_reference(w, ws, stage):
     lo, hi = w & 15, w >> 4
     remap = lambda c: c + np.where((c & 6) != 0, 2, 0).astype(np.uint8)
     nonfinite = ((lo & 6) == 6) | ((hi & 6) == 6)
+    bad_row = nonfinite.any(axis=2) | (ws < 64).any(axis=2) | (ws > 190).any(axis=2)
     for e in range(E):
         for u in range(units):
+            rows_u = [(t >> 1) * ncols + u * 64 + (t & 1) * 32 + n if stage == 0 else u * 128 + t * 32 + n
+                      for t in range(4) for n in range(32)]
+            raw = any(r < rows and bad_row[e, r] for r in rows_u)
             for t in range(4):
                 for n in range(32):
                     row = (t >> 1) * ncols + u * 64 + (t & 1) * 32 + n if stage == 0 else u * 128 + t * 32 + n
@@ -67,10 +73,10 @@ def _prepack_reference(w, ws, stage):
                             sc_view[lane, half, t] = 127
                             continue
                         piece = w[e, row, g * 16:(g + 1) * 16]
-                        packed = remap(piece & 15) | (remap(piece >> 4) << 4)
+                        packed = piece if raw else remap(piece & 15) | (remap(piece >> 4) << 4)
                         off = ((half * 4 + t) * 64 + lane) * 16
                         out[e, u, ks, off:off + 16] = packed
-                        sc_view[lane, half, t] = (int(ws[e, row, g]) - 1) & 0xFF
+                        sc_view[lane, half, t] = int(ws[e, row, g]) if raw else (int(ws[e, row, g]) - 1) & 0xFF
     return out, flags
 
 
@@ -94,9 +100,8 @@ def test_prepack_layout_bitwise(hip_lib, stage, rows, K):
     ref, flags = _prepack_reference(w, ws, stage)
     got = buf.cpu().numpy()
     body = ref.size
-    flagged = np.repeat(flags.ravel().astype(bool), ref.shape[2] * 8704)
-    # flagged units are never read in packed form; the others must match byte for byte
-    assert np.array_equal(got[:body][~flagged], ref.ravel()[~flagged])
+    # byte for byte, the flagged units (raw codes and scale bytes for the exact paths) included
+    assert np.array_equal(got[:body], ref.ravel())
     f_off = (body + 255) // 256 * 256
     assert np.array_equal(got[f_off:f_off + flags.size], flags.ravel())
     assert flags.sum() == 3
@@ -184,15 +189,18 @@ def _down_ex(lib):
     return fn
 
 
-@pytest.mark.parametrize("path", ["packed", "packed3", "packed2", "workspace", "plain", "resident"])
+@pytest.mark.parametrize("path", ["packed", "packed3", "packed2", "workspace", "plain", "resident",
+                                  "packed_alone", "resident_packed_alone"])
 def test_onehot_rows_read_back_the_dequantised_weights(hip_lib, path):
     """act rows with a single 1.0 at column k, routing weight 1: out[t, :] is column k of
     the expert's dequantised W2, so every value the GEMM multiplies by is compared with the
     oracle bit for bit.  Expert 0: the 12 finite codes with scale bytes 64, 65, 127, 189,
     190 (the scaled-MFMA path); expert 1: all 16 codes and scale bytes 0, 1, 63, 191, 200,
-    255 (flagged: the exact path)."""
+    255 (flagged: the exact path).  The paths "..._alone" pass the prepacked form and no raw
+    tensors: the flagged units' raw codes and scale bytes are then read from it."""
     E, H = 2, 192
-    I = 256 if path == "resident" else 576
+    alone = path.endswith("_alone")
+    I = 256 if path.startswith("resident") else 576
     M = E * I
     rng = np.random.default_rng(11)
     fin = np.array(synth.FINITE_CODES, dtype=np.uint8)
@@ -210,8 +218,9 @@ def test_onehot_rows_read_back_the_dequantised_weights(hip_lib, path):
     w2s[1] = np.array([0, 1, 63, 191, 200, 255], dtype=np.uint8)[rng.integers(0, 6, (H, I // 32))]
     ids = (np.arange(M) // I).astype(np.int32).reshape(M, 1)
     fe = ve.FusedExperts(to_dev(np.zeros((E, 2 * I, H // 2), np.uint8)), to_dev(np.zeros((E, 2 * I, H // 32), np.uint8)),
-                         to_dev(w2), to_dev(w2s), scratch=ve.CaptureSafeScratch(), prepack=path.startswith("packed"))
-    bs = 16 if path == "resident" else 128
+                         to_dev(w2), to_dev(w2s), scratch=ve.CaptureSafeScratch(),
+                         prepack=path.startswith("packed") or alone, keep_raw=not alone)
+    bs = 16 if path.startswith("resident") else 128
     sids, eids, out_em, max_em = fe.align(to_dev(ids), bs)
     torch.cuda.synchronize()
     s_np = sids.cpu().numpy()
@@ -222,12 +231,13 @@ def test_onehot_rows_read_back_the_dequantised_weights(hip_lib, path):
     tw = torch.ones((M, 1), dtype=torch.float32, device=dev())
     out = torch.full((M, H), float("nan"), dtype=torch.float32, device=dev())
     ws, need = None, 0
-    if path != "plain" and path != "resident":
+    if path != "plain" and not path.startswith("resident"):
         need = int(fe.ws_bytes_fn(M, H, I, 1, max_em))
         ws = torch.empty(need, dtype=torch.uint8, device=dev())
     flags = ve.MOE_OVERWRITE_OUT | (ve.MOE_SPLIT2 if path == "packed2" else ve.MOE_SPLIT3 if path == "packed3" else 0)
     hip_lib.vk_set_last_error(0, b"")
-    _down_ex(hip_lib)(d_act.data_ptr(), fe.w2.data_ptr(), fe.w2_scale.data_ptr(), tw.data_ptr(),
+    _down_ex(hip_lib)(d_act.data_ptr(), None if alone else fe.w2.data_ptr(),
+                      None if alone else fe.w2_scale.data_ptr(), tw.data_ptr(),
                       out.data_ptr(), M, H, I, 1, sids.data_ptr(), eids.data_ptr(), max_em, None, bs,
                       None if ws is None else ws.data_ptr(), need, flags,
                       None if fe.w2_packed is None else fe.w2_packed.data_ptr(), E, None)
@@ -253,7 +263,8 @@ def _bf16_order(bits):
     return np.where(b & 0x8000, -(b & 0x7FFF), b & 0x7FFF)
 
 
-@pytest.mark.parametrize("path", ["packed", "packed3", "packed2", "workspace", "plain", "resident"])
+@pytest.mark.parametrize("path", ["packed", "packed3", "packed2", "workspace", "plain", "resident",
+                                  "packed_alone", "resident_packed_alone"])
 def test_onehot_rows_through_the_first_stage(hip_lib, path):
     """A rows with a single 1.0 at column k: the gate and up sums of sorted row r are single
     exact products, W13[e, c, k] and W13[e, I + c, k], so act[r, c] = bf16(silu(g) u) pins
@@ -267,7 +278,8 @@ def test_onehot_rows_through_the_first_stage(hip_lib, path):
     in the last place of the oracle's everywhere, and bit-equal in at least 99 % of the
     values."""
     E, I = 2, 192
-    H = 256 if path == "resident" else 576
+    alone = path.endswith("_alone")
+    H = 256 if path.startswith("resident") else 576
     M = E * H
     rng = np.random.default_rng(23)
     fin = np.array(synth.FINITE_CODES, dtype=np.uint8)
@@ -289,12 +301,12 @@ def test_onehot_rows_through_the_first_stage(hip_lib, path):
     ids = (np.arange(M) // H).astype(np.int32).reshape(M, 1)
     A = np.zeros((M, H), dtype=np.uint16)
     A[np.arange(M), np.arange(M) % H] = 0x3F80                        # 1.0
-    kw = dict(prepack=path.startswith("packed"))
+    kw = dict(prepack=path.startswith("packed") or alone, keep_raw=not alone)
     if path in ("packed2", "packed3"):
         kw["split_terms"] = int(path[-1])
     fe = ve.FusedExperts(to_dev(w13), to_dev(w13s), to_dev(w2), to_dev(w2s), scratch=ve.CaptureSafeScratch(), **kw)
     fe.use_workspace = path not in ("plain", "resident")
-    bs = 16 if path == "resident" else 128
+    bs = 16 if path.startswith("resident") else 128
     d_ids = to_dev(ids)
     sids, eids, out_em, max_em = fe.align(d_ids, bs)
     fe.apply(to_dev(A, torch.bfloat16), d_ids, None, block_size=bs)

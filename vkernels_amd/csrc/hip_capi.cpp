@@ -55,13 +55,25 @@ namespace {
 // Shared contract check of the three layer entry points.  They return void
 // like the reference's launcher; a violation is recorded for vk_last_error()
 // and nothing is launched.
-bool layer_args_ok(const char* who, bool need13, bool need2, const vk::FusedMoeArgs& a) {
+// A call that passes the prepacked weights in place of the raw tensors (all four null).
+bool packed_weights_alone(const void* w13, const void* w13_scale, const void* w2, const void* w2_scale,
+                          const void* w13_packed, const void* w2_packed) {
+  return w13 == nullptr && w13_scale == nullptr && w2 == nullptr && w2_scale == nullptr &&
+         w13_packed != nullptr && w2_packed != nullptr;
+}
+const char* const kPackedOnlyNeeds =
+    "a call without the raw weights needs shapes the decode kernels take or, beyond them, the "
+    "workspace of vk_hip_fused_moe_mxfp4_workspace_bytes (16-byte aligned)";
+
+// packed_only: the call passes the prepacked weights in place of the raw tensors.
+bool layer_args_ok(const char* who, bool need13, bool need2, const vk::FusedMoeArgs& a,
+                   bool packed_only = false) {
   const char* why = nullptr;
   if (a.sorted_ids == nullptr || a.expert_ids == nullptr || a.act == nullptr)
     why = "buffers must not be null";
-  else if (need13 && (a.A == nullptr || a.w13 == nullptr || a.w13_scale == nullptr))
+  else if (need13 && (a.A == nullptr || (!packed_only && (a.w13 == nullptr || a.w13_scale == nullptr))))
     why = "buffers must not be null";
-  else if (need2 && (a.w2 == nullptr || a.w2_scale == nullptr || a.topk_w == nullptr ||
+  else if (need2 && ((!packed_only && (a.w2 == nullptr || a.w2_scale == nullptr)) || a.topk_w == nullptr ||
                      a.out == nullptr))
     why = "buffers must not be null";
   else if (a.hidden <= 0 || a.ispp <= 0 || a.hidden % 64 != 0 || a.ispp % 64 != 0)
@@ -191,7 +203,8 @@ void vk_hip_fused_moe_mxfp4_prepacked(
       fused_args(A, w13, w13_scale, w2, w2_scale, topk_w, act_scratch, out, M, hidden, ispp,
                  top_k, sorted_ids, expert_ids, EM, swiglu_limit, activation, beta, linear_beta,
                  b13, b2, block_size, workspace, workspace_bytes, flags);
-  if (!layer_args_ok("vk_hip_fused_moe_mxfp4_prepacked", true, true, a)) return;
+  const bool packed_only = packed_weights_alone(w13, w13_scale, w2, w2_scale, w13_packed, w2_packed);
+  if (!layer_args_ok("vk_hip_fused_moe_mxfp4_prepacked", true, true, a, packed_only)) return;
   if ((w13_packed == nullptr) != (w2_packed == nullptr) || (w13_packed != nullptr && num_experts <= 0)) {
     vk_set_last_error(VK_ERROR_INVALID_ARGUMENT,
                       "vk_hip_fused_moe_mxfp4_prepacked: both packed buffers (or neither) and a "
@@ -201,6 +214,10 @@ void vk_hip_fused_moe_mxfp4_prepacked(
   a.w13_packed = static_cast<const uint8_t*>(w13_packed);
   a.w2_packed = static_cast<const uint8_t*>(w2_packed);
   a.num_experts = num_experts;
+  if (packed_only && !vk::fused_moe_packed_only_ok(a)) {
+    vk_set_last_error(VK_ERROR_INVALID_ARGUMENT, kPackedOnlyNeeds);
+    return;
+  }
   const hipError_t before = hipPeekAtLastError();
   vk::launch_fused_moe(a, static_cast<hipStream_t>(stream));
   note_launch_error("vk_hip_fused_moe_mxfp4_prepacked", before);
@@ -222,10 +239,15 @@ void vk_hip_moe_down_mxfp4_ex(
   a.workspace = workspace; a.workspace_bytes = workspace_bytes; a.flags = flags;
   a.w2_packed = static_cast<const uint8_t*>(w2_packed);
   a.num_experts = num_experts;
-  if (!layer_args_ok("vk_hip_moe_down_mxfp4_ex", false, true, a)) return;
+  const bool packed_only = w2 == nullptr && w2_scale == nullptr && w2_packed != nullptr;
+  if (!layer_args_ok("vk_hip_moe_down_mxfp4_ex", false, true, a, packed_only)) return;
   if (w2_packed != nullptr && num_experts <= 0) {
     vk_set_last_error(VK_ERROR_INVALID_ARGUMENT,
                       "vk_hip_moe_down_mxfp4_ex: num_experts must be positive with packed weights");
+    return;
+  }
+  if (packed_only && !vk::moe_down_packed_only_ok(a)) {
+    vk_set_last_error(VK_ERROR_INVALID_ARGUMENT, kPackedOnlyNeeds);
     return;
   }
   const hipError_t before = hipPeekAtLastError();
@@ -756,7 +778,8 @@ int vk_hip_moe_route_layer_mxfp4(
                  block_size, workspace, workspace_bytes, flags);
   if (max_EM <= 0 || block_size <= 0 || max_EM % block_size != 0)
     return fail(VK_ERROR_INVALID_ARGUMENT, "vk_hip_moe_route_layer_mxfp4: block_size must divide max_EM");
-  if (!layer_args_ok("vk_hip_moe_route_layer_mxfp4", true, true, a)) return VK_ERROR_INVALID_ARGUMENT;
+  const bool packed_only = packed_weights_alone(w13, w13_scale, w2, w2_scale, w13_packed, w2_packed);
+  if (!layer_args_ok("vk_hip_moe_route_layer_mxfp4", true, true, a, packed_only)) return VK_ERROR_INVALID_ARGUMENT;
   if (logits == nullptr || topk_ids == nullptr || out_EM == nullptr)
     return fail(VK_ERROR_INVALID_ARGUMENT, "vk_hip_moe_route_layer_mxfp4: logits/topk_ids/out_EM must not be null");
   if ((w13_packed == nullptr) != (w2_packed == nullptr) || (w13_packed != nullptr && num_local_experts <= 0))
@@ -766,6 +789,7 @@ int vk_hip_moe_route_layer_mxfp4(
   a.w13_packed = static_cast<const uint8_t*>(w13_packed);
   a.w2_packed = static_cast<const uint8_t*>(w2_packed);
   a.num_experts = num_local_experts;
+  if (packed_only && !vk::fused_moe_packed_only_ok(a)) return fail(VK_ERROR_INVALID_ARGUMENT, kPackedOnlyNeeds);
   if (num_experts > 0 && top_k <= num_experts && local_n >= 0 && local_n <= num_experts) {
     vk::RoutedArgs r{};
     r.logits = logits; r.expert_map = expert_map; r.topk_ids = topk_ids; r.topk_w = topk_w;

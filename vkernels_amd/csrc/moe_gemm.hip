@@ -43,6 +43,7 @@
 
 #include "moe_common.hpp"
 #include "moe_heuristics.hpp"
+#include "moe_prefill_layout.hpp"
 #include "moe_route.hpp"
 #include "moe_tuning.hpp"
 #include "mxfp4.hpp"
@@ -56,6 +57,12 @@ struct GemmArgs {
   const uint16_t* A;        // stage 0: activations [M, K]; stage 1: act [EM, K]
   const uint8_t* W;         // [E, rows_w, K/2]
   const uint8_t* Ws;        // [E, rows_w, K/32]
+  // The same weights in the prepacked form (moe_prefill_layout.hpp), for the decode
+  // kernels' packed instantiations, which read nothing of W / Ws: the blocks, the flag
+  // byte of every (expert, packed unit), packed units per expert.
+  const uint8_t* Wp;
+  const uint8_t* Wpf;
+  int p_units;
   const int32_t* sorted_ids;
   const int32_t* expert_ids;
   const float* topk_w;      // stage 1
@@ -217,6 +224,51 @@ __device__ __forceinline__ void unit_tiles(const GemmArgs& p, int e, int unit, i
   }
 }
 
+// The same for the prepacked form.  A decode tile (16 weight rows from row c of the gate,
+// up or down matrix, c a multiple of 16) lies inside one 32-row tile of one packed unit:
+// unit c / 64 (gate / up: tiles 0, 1 / 2, 3 of it) or c / 128 (down), rows c % 32 .. + 15
+// of tile (c % 64) / 32 resp. (c % 128) / 32.  Lane (ln, lq) takes K block lq of row ln of
+// the step: half lq / 2, lane (lq % 2, c % 32 + ln) of the packed tile.  w_rows / s_rows
+// point at that lane's 16 code bytes and at the four scale bytes of its half (the tile's
+// is byte shift / 8 of them) in the unit's first K step; every further step is
+// kMxStepBytes on.  pu = the packed unit (the same for all tiles of a decode unit).
+template <int STAGE, int NT>
+__device__ __forceinline__ void unit_tiles_packed(const GemmArgs& p, int e, int unit, int lane, int nsteps,
+                                                  const uint8_t* (&w_rows)[NT],
+                                                  const uint8_t* (&s_rows)[NT], int (&shift)[NT],
+                                                  int (&col0)[NT], int& pu) {
+  static_assert(NT <= 2, "a decode unit lies inside one packed unit");
+  const int ln = lane & 15, lq = lane >> 4;
+#pragma unroll
+  for (int t = 0; t < NT; ++t) {
+    int c, ptile;
+    if (STAGE == 0) {
+      const int half = t / (NT / 2), tt = t % (NT / 2);
+      col0[t] = unit * (8 * NT) + tt * 16;
+      c = col0[t];
+      pu = c >> 6;
+      ptile = half * 2 + ((c & 63) >> 5);
+    } else {
+      col0[t] = unit * (16 * NT) + t * 16;
+      c = col0[t];
+      pu = c >> 7;
+      ptile = (c & 127) >> 5;
+    }
+    const int ln32 = (c & 31) + ln;
+    const uint8_t* ub = p.Wp + mx_unit_offset(e, p.p_units, pu, nsteps);
+    w_rows[t] = ub + (lq >> 1) * 4096 + ptile * 1024 + (lq & 1) * 512 + ln32 * 16;
+    s_rows[t] = ub + 8192 + ((lq & 1) * 32 + ln32) * 8 + (lq >> 1) * 4;
+    shift[t] = 8 * ptile;
+  }
+}
+
+// Flag byte of a packed unit (1 = it holds a code or a scale byte the fast path does not
+// take, and its codes and scale bytes are the raw tensors').  The index is uniform.
+__device__ __forceinline__ bool packed_unit_flagged(const GemmArgs& p, int e, int pu) {
+  const int idx = __builtin_amdgcn_readfirstlane(e * p.p_units + pu);
+  return p.Wpf[idx] != 0;
+}
+
 // ---------------------------------------------------------------------------
 // Decode kernel ("resident"): one workgroup per compute unit, the activation
 // rows of a run resident in LDS for the whole K dimension, no barrier inside
@@ -308,6 +360,12 @@ __device__ __forceinline__ i32x8 fp4_operand(u32x4 w) {
   return __builtin_shufflevector(y, y, 0, 1, 2, 3, -1, -1, -1, -1);
 }
 
+// The same for codes that are on the OCP code points already (the prepacked form).
+__device__ __forceinline__ i32x8 fp4_operand_packed(u32x4 w) {
+  const i32x4 y = {(int)w[0], (int)w[1], (int)w[2], (int)w[3]};
+  return __builtin_shufflevector(y, y, 0, 1, 2, 3, -1, -1, -1, -1);
+}
+
 // First item of part `i` when `total` items are cut into `parts` contiguous
 // slices whose sizes differ by at most one.
 __device__ __forceinline__ int slice_begin(int total, int i, int parts) {
@@ -353,6 +411,44 @@ __device__ __forceinline__ void exact_unit_global(const uint8_t* const (&w_rows)
         if (ok) {
           x = *reinterpret_cast<const uint32_t*>(w_rows[t] + (size_t)g * 16 + d * 4);
           sc = s_rows[t][g];
+        }
+        acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(dequant8_exact(x, sc)),
+                                                         as_bf16x8(av), acc[t], 0, 0, 0);
+      }
+    }
+  }
+}
+
+// The same from the prepacked form (pointers of unit_tiles_packed).  raw: the unit is
+// flagged and holds the raw codes and scale bytes; otherwise the move onto the OCP code
+// points and the decrement of the scale byte are undone (all codes of such a unit are finite).
+template <int NT>
+__device__ __forceinline__ void exact_unit_packed(const uint8_t* const (&w_rows)[NT],
+                                                  const uint8_t* const (&s_rows)[NT],
+                                                  const int (&shift)[NT], bool raw, const uint16_t* a_row,
+                                                  int K, int lane, f32x4 (&acc)[NT]) {
+  const int lq = lane >> 4;
+  const int groups = K / 32;
+#pragma unroll
+  for (int t = 0; t < NT; ++t) acc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll 1
+  for (int ks = 0; ks * 4 < groups; ++ks) {
+    const int g = ks * 4 + lq;
+    const bool ok = g < groups;
+#pragma unroll 1
+    for (int d = 0; d < 4; ++d) {
+      u32x4 av = {0u, 0u, 0u, 0u};
+      if (ok && a_row != nullptr) av = *reinterpret_cast<const u32x4*>(a_row + g * 32 + d * 8);
+#pragma unroll
+      for (int t = 0; t < NT; ++t) {
+        uint32_t x = 0u, sc = 127u;
+        if (ok) {
+          x = *reinterpret_cast<const uint32_t*>(w_rows[t] + (size_t)ks * kMxStepBytes + d * 4);
+          sc = (*reinterpret_cast<const uint32_t*>(s_rows[t] + (size_t)ks * kMxStepBytes) >> shift[t]) & 0xFFu;
+          if (!raw) {
+            x -= (x & 0x44444444u) >> 1;
+            sc = (sc + 1u) & 0xFFu;
+          }
         }
         acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(dequant8_exact(x, sc)),
                                                          as_bf16x8(av), acc[t], 0, 0, 0);
@@ -422,9 +518,17 @@ __device__ __forceinline__ void lds_barrier() {
   __asm__ volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
 }
 
-template <int STAGE, int WAVES, int NT, int D, bool KSPLIT = false, bool ROUTE = false>
+// PACKED: the weights are read from the prepacked form (GemmArgs::Wp) and W / Ws not at
+// all, so that a caller who prepacks needs no second copy of the weights.  A lane's 16
+// code bytes of a K step are where unit_tiles_packed says, already on the OCP code points,
+// and the scale bytes (already less one) come with the step, four to a lane, so there is
+// no scale block to park in LDS and nothing to check in the loop: a unit that needs the
+// exact path carries a flag, looked up when the unit is begun.
+template <int STAGE, int WAVES, int NT, int D, bool KSPLIT = false, bool ROUTE = false, bool PACKED = false>
 __global__ __launch_bounds__(64 * WAVES) void stream_resident_kernel(GemmArgs p) {
   static_assert(!ROUTE || STAGE == 0, "the routed form is the first stage's");
+  static_assert(!PACKED || (WAVES * (STAGE == 0 ? 8 * NT : 16 * NT)) % (STAGE == 0 ? 64 : 128) == 0,
+                "a wavefront's consecutive units are whole packed units apart");
   extern __shared__ u32x4 b_lds[];  // [nsteps][2][2][64] operand planes, block scales, weight scales
   __shared__ int run_block0[kMaxRuns];
   __shared__ int run_expert[kMaxRuns];
@@ -451,11 +555,15 @@ __global__ __launch_bounds__(64 * WAVES) void stream_resident_kernel(GemmArgs p)
   const int units = STAGE == 0 ? p.ncols / (8 * NT) : p.ncols / (16 * NT);
   const int sc_tile_bytes = 16 * groups;  // scale bytes of one 16-row tile
   uint8_t* bsc_lds = reinterpret_cast<uint8_t*>(b_lds + (size_t)nsteps * 256);  // [nsteps][64]
-  uint8_t* sc_lds = bsc_lds + (size_t)nsteps * 64 + (size_t)wave * NT * sc_tile_bytes;
+  uint8_t* sc_lds = bsc_lds + (size_t)nsteps * 64 + (size_t)wave * NT * sc_tile_bytes;  // (not PACKED)
   // rows of W between the units a wavefront takes one after the other
   const size_t unit_stride_rows = (size_t)WAVES * (STAGE == 0 ? 8 * NT : 16 * NT);
-  const size_t w_unit_stride = unit_stride_rows * (size_t)(K / 2);
+  // packed units between them, and the bytes: of W (PACKED: of the packed form) and of Ws
+  constexpr int kPackedStride = WAVES * (STAGE == 0 ? 8 * NT : 16 * NT) / (STAGE == 0 ? 64 : 128);
+  const size_t w_unit_stride = PACKED ? (size_t)kPackedStride * (size_t)nsteps * (size_t)kMxStepBytes
+                                      : unit_stride_rows * (size_t)(K / 2);
   const size_t s_unit_stride = unit_stride_rows * (size_t)groups;
+  constexpr int kNS = PACKED ? (STAGE == 0 ? NT / 2 : NT) : 1;  // scale words of a K step a lane loads
 
   // Order of the start: what memory must bring is asked for first (wavefront 0: the experts
   // of the first 64 blocks, for the run list; the others: the head of sorted_ids, which
@@ -708,6 +816,7 @@ __global__ __launch_bounds__(64 * WAVES) void stream_resident_kernel(GemmArgs p)
 
   struct Stage {
     u32x4 w[NT];
+    uint32_t s[kNS];  // PACKED: the scale bytes of the step (tile t: word t % kNS, byte shift[t] / 8)
   };
   int pass_no = 0;
 
@@ -748,20 +857,34 @@ __global__ __launch_bounds__(64 * WAVES) void stream_resident_kernel(GemmArgs p)
     const uint8_t* cw[NT];
     const uint8_t* cs[NT];
     int col0[NT];
+    int shift[NT];         // PACKED: where a tile's scale byte is in the step's word
+    int cur_pu = 0;        // PACKED: packed unit of the unit being computed ...
+    bool cur_flag = false; // ... and its flag
 
     // ---- load cursor: runs D steps ahead and crosses unit boundaries -----
     const uint8_t* lrow[NT];
+    const uint8_t* lsc[kNS];
 #pragma unroll
     for (int t = 0; t < NT; ++t) lrow[t] = nullptr;
+#pragma unroll
+    for (int j = 0; j < kNS; ++j) lsc[j] = nullptr;
     int ld_ks = 0;
     int ld_units = 0;  // units the cursor has not finished, the current one included
     auto issue = [&](Stage& st) {
       // lanes past the end of a partial last step re-read the last group: the
       // operand planes there are zero, so what they load does not matter
-      const int g = min(ld_ks * 4 + lq, groups - 1);
+      if constexpr (PACKED) {  // (the packed form is padded to whole K steps with zero codes)
+        const size_t step = (size_t)ld_ks * (size_t)kMxStepBytes;
 #pragma unroll
-      for (int t = 0; t < NT; ++t)
-        st.w[t] = *reinterpret_cast<const u32x4*>(lrow[t] + (size_t)g * 16);
+        for (int t = 0; t < NT; ++t) st.w[t] = *reinterpret_cast<const u32x4*>(lrow[t] + step);
+#pragma unroll
+        for (int j = 0; j < kNS; ++j) st.s[j] = *reinterpret_cast<const uint32_t*>(lsc[j] + step);
+      } else {
+        const int g = min(ld_ks * 4 + lq, groups - 1);
+#pragma unroll
+        for (int t = 0; t < NT; ++t)
+          st.w[t] = *reinterpret_cast<const u32x4*>(lrow[t] + (size_t)g * 16);
+      }
       if constexpr (KSPLIT) {
         if (++ld_ks == k_end) ld_ks = k_end - 1;  // past this wavefront's part: stay on its last step
       } else if (++ld_ks == nsteps) {  // uniform, no memory operation inside
@@ -770,6 +893,10 @@ __global__ __launch_bounds__(64 * WAVES) void stream_resident_kernel(GemmArgs p)
           ld_ks = 0;
 #pragma unroll
           for (int t = 0; t < NT; ++t) lrow[t] += w_unit_stride;
+          if constexpr (PACKED) {
+#pragma unroll
+            for (int j = 0; j < kNS; ++j) lsc[j] += w_unit_stride;
+          }
         } else {
           ld_ks = nsteps - 1;  // past the last unit: stay on its last step
         }
@@ -785,11 +912,13 @@ __global__ __launch_bounds__(64 * WAVES) void stream_resident_kernel(GemmArgs p)
     u32x4 scn[kScMax];
     const uint8_t* sc_unit = nullptr;  // scale bytes of the first tile of the unit being computed
     auto fetch_scales = [&](size_t ahead) {
+      if constexpr (PACKED) return;
 #pragma unroll
       for (int j = 0; j < kScMax; ++j)
         scn[j] = *reinterpret_cast<const u32x4*>(sc_unit + ahead + sc_piece[j]);
     };
     auto park_scales = [&]() {
+      if constexpr (PACKED) return;
 #pragma unroll
       for (int j = 0; j < kScMax; ++j) {
         const int piece = lane + 64 * j;
@@ -804,8 +933,15 @@ __global__ __launch_bounds__(64 * WAVES) void stream_resident_kernel(GemmArgs p)
     // written; a wavefront without units loads the slice's first unit and drops it.
     Stage st[D];
     auto prime = [&]() {
-      unit_tiles<STAGE, NT>(p, e, n_my > 0 ? first : u0, ln, cw, cs, col0);
-      sc_unit = cs[0] - (size_t)ln * groups;
+      if constexpr (PACKED) {
+        unit_tiles_packed<STAGE, NT>(p, e, n_my > 0 ? first : u0, lane, nsteps, cw, cs, shift, col0, cur_pu);
+        cur_flag = packed_unit_flagged(p, e, cur_pu);
+#pragma unroll
+        for (int j = 0; j < kNS; ++j) lsc[j] = cs[j];
+      } else {
+        unit_tiles<STAGE, NT>(p, e, n_my > 0 ? first : u0, ln, cw, cs, col0);
+        sc_unit = cs[0] - (size_t)ln * groups;
+      }
 #pragma unroll
       for (int t = 0; t < NT; ++t) lrow[t] = cw[t];
       ld_ks = KSPLIT ? k_begin : 0;
@@ -970,11 +1106,15 @@ __global__ __launch_bounds__(64 * WAVES) void stream_resident_kernel(GemmArgs p)
           int sa[NT];
 #pragma unroll
           for (int t = 0; t < NT; ++t) {
-            const uint32_t sb = sc_lds[t * sc_tile_bytes + ln * groups + g];
-            bad |= (uint32_t)((sb - kScaleLo) > (kScaleHi - kScaleLo));
-            bad |= fp4x8_nonfinite(sg.w[t][0]) | fp4x8_nonfinite(sg.w[t][1]) |
-                   fp4x8_nonfinite(sg.w[t][2]) | fp4x8_nonfinite(sg.w[t][3]);
-            sa[t] = (int)sb - 1;
+            if constexpr (PACKED) {
+              sa[t] = (int)((sg.s[t % kNS] >> shift[t]) & 0xFFu);
+            } else {
+              const uint32_t sb = sc_lds[t * sc_tile_bytes + ln * groups + g];
+              bad |= (uint32_t)((sb - kScaleLo) > (kScaleHi - kScaleLo));
+              bad |= fp4x8_nonfinite(sg.w[t][0]) | fp4x8_nonfinite(sg.w[t][1]) |
+                     fp4x8_nonfinite(sg.w[t][2]) | fp4x8_nonfinite(sg.w[t][3]);
+              sa[t] = (int)sb - 1;
+            }
           }
           const int sbh = bsc_lds[ks * 64 + lane];
           const int sbl = sbh - 4;
@@ -984,7 +1124,7 @@ __global__ __launch_bounds__(64 * WAVES) void stream_resident_kernel(GemmArgs p)
           const i32x8 bl = fp8_operand(l0, l1);
           i32x8 wa[NT];
 #pragma unroll
-          for (int t = 0; t < NT; ++t) wa[t] = fp4_operand(sg.w[t]);
+          for (int t = 0; t < NT; ++t) wa[t] = PACKED ? fp4_operand_packed(sg.w[t]) : fp4_operand(sg.w[t]);
           // the two MFMAs of an accumulator are kept NT instructions apart
 #pragma unroll
           for (int t = 0; t < NT; ++t)
@@ -1029,7 +1169,7 @@ __global__ __launch_bounds__(64 * WAVES) void stream_resident_kernel(GemmArgs p)
                 for (int t = 0; t < NT; ++t) acc[t] += part[(w2 * NT + t) * 64 + lane];
                 any_bad |= ks_bad[w2] != 0;
               }
-              if (any_bad)
+              if (any_bad || (PACKED && cur_flag))
                 redo = 1ull;
               else if (my_flat >= 0)
                 epilogue_tile<STAGE, NT>(p, e, acc, col0, my_flat, srow, lq);
@@ -1062,7 +1202,7 @@ __global__ __launch_bounds__(64 * WAVES) void stream_resident_kernel(GemmArgs p)
                   // unit's last K step could run: the pass's mark is complete.)  A unit of a
                   // marked pass, or one that met a code or scale outside the fast path's
                   // domain, is redone after the stream, so the hot loop stays small
-                  if (__ballot(bad != 0u) != 0ull || pass_slow[flag] != 0)
+                  if (__ballot(bad != 0u) != 0ull || pass_slow[flag] != 0 || (PACKED && cur_flag))
                     redo |= 1ull << cunit;
                   else if (my_flat >= 0)
                     epilogue_tile<STAGE, NT>(p, e, acc, col0, my_flat, srow, lq);
@@ -1071,11 +1211,16 @@ __global__ __launch_bounds__(64 * WAVES) void stream_resident_kernel(GemmArgs p)
 #pragma unroll
                     for (int t = 0; t < NT; ++t) {
                       cw[t] += w_unit_stride;
-                      cs[t] += s_unit_stride;
+                      cs[t] += PACKED ? w_unit_stride : s_unit_stride;
                       col0[t] += WAVES * (STAGE == 0 ? 8 * NT : 16 * NT);
                     }
-                    sc_unit += s_unit_stride;
-                    if (cunit + 1 < n_my) fetch_scales(s_unit_stride);
+                    if constexpr (PACKED) {
+                      cur_pu += kPackedStride;
+                      cur_flag = packed_unit_flagged(p, e, cur_pu);
+                    } else {
+                      sc_unit += s_unit_stride;
+                      if (cunit + 1 < n_my) fetch_scales(s_unit_stride);
+                    }
                   }
                   cks = 0;
                   bad = 0u;
@@ -1096,8 +1241,13 @@ __global__ __launch_bounds__(64 * WAVES) void stream_resident_kernel(GemmArgs p)
           while (redo != 0ull) {
             const int idx = __builtin_ctzll(redo);
             redo &= redo - 1ull;
-            unit_tiles<STAGE, NT>(p, e, first + idx * WAVES, ln, cw, cs, col0);
-            exact_unit_global<NT>(cw, cs, a_row, K, lane, acc);
+            if constexpr (PACKED) {
+              unit_tiles_packed<STAGE, NT>(p, e, first + idx * WAVES, lane, nsteps, cw, cs, shift, col0, cur_pu);
+              exact_unit_packed<NT>(cw, cs, shift, packed_unit_flagged(p, e, cur_pu), a_row, K, lane, acc);
+            } else {
+              unit_tiles<STAGE, NT>(p, e, first + idx * WAVES, ln, cw, cs, col0);
+              exact_unit_global<NT>(cw, cs, a_row, K, lane, acc);
+            }
             if (my_flat >= 0) epilogue_tile<STAGE, NT>(p, e, acc, col0, my_flat, srow, lq);
           }
         }
@@ -1879,11 +2029,11 @@ constexpr size_t kResidentLdsLimit = 150 * 1024;  // dynamic LDS the resident ke
 
 // True when the device grants the kernel its dynamic LDS (asked once per kernel;
 // a refusal makes the caller take the other variant).
-template <int STAGE, int WAVES, int NT, int D, bool KSPLIT = false, bool ROUTE = false>
+template <int STAGE, int WAVES, int NT, int D, bool KSPLIT = false, bool ROUTE = false, bool PACKED = false>
 bool resident_kernel_ready() {
   static const bool configured = [] {
     const hipError_t err = hipFuncSetAttribute(
-        reinterpret_cast<const void*>(stream_resident_kernel<STAGE, WAVES, NT, D, KSPLIT, ROUTE>),
+        reinterpret_cast<const void*>(stream_resident_kernel<STAGE, WAVES, NT, D, KSPLIT, ROUTE, PACKED>),
         hipFuncAttributeMaxDynamicSharedMemorySize, (int)kResidentLdsLimit);
     if (err != hipSuccess) (void)hipGetLastError();  // not left for the next caller to find
     return err == hipSuccess;
@@ -1891,18 +2041,24 @@ bool resident_kernel_ready() {
   return configured;
 }
 
-template <int STAGE, int WAVES, int NT, int D, bool KSPLIT = false, bool ROUTE = false>
+template <int STAGE, int WAVES, int NT, int D, bool KSPLIT = false, bool ROUTE = false, bool PACKED = false>
 bool launch_resident(const GemmArgs& g, size_t lds, hipStream_t stream) {
-  if (!resident_kernel_ready<STAGE, WAVES, NT, D, KSPLIT, ROUTE>()) return false;
-  hipLaunchKernelGGL((stream_resident_kernel<STAGE, WAVES, NT, D, KSPLIT, ROUTE>), dim3(num_compute_units()),
+  if (!resident_kernel_ready<STAGE, WAVES, NT, D, KSPLIT, ROUTE, PACKED>()) return false;
+  hipLaunchKernelGGL((stream_resident_kernel<STAGE, WAVES, NT, D, KSPLIT, ROUTE, PACKED>), dim3(num_compute_units()),
                      dim3(64 * WAVES), lds, stream, g);
   return true;
 }
 
 // Launch shape of one stage.  variant kMoeVariantLds = the tile kernel.
+// The shapes the packed instantiations of the resident kernel exist for: the ones the
+// compiled-in rules return (a record of the tuning store is for the raw form's shapes).
+#define VK_PACKED_VARIANTS(X) X(0, 8, 2, 2) X(0, 4, 2, 8) X(1, 8, 1, 4) X(1, 8, 2, 4) X(1, 8, 1, 6)
+#define VK_PACKED_KSPLIT_VARIANTS(X) X(0, 8, 2, 4) X(1, 8, 1, 8) X(1, 8, 2, 4)
+
 struct StagePlan {
   int variant, waves, nt, depth;
   bool ksplit;  // the resident kernel with K shared between the wavefronts of a unit
+  bool packed;  // ... reading the prepacked form (the stage has no raw weights)
   size_t resident_lds;
 };
 
@@ -1910,9 +2066,11 @@ template <int STAGE>
 StagePlan plan_stage(const GemmArgs& g) {
   // a record of the tuning store first, then the compiled-in rules
   MoeTile tile;
-  if (!moe_tuning_find(STAGE, g.K, g.ncols, g.n_flat, &tile))
+  const bool packed = g.W == nullptr && g.Wp != nullptr;
+  if (packed || !moe_tuning_find(STAGE, g.K, g.ncols, g.n_flat, &tile))
     tile = pick_moe_tile(g.n_flat, g.K, g.ncols, STAGE);
   StagePlan pl;
+  pl.packed = packed;
   pl.ksplit = tile.variant == kMoeVariantResidentKSplit;
   pl.variant = pl.ksplit ? (int)kMoeVariantResident : tile.variant;
   pl.nt = tile.nt;
@@ -1921,12 +2079,13 @@ StagePlan plan_stage(const GemmArgs& g) {
   const int groups = g.K / 32;
   const int nsteps = (groups + 3) / 4;
   // operand planes + block scales + one weight-scale region per wavefront
-  pl.resident_lds = (size_t)nsteps * (4096 + 64) + (size_t)pl.waves * pl.nt * 16 * groups;
+  pl.resident_lds = (size_t)nsteps * (4096 + 64) + (packed ? 0 : (size_t)pl.waves * pl.nt * 16 * groups);
   // (K split: the partial sums of the wavefronts, 1 KB a tile, lie over the operand planes)
   if (pl.ksplit && (size_t)nsteps * 4096 < (size_t)pl.waves * pl.nt * 1024) pl.ksplit = false;
   const int res_units = STAGE == 0 ? g.ncols / (8 * pl.nt) : g.ncols / (16 * pl.nt);
   if (pl.resident_lds > kResidentLdsLimit || g.num_blocks > kMaxRuns ||
-      pl.nt * groups > 64 * resident_scale_pieces(pl.waves) ||
+      (!packed && pl.nt * groups > 64 * resident_scale_pieces(pl.waves)) ||
+      (packed && STAGE == 0 && g.ncols % 64 != 0) ||  // (what the prepacked form asks of the first stage)
       (res_units + pl.waves - 1) / pl.waves > 64 ||  // one bit per unit in a wavefront's redo mask
       nsteps * 4 > resident_batch(pl.waves) * pl.waves)  // the rows are staged in one batch
     pl.variant = kMoeVariantLds;
@@ -1953,6 +2112,25 @@ bool wide_kernel_applies(const GemmArgs& g) { return g.Aq != nullptr; }
 
 template <int STAGE>
 void launch_stage(const GemmArgs& g, const StagePlan& pl, hipStream_t stream) {
+  if (pl.packed) {  // (the callers keep stages that are not resident away from here)
+#define VK_RESIDENT(S_, W_, NT_, D_) \
+  if constexpr (STAGE == S_) { \
+    if (pl.ksplit && pl.waves == W_ && pl.nt == NT_ && pl.depth == D_ && \
+        launch_resident<S_, W_, NT_, D_, true, false, true>(g, pl.resident_lds, stream)) \
+      return; \
+  }
+    VK_PACKED_KSPLIT_VARIANTS(VK_RESIDENT)
+#undef VK_RESIDENT
+#define VK_RESIDENT(S_, W_, NT_, D_) \
+  if constexpr (STAGE == S_) { \
+    if (!pl.ksplit && pl.waves == W_ && pl.nt == NT_ && pl.depth == D_ && \
+        launch_resident<S_, W_, NT_, D_, false, false, true>(g, pl.resident_lds, stream)) \
+      return; \
+  }
+    VK_PACKED_VARIANTS(VK_RESIDENT)
+#undef VK_RESIDENT
+    return;
+  }
   if (pl.variant == kMoeVariantResident) {
 #define VK_RESIDENT(S_, W_, NT_, D_) \
   if constexpr (STAGE == S_) { \
@@ -2054,6 +2232,11 @@ GemmArgs gateup_args(const FusedMoeArgs& a) {
   g.A = a.A;
   g.W = a.w13;
   g.Ws = a.w13_scale;
+  if (a.w13_packed != nullptr) {
+    g.p_units = mx_units(0, a.ispp);
+    g.Wp = a.w13_packed;
+    g.Wpf = a.w13_packed + mx_packed_body_bytes(a.num_experts, g.p_units, mx_kp(a.hidden) / 128);
+  }
   g.bias = a.b13;
   g.K = a.hidden;
   g.a_stride = a.hidden;
@@ -2066,6 +2249,11 @@ GemmArgs down_args(const FusedMoeArgs& a) {
   g.A = a.act;
   g.W = a.w2;
   g.Ws = a.w2_scale;
+  if (a.w2_packed != nullptr) {
+    g.p_units = mx_units(1, a.hidden);
+    g.Wp = a.w2_packed;
+    g.Wpf = a.w2_packed + mx_packed_body_bytes(a.num_experts, g.p_units, mx_kp(a.ispp) / 128);
+  }
   g.bias = a.b2;
   g.K = a.ispp;
   g.a_stride = a.ispp;
@@ -2074,6 +2262,26 @@ GemmArgs down_args(const FusedMoeArgs& a) {
 }
 
 }  // namespace
+
+// A call that passes the prepacked weights alone (w13 / w2 null): true when the library
+// can run it -- both stages on the decode kernels' packed forms, or the workspace the
+// prepacked kernels need.
+bool fused_moe_packed_only_ok(const FusedMoeArgs& a) {
+  if (a.w13_packed == nullptr || a.w2_packed == nullptr || a.num_experts <= 0) return false;
+  if (a.M <= 0 || a.EM <= 0 || a.block_size <= 0) return true;  // nothing will run
+  const GemmArgs g0 = gateup_args(a), g1 = down_args(a);
+  const StagePlan p0 = plan_stage<0>(g0), p1 = plan_stage<1>(g1);
+  if (p0.variant == kMoeVariantResident && p1.variant == kMoeVariantResident) return true;
+  return fused_moe_prepacked_takes(a, true);
+}
+
+bool moe_down_packed_only_ok(const FusedMoeArgs& a) {
+  if (a.w2_packed == nullptr || a.num_experts <= 0) return false;
+  if (a.M <= 0 || a.EM <= 0 || a.block_size <= 0) return true;
+  const GemmArgs g = down_args(a);
+  if (plan_stage<1>(g).variant == kMoeVariantResident) return true;
+  return fused_moe_prepacked_takes(a, false);
+}
 
 size_t fused_moe_workspace_bytes(int M, int hidden, int ispp, int top_k, int EM) {
   if (M <= 0 || EM <= 0 || hidden <= 0 || ispp <= 0 || top_k <= 0) return 0;
@@ -2114,6 +2322,13 @@ bool prepare_moe_kernels() {
   VK_KSPLIT_VARIANTS(VK_READY)
 #undef VK_READY
   ok = resident_kernel_ready<0, 8, 2, 4, true, true>() && resident_kernel_ready<0, 8, 2, 2, false, true>() && ok;
+#define VK_READY(S_, W_, NT_, D_) ok = resident_kernel_ready<S_, W_, NT_, D_, false, false, true>() && ok;
+  VK_PACKED_VARIANTS(VK_READY)
+#undef VK_READY
+#define VK_READY(S_, W_, NT_, D_) ok = resident_kernel_ready<S_, W_, NT_, D_, true, false, true>() && ok;
+  VK_PACKED_KSPLIT_VARIANTS(VK_READY)
+#undef VK_READY
+  ok = resident_kernel_ready<0, 8, 2, 4, true, true, true>() && resident_kernel_ready<0, 8, 2, 2, false, true, true>() && ok;
   MoeTile unused;
   (void)moe_tuning_find(0, 64, 64, 1, &unused);  // reads the tuning store now rather than on the first launch
   return ok;
@@ -2157,10 +2372,13 @@ bool launch_routed_moe(const FusedMoeArgs& a, const RoutedArgs& r, hipStream_t s
     g0.zero_count = (long long)a.M * a.hidden;
   }
   bool launched = false;
+  if (p0.packed != p1.packed) return false;  // (both packed forms or neither)
   if (p0.ksplit && p0.waves == 8 && p0.nt == 2 && p0.depth == 4)
-    launched = launch_resident<0, 8, 2, 4, true, true>(g0, p0.resident_lds, stream);
+    launched = p0.packed ? launch_resident<0, 8, 2, 4, true, true, true>(g0, p0.resident_lds, stream)
+                         : launch_resident<0, 8, 2, 4, true, true>(g0, p0.resident_lds, stream);
   else if (!p0.ksplit && p0.waves == 8 && p0.nt == 2 && p0.depth == 2)
-    launched = launch_resident<0, 8, 2, 2, false, true>(g0, p0.resident_lds, stream);
+    launched = p0.packed ? launch_resident<0, 8, 2, 2, false, true, true>(g0, p0.resident_lds, stream)
+                         : launch_resident<0, 8, 2, 2, false, true>(g0, p0.resident_lds, stream);
   if (!launched) return false;
   g1.topk_w = r.topk_w;
   launch_stage<1>(g1, p1, stream);
@@ -2244,6 +2462,15 @@ void launch_fused_moe(const FusedMoeArgs& a, hipStream_t stream) {
       p1.variant != kMoeVariantResident &&
       launch_fused_moe_prepacked(a, stream))
     return;
+  // Without raw weights the decode kernels' packed forms take the call when both stages
+  // are theirs, and the prepacked kernels any other (fused_moe_packed_only_ok has checked
+  // that they can: the tile kernels below read raw weights).
+  if (p0.packed || p1.packed) {
+    if (p0.variant != kMoeVariantResident || p1.variant != kMoeVariantResident) {
+      (void)launch_fused_moe_prepacked(a, stream);
+      return;
+    }
+  }
   Workspace w;
   bool combine = false;
   bool split_act_between = false;

@@ -125,14 +125,19 @@ __global__ __launch_bounds__(256) void prepack_flag_kernel(const uint8_t* __rest
 
 // One workgroup per (K step, unit, expert): 512 pieces of 16 bytes (codes on the
 // OCP points) and 64 x 8 scale bytes (decremented), zero codes / neutral scales
-// where the unit or K is ragged.
+// where the unit or K is ragged.  A flagged unit keeps the codes and the scale bytes
+// as they are in W / Ws: no fast path multiplies them, and the exact paths, which read
+// the packed form as well, need the codes the move onto the OCP points would merge
+// (the inf / NaN codes carry into the sign bit).
 __global__ __launch_bounds__(256) void prepack_kernel(const uint8_t* __restrict__ W,
                                                       const uint8_t* __restrict__ Ws,
-                                                      uint8_t* __restrict__ packed, int stage,
+                                                      uint8_t* __restrict__ packed,
+                                                      const uint8_t* __restrict__ flags, int stage,
                                                       int rows_w, int ncols, int K, int units,
                                                       int ksteps) {
   const int kstep = blockIdx.x, unit = blockIdx.y, e = blockIdx.z;
   const int groups = K / 32;
+  const bool raw = flags[(size_t)e * units + unit] != 0;  // uniform
   uint8_t* dst = packed + mx_unit_offset(e, units, unit, ksteps) + (size_t)kstep * (size_t)kMxStepBytes;
 #pragma unroll
   for (int i = 0; i < 2; ++i) {
@@ -144,8 +149,10 @@ __global__ __launch_bounds__(256) void prepack_kernel(const uint8_t* __restrict_
     if (row < rows_w && g < groups) {
       const size_t r = (size_t)e * (size_t)rows_w + (size_t)row;
       v = *reinterpret_cast<const u32x4*>(W + r * (size_t)(K / 2) + (size_t)g * 16);
+      if (!raw) {
 #pragma unroll
-      for (int j = 0; j < 4; ++j) v[j] = fp4x8_to_ocp_doubled(v[j]);
+        for (int j = 0; j < 4; ++j) v[j] = fp4x8_to_ocp_doubled(v[j]);
+      }
     }
     *reinterpret_cast<u32x4*>(dst + (size_t)pc * 16) = v;
   }
@@ -160,7 +167,7 @@ __global__ __launch_bounds__(256) void prepack_kernel(const uint8_t* __restrict_
         const int g = kstep * 4 + half * 2 + (lane >> 5);
         uint32_t s = 127u;
         if (row < rows_w && g < groups)
-          s = ((uint32_t)Ws[((size_t)e * (size_t)rows_w + (size_t)row) * (size_t)groups + g] - 1u) & 0xFFu;
+          s = ((uint32_t)Ws[((size_t)e * (size_t)rows_w + (size_t)row) * (size_t)groups + g] - (raw ? 0u : 1u)) & 0xFFu;
         s8[half] |= s << (8 * t);
       }
     *reinterpret_cast<u32x2*>(dst + 8192 + lane * 8) = u32x2{s8[0], s8[1]};
@@ -403,26 +410,21 @@ __global__ __launch_bounds__(256) void quant_rows_w4_kernel(const uint16_t* __re
 // a_row: the bf16 row of this lane's activation row, or null for a padding row.
 // q_row (W4A4 mode): the row's quantised plane instead; its values are decoded exactly.
 template <int STAGE>
-__device__ __forceinline__ void exact_unit_mx(const MxArgs& p, int e, int unit, const uint16_t* a_row,
+__device__ __forceinline__ void exact_unit_mx(const MxArgs& p, int e, int unit, bool w_raw, const uint16_t* a_row,
                                               const uint8_t* q_row, int lane, f32x16 (&acc)[4]) {
+  // The weights come from the packed form: K block g of row n of tile t is the 16 bytes
+  // at step g / 4, half (g / 2) % 2, lane (g % 2, n) of the tile, its scale byte the one
+  // for (half, t) of that lane's eight.  A flagged unit (w_raw) holds the codes and
+  // scale bytes of the raw tensors; any other the codes moved onto the OCP points and
+  // the scale bytes less one, both undone here (all its codes are finite).
   const int n = lane & 31, hh = lane >> 5;
-  const int rows_w = STAGE == 0 ? 2 * p.ncols : p.ncols;
   const int K = p.K;
-  const uint8_t* w_row[4];
-  const uint8_t* s_row[4];
+  const int nsteps = mx_kp(K) / 128;
+  const uint8_t* const ub = p.Wp + mx_unit_offset(e, p.units, unit, nsteps);
 #pragma unroll
-  for (int t = 0; t < 4; ++t) {
-    const int row = mx_weight_row(STAGE, p.ncols, unit, t, n);
-    w_row[t] = nullptr;
-    s_row[t] = nullptr;
-    if (row < rows_w) {
-      const size_t r = (size_t)e * (size_t)rows_w + (size_t)row;
-      w_row[t] = p.W + r * (size_t)(K / 2);
-      s_row[t] = p.Ws + r * (size_t)(K / 32);
-    }
+  for (int t = 0; t < 4; ++t)
 #pragma unroll
     for (int i = 0; i < 16; ++i) acc[t][i] = 0.f;
-  }
 #pragma unroll 1
   for (int s = 0; s < K / 16; ++s) {  // 16 values of K: lane half hh takes 8 of them
     const int k = 16 * s + 8 * hh;
@@ -434,11 +436,18 @@ __device__ __forceinline__ void exact_unit_mx(const MxArgs& p, int e, int unit, 
       c -= (c & 0x44444444u) >> 1;
       av = dequant8_exact(c, ((uint32_t)blk[16] + 1u) & 0xFFu);
     }
+    const int g = k >> 5;
+    const uint8_t* const sb = ub + (size_t)(g >> 2) * kMxStepBytes;
+    const int half = (g >> 1) & 1, lane_p = (g & 1) * 32 + n;
 #pragma unroll
     for (int t = 0; t < 4; ++t) {
-      u32x4 wv = {0u, 0u, 0u, 0u};
-      if (w_row[t] != nullptr)
-        wv = dequant8_exact(*reinterpret_cast<const uint32_t*>(w_row[t] + k / 2), s_row[t][k >> 5]);
+      uint32_t c = *reinterpret_cast<const uint32_t*>(sb + half * 4096 + t * 1024 + lane_p * 16 + ((k & 31) >> 1));
+      uint32_t sc = sb[8192 + lane_p * 8 + half * 4 + t];
+      if (!w_raw) {
+        c -= (c & 0x44444444u) >> 1;
+        sc = (sc + 1u) & 0xFFu;
+      }
+      const u32x4 wv = dequant8_exact(c, sc);
       acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_bf16x8(wv), as_bf16x8(av), acc[t], 0, 0, 0);
     }
   }
@@ -822,7 +831,7 @@ __global__ __launch_bounds__(64 * kMxWaves) void tile_mx_kernel(MxArgs p) {
           if (TERMS == 1) q_row = p.Aq + grow * (size_t)Kp;
           else a_row = p.A + grow * (size_t)p.a_stride;
         }
-        exact_unit_mx<STAGE>(p, e, unit, a_row, q_row, lane, tile);
+        exact_unit_mx<STAGE>(p, e, unit, w_slow, a_row, q_row, lane, tile);
       }
       if constexpr (PREACT) {
         // the accumulators as they are: 64 columns (two tiles) at a time through the
@@ -1069,7 +1078,7 @@ void launch_moe_prepack(const uint8_t* w, const uint8_t* w_scale, int num_expert
   hipLaunchKernelGGL(prepack_flag_kernel, dim3(units, num_experts), dim3(256), 0, stream, w, w_scale,
                      flags, stage, rows, ncols, K, units);
   hipLaunchKernelGGL(prepack_kernel, dim3(ksteps, units, num_experts), dim3(256), 0, stream, w,
-                     w_scale, packed, stage, rows, ncols, K, units, ksteps);
+                     w_scale, packed, flags, stage, rows, ncols, K, units, ksteps);
 }
 
 // ---- workspace of the prepacked path -------------------------------------------
@@ -1203,6 +1212,13 @@ bool launch_fused_moe_prepacked(const FusedMoeArgs& a, hipStream_t stream) {
   mx_stage0(a, pl, stream);
   mx_stage1(a, pl, stream);
   return true;
+}
+
+// True when launch_fused_moe_prepacked (both_stages) or launch_moe_down_prepacked would
+// take the call (nothing is enqueued).
+bool fused_moe_prepacked_takes(const FusedMoeArgs& a, bool both_stages) {
+  MxPlan pl;
+  return mx_plan(a, both_stages, pl);
 }
 
 // The second stage alone (act is the caller's), likewise.

@@ -90,6 +90,11 @@ void launch_moe_prepack(const uint8_t* w, const uint8_t* w_scale, int num_expert
                         int stage, uint8_t* packed, hipStream_t stream);
 size_t mx_workspace_bytes(int M, int hidden, int ispp, int top_k, int EM);
 bool launch_fused_moe_prepacked(const FusedMoeArgs& a, hipStream_t stream);
+bool fused_moe_prepacked_takes(const FusedMoeArgs& a, bool both_stages);
+// A call with the prepacked weights alone (w13 / w2 null): can the library run it?
+// (the layer; the second stage alone)
+bool fused_moe_packed_only_ok(const FusedMoeArgs& a);
+bool moe_down_packed_only_ok(const FusedMoeArgs& a);
 bool launch_moe_down_prepacked(const FusedMoeArgs& a, hipStream_t stream);
 void launch_split_rows_fp6(const uint16_t* x, int rows, int K, int terms, uint8_t* xq, uint8_t* row_bad,
                            hipStream_t stream);

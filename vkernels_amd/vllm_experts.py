@@ -424,12 +424,16 @@ class FusedExperts:
 
     Weights keep the raw serving layout: ``w13`` [E, 2*I, H/2] uint8 with gate
     rows first, ``w2`` [E, H, I/2] uint8, ue8m0 scales [.., K/32] uint8.
+    ``prepack=True`` adds the prepacked form (1.0625 x the bytes of codes and scales);
+    with ``keep_raw=False`` the raw tensors are let go of after the packing and every
+    call runs on the prepacked form alone.
     """
 
     def __init__(self, w13, w13_scale, w2, w2_scale, *, b13=None, b2=None, activation="swiglu",
                  swiglu_limit: float = 0.0, beta: float = 4.0, linear_beta: float = 25.0,
                  expert_map=None, local_num_experts=None, scratch: CaptureSafeScratch | None = None,
-                 prepack: bool = False, split_terms: int | None = None, w4a4: bool = False):
+                 prepack: bool = False, split_terms: int | None = None, w4a4: bool = False,
+                 keep_raw: bool = True):
         torch = _require_torch()
         self.torch = torch
         self.lib = load_libvkernels_hip()
@@ -481,8 +485,19 @@ class FusedExperts:
             raise ValueError("w4a4=True needs prepack=True")
         self.w13_packed = self.w2_packed = None
         self.moe_prepacked_fn = None
+        if not keep_raw and not prepack:
+            raise ValueError("keep_raw=False needs prepack=True")
         if prepack:
             self.prepack()
+        if not keep_raw:
+            # One copy of the weights: every kernel family reads the prepacked form (the
+            # decode kernels their packed instantiations, the exact paths the raw codes a
+            # flagged unit keeps), so the references to the raw tensors are dropped here
+            # and the calls pass null for them.  The caller drops its own to free the memory.
+            if not self.use_workspace or self.moe_prepacked_fn is None:
+                raise RuntimeError("keep_raw=False needs the workspace entry points")
+            torch.cuda.current_stream().synchronize()  # the packing kernels have read them
+            self.w13 = self.w13_scale = self.w2 = self.w2_scale = None
 
     def prepack(self):
         """Build the prepacked copies of w13 and w2 (idempotent)."""
