@@ -16,7 +16,10 @@ The metric has two halves, and one JSON line carries both:
   weight bytes): algorithmic HBM bytes per launch over its mean duration,
   measured with events on the launch stream in a second loop of the same
   steps, against the 8 TB/s peak.  Weight sets are rotated between steps so
-  that the 256 MB Infinity Cache cannot serve the 423 MB of weights twice;
+  that the 256 MB Infinity Cache cannot serve the 423 MB of weights twice.
+  The weights are prepacked at load time and the raw tensors let go of (one
+  copy: the decode kernels stream the prepacked form; --no-prepack measures
+  the raw form, --keep-raw keeps both);
 * `prefill` is the prefill-shaped workload that is bound by the matrix cores
   (hidden 7168, intermediate 2048, 256 experts, top-8, T = 16384) on weights
   prepacked at load time: tokens/s of the whole step and a `roofline` whose
@@ -30,6 +33,7 @@ decode workload, single-threaded and on all host cores.
 from __future__ import annotations
 
 import argparse
+import ctypes
 import hashlib
 import json
 import os
@@ -58,10 +62,9 @@ def parse_args():
                     help="FP6 terms per activation on the prepacked path: 0 = the library's default "
                          "(3 in the first stage, 2 in the second), 2 or 3 = that many in both")
     ap.add_argument("--no-prepack", action="store_true", help="raw weights only, also for prefill sizes")
-    ap.add_argument("--packed-only", action="store_true",
-                    help="one copy of the weights: prepack at every size and let go of the raw tensors "
-                         "(decode sizes then run the decode kernels' packed instantiations; the "
-                         "`roofline` of such a record is over the fused call, both stages)")
+    ap.add_argument("--keep-raw", action="store_true",
+                    help="keep the raw weight tensors beside the prepacked form (the default lets go of them: "
+                         "one copy of the weights, every kernel reads the prepacked form)")
     ap.add_argument("--no-workspace", action="store_true",
                     help="call the reference's own symbol (no workspace, raw weights)")
     ap.add_argument("--no-modes", action="store_true",
@@ -167,8 +170,8 @@ def run_workload(args, workload, steps, warmup, prepack, split_terms=None, w4a4=
     dev = torch.device("cuda", 0)
     H, I, k = cfg.H, cfg.I, cfg.top_k
     prefill = T * k > 512  # the library's own split between its decode and tile kernels
-    packed_only = args.packed_only and prepack and not args.no_workspace
-    prepack = prepack and (prefill or packed_only) and not args.no_workspace
+    prepack = prepack and not args.no_workspace   # at every size: the decode kernels read the prepacked form too
+    packed_only = prepack and not args.keep_raw
     terms = args.split_terms if split_terms is None else split_terms   # 0 = the library's default
 
     per_set = synth.algorithmic_bytes(H, I, cfg.E, k, 0, cfg.E)
@@ -201,8 +204,8 @@ def run_workload(args, workload, steps, warmup, prepack, split_terms=None, w4a4=
     out = torch.empty((T, H), dtype=torch.float32, device=dev)
     bs = args.block_size or ve.default_block_size(T, k)
     lib = ve.load_libvkernels_hip()
-    lib.vk_hip_moe_gateup_mxfp4.restype = None
-    lib.vk_hip_moe_down_mxfp4.restype = None
+    lib.vk_hip_moe_gateup_mxfp4_ex.restype = None
+    lib.vk_hip_moe_down_mxfp4_ex.restype = None
 
     def step(i, events=None):
         fe = experts[i % n_sets]
@@ -219,7 +222,7 @@ def run_workload(args, workload, steps, warmup, prepack, split_terms=None, w4a4=
         # same launches, with events around the two GEMM stages (decode) or around
         # the fused call (prefill-sized batches, which run with a workspace)
         sids, eids, _, max_em = fe.align(ids, bs)
-        if prefill or packed_only:
+        if prefill:
             events[0].record()
             events[1].record()
             if args.no_workspace:
@@ -232,14 +235,16 @@ def run_workload(args, workload, steps, warmup, prepack, split_terms=None, w4a4=
         st = ve._P(torch.cuda.current_stream().cuda_stream)
         e0, e1, e2 = events
         e0.record()
-        lib.vk_hip_moe_gateup_mxfp4(
+        lib.vk_hip_moe_gateup_mxfp4_ex(
             ve._ptr(A), ve._ptr(fe.w13), ve._ptr(fe.w13_scale), ve._ptr(act), T, H, I,
             k, ve._ptr(sids), ve._ptr(eids), max_em, ve._F(float(fe.swiglu_limit)), fe.activation,
-            ve._F(float(fe.beta)), ve._F(float(fe.linear_beta)), ve._ptr(fe.b13), bs, st)
+            ve._F(float(fe.beta)), ve._F(float(fe.linear_beta)), ve._ptr(fe.b13), bs,
+            ve._ptr(fe.w13_packed), fe.E, st)
         e1.record()
-        lib.vk_hip_moe_down_mxfp4(
+        lib.vk_hip_moe_down_mxfp4_ex(
             ve._ptr(act), ve._ptr(fe.w2), ve._ptr(fe.w2_scale), ve._ptr(w), ve._ptr(out), T,
-            H, I, k, ve._ptr(sids), ve._ptr(eids), max_em, ve._ptr(fe.b2), bs, st)
+            H, I, k, ve._ptr(sids), ve._ptr(eids), max_em, ve._ptr(fe.b2), bs, None, ctypes.c_size_t(0),
+            ctypes.c_uint(0), ve._ptr(fe.w2_packed), fe.E, st)
         e2.record()
 
     for i in range(warmup):
@@ -323,19 +328,11 @@ def run_workload(args, workload, steps, warmup, prepack, split_terms=None, w4a4=
             "flops_per_launch": flops, "avg_launch_us": down_avg * 1e3,
             "median_launch_us": down_ms[len(down_ms) // 2] * 1e3,
         }
-    elif packed_only:
-        achieved = (gate_bytes + down_bytes) / (down_avg * 1e-3) / 1e9
-        roofline = {
-            "bound": "hbm", "kernel": "vk_hip_fused_moe_mxfp4_prepacked without raw weights (stream_resident_kernel<0, "
-                                      "..., PACKED> + stream_resident_kernel<1, ..., PACKED>)",
-            "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
-            "traffic": None, "bytes_per_launch": gate_bytes + down_bytes, "avg_launch_us": down_avg * 1e3,
-            "median_launch_us": down_ms[len(down_ms) // 2] * 1e3,
-        }
     else:
         achieved = gate_bytes / (gate_avg * 1e-3) / 1e9
         roofline = {
-            "bound": "hbm", "kernel": "stream_resident_kernel<0, ...> (gate/up grouped GEMM + SwiGLU)",
+            "bound": "hbm", "kernel": "stream_resident_kernel<0, ...> (gate/up grouped GEMM + SwiGLU"
+                                      + (", weights read from the prepacked form)" if prepack else ")"),
             "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
             "frac": achieved / HBM_PEAK_GBS, "traffic": measured_traffic(workload),
             "bytes_per_launch": gate_bytes, "avg_launch_us": gate_avg * 1e3,
@@ -352,7 +349,7 @@ def run_workload(args, workload, steps, warmup, prepack, split_terms=None, w4a4=
             "workload": f"{cfg.name} T={T}: hidden {H}, intermediate {I}, {cfg.E} experts, "
                         f"top-{k}, MXFP4 weights, bf16 activations, {cfg.logits} routing",
             "block_size": bs, "active_experts": active, "weight_sets": n_sets,
-            "weights": "prepacked at load time, raw tensors let go of" if packed_only
+            "weights": "prepacked at load time, one copy (the raw tensors let go of)" if packed_only
                        else "prepacked at load time (+ raw)" if prepack else "raw",
             "epilogue": args.epilogue,
         },
@@ -361,11 +358,13 @@ def run_workload(args, workload, steps, warmup, prepack, split_terms=None, w4a4=
             "algorithmic_bytes": layer_bytes, "algorithmic_flops": flops,
             "hbm_frac_whole_step": layer_bytes / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS,
             "fp4_mfma_frac_whole_step": flops / (ms_per_step * 1e-3) / 1e12 / FP4_PEAK_TFLOPS,
-            "down_kernel_avg_us": None if prefill or packed_only else down_avg * 1e3,
-            "down_kernel_gbs": None if prefill or packed_only else down_bytes / (down_avg * 1e-3) / 1e9,
+            "down_kernel_avg_us": None if prefill else down_avg * 1e3,
+            "down_kernel_gbs": None if prefill else down_bytes / (down_avg * 1e-3) / 1e9,
         },
     }
-    if prepack:
+    if prepack and not prefill:
+        rec["config"]["activations"] = "bf16 split exactly into two E4M3 terms per block of 32 (decode kernels)"
+    elif prepack:
         rec["config"]["activations"] = (
             "MXFP4 (reference mxfp4_moe_quant), one FP4 x FP4 MFMA per product" if w4a4 else
             f"bf16 as {terms} FP6 E2M3 terms per block of 32 in both stages" if terms else

@@ -186,13 +186,23 @@ void vk_hip_fused_moe_mxfp4_ex(
  * 8 operand tiles of 64 lanes x 16 bytes in lane order (codes moved onto the
  * OCP FP4 code points), then 8 scale bytes per lane (decremented by one); then
  * one flag byte per unit marking units whose weights hold an inf/NaN code or a
- * scale byte outside [64, 190] (computed from the raw weights by the exact
- * path).  Returns VK_OK or a VK_ERROR_* code.
+ * scale byte outside [64, 190]: such a unit is computed by the exact path, and
+ * its blocks hold the codes and scale bytes as they are in w / w_scale (the move
+ * onto the OCP points would merge the inf / NaN codes with others).  Returns VK_OK
+ * or a VK_ERROR_* code.
  *
  * vk_hip_fused_moe_mxfp4_prepacked is vk_hip_fused_moe_mxfp4_ex with the two
  * packed buffers (NULL, NULL = vk_hip_fused_moe_mxfp4_ex exactly) and the
- * number of experts in the weight tensors.  The raw weights are still required:
- * decode-sized calls and the exact path read them.  On the packed path the bf16
+ * number of experts in the weight tensors.  With the packed buffers every kernel
+ * family reads the prepacked form: decode-sized calls run decode kernels that
+ * stream it (faster than the raw form's: the scale bytes come with the codes
+ * and nothing is checked or moved in the loop), and both exact paths read it as
+ * well.  The raw tensors are therefore optional: w13, w13_scale, w2 and w2_scale
+ * may all be NULL (one copy of the weights), provided the call is one the decode
+ * kernels take (up to 512 routed rows, hidden <= 4096 for the first stage and
+ * ispp <= 3072 for the second) or the workspace is given; otherwise the call is
+ * refused with VK_ERROR_INVALID_ARGUMENT in the error state.  On the packed path of
+ * prefill-sized calls the bf16
  * activations are multiplied as a sum of FP6 (E2M3) terms per block of 32 along K,
  * each term with a block scale of its own: three terms (exact unless an element
  * lies more than 2^-13 below its block's largest) in the first stage, whose
@@ -270,7 +280,9 @@ int vk_hip_init(void);
  * vk_hip_moe_tile_query writes the shape a call of this problem size would be
  * planned with and returns 1 when it comes from the tuning store, 0 from the
  * compiled-in rules (a launcher still falls back to the tile kernels where a
- * shape does not fit the device's LDS).
+ * shape does not fit the device's LDS); stage 2 / 3 ask for stage 0 / 1 of a call
+ * that gives the prepacked weights, whose decode kernels have rules of their own
+ * (the store's records are shared).
  * vk_hip_moe_tile_set puts a record for (stage, K, ncols, bucket of n_flat)
  * into the process's store (shape null: removes it); VK_ERROR_INVALID_ARGUMENT
  * for a shape that is not a candidate.  vk_hip_moe_tuning_load reads
@@ -346,10 +358,24 @@ void vk_hip_moe_down_mxfp4(
     const float* b2, int block_size, void* stream);
 
 /*
+ * Additive: vk_hip_moe_gateup_mxfp4 with the prepacked gate/up weights (NULL = raw
+ * weights only).  With them, decode-sized calls run the decode kernels that read the
+ * prepacked form, as the fused call does, and w13 / w13_scale may then be NULL; larger
+ * calls run the raw-weight kernels and need the raw tensors.
+ */
+void vk_hip_moe_gateup_mxfp4_ex(
+    const uint16_t* A, const uint8_t* w13, const uint8_t* w13_scale,
+    uint16_t* act_scratch, int M, int hidden, int ispp, int top_k,
+    const int32_t* sorted_ids, const int32_t* expert_ids, int EM,
+    float swiglu_limit, int activation, float beta, float linear_beta,
+    const float* b13, int block_size, const void* w13_packed, int num_experts, void* stream);
+
+/*
  * Additive: vk_hip_moe_down_mxfp4 with the optional arguments of the fused
  * entry points: a caller-owned workspace (size as for vk_hip_fused_moe_mxfp4_ws),
  * flags (VK_HIP_MOE_OVERWRITE_OUT, VK_HIP_MOE_SPLIT2) and the prepacked down
- * weights (NULL = raw weights only).  It runs the second stage exactly as the
+ * weights (NULL = raw weights only; with them w2 / w2_scale may be NULL when the
+ * call is decode-sized or the workspace is given).  It runs the second stage exactly as the
  * fused call does for the same arguments, so a tensor-parallel caller can sum
  * `act` contributions between the stages and a test can feed the second stage
  * chosen `act` rows.  Device counterpart of moe_down_cpu + moe_combine_cpu,

@@ -583,8 +583,10 @@ int vk_hip_moe_tile_candidates(int stage, int* shapes, int capacity) {
 
 int vk_hip_moe_tile_query(int stage, int K, int ncols, int n_flat, int* shape) {
   vk::MoeTile t;
+  const bool packed = stage == 2 || stage == 3;  // the stage on the prepacked form
+  if (packed) stage -= 2;
   const bool stored = vk::moe_tuning_find(stage, K, ncols, n_flat, &t);
-  if (!stored) t = vk::pick_moe_tile(n_flat, K, ncols, stage);
+  if (!stored) t = vk::pick_moe_tile(n_flat, K, ncols, stage, packed);
   if (shape != nullptr) {
     shape[0] = t.variant; shape[1] = t.waves; shape[2] = t.nt; shape[3] = t.depth;
   }
@@ -670,6 +672,39 @@ void vk_hip_moe_gateup_mxfp4(
   const hipError_t before = hipPeekAtLastError();
   vk::launch_moe_gateup(a, static_cast<hipStream_t>(stream));
   note_launch_error("vk_hip_moe_gateup_mxfp4", before);
+}
+
+void vk_hip_moe_gateup_mxfp4_ex(
+    const uint16_t* A, const uint8_t* w13, const uint8_t* w13_scale,
+    uint16_t* act_scratch, int M, int hidden, int ispp, int top_k,
+    const int32_t* sorted_ids, const int32_t* expert_ids, int EM,
+    float swiglu_limit, int activation, float beta, float linear_beta,
+    const float* b13, int block_size, const void* w13_packed, int num_experts, void* stream) {
+  if (M <= 0 || EM <= 0) return;
+  vk::FusedMoeArgs a{};
+  a.A = A; a.w13 = w13; a.w13_scale = w13_scale; a.act = act_scratch;
+  a.sorted_ids = sorted_ids; a.expert_ids = expert_ids; a.b13 = b13;
+  a.M = M; a.hidden = hidden; a.ispp = ispp; a.top_k = top_k; a.EM = EM;
+  a.block_size = block_size; a.swiglu_limit = swiglu_limit; a.beta = beta;
+  a.linear_beta = linear_beta; a.activation = activation;
+  a.w13_packed = static_cast<const uint8_t*>(w13_packed);
+  a.num_experts = num_experts;
+  const bool packed_only = w13 == nullptr && w13_scale == nullptr && w13_packed != nullptr;
+  if (!layer_args_ok("vk_hip_moe_gateup_mxfp4_ex", true, false, a, packed_only)) return;
+  if (w13_packed != nullptr && num_experts <= 0) {
+    vk_set_last_error(VK_ERROR_INVALID_ARGUMENT,
+                      "vk_hip_moe_gateup_mxfp4_ex: num_experts must be positive with packed weights");
+    return;
+  }
+  if (packed_only && !vk::moe_gateup_packed_only_ok(a)) {
+    vk_set_last_error(VK_ERROR_INVALID_ARGUMENT,
+                      "vk_hip_moe_gateup_mxfp4_ex: without the raw weights the first stage alone runs "
+                      "at decode sizes only");
+    return;
+  }
+  const hipError_t before = hipPeekAtLastError();
+  vk::launch_moe_gateup(a, static_cast<hipStream_t>(stream));
+  note_launch_error("vk_hip_moe_gateup_mxfp4_ex", before);
 }
 
 void vk_hip_moe_down_mxfp4(

@@ -2050,15 +2050,10 @@ bool launch_resident(const GemmArgs& g, size_t lds, hipStream_t stream) {
 }
 
 // Launch shape of one stage.  variant kMoeVariantLds = the tile kernel.
-// The shapes the packed instantiations of the resident kernel exist for: the ones the
-// compiled-in rules return (a record of the tuning store is for the raw form's shapes).
-#define VK_PACKED_VARIANTS(X) X(0, 8, 2, 2) X(0, 4, 2, 8) X(1, 8, 1, 4) X(1, 8, 2, 4) X(1, 8, 1, 6)
-#define VK_PACKED_KSPLIT_VARIANTS(X) X(0, 8, 2, 4) X(1, 8, 1, 8) X(1, 8, 2, 4)
-
 struct StagePlan {
   int variant, waves, nt, depth;
   bool ksplit;  // the resident kernel with K shared between the wavefronts of a unit
-  bool packed;  // ... reading the prepacked form (the stage has no raw weights)
+  bool packed;  // ... reading the prepacked form (whenever the caller gives it)
   size_t resident_lds;
 };
 
@@ -2066,9 +2061,11 @@ template <int STAGE>
 StagePlan plan_stage(const GemmArgs& g) {
   // a record of the tuning store first, then the compiled-in rules
   MoeTile tile;
-  const bool packed = g.W == nullptr && g.Wp != nullptr;
-  if (packed || !moe_tuning_find(STAGE, g.K, g.ncols, g.n_flat, &tile))
-    tile = pick_moe_tile(g.n_flat, g.K, g.ncols, STAGE);
+  // The prepacked form whenever the caller gives it: its decode kernels are the faster
+  // ones (no scale block to park, nothing to check or fix in the loop).
+  const bool packed = g.Wp != nullptr && !(STAGE == 0 && g.ncols % 64 != 0);
+  if (!moe_tuning_find(STAGE, g.K, g.ncols, g.n_flat, &tile))
+    tile = pick_moe_tile(g.n_flat, g.K, g.ncols, STAGE, packed);
   StagePlan pl;
   pl.packed = packed;
   pl.ksplit = tile.variant == kMoeVariantResidentKSplit;
@@ -2085,7 +2082,6 @@ StagePlan plan_stage(const GemmArgs& g) {
   const int res_units = STAGE == 0 ? g.ncols / (8 * pl.nt) : g.ncols / (16 * pl.nt);
   if (pl.resident_lds > kResidentLdsLimit || g.num_blocks > kMaxRuns ||
       (!packed && pl.nt * groups > 64 * resident_scale_pieces(pl.waves)) ||
-      (packed && STAGE == 0 && g.ncols % 64 != 0) ||  // (what the prepacked form asks of the first stage)
       (res_units + pl.waves - 1) / pl.waves > 64 ||  // one bit per unit in a wavefront's redo mask
       nsteps * 4 > resident_batch(pl.waves) * pl.waves)  // the rows are staged in one batch
     pl.variant = kMoeVariantLds;
@@ -2112,22 +2108,23 @@ bool wide_kernel_applies(const GemmArgs& g) { return g.Aq != nullptr; }
 
 template <int STAGE>
 void launch_stage(const GemmArgs& g, const StagePlan& pl, hipStream_t stream) {
-  if (pl.packed) {  // (the callers keep stages that are not resident away from here)
+  // (a stage without raw weights that is not resident is kept away from here by the callers)
+  if (pl.packed && pl.variant == kMoeVariantResident) {
 #define VK_RESIDENT(S_, W_, NT_, D_) \
   if constexpr (STAGE == S_) { \
     if (pl.ksplit && pl.waves == W_ && pl.nt == NT_ && pl.depth == D_ && \
         launch_resident<S_, W_, NT_, D_, true, false, true>(g, pl.resident_lds, stream)) \
       return; \
   }
-    VK_PACKED_KSPLIT_VARIANTS(VK_RESIDENT)
+    VK_KSPLIT_VARIANTS(VK_RESIDENT)
 #undef VK_RESIDENT
 #define VK_RESIDENT(S_, W_, NT_, D_) \
   if constexpr (STAGE == S_) { \
-    if (!pl.ksplit && pl.waves == W_ && pl.nt == NT_ && pl.depth == D_ && \
+    if (pl.waves == W_ && pl.nt == NT_ && pl.depth == D_ && \
         launch_resident<S_, W_, NT_, D_, false, false, true>(g, pl.resident_lds, stream)) \
       return; \
   }
-    VK_PACKED_VARIANTS(VK_RESIDENT)
+    VK_RESIDENT_VARIANTS(VK_RESIDENT)
 #undef VK_RESIDENT
     return;
   }
@@ -2275,6 +2272,14 @@ bool fused_moe_packed_only_ok(const FusedMoeArgs& a) {
   return fused_moe_prepacked_takes(a, true);
 }
 
+bool moe_gateup_packed_only_ok(const FusedMoeArgs& a) {
+  if (a.w13_packed == nullptr || a.num_experts <= 0) return false;
+  if (a.M <= 0 || a.EM <= 0 || a.block_size <= 0) return true;
+  const GemmArgs g = gateup_args(a);
+  const StagePlan pl = plan_stage<0>(g);
+  return pl.packed && pl.variant == kMoeVariantResident;
+}
+
 bool moe_down_packed_only_ok(const FusedMoeArgs& a) {
   if (a.w2_packed == nullptr || a.num_experts <= 0) return false;
   if (a.M <= 0 || a.EM <= 0 || a.block_size <= 0) return true;
@@ -2323,10 +2328,10 @@ bool prepare_moe_kernels() {
 #undef VK_READY
   ok = resident_kernel_ready<0, 8, 2, 4, true, true>() && resident_kernel_ready<0, 8, 2, 2, false, true>() && ok;
 #define VK_READY(S_, W_, NT_, D_) ok = resident_kernel_ready<S_, W_, NT_, D_, false, false, true>() && ok;
-  VK_PACKED_VARIANTS(VK_READY)
+  VK_RESIDENT_VARIANTS(VK_READY)
 #undef VK_READY
 #define VK_READY(S_, W_, NT_, D_) ok = resident_kernel_ready<S_, W_, NT_, D_, true, false, true>() && ok;
-  VK_PACKED_KSPLIT_VARIANTS(VK_READY)
+  VK_KSPLIT_VARIANTS(VK_READY)
 #undef VK_READY
   ok = resident_kernel_ready<0, 8, 2, 4, true, true, true>() && resident_kernel_ready<0, 8, 2, 2, false, true, true>() && ok;
   MoeTile unused;
@@ -2465,11 +2470,9 @@ void launch_fused_moe(const FusedMoeArgs& a, hipStream_t stream) {
   // Without raw weights the decode kernels' packed forms take the call when both stages
   // are theirs, and the prepacked kernels any other (fused_moe_packed_only_ok has checked
   // that they can: the tile kernels below read raw weights).
-  if (p0.packed || p1.packed) {
-    if (p0.variant != kMoeVariantResident || p1.variant != kMoeVariantResident) {
-      (void)launch_fused_moe_prepacked(a, stream);
-      return;
-    }
+  if (a.w13 == nullptr && (p0.variant != kMoeVariantResident || p1.variant != kMoeVariantResident)) {
+    (void)launch_fused_moe_prepacked(a, stream);
+    return;
   }
   Workspace w;
   bool combine = false;

@@ -111,7 +111,10 @@ struct MoeTileRule {
 // part of K each.  Only the shapes whose rows of K values need 8 wavefronts to stage have it.
 constexpr int kMoeComputeUnits = 256;  // of the device the rules were swept on
 
-inline MoeTile pick_moe_tile(int n_flat, int K, int ncols, int stage) {
+// packed: the stage reads the prepacked form (its decode kernels have no scale block in
+// LDS and fewer registers in use, so their best shapes are swept separately).
+inline MoeTile pick_moe_tile(int n_flat, int K, int ncols, int stage, bool packed = false) {
+  (void)packed;
   if (n_flat <= kMoeDecodeMaxRows && K >= 1024 && K <= 3072) {
     const long long spare = (long long)kMoeComputeUnits * 4;  // half of 8 wavefronts per compute unit
     if (stage == 0 && (long long)n_flat * (ncols / 16) <= spare)

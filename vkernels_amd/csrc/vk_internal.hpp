@@ -94,6 +94,7 @@ bool fused_moe_prepacked_takes(const FusedMoeArgs& a, bool both_stages);
 // A call with the prepacked weights alone (w13 / w2 null): can the library run it?
 // (the layer; the second stage alone)
 bool fused_moe_packed_only_ok(const FusedMoeArgs& a);
+bool moe_gateup_packed_only_ok(const FusedMoeArgs& a);  // (decode sizes only)
 bool moe_down_packed_only_ok(const FusedMoeArgs& a);
 bool launch_moe_down_prepacked(const FusedMoeArgs& a, hipStream_t stream);
 void launch_split_rows_fp6(const uint16_t* x, int rows, int K, int terms, uint8_t* xq, uint8_t* row_bad,

@@ -4,6 +4,7 @@ the winners go to the tuning store the library reads (moe_fused.gfx950.tune).
 
     python -m vkernels_amd.tune_moe                      # the default shapes, markdown to stdout
     python -m vkernels_amd.tune_moe --store ~/.cache/vkernels/tuning --shapes 2880x2880x32x4
+    python -m vkernels_amd.tune_moe --packed             # the decode kernels that read the prepacked form
 
 A shape is HIDDENxINTERMEDIATExEXPERTSxTOP_K; each is swept at the token counts of
 --tokens.  One stage call is timed with HIP events over `--iters` launches that rotate
@@ -32,8 +33,21 @@ def time_stage(torch, ve, lib, fe_sets, stage, A, ids, tw, out, bs, iters):
     st = ve._P(torch.cuda.current_stream().cuda_stream)
     lib.vk_hip_moe_gateup_mxfp4.restype = None
     lib.vk_hip_moe_down_mxfp4.restype = None
+    lib.vk_hip_moe_gateup_mxfp4_ex.restype = None
+    lib.vk_hip_moe_down_mxfp4_ex.restype = None
 
     def call(f):
+        if f.w13_packed is not None:   # the prepacked form alone
+            if stage == 0:
+                lib.vk_hip_moe_gateup_mxfp4_ex(ve._ptr(A), None, None, ve._ptr(act), T, H, f.ispp, k, ve._ptr(sids),
+                                               ve._ptr(eids), max_em, ve._F(0.0), 0, ve._F(4.0), ve._F(25.0), None,
+                                               bs, ve._ptr(f.w13_packed), f.E, st)
+            else:
+                lib.vk_hip_moe_down_mxfp4_ex(ve._ptr(act), None, None, ve._ptr(tw), ve._ptr(out), T, H, f.ispp, k,
+                                             ve._ptr(sids), ve._ptr(eids), max_em, None, bs, None,
+                                             ve.ctypes.c_size_t(0), ve.ctypes.c_uint(0), ve._ptr(f.w2_packed),
+                                             f.E, st)
+            return
         if stage == 0:
             lib.vk_hip_moe_gateup_mxfp4(ve._ptr(A), ve._ptr(f.w13), ve._ptr(f.w13_scale), ve._ptr(act), T, H,
                                         f.ispp, k, ve._ptr(sids), ve._ptr(eids), max_em, ve._F(0.0), 0,
@@ -59,6 +73,9 @@ def main() -> None:
     ap.add_argument("--tokens", nargs="*", type=int, default=list(DEFAULT_TOKENS))
     ap.add_argument("--iters", type=int, default=40)
     ap.add_argument("--store", default=None, help="directory to write moe_fused.gfx950.tune into")
+    ap.add_argument("--packed", action="store_true",
+                    help="sweep the decode kernels that read the prepacked form (the weights are prepacked "
+                         "and the raw tensors let go of); shapes they do not take are skipped")
     args = ap.parse_args()
 
     import numpy as np
@@ -79,7 +96,9 @@ def main() -> None:
         fe_sets = []
         for s in range(min(n_sets, 8)):
             w = synth.make_weights(E, H, I, 900 + s, device=dev)
-            fe_sets.append(ve.FusedExperts(w.w13, w.w13_scale, w.w2, w.w2_scale))
+            fe_sets.append(ve.FusedExperts(w.w13, w.w13_scale, w.w2, w.w2_scale, prepack=args.packed,
+                                           keep_raw=not args.packed))
+            del w
         for T in args.tokens:
             if T * k > 512:
                 continue   # the tile kernels' side of the split: nothing to choose between
@@ -89,11 +108,19 @@ def main() -> None:
             out = torch.zeros((T, H), dtype=torch.float32, device=dev)
             bs = ve.default_block_size(T, k)
             for stage, K, ncols in ((0, H, I), (1, I, H)):
-                rule, _ = ve.moe_tile_query(stage, K, ncols, T * k)
+                rule, _ = ve.moe_tile_query(stage, K, ncols, T * k, packed=args.packed)
                 times = {}
                 for cand in ve.moe_tile_candidates(stage):
+                    if args.packed and cand[0] == 0:
+                        continue   # the tile kernels read the raw tensors
                     ve.moe_tile_set(stage, K, ncols, T * k, cand)
-                    times[cand] = time_stage(torch, ve, lib, fe_sets, stage, A, ids, tw, out, bs, args.iters)
+                    lib.vk_set_last_error(0, b"")
+                    t = time_stage(torch, ve, lib, fe_sets, stage, A, ids, tw, out, bs, args.iters)
+                    if int(lib.vk_last_error_code()) == 0:   # (refused: a shape the packed kernels do not take)
+                        times[cand] = t
+                if rule not in times:
+                    ve.moe_tile_set(stage, K, ncols, T * k, None)
+                    continue
                 best = min(times, key=times.get)
                 # keep the rule's shape unless another is faster by more than the noise of the measurement
                 keep = rule if times[rule] <= 1.02 * times[best] else best
