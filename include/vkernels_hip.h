@@ -592,11 +592,14 @@ int vk_hip_moe_route_align(const float* logits, int32_t T, int32_t E, int32_t to
  * (logits [M, num_experts] in; topk_ids, topk_w, sorted_ids [max_EM], expert_ids
  * [max_EM / block_size], out_EM out, written as that call writes them) and of
  * vk_hip_fused_moe_mxfp4_prepacked (the layer's buffers, workspace, flags, optional
- * prepacked weights of num_local_experts experts).  For a handful of tokens (M <= 16,
- * M * top_k <= 128, num_experts <= 256, block_size 16, shapes the decode kernels take)
- * the first stage's kernel routes and aligns for itself and the step is two launches;
- * every other call runs vk_hip_moe_route_align and then the layer, so the results are
- * the same either way: the routing tables bit for bit, `out` as the layer computes it.
+ * prepacked weights of num_local_experts experts; with them the raw tensors may be
+ * NULL as for vk_hip_fused_moe_mxfp4_prepacked).  Up to 256 routed rows (M * top_k),
+ * with num_experts <= 256, block_size 16 and shapes the decode kernels take, the
+ * first stage's kernel aligns for itself: for a handful of tokens (M <= 16) it routes
+ * as well and the step is two launches; beyond, the router has its launch and the step
+ * is three.  Every other call runs vk_hip_moe_route_align and then the layer.  The
+ * results are the same either way: the routing tables bit for bit, `out` as the layer
+ * computes it.
  * M = 0 writes the alignment's sentinels and EM and leaves `out` as it is.  Returns
  * VK_OK or a VK_ERROR_* code; asynchronous on `stream`, no allocation.
  */

@@ -1,10 +1,12 @@
 """GPU parity of vk_hip_moe_route_layer_mxfp4 (router, alignment and the layer behind one
 call) through the C ABI.  For a handful of tokens the first stage's kernel routes and aligns
-for itself; the tables it leaves (topk_ids, topk_w, sorted_ids, expert_ids, EM) must be the
-oracle's bit for bit, every entry up to max_EM, exactly as the separate calls leave them, and
-the layer's output inside the same bounds as theirs.  Shapes either side of every limit of
-the two-launch form (16 tokens, 128 routed rows, 256 experts, K = 3072, a block size other
-than 16), which run the separate kernels behind the same entry point."""
+for itself; up to 256 routed rows the router has its launch and the first stage's kernel
+aligns from its ids.  The tables left (topk_ids, topk_w, sorted_ids, expert_ids, EM) must be
+the oracle's bit for bit, every entry up to max_EM, exactly as the separate calls leave them,
+and the layer's output inside the same bounds as theirs.  Shapes either side of every limit
+of these forms (16 tokens, 256 routed rows, 256 experts, K = 3072 / 4096, a block size other
+than 16), which run the separate kernels behind the same entry point; on the raw tensors and
+on the prepacked form."""
 from __future__ import annotations
 
 import numpy as np
@@ -56,6 +58,18 @@ def test_route_layer_config1(T):
     _check(cfg, T, cfgs._weights(cfg, 1500), 6100 + T)
 
 
+@pytest.mark.parametrize("name,T", [("c1", 17), ("c1", 33), ("c1", 64), ("c1", 65), ("c2", 64), ("c4", 33),
+                                    ("c4", 42), ("c4", 43), ("c0", 128)])
+@pytest.mark.parametrize("packed", [False, True])
+def test_route_layer_aligning_in_the_first_stage(name, T, packed):
+    """More than 16 tokens, up to 256 routed rows (c1 T=64, c4 T=42, c0 T=128 are the last that
+    fit; c1 T=65 and c4 T=43 the first that do not): the router's launch, then the first stage
+    aligning for itself."""
+    cfg = synth.CONFIGS[name]
+    kw = dict(prepack=True, keep_raw=False) if packed else {}
+    _check(cfg, T, cfgs._weights(cfg), 6150 + T, **kw)
+
+
 @pytest.mark.parametrize("T", [1, 7, 16, 33])
 def test_route_layer_config2_zipf(T):
     cfg = synth.CONFIGS["c2"]       # 128 experts, a few of them popular
@@ -97,8 +111,9 @@ def test_route_layer_with_an_expert_map():
     local_n = cfg.E // 2
     emap = np.full(cfg.E, -1, dtype=np.int32)
     emap[np.sort(rng.permutation(cfg.E)[:local_n])] = np.arange(local_n, dtype=np.int32)
-    for T in (1, 9, 40):
+    for T in (1, 9, 40, 64):
         _check(cfg, T, cfgs._weights(cfg, 1500), 6600 + T, expert_map=emap, local_n=local_n)
+    _check(cfg, 50, cfgs._weights(cfg, 1500), 6650, expert_map=emap, local_n=local_n, prepack=True, keep_raw=False)
 
 
 def test_route_layer_equals_the_separate_calls():
@@ -106,7 +121,7 @@ def test_route_layer_equals_the_separate_calls():
     differs by the spread of the second stage's atomic adds only."""
     cfg = synth.CONFIGS["c1"]
     w = cfgs._weights(cfg, 1500)
-    for T in (1, 4, 16):
+    for T in (1, 4, 16, 48):
         A_bits, lg = cfgs._inputs(cfg, T, 6700 + T)
         fe = ve.FusedExperts(w.w13, w.w13_scale, w.w2, w.w2_scale, scratch=ve.CaptureSafeScratch())
         A, d_lg = to_dev(A_bits, torch.bfloat16), to_dev(lg)

@@ -507,7 +507,12 @@ __host__ __device__ constexpr int resident_batch(int waves) { return waves == 4 
 // ranks every routed row inside its expert's blocks, all in LDS, which is what
 // route_align_kernel does per workgroup as well; workgroup 0 also writes topk_ids, topk_w,
 // sorted_ids, expert_ids and EM out, exactly as vk_hip_moe_route_align leaves them.
-constexpr int kRouteMaxRows = 128, kRouteMaxExperts = 256, kRoutePer = kRouteMaxExperts / 64;
+// ROUTE = 2 is the same without the router: topk_ids comes from the router's own launch
+// (with more than a handful of tokens every workgroup routing all of them costs more than
+// that launch) and the kernel only aligns, which saves the alignment's launch and this
+// kernel's listing of the runs.
+constexpr int kRouteMaxRows = 256, kRouteMaxExperts = 256, kRoutePer = kRouteMaxExperts / 64;
+constexpr int kRouteMaxTokens = 16;  // ROUTE = 1: tokens every workgroup routes for itself
 
 // A workgroup barrier for LDS alone.  __syncthreads() is a workgroup-wide fence as well,
 // which makes a wavefront wait for every global load it has in flight (s_waitcnt vmcnt(0)):
@@ -524,9 +529,9 @@ __device__ __forceinline__ void lds_barrier() {
 // and the scale bytes (already less one) come with the step, four to a lane, so there is
 // no scale block to park in LDS and nothing to check in the loop: a unit that needs the
 // exact path carries a flag, looked up when the unit is begun.
-template <int STAGE, int WAVES, int NT, int D, bool KSPLIT = false, bool ROUTE = false, bool PACKED = false>
+template <int STAGE, int WAVES, int NT, int D, bool KSPLIT = false, int ROUTE = 0, bool PACKED = false>
 __global__ __launch_bounds__(64 * WAVES) void stream_resident_kernel(GemmArgs p) {
-  static_assert(!ROUTE || STAGE == 0, "the routed form is the first stage's");
+  static_assert(ROUTE == 0 || STAGE == 0, "the routed form is the first stage's");
   static_assert(!PACKED || (WAVES * (STAGE == 0 ? 8 * NT : 16 * NT)) % (STAGE == 0 ? 64 : 128) == 0,
                 "a wavefront's consecutive units are whole packed units apart");
   extern __shared__ u32x4 b_lds[];  // [nsteps][2][2][64] operand planes, block scales, weight scales
@@ -537,7 +542,7 @@ __global__ __launch_bounds__(64 * WAVES) void stream_resident_kernel(GemmArgs p)
   // block of the expert), the 16 flat indices of every run (0xFF = padding), the run count
   __shared__ short rt_le[ROUTE ? kRouteMaxRows : 1];
   __shared__ int rt_hist[ROUTE ? kRouteMaxExperts : 1];
-  __shared__ unsigned char run_ids[ROUTE ? kRouteMaxRows * 16 : 1];
+  __shared__ unsigned short run_ids[ROUTE ? kRouteMaxRows * 16 : 1];
   __shared__ int rt_runs;
   __shared__ int slice_sh[2];           // this workgroup's slice of the (run, unit) space
   __shared__ int pass_slow[2];          // set while staging: this pass takes the exact path
@@ -580,8 +585,19 @@ __global__ __launch_bounds__(64 * WAVES) void stream_resident_kernel(GemmArgs p)
     // ---- router: a wavefront per token; the table of local experts stays in LDS ----
     const int n_flat = p.n_flat, top_k = p.top_k, T = n_flat / top_k;
     for (int i = tid; i < kRouteMaxExperts; i += 64 * WAVES) rt_hist[i] = 0;
-    for (int i = tid; i < kRouteMaxRows * 16; i += 64 * WAVES) run_ids[i] = 0xFF;
-    for (int token = wave; token < T; token += WAVES) {  // uniform per wavefront
+    for (int i = tid; i < kRouteMaxRows * 16; i += 64 * WAVES) run_ids[i] = 0xFFFF;
+    if constexpr (ROUTE == 2) {  // the ids are the router's: the local expert of every routed row
+      for (int i = tid; i < n_flat; i += 64 * WAVES) {
+        const int id = p.rt_topk_ids[i];
+        int le = -1;
+        if (id >= 0 && id < p.rt_experts) {
+          le = p.rt_expert_map != nullptr ? p.rt_expert_map[id] : id;
+          if (le < 0 || le >= p.rt_local_n) le = -1;
+        }
+        rt_le[i] = (short)le;
+      }
+    }
+    for (int token = wave; ROUTE == 1 && token < T; token += WAVES) {  // uniform per wavefront
       int my_id;
       float my_w;
       route_token<kRoutePer>(p.rt_logits + (size_t)token * p.rt_experts, p.rt_experts, top_k,
@@ -643,7 +659,7 @@ __global__ __launch_bounds__(64 * WAVES) void stream_resident_kernel(GemmArgs p)
       if (le >= 0) {
         int rank = 0;
         for (int j = 0; j < i; ++j) rank += rt_le[j] == le ? 1 : 0;
-        run_ids[rt_hist[le] * 16 + rank] = (unsigned char)i;
+        run_ids[rt_hist[le] * 16 + rank] = (unsigned short)i;
       }
     }
     __syncthreads();
@@ -653,7 +669,7 @@ __global__ __launch_bounds__(64 * WAVES) void stream_resident_kernel(GemmArgs p)
       if (tid == 0) *p.rt_out_em = em;
       for (int r = tid; r < p.rt_max_em; r += 64 * WAVES) {
         int id = n_flat;
-        if (r < n_runs * 16 && run_ids[r] != 0xFF) id = run_ids[r];
+        if (r < n_runs * 16 && run_ids[r] != 0xFFFF) id = run_ids[r];
         p.rt_sorted_ids[r] = id;
       }
       for (int b = tid; b < p.rt_max_em / 16; b += 64 * WAVES) p.rt_expert_ids[b] = b < n_runs ? run_expert[b] : -1;
@@ -960,7 +976,7 @@ __global__ __launch_bounds__(64 * WAVES) void stream_resident_kernel(GemmArgs p)
         // uniform: the first rows a workgroup stages come from the copy in LDS
         if constexpr (ROUTE) {
           const int x = run_ids[at];  // (a run is a block of 16 rows: index = the sorted row)
-          fl = x == 0xFF ? -1 : x;
+          fl = x == 0xFFFF ? -1 : x;
         } else if (pass_no == 0 && run_row0 + tile0 * 16 + 64 <= ids_cached) {
           fl = ids_lds[at];
         } else {
@@ -2026,22 +2042,25 @@ int num_compute_units() {
 }
 
 constexpr size_t kResidentLdsLimit = 150 * 1024;  // dynamic LDS the resident kernel may ask for
+// ... and its routed forms, whose tables are 10 KB of static LDS over the plain form's
+constexpr size_t kRoutedStaticLds = 10 * 1024;
+constexpr size_t kRoutedLdsLimit = kResidentLdsLimit - kRoutedStaticLds;
 
 // True when the device grants the kernel its dynamic LDS (asked once per kernel;
 // a refusal makes the caller take the other variant).
-template <int STAGE, int WAVES, int NT, int D, bool KSPLIT = false, bool ROUTE = false, bool PACKED = false>
+template <int STAGE, int WAVES, int NT, int D, bool KSPLIT = false, int ROUTE = 0, bool PACKED = false>
 bool resident_kernel_ready() {
   static const bool configured = [] {
     const hipError_t err = hipFuncSetAttribute(
         reinterpret_cast<const void*>(stream_resident_kernel<STAGE, WAVES, NT, D, KSPLIT, ROUTE, PACKED>),
-        hipFuncAttributeMaxDynamicSharedMemorySize, (int)kResidentLdsLimit);
+        hipFuncAttributeMaxDynamicSharedMemorySize, (int)(ROUTE != 0 ? kRoutedLdsLimit : kResidentLdsLimit));
     if (err != hipSuccess) (void)hipGetLastError();  // not left for the next caller to find
     return err == hipSuccess;
   }();
   return configured;
 }
 
-template <int STAGE, int WAVES, int NT, int D, bool KSPLIT = false, bool ROUTE = false, bool PACKED = false>
+template <int STAGE, int WAVES, int NT, int D, bool KSPLIT = false, int ROUTE = 0, bool PACKED = false>
 bool launch_resident(const GemmArgs& g, size_t lds, hipStream_t stream) {
   if (!resident_kernel_ready<STAGE, WAVES, NT, D, KSPLIT, ROUTE, PACKED>()) return false;
   hipLaunchKernelGGL((stream_resident_kernel<STAGE, WAVES, NT, D, KSPLIT, ROUTE, PACKED>), dim3(num_compute_units()),
@@ -2113,7 +2132,7 @@ void launch_stage(const GemmArgs& g, const StagePlan& pl, hipStream_t stream) {
 #define VK_RESIDENT(S_, W_, NT_, D_) \
   if constexpr (STAGE == S_) { \
     if (pl.ksplit && pl.waves == W_ && pl.nt == NT_ && pl.depth == D_ && \
-        launch_resident<S_, W_, NT_, D_, true, false, true>(g, pl.resident_lds, stream)) \
+        launch_resident<S_, W_, NT_, D_, true, 0, true>(g, pl.resident_lds, stream)) \
       return; \
   }
     VK_KSPLIT_VARIANTS(VK_RESIDENT)
@@ -2121,7 +2140,7 @@ void launch_stage(const GemmArgs& g, const StagePlan& pl, hipStream_t stream) {
 #define VK_RESIDENT(S_, W_, NT_, D_) \
   if constexpr (STAGE == S_) { \
     if (pl.waves == W_ && pl.nt == NT_ && pl.depth == D_ && \
-        launch_resident<S_, W_, NT_, D_, false, false, true>(g, pl.resident_lds, stream)) \
+        launch_resident<S_, W_, NT_, D_, false, 0, true>(g, pl.resident_lds, stream)) \
       return; \
   }
     VK_RESIDENT_VARIANTS(VK_RESIDENT)
@@ -2326,38 +2345,43 @@ bool prepare_moe_kernels() {
 #define VK_READY(S_, W_, NT_, D_) ok = resident_kernel_ready<S_, W_, NT_, D_, true>() && ok;
   VK_KSPLIT_VARIANTS(VK_READY)
 #undef VK_READY
-  ok = resident_kernel_ready<0, 8, 2, 4, true, true>() && resident_kernel_ready<0, 8, 2, 2, false, true>() && ok;
-#define VK_READY(S_, W_, NT_, D_) ok = resident_kernel_ready<S_, W_, NT_, D_, false, false, true>() && ok;
+  ok = resident_kernel_ready<0, 8, 2, 4, true, 1>() && resident_kernel_ready<0, 8, 2, 2, false, 1>() && ok;
+  ok = resident_kernel_ready<0, 8, 2, 2, false, 2>() && resident_kernel_ready<0, 4, 2, 8, false, 2>() && ok;
+#define VK_READY(S_, W_, NT_, D_) ok = resident_kernel_ready<S_, W_, NT_, D_, false, 0, true>() && ok;
   VK_RESIDENT_VARIANTS(VK_READY)
 #undef VK_READY
-#define VK_READY(S_, W_, NT_, D_) ok = resident_kernel_ready<S_, W_, NT_, D_, true, false, true>() && ok;
+#define VK_READY(S_, W_, NT_, D_) ok = resident_kernel_ready<S_, W_, NT_, D_, true, 0, true>() && ok;
   VK_KSPLIT_VARIANTS(VK_READY)
 #undef VK_READY
-  ok = resident_kernel_ready<0, 8, 2, 4, true, true, true>() && resident_kernel_ready<0, 8, 2, 2, false, true, true>() && ok;
+  ok = resident_kernel_ready<0, 8, 2, 4, true, 1, true>() && resident_kernel_ready<0, 8, 2, 2, false, 1, true>() && ok;
+  ok = resident_kernel_ready<0, 8, 2, 2, false, 2, true>() && resident_kernel_ready<0, 4, 2, 8, false, 2, true>() && ok;
   MoeTile unused;
   (void)moe_tuning_find(0, 64, 64, 1, &unused);  // reads the tuning store now rather than on the first launch
   return ok;
 }
 
-// Router, alignment and the layer for a handful of tokens in two launches: the first
-// stage's decode kernel routes and aligns for itself (its routed form) and workgroup 0
-// writes the tables out, the second stage reads them.  False (nothing enqueued) when the
-// call is not one the routed form takes: more than 16 tokens or kRouteMaxRows routed rows,
+// Router, alignment and the layer with the alignment inside the first stage's decode
+// kernel (its routed forms), whose workgroup 0 writes the tables out for the second stage
+// and the caller.  Up to kRouteMaxTokens tokens the kernel routes as well: two launches a
+// step.  Beyond, up to kRouteMaxRows routed rows, the router has its launch and the kernel
+// aligns from its ids: three launches instead of four, and no run listing in the kernel.
+// False (nothing enqueued) when the call is not one these forms take: more routed rows or
 // more than kRouteMaxExperts experts, a block size other than 16, a first stage whose
-// launch shape has no routed form, or LDS that does not hold its tables as well.
+// launch shape has no routed form, or LDS that does not hold the tables as well.
 bool launch_routed_moe(const FusedMoeArgs& a, const RoutedArgs& r, hipStream_t stream) {
-  if (a.M <= 0 || a.M > 16 || a.M * a.top_k > kRouteMaxRows || r.num_experts > kRouteMaxExperts ||
-      r.num_experts <= 0 || a.top_k > 64 || a.top_k > r.num_experts || a.block_size != 16 ||
+  if (a.M <= 0 || a.M * a.top_k > kRouteMaxRows || r.num_experts > kRouteMaxExperts ||
+      r.num_experts <= 0 || a.top_k > r.num_experts || a.block_size != 16 ||
       r.max_EM < 16 || r.max_EM % 16 != 0 || r.max_EM / 16 > kMaxRuns)
     return false;
+  const bool route_inside = a.M <= kRouteMaxTokens && a.top_k <= 64;
   FusedMoeArgs b = a;
   b.EM = r.max_EM;
   GemmArgs g0 = gateup_args(b);
   GemmArgs g1 = down_args(b);
   const StagePlan p0 = plan_stage<0>(g0), p1 = plan_stage<1>(g1);
   if (p0.variant != kMoeVariantResident || p1.variant != kMoeVariantResident) return false;
-  constexpr size_t kRoutedStaticLds = 6 * 1024;  // the routed form's tables, over the plain form's
-  if (p0.resident_lds + kRoutedStaticLds + 8 * 1024 > 160 * 1024) return false;
+  if (p0.packed != p1.packed) return false;  // (both packed forms or neither)
+  if (p0.resident_lds > kRoutedLdsLimit) return false;
   g0.rt_logits = r.logits;
   g0.rt_expert_map = r.expert_map;
   g0.rt_topk_ids = r.topk_ids;
@@ -2376,15 +2400,37 @@ bool launch_routed_moe(const FusedMoeArgs& a, const RoutedArgs& r, hipStream_t s
     g0.zero_out = a.out;
     g0.zero_count = (long long)a.M * a.hidden;
   }
-  bool launched = false;
-  if (p0.packed != p1.packed) return false;  // (both packed forms or neither)
-  if (p0.ksplit && p0.waves == 8 && p0.nt == 2 && p0.depth == 4)
-    launched = p0.packed ? launch_resident<0, 8, 2, 4, true, true, true>(g0, p0.resident_lds, stream)
-                         : launch_resident<0, 8, 2, 4, true, true>(g0, p0.resident_lds, stream);
-  else if (!p0.ksplit && p0.waves == 8 && p0.nt == 2 && p0.depth == 2)
-    launched = p0.packed ? launch_resident<0, 8, 2, 2, false, true, true>(g0, p0.resident_lds, stream)
-                         : launch_resident<0, 8, 2, 2, false, true>(g0, p0.resident_lds, stream);
-  if (!launched) return false;
+  // the routed instantiation of the planned shape: is it there and ready?
+  const int shape = p0.ksplit && p0.waves == 8 && p0.nt == 2 && p0.depth == 4 ? 1
+                    : !p0.ksplit && p0.waves == 8 && p0.nt == 2 && p0.depth == 2 ? 2
+                    : !p0.ksplit && p0.waves == 4 && p0.nt == 2 && p0.depth == 8 ? 3 : 0;
+  bool ready = false;
+  if (route_inside) {
+    if (shape == 1) ready = p0.packed ? resident_kernel_ready<0, 8, 2, 4, true, 1, true>() : resident_kernel_ready<0, 8, 2, 4, true, 1>();
+    if (shape == 2) ready = p0.packed ? resident_kernel_ready<0, 8, 2, 2, false, 1, true>() : resident_kernel_ready<0, 8, 2, 2, false, 1>();
+  } else {
+    if (shape == 2) ready = p0.packed ? resident_kernel_ready<0, 8, 2, 2, false, 2, true>() : resident_kernel_ready<0, 8, 2, 2, false, 2>();
+    if (shape == 3) ready = p0.packed ? resident_kernel_ready<0, 4, 2, 8, false, 2, true>() : resident_kernel_ready<0, 4, 2, 8, false, 2>();
+  }
+  if (!ready) return false;
+  if (route_inside) {
+    if (shape == 1) {
+      if (p0.packed) launch_resident<0, 8, 2, 4, true, 1, true>(g0, p0.resident_lds, stream);
+      else launch_resident<0, 8, 2, 4, true, 1>(g0, p0.resident_lds, stream);
+    } else {
+      if (p0.packed) launch_resident<0, 8, 2, 2, false, 1, true>(g0, p0.resident_lds, stream);
+      else launch_resident<0, 8, 2, 2, false, 1>(g0, p0.resident_lds, stream);
+    }
+  } else {
+    launch_route_topk(r.logits, a.M, r.num_experts, a.top_k, r.renormalize, r.topk_ids, r.topk_w, stream);
+    if (shape == 2) {
+      if (p0.packed) launch_resident<0, 8, 2, 2, false, 2, true>(g0, p0.resident_lds, stream);
+      else launch_resident<0, 8, 2, 2, false, 2>(g0, p0.resident_lds, stream);
+    } else {
+      if (p0.packed) launch_resident<0, 4, 2, 8, false, 2, true>(g0, p0.resident_lds, stream);
+      else launch_resident<0, 4, 2, 8, false, 2>(g0, p0.resident_lds, stream);
+    }
+  }
   g1.topk_w = r.topk_w;
   launch_stage<1>(g1, p1, stream);
   return true;
