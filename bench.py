@@ -202,7 +202,7 @@ def run_workload(args, workload, steps, warmup, prepack, split_terms=None, w4a4=
     A = torch.from_numpy(A_bits.view(np.int16)).view(torch.bfloat16).to(dev)
     logits = torch.from_numpy(logits_np).to(dev)
     out = torch.empty((T, H), dtype=torch.float32, device=dev)
-    bs = args.block_size or ve.default_block_size(T, k)
+    bs = args.block_size or experts[0].block_size_for(T, k)
     lib = ve.load_libvkernels_hip()
     lib.vk_hip_moe_gateup_mxfp4_ex.restype = None
     lib.vk_hip_moe_down_mxfp4_ex.restype = None

@@ -269,6 +269,11 @@ int vk_hip_init(void);
  * vk_hip_moe_default_block_size: the alignment block the kernels like best for
  * M tokens routed to top_k experts each (what to pass to
  * vk_hip_moe_align_block_size and on to the layer).  Any multiple of 16 works.
+ * vk_hip_moe_default_block_size_ex: the same for a caller that gives the prepacked
+ * weights of num_local_experts experts of a hidden x ispp layer: what decides between
+ * the decode kernels (blocks of 16) and the tile kernels (blocks of 128) is then rows per
+ * expert, and with blocks of 16 the decode kernels also take calls beyond 512 routed
+ * rows, up to 9 per expert (where they take the layer's widths at all).
  *
  * A launch shape is four ints {variant, wavefronts, tiles, depth}: variant 2 =
  * the decode kernel (one workgroup per compute unit, a run's rows resident in
@@ -293,6 +298,7 @@ int vk_hip_init(void);
  * returns the length the whole text needs.
  */
 int vk_hip_moe_default_block_size(int M, int top_k);
+int vk_hip_moe_default_block_size_ex(int M, int top_k, int num_local_experts, int hidden, int ispp);
 int vk_hip_moe_tile_candidates(int stage, int* shapes, int capacity);
 int vk_hip_moe_tile_query(int stage, int K, int ncols, int n_flat, int* shape);
 int vk_hip_moe_tile_set(int stage, int K, int ncols, int n_flat, const int* shape);

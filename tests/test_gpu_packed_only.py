@@ -56,6 +56,23 @@ def test_prefill_sizes_on_the_packed_form_alone(name, T):
     assert np.all(np.isfinite(a["out"]))
 
 
+@pytest.mark.parametrize("name,T", [("c4", 96), ("c2", 256), ("c2", 288)])
+def test_few_rows_per_expert_beyond_512_rows(name, T):
+    """A caller that gives the prepacked weights gets blocks of 16 and the decode kernels up to
+    9 routed rows per expert (576 rows on 64 experts; 1024 and 1152 on 128 with a few popular
+    ones, where some experts have a dozen passes): the exact-split bounds hold, and the call
+    with blocks of 128 (the prepacked tile kernels) agrees."""
+    cfg = synth.CONFIGS[name]
+    w = cfgs._weights(cfg)
+    A, lg = cfgs._inputs(cfg, T, 6300 + T)
+    g, wn = cfgs._check(cfg, T, w, A, lg, gpu_kw=PACKED_ONLY, tight=True,
+                        block_size=ve.default_block_size(T, cfg.top_k, packed_experts=cfg.E, hidden=cfg.H, ispp=cfg.I))
+    assert g["bs"] == 16 and T * cfg.top_k > 512
+    t = cfgs._run_gpu(cfg, w, A, lg, 128, True, **PACKED_ONLY)
+    m, l2, nf = error_metrics(g["out"], t["out"])
+    assert nf and l2 <= 1.5e-3, (m, l2)
+
+
 @pytest.mark.parametrize("T", [4, 300])
 def test_values_outside_the_range_on_the_packed_form_alone(T):
     """inf/NaN codes and out-of-range scale bytes in some experts (flagged units, which keep

@@ -50,6 +50,17 @@ def test_default_block_size():
     assert ve.default_block_size(64, 4) == 16 and ve.default_block_size(128, 4) == 16
     assert ve.default_block_size(129, 4) == 128 and ve.default_block_size(2047, 8) == 128
     assert ve.default_block_size(2048, 8) == 128 and ve.default_block_size(16384, 8) == 128
+    # a caller that gives the prepacked weights: by rows per expert as well (9), as long as
+    # the runs (a block per 16 rows and one more per expert) fit the decode kernels' list of 512
+    # and the decode kernels take the layer's widths
+    c4 = dict(packed_experts=64, hidden=4096, ispp=1536)
+    assert ve.default_block_size(96, 6, **c4) == 16 and ve.default_block_size(97, 6, **c4) == 128     # 576 / 582 rows
+    c2 = dict(packed_experts=128, hidden=2880, ispp=2880)
+    assert ve.default_block_size(288, 4, **c2) == 16 and ve.default_block_size(289, 4, **c2) == 128
+    assert ve.default_block_size(128, 4, packed_experts=8, hidden=2880, ispp=2880) == 16   # 512 rows: decode-sized anyway
+    assert ve.default_block_size(129, 4, packed_experts=8, hidden=2880, ispp=2880) == 128
+    assert ve.default_block_size(250, 8, packed_experts=256, hidden=7168, ispp=2048) == 128   # rows too wide for them
+    assert ve.default_block_size(512, 8, packed_experts=500, hidden=2880, ispp=2880) == 128   # room for 12 runs only
 
 
 @pytest.mark.parametrize("M,top_k,E,bs", [(1, 1, 8, 16), (4, 2, 8, 16), (64, 4, 32, 64),

@@ -565,6 +565,11 @@ int vk_hip_moe_default_block_size(int M, int top_k) {
   return vk::moe_default_block_size(M < 0 ? 0 : M, top_k < 0 ? 0 : top_k);
 }
 
+int vk_hip_moe_default_block_size_ex(int M, int top_k, int num_local_experts, int hidden, int ispp) {
+  return vk::moe_default_block_size(M < 0 ? 0 : M, top_k < 0 ? 0 : top_k,
+                                    num_local_experts < 0 ? 0 : num_local_experts, hidden, ispp);
+}
+
 int vk_hip_moe_tile_candidates(int stage, int* shapes, int capacity) {
   size_t n = 0;
   const vk::MoeTileCandidate* table = vk::moe_tile_candidates(&n);

@@ -63,6 +63,7 @@ struct GemmArgs {
   const uint8_t* Wp;
   const uint8_t* Wpf;
   int p_units;
+  int p_experts;            // experts in the prepacked weights
   const int32_t* sorted_ids;
   const int32_t* expert_ids;
   const float* topk_w;      // stage 1
@@ -335,7 +336,7 @@ __device__ __forceinline__ bool packed_unit_flagged(const GemmArgs& p, int e, in
 // 16 h + 15).  Planes past K are zero, so the last, partial K step needs no
 // masking of the weight side.
 // ---------------------------------------------------------------------------
-constexpr int kMaxRuns = 512;   // runs the resident kernel can list in LDS
+constexpr int kMaxRuns = kMoeMaxRuns;   // runs the resident kernel can list in LDS
 // 16-byte scale pieces of a unit a lane holds: NT * K/32 <= 64 * resident_scale_pieces.
 // Workgroups of 8 wavefronts stage K <= 3072 (resident_batch), 96 groups, and have
 // 256 registers a lane: three pieces are enough there, and a fourth would cost four registers.
@@ -2084,7 +2085,7 @@ StagePlan plan_stage(const GemmArgs& g) {
   // ones (no scale block to park, nothing to check or fix in the loop).
   const bool packed = g.Wp != nullptr && !(STAGE == 0 && g.ncols % 64 != 0);
   if (!moe_tuning_find(STAGE, g.K, g.ncols, g.n_flat, &tile))
-    tile = pick_moe_tile(g.n_flat, g.K, g.ncols, STAGE, packed);
+    tile = pick_moe_tile(g.n_flat, g.K, g.ncols, STAGE, packed, packed && g.block_size == 16 ? g.p_experts : 0);
   StagePlan pl;
   pl.packed = packed;
   pl.ksplit = tile.variant == kMoeVariantResidentKSplit;
@@ -2250,6 +2251,7 @@ GemmArgs gateup_args(const FusedMoeArgs& a) {
   g.Ws = a.w13_scale;
   if (a.w13_packed != nullptr) {
     g.p_units = mx_units(0, a.ispp);
+    g.p_experts = a.num_experts;
     g.Wp = a.w13_packed;
     g.Wpf = a.w13_packed + mx_packed_body_bytes(a.num_experts, g.p_units, mx_kp(a.hidden) / 128);
   }
@@ -2267,6 +2269,7 @@ GemmArgs down_args(const FusedMoeArgs& a) {
   g.Ws = a.w2_scale;
   if (a.w2_packed != nullptr) {
     g.p_units = mx_units(1, a.hidden);
+    g.p_experts = a.num_experts;
     g.Wp = a.w2_packed;
     g.Wpf = a.w2_packed + mx_packed_body_bytes(a.num_experts, g.p_units, mx_kp(a.ispp) / 128);
   }

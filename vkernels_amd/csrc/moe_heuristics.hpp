@@ -71,6 +71,25 @@ inline bool is_moe_tile_candidate(int stage, const MoeTile& tile) {
 // experts have several 16-row passes and the tile kernels, which keep a 128-row window
 // per workgroup, read each weight byte once per window instead of once per pass.
 constexpr int kMoeDecodeMaxRows = 512;
+// A caller that gives the prepacked weights also says how many experts they hold, and
+// what decides between the families is rows per expert, not rows: a pass per 16 rows of an
+// expert against a window per expert.  With blocks of 16 the decode kernels then take
+// calls of up to this many routed rows per expert as well (measured on the prepacked
+// form, decode against tile kernels: 600 rows on 64 experts, 9.4 each, 164 against 195 us;
+// 636 rows, 9.9 each, 183 against 194 us; 1024 rows on 128 experts with a few popular ones,
+// 8 each, 226 against 255 us -- but 1280 rows there, 10 each, 272 against 256 us; 1530 on
+// 64, 24 each, 263 against 204 us; 1024 on 32: 199 against 156 us) -- as long as the runs
+// (a block of 16 per pass, one more per expert for its partly filled one) fit the run list.
+constexpr int kMoeDecodeRowsPerExpert = 9;
+constexpr int kMoeMaxRuns = 512;  // runs the decode kernel lists in LDS
+
+inline int moe_decode_max_rows(int packed_experts) {
+  if (packed_experts <= 0) return kMoeDecodeMaxRows;
+  const long long by_expert = (long long)kMoeDecodeRowsPerExpert * packed_experts;
+  const long long by_runs = 16ll * (kMoeMaxRuns - packed_experts);
+  const long long m = by_expert < by_runs ? by_expert : by_runs;
+  return m > kMoeDecodeMaxRows ? (int)m : kMoeDecodeMaxRows;
+}
 
 // One row of the decision table: the first row whose bounds hold decides.
 struct MoeTileRule {
@@ -113,8 +132,11 @@ constexpr int kMoeComputeUnits = 256;  // of the device the rules were swept on
 
 // packed: the stage reads the prepacked form (its decode kernels have no scale block in
 // LDS and fewer registers in use, so their best shapes are swept separately).
-inline MoeTile pick_moe_tile(int n_flat, int K, int ncols, int stage, bool packed = false) {
-  (void)packed;
+// packed_experts: their number when the call also comes in blocks of 16 (else 0): the
+// decode range then follows moe_decode_max_rows.
+inline MoeTile pick_moe_tile(int n_flat, int K, int ncols, int stage, bool packed = false,
+                             int packed_experts = 0) {
+  const int max_rows = moe_decode_max_rows(packed ? packed_experts : 0);
   if (n_flat <= kMoeDecodeMaxRows && K >= 1024 && K <= 3072) {
     const long long spare = (long long)kMoeComputeUnits * 4;  // half of 8 wavefronts per compute unit
     if (stage == 0 && (long long)n_flat * (ncols / 16) <= spare)
@@ -124,12 +146,12 @@ inline MoeTile pick_moe_tile(int n_flat, int K, int ncols, int stage, bool packe
     if (stage == 1 && (long long)n_flat * (ncols / 32) <= spare)
       return MoeTile{kMoeVariantResidentKSplit, 8, 2, 4};
   }
-  static const MoeTileRule rules[] = {
-      {0, kMoeDecodeMaxRows, 3072, {kMoeVariantResident, 8, 2, 2}},
-      {0, kMoeDecodeMaxRows, 4096, {kMoeVariantResident, 4, 2, 8}},
-      {1, kMoeDecodeMaxRows, 1024, {kMoeVariantResident, 8, 1, 4}},
+  const MoeTileRule rules[] = {
+      {0, max_rows, 3072, {kMoeVariantResident, 8, 2, 2}},
+      {0, max_rows, 4096, {kMoeVariantResident, 4, 2, 8}},
+      {1, max_rows, 1024, {kMoeVariantResident, 8, 1, 4}},
       {1, 24, 3072, {kMoeVariantResident, 8, 2, 4}},
-      {1, kMoeDecodeMaxRows, 3072, {kMoeVariantResident, 8, 1, 6}},
+      {1, max_rows, 3072, {kMoeVariantResident, 8, 1, 6}},
   };
   for (const MoeTileRule& r : rules)
     if (r.stage == stage && n_flat <= r.max_rows && K <= r.max_k) return r.tile;
@@ -141,9 +163,16 @@ inline MoeTile pick_moe_tile(int n_flat, int K, int ncols, int stage, bool packe
 // passes of every expert exactly and pad least.  Tile kernels: a workgroup takes a
 // window of 128 sorted rows of one expert, so blocks of 128 give every expert windows of
 // its own (0.5 to 8 % faster than blocks of 64 from 16 to 770 rows per expert).
-inline int moe_default_block_size(int M, int top_k) {
+// packed_experts, hidden, ispp: the number of (local) experts and the layer's widths when
+// the caller gives the prepacked weights, 0 otherwise: beyond kMoeDecodeMaxRows rows the
+// blocks are 16 only where the decode kernels take both stages.
+inline int moe_default_block_size(int M, int top_k, int packed_experts = 0, int hidden = 0, int ispp = 0) {
   const long long n = (long long)M * (long long)top_k;
-  return n <= kMoeDecodeMaxRows ? 16 : 128;
+  if (n <= kMoeDecodeMaxRows) return 16;
+  if (packed_experts <= 0 || hidden <= 0 || ispp <= 0 || n > moe_decode_max_rows(packed_experts)) return 128;
+  const bool decode = pick_moe_tile((int)n, hidden, ispp, 0, true, packed_experts).variant != kMoeVariantLds &&
+                      pick_moe_tile((int)n, ispp, hidden, 1, true, packed_experts).variant != kMoeVariantLds;
+  return decode ? 16 : 128;
 }
 
 }  // namespace vk

@@ -351,17 +351,24 @@ def _stream(torch):
 _scratch = CaptureSafeScratch()
 
 
-def default_block_size(M: int, top_k: int | None = None, lib=None) -> int:
+def default_block_size(M: int, top_k: int | None = None, lib=None, packed_experts: int = 0,
+                       hidden: int = 0, ispp: int = 0) -> int:
     """The reference's policy: 16-row alignment for decode batches, 64 above
     (vllm_experts.py:846).  With top_k given the library is asked what its kernels
     like best (vk_hip_moe_default_block_size: 16 while M * top_k routed rows run the
-    decode kernels, blocks of 128 for the tile kernels' windows beyond)."""
+    decode kernels, blocks of 128 for the tile kernels' windows beyond; packed_experts,
+    hidden, ispp: the number of local experts and the layer's widths of a caller that gives
+    the prepacked weights, for whom the decode kernels' range follows the rows per expert)."""
     if top_k is not None:
         lib = load_libvkernels_hip() if lib is None else lib
         fn = getattr(lib, "vk_hip_moe_default_block_size", None)
         if fn is None:
             raise RuntimeError("the loaded libvkernels_hip has no vk_hip_moe_default_block_size; "
                                "pass block_size, or call default_block_size(M) for the reference's policy")
+        if packed_experts > 0:
+            fn = lib.vk_hip_moe_default_block_size_ex
+            fn.restype, fn.argtypes = _I, [_I, _I, _I, _I, _I]
+            return int(fn(int(M), int(top_k), int(packed_experts), int(hidden), int(ispp)))
         fn.restype, fn.argtypes = _I, [_I, _I]
         return int(fn(int(M), int(top_k)))
     return 16 if M <= 32 else 64
@@ -500,6 +507,13 @@ class FusedExperts:
             torch.cuda.current_stream().synchronize()  # the packing kernels have read them
             self.w13 = self.w13_scale = self.w2 = self.w2_scale = None
 
+    def block_size_for(self, M: int, top_k: int) -> int:
+        """The alignment block the library's kernels like best for M tokens on these weights
+        (with prepacked weights the library is told how many experts they hold)."""
+        return default_block_size(M, top_k, self.lib,
+                                  packed_experts=self.local_n if self.w13_packed is not None else 0,
+                                  hidden=self.hidden, ispp=self.ispp)
+
     def prepack(self):
         """Build the prepacked copies of w13 and w2 (idempotent)."""
         if self.w13_packed is not None:
@@ -563,7 +577,7 @@ class FusedExperts:
         torch = self.torch
         T, E = logits.shape
         dev = logits.device
-        block_size = default_block_size(T, top_k) if block_size is None else block_size
+        block_size = self.block_size_for(T, top_k) if block_size is None else block_size
         if block_size <= 0 or block_size % 16 != 0:
             raise ValueError(f"block_size must be a positive multiple of 16, got {block_size}")
         logits = logits.contiguous()
@@ -597,7 +611,7 @@ class FusedExperts:
             raise ValueError(f"hidden size {K} does not match the weights ({self.hidden})")
         top_k = topk_ids.shape[1]
         dev = hidden_states.device
-        block_size = default_block_size(M, top_k) if block_size is None else block_size
+        block_size = self.block_size_for(M, top_k) if block_size is None else block_size
         if block_size <= 0 or block_size % 16 != 0:
             raise ValueError(f"block_size must be a positive multiple of 16, got {block_size}")
         hidden_states = hidden_states.contiguous()
@@ -688,7 +702,7 @@ class FusedExperts:
             raise ValueError(f"hidden size {K} does not match the weights ({self.hidden})")
         E = router_logits.shape[1]
         dev = hidden_states.device
-        block_size = default_block_size(M, top_k) if block_size is None else block_size
+        block_size = self.block_size_for(M, top_k) if block_size is None else block_size
         if block_size <= 0 or block_size % 16 != 0:
             raise ValueError(f"block_size must be a positive multiple of 16, got {block_size}")
         hidden_states = hidden_states.contiguous()
