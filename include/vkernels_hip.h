@@ -508,13 +508,17 @@ int vk_hip_moe_combine(const float* partial, const float* b2, const float* topk_
  * Additive: the two GEMM stages of the split above on prepacked weights, so that a
  * tensor-parallel caller at prefill sizes runs the FP4-rate kernels as the fused call
  * does.  w13_packed / w2_packed: vk_hip_moe_prepack_weights of the rank's shard
- * (K = hidden_k / ispp_k) of num_experts experts; the raw shard is still read where a
- * unit or a row leaves the fast path's range.  workspace:
+ * (K = hidden_k / ispp_k) of num_experts experts.  With it the raw shard (w13 /
+ * w13_scale, w2 / w2_scale) may be NULL: the exact paths read the packed form, and calls
+ * of up to 512 routed rows run the decode kernels on it; a call that would need the raw
+ * shard (no workspace at prefill sizes, a slice too wide for the decode kernels) is then
+ * refused with VK_ERROR_INVALID_ARGUMENT.  workspace:
  * vk_hip_moe_preact_workspace_bytes(stage, M, EM, k_dim) bytes, 16-byte aligned (the
  * split rows of the K slice).  flags: VK_HIP_MOE_SPLIT2 / _SPLIT3 as for the layer
  * (default: three FP6 terms per activation in the first stage, two in the second).
- * Calls of up to 512 routed rows, or without packed weights or workspace, run as
- * vk_hip_moe_gateup_preact / vk_hip_moe_down_preact do.  Same outputs, same rules:
+ * Calls of up to 512 routed rows, or without packed weights or workspace, run the decode
+ * or raw-weight kernels as vk_hip_moe_gateup_preact / vk_hip_moe_down_preact do (the
+ * decode kernels on the packed shard where it is given).  Same outputs, same rules:
  * routed rows only are written.
  */
 size_t vk_hip_moe_preact_workspace_bytes(int stage, int M, int EM, int k_dim);

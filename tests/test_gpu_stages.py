@@ -243,13 +243,16 @@ PREPACKED3_MAX_TOL, PREPACKED3_L2_TOL = 2e-3, 2e-4
 PREPACKED2_MAX_TOL, PREPACKED2_L2_TOL = 2e-2, 2e-3
 
 
-@pytest.mark.parametrize("name,T,bs,tp", [("c1", 300, 128, 1), ("c1", 600, 128, 2), ("c4", 255, 64, 3)])
-def test_prepacked_stages_against_the_oracle_and_in_composition(hip_lib, name, T, bs, tp):
+@pytest.mark.parametrize("name,T,bs,tp,raw", [("c1", 300, 128, 1, True), ("c1", 600, 128, 2, True),
+                                              ("c4", 255, 64, 3, True), ("c1", 600, 128, 2, False),
+                                              ("c4", 255, 64, 3, False), ("c1", 48, 16, 2, False)])
+def test_prepacked_stages_against_the_oracle_and_in_composition(hip_lib, name, T, bs, tp, raw):
     """vk_hip_moe_gateup_preact_prepacked / _down_preact_prepacked: every rank's K slice of the
     weights prepacked as its own shard, the A / act slice addressed inside the full rows; each
     stage against the oracle's function of the same name on the same slice (rows that are not
     routed left as they were), and the composition (slices summed, epilogues once) against
-    the fused oracle."""
+    the fused oracle.  raw = False: the shard's raw tensors are not passed (one copy of the
+    weights; decode-sized calls then run the decode kernels on the prepacked shard)."""
     lib = _prepacked_fns(hip_lib)
     cfg = synth.CONFIGS[name]
     H, I, k = cfg.H, cfg.I, cfg.top_k
@@ -277,7 +280,8 @@ def test_prepacked_stages_against_the_oracle_and_in_composition(hip_lib, name, T
         ws = torch.empty(need, dtype=torch.uint8, device=dev())
         part = torch.full((em, 2 * I), 7.0, dtype=torch.float32, device=dev())
         assert lib.vk_hip_moe_gateup_preact_prepacked(
-            d_A.data_ptr(), d_w.data_ptr(), d_s.data_ptr(), packed.data_ptr(), cfg.E, d_sids.data_ptr(),
+            d_A.data_ptr(), d_w.data_ptr() if raw else None, d_s.data_ptr() if raw else None, packed.data_ptr(),
+            cfg.E, d_sids.data_ptr(),
             d_eids.data_ptr(), part.data_ptr(), T, H, I, k, em, k_base, k_dim, bs, ws.data_ptr(), need, 0,
             None) == 0, ve.last_error(lib)
         torch.cuda.synchronize()
@@ -310,7 +314,8 @@ def test_prepacked_stages_against_the_oracle_and_in_composition(hip_lib, name, T
                                     (0, (PREPACKED2_MAX_TOL, PREPACKED2_L2_TOL))):
             part = torch.full((em, H), -3.0, dtype=torch.float32, device=dev())
             assert lib.vk_hip_moe_down_preact_prepacked(
-                act.data_ptr(), d_w.data_ptr(), d_s.data_ptr(), packed.data_ptr(), cfg.E, d_sids.data_ptr(),
+                act.data_ptr(), d_w.data_ptr() if raw else None, d_s.data_ptr() if raw else None, packed.data_ptr(),
+                cfg.E, d_sids.data_ptr(),
                 d_eids.data_ptr(), part.data_ptr(), T, I, H, k, em, k_base, k_dim, bs, ws.data_ptr(), need, flags,
                 None) == 0, ve.last_error(lib)
             torch.cuda.synchronize()

@@ -418,8 +418,9 @@ int preact_any(const char* who, int stage, const uint16_t* a, const uint8_t* w, 
   if (const char* why = stage_shape_error(M, width_a, ncols, top_k, EM, k_base, k_dim, block_size))
     return fail(VK_ERROR_INVALID_ARGUMENT, (std::string(who) + ": " + why).c_str());
   if (M == 0 || EM == 0) return VK_OK;
-  if (a == nullptr || w == nullptr || w_scale == nullptr || sorted_ids == nullptr || expert_ids == nullptr ||
-      preact == nullptr)
+  const bool raw_given = w != nullptr && w_scale != nullptr;
+  if (a == nullptr || (!raw_given && (packed == nullptr || w != nullptr || w_scale != nullptr)) ||
+      sorted_ids == nullptr || expert_ids == nullptr || preact == nullptr)
     return fail(VK_ERROR_INVALID_ARGUMENT, (std::string(who) + ": buffers must not be null").c_str());
   if (packed != nullptr && num_experts <= 0)
     return fail(VK_ERROR_INVALID_ARGUMENT, (std::string(who) + ": num_experts must be positive with packed weights").c_str());
@@ -430,9 +431,11 @@ int preact_any(const char* who, int stage, const uint16_t* a, const uint8_t* w, 
         vk::launch_moe_preact_prepacked(stage, a, static_cast<const uint8_t*>(packed), w, w_scale, sorted_ids,
                                         expert_ids, preact, M, width_a, ncols, top_k, EM, k_base, k_dim,
                                         block_size, num_experts, workspace, workspace_bytes, flags,
-                                        static_cast<hipStream_t>(stream))))
-    vk::launch_moe_preact(stage, a, w, w_scale, sorted_ids, expert_ids, preact, M, width_a, ncols, top_k, EM,
-                          k_base, k_dim, block_size, static_cast<hipStream_t>(stream));
+                                        static_cast<hipStream_t>(stream))) &&
+      !vk::launch_moe_preact(stage, a, w, w_scale, sorted_ids, expert_ids, preact, M, width_a, ncols, top_k, EM,
+                             k_base, k_dim, block_size, static_cast<hipStream_t>(stream),
+                             static_cast<const uint8_t*>(packed), num_experts))
+    return fail(VK_ERROR_INVALID_ARGUMENT, (std::string(who) + ": " + kPackedOnlyNeeds).c_str());
   return stage_launch_status(who, before);
 }
 

@@ -28,7 +28,11 @@
 //     requires `out` to be accumulated into.
 //
 // stream_resident_kernel: decode (few rows per expert, K up to 3072): HBM
-//   bound, one workgroup per compute unit, all of K of 16 rows resident.
+//   bound, one workgroup per compute unit, all of K of 16 rows resident.  It has
+//   a second form that reads the weights from the prepacked layout of
+//   moe_prefill_layout.hpp instead (taken whenever the caller gives it: the
+//   scale bytes then come with the codes and nothing is checked or moved in the
+//   loop), and forms that align, or route and align, for themselves.
 // tile_wide_kernel: everything else when the caller lends a workspace (and K >=
 //   512): 128 rows x 16 weight tiles per workgroup, rows pre-split in the
 //   workspace, operands brought to LDS by DMA three K steps ahead; the second
@@ -2451,17 +2455,26 @@ void launch_moe_gateup(const FusedMoeArgs& a, hipStream_t stream) {
 // are the rank's shard [E, rows, k_dim / 2] and [E, rows, k_dim / 32].  stage 0: rows =
 // 2 * ncols, preact [EM, 2 * ncols] (gate columns, then up columns); stage 1: rows =
 // ncols, preact [EM, ncols].  Routed rows are written, the others left as they are.
-// Runs the decode kernel or the plain tile kernel (no workspace, raw weights).
-void launch_moe_preact(int stage, const uint16_t* a, const uint8_t* w, const uint8_t* w_scale,
+// Runs the decode kernel or the plain tile kernel (no workspace).  packed (optional): the
+// shard in the prepacked form, which the decode kernels then read; w / w_scale may be null
+// with it, and the call is then refused (false, nothing enqueued) where the decode kernels
+// do not take it.
+bool launch_moe_preact(int stage, const uint16_t* a, const uint8_t* w, const uint8_t* w_scale,
                        const int32_t* sorted_ids, const int32_t* expert_ids, float* preact, int M,
                        int a_stride, int ncols, int top_k, int EM, int k_base, int k_dim, int block_size,
-                       hipStream_t stream) {
-  if (M <= 0 || EM <= 0 || block_size <= 0) return;
+                       hipStream_t stream, const uint8_t* packed, int num_experts) {
+  if (M <= 0 || EM <= 0 || block_size <= 0) return true;
   GemmArgs g{};
   g.A = a + k_base;
   g.a_stride = a_stride;
   g.W = w;
   g.Ws = w_scale;
+  if (packed != nullptr && num_experts > 0) {
+    g.p_units = mx_units(stage, ncols);
+    g.p_experts = num_experts;
+    g.Wp = packed;
+    g.Wpf = packed + mx_packed_body_bytes(num_experts, g.p_units, mx_kp(k_dim) / 128);
+  }
   g.sorted_ids = sorted_ids;
   g.expert_ids = expert_ids;
   g.preact = preact;
@@ -2471,8 +2484,11 @@ void launch_moe_preact(int stage, const uint16_t* a, const uint8_t* w, const uin
   g.ncols = ncols;
   g.num_blocks = EM / block_size;
   g.block_size = block_size;
-  if (stage == 0) launch_stage<0>(g, plan_stage<0>(g), stream);
-  else launch_stage<1>(g, plan_stage<1>(g), stream);
+  const StagePlan pl = stage == 0 ? plan_stage<0>(g) : plan_stage<1>(g);
+  if (w == nullptr && !(pl.packed && pl.variant == kMoeVariantResident)) return false;
+  if (stage == 0) launch_stage<0>(g, pl, stream);
+  else launch_stage<1>(g, pl, stream);
+  return true;
 }
 
 // The second stage alone.  With a workspace (and packed weights) it runs as in the

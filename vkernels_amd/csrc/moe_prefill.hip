@@ -26,7 +26,9 @@
 // [kScaleLo, kScaleHi] (flagged when the weights are prepacked) and segments
 // with a row whose blocks are outside the representable range (flagged when
 // the rows are split) are recomputed by exact_unit_mx: integer-exact
-// dequantisation of the raw weights, bf16 MFMAs, bf16 rows from global memory.
+// dequantisation of the weights as the raw tensors hold them (read back from the
+// prepacked form: a flagged unit keeps them there as they are, any other has
+// the move onto the OCP points undone), bf16 MFMAs, bf16 rows from global memory.
 //
 // Work split.  A workgroup of 4 wavefronts (one per SIMD, 512 registers each)
 // takes a window of 128 sorted rows -- cut into segments of consecutive blocks
@@ -76,8 +78,6 @@ typedef __attribute__((ext_vector_type(32))) __bf16 bf16x32;
 struct MxArgs {
   const uint8_t* Wp;       // prepacked weights of the stage
   const uint8_t* Wflags;   // [E, units]: 1 = the unit takes the exact path
-  const uint8_t* W;        // raw weights [E, rows_w, K/2] and scales [E, rows_w, K/32] (exact path)
-  const uint8_t* Ws;
   const uint16_t* A;       // bf16 rows (exact path): stage 0 A [M, K], stage 1 act [EM, K]
   const uint8_t* Aq;       // split rows: row r = TERMS planes of Kp bytes at r * TERMS * Kp
   const uint8_t* row_bad;  // per row of Aq: 1 = outside the split's range
@@ -1048,9 +1048,9 @@ MxArgs mx_args(const FusedMoeArgs& a, int stage) {
   g.linear_beta = a.linear_beta;
   g.activation = a.activation;
   if (stage == 0) {
-    g.A = a.A; g.W = a.w13; g.Ws = a.w13_scale; g.bias = a.b13; g.K = a.hidden; g.ncols = a.ispp;
+    g.A = a.A; g.bias = a.b13; g.K = a.hidden; g.ncols = a.ispp;
   } else {
-    g.A = a.act; g.W = a.w2; g.Ws = a.w2_scale; g.bias = a.b2; g.K = a.ispp; g.ncols = a.hidden;
+    g.A = a.act; g.bias = a.b2; g.K = a.ispp; g.ncols = a.hidden;
   }
   g.a_stride = g.K;
   return g;
@@ -1245,6 +1245,8 @@ bool launch_moe_preact_prepacked(int stage, const uint16_t* a, const uint8_t* pa
                                  float* preact, int M, int a_stride, int ncols, int top_k, int EM, int k_base,
                                  int k_dim, int block_size, int num_experts, void* workspace,
                                  size_t workspace_bytes, unsigned flags, hipStream_t stream) {
+  (void)w;  // (the exact path reads the packed form as well; the raw shard serves the
+  (void)w_scale;  // small calls, which the caller runs on the raw-weight kernels)
   if (M <= 0 || EM <= 0 || block_size <= 0 || packed == nullptr || workspace == nullptr) return false;
   if (workspace_bytes < mx_preact_workspace_bytes(stage, M, EM, k_dim) ||
       (reinterpret_cast<uintptr_t>(workspace) & 15) != 0)
@@ -1270,8 +1272,6 @@ bool launch_moe_preact_prepacked(int stage, const uint16_t* a, const uint8_t* pa
   g.block_size = block_size;
   g.A = a + k_base;
   g.a_stride = a_stride;
-  g.W = w;
-  g.Ws = w_scale;
   g.K = k_dim;
   g.ncols = ncols;
   g.preact = preact;

@@ -105,10 +105,10 @@ bool prepare_mx_kernels();
 // (sorted_ids null = token order), routed combine in gather form (pos: M * top_k ints).
 void launch_mxfp4_quant(const uint16_t* A, const int32_t* sorted_ids, uint8_t* packed, uint8_t* scales,
                         int rows, int hidden, int top_k, int n_flat, hipStream_t stream);
-void launch_moe_preact(int stage, const uint16_t* a, const uint8_t* w, const uint8_t* w_scale,
+bool launch_moe_preact(int stage, const uint16_t* a, const uint8_t* w, const uint8_t* w_scale,
                        const int32_t* sorted_ids, const int32_t* expert_ids, float* preact, int M,
                        int a_stride, int ncols, int top_k, int EM, int k_base, int k_dim, int block_size,
-                       hipStream_t stream);
+                       hipStream_t stream, const uint8_t* packed = nullptr, int num_experts = 0);
 // The same on prepacked weights (the FP4-rate kernels of moe_prefill.hip; `packed` from
 // launch_moe_prepack for the shard [num_experts, rows, k_dim / 2]); false = nothing enqueued.
 size_t mx_preact_workspace_bytes(int stage, int M, int EM, int k_dim);
