@@ -267,11 +267,17 @@ __device__ __forceinline__ void unit_tiles_packed(const GemmArgs& p, int e, int 
   }
 }
 
-// Flag byte of a packed unit (1 = it holds a code or a scale byte the fast path does not
-// take, and its codes and scale bytes are the raw tensors').  The index is uniform.
-__device__ __forceinline__ bool packed_unit_flagged(const GemmArgs& p, int e, int pu) {
+// Flag byte of a packed unit (non-zero = it holds a code or a scale byte the fast path does
+// not take, and its codes and scale bytes are the raw tensors').  The index is uniform, so
+// the word that holds the byte comes through the scalar path (a read of memory that no
+// kernel writes while this one runs; the flags start on a multiple of 256 bytes and are
+// padded to one): it does not queue with the vector loads, and a wait for it waits for
+// nothing else.  The caller keeps the word and looks at it when the unit is complete.
+__device__ __forceinline__ uint32_t packed_unit_flag(const GemmArgs& p, int e, int pu) {
+  typedef const __attribute__((address_space(4))) uint32_t* const_u32_ptr;
   const int idx = __builtin_amdgcn_readfirstlane(e * p.p_units + pu);
-  return p.Wpf[idx] != 0;
+  const uintptr_t word = reinterpret_cast<uintptr_t>(p.Wpf) + (uintptr_t)(idx & ~3);
+  return (*(const_u32_ptr)word >> (8 * (idx & 3))) & 0xFFu;
 }
 
 // ---------------------------------------------------------------------------
@@ -537,6 +543,7 @@ __device__ __forceinline__ void lds_barrier() {
 template <int STAGE, int WAVES, int NT, int D, bool KSPLIT = false, int ROUTE = 0, bool PACKED = false>
 __global__ __launch_bounds__(64 * WAVES) void stream_resident_kernel(GemmArgs p) {
   static_assert(ROUTE == 0 || STAGE == 0, "the routed form is the first stage's");
+  static_assert(ROUTE == 0 || 64 * WAVES >= kRouteMaxRows, "a lane per routed row");
   static_assert(!PACKED || (WAVES * (STAGE == 0 ? 8 * NT : 16 * NT)) % (STAGE == 0 ? 64 : 128) == 0,
                 "a wavefront's consecutive units are whole packed units apart");
   extern __shared__ u32x4 b_lds[];  // [nsteps][2][2][64] operand planes, block scales, weight scales
@@ -548,6 +555,8 @@ __global__ __launch_bounds__(64 * WAVES) void stream_resident_kernel(GemmArgs p)
   __shared__ short rt_le[ROUTE ? kRouteMaxRows : 1];
   __shared__ int rt_hist[ROUTE ? kRouteMaxExperts : 1];
   __shared__ unsigned short run_ids[ROUTE ? kRouteMaxRows * 16 : 1];
+  // ... rows of every local expert among the 64 routed rows a wavefront ranks
+  __shared__ int rt_cnt[ROUTE ? kRouteMaxRows / 64 : 1][ROUTE ? kRouteMaxExperts : 1];
   __shared__ int rt_runs;
   __shared__ int slice_sh[2];           // this workgroup's slice of the (run, unit) space
   __shared__ int pass_slow[2];          // set while staging: this pass takes the exact path
@@ -589,19 +598,19 @@ __global__ __launch_bounds__(64 * WAVES) void stream_resident_kernel(GemmArgs p)
   if constexpr (ROUTE) {
     // ---- router: a wavefront per token; the table of local experts stays in LDS ----
     const int n_flat = p.n_flat, top_k = p.top_k, T = n_flat / top_k;
-    for (int i = tid; i < kRouteMaxExperts; i += 64 * WAVES) rt_hist[i] = 0;
-    for (int i = tid; i < kRouteMaxRows * 16; i += 64 * WAVES) run_ids[i] = 0xFFFF;
-    if constexpr (ROUTE == 2) {  // the ids are the router's: the local expert of every routed row
-      for (int i = tid; i < n_flat; i += 64 * WAVES) {
-        const int id = p.rt_topk_ids[i];
-        int le = -1;
+    // (routed rows: at most kRouteMaxRows, a lane each: row tid)
+    int my_le = -1;  // ROUTE == 2: the local expert of row tid
+    if constexpr (ROUTE == 2) {  // the ids are the router's; asked for first, the tables cleared meanwhile
+      if (tid < n_flat) {
+        const int id = p.rt_topk_ids[tid];
         if (id >= 0 && id < p.rt_experts) {
-          le = p.rt_expert_map != nullptr ? p.rt_expert_map[id] : id;
-          if (le < 0 || le >= p.rt_local_n) le = -1;
+          my_le = p.rt_expert_map != nullptr ? p.rt_expert_map[id] : id;
+          if (my_le < 0 || my_le >= p.rt_local_n) my_le = -1;
         }
-        rt_le[i] = (short)le;
       }
     }
+    for (int i = tid; i < (kRouteMaxRows / 64) * kRouteMaxExperts; i += 64 * WAVES) (&rt_cnt[0][0])[i] = 0;
+    for (int i = tid; i < kRouteMaxRows * 8; i += 64 * WAVES) reinterpret_cast<uint32_t*>(run_ids)[i] = 0xFFFFFFFFu;
     for (int token = wave; ROUTE == 1 && token < T; token += WAVES) {  // uniform per wavefront
       int my_id;
       float my_w;
@@ -620,11 +629,22 @@ __global__ __launch_bounds__(64 * WAVES) void stream_resident_kernel(GemmArgs p)
         }
       }
     }
-    __syncthreads();
-    // ---- rows per local expert ----
-    for (int i = tid; i < n_flat; i += 64 * WAVES) {
-      const int le = rt_le[i];
-      if (le >= 0) atomicAdd(&rt_hist[le], 1);
+    __syncthreads();  // (the tables are cleared; ROUTE == 1: rt_le is written)
+    // ---- every routed row among the rows of its expert: lane = row tid; the lanes of a
+    // wavefront with the same expert are found with a ballot per bit of the expert's
+    // number, the row's rank among them is the count of the lower lanes, and their number
+    // goes to the wavefront's line of rt_cnt ----
+    if constexpr (ROUTE == 1) my_le = tid < n_flat ? (int)rt_le[tid] : -1;
+    int my_rank = 0;
+    if (tid < kRouteMaxRows) {  // uniform per wavefront
+      unsigned long long same = __ballot(my_le >= 0);
+#pragma unroll
+      for (int b = 0; b < 8; ++b) {  // kRouteMaxExperts = 2^8
+        const unsigned long long set = __ballot(((my_le >> b) & 1) != 0);
+        same &= ((my_le >> b) & 1) != 0 ? set : ~set;
+      }
+      my_rank = (int)__popcll(same & ((1ull << lane) - 1ull));
+      if (my_le >= 0 && my_rank == 0) rt_cnt[tid >> 6][my_le] = (int)__popcll(same);
     }
     __syncthreads();
     // ---- first block of every expert (wavefront 0: a scan of the blocks, 64 experts a trip) ----
@@ -632,7 +652,11 @@ __global__ __launch_bounds__(64 * WAVES) void stream_resident_kernel(GemmArgs p)
       int blocks = 0;
       for (int base = 0; base < p.rt_local_n; base += 64) {
         const int e = base + lane;
-        const int c = e < p.rt_local_n ? rt_hist[e] : 0;
+        int c = 0;
+        if (e < p.rt_local_n) {
+#pragma unroll
+          for (int w = 0; w < kRouteMaxRows / 64; ++w) c += rt_cnt[w][e];
+        }
         const int nb_e = (c + 15) >> 4;
         int incl = nb_e;
 #pragma unroll
@@ -659,13 +683,10 @@ __global__ __launch_bounds__(64 * WAVES) void stream_resident_kernel(GemmArgs p)
     __syncthreads();
     // ---- place of every routed row: its rank among the rows of its expert ----
     const int n_runs = rt_runs;
-    for (int i = tid; i < n_flat; i += 64 * WAVES) {
-      const int le = rt_le[i];
-      if (le >= 0) {
-        int rank = 0;
-        for (int j = 0; j < i; ++j) rank += rt_le[j] == le ? 1 : 0;
-        run_ids[rt_hist[le] * 16 + rank] = (unsigned short)i;
-      }
+    if (my_le >= 0) {  // (rows in ascending order inside an expert: those of the wavefronts before, then the lower lanes)
+      int rank = my_rank;
+      for (int w = 0; w < (tid >> 6); ++w) rank += rt_cnt[w][my_le];
+      run_ids[rt_hist[my_le] * 16 + rank] = (unsigned short)tid;
     }
     __syncthreads();
     // ---- workgroup 0: the tables for the second stage and the caller ----
@@ -880,7 +901,7 @@ __global__ __launch_bounds__(64 * WAVES) void stream_resident_kernel(GemmArgs p)
     int col0[NT];
     int shift[NT];         // PACKED: where a tile's scale byte is in the step's word
     int cur_pu = 0;        // PACKED: packed unit of the unit being computed ...
-    bool cur_flag = false; // ... and its flag
+    uint32_t cur_flag = 0u;  // ... and its flag (packed_unit_flag)
 
     // ---- load cursor: runs D steps ahead and crosses unit boundaries -----
     const uint8_t* lrow[NT];
@@ -956,7 +977,7 @@ __global__ __launch_bounds__(64 * WAVES) void stream_resident_kernel(GemmArgs p)
     auto prime = [&]() {
       if constexpr (PACKED) {
         unit_tiles_packed<STAGE, NT>(p, e, n_my > 0 ? first : u0, lane, nsteps, cw, cs, shift, col0, cur_pu);
-        cur_flag = packed_unit_flagged(p, e, cur_pu);
+        cur_flag = packed_unit_flag(p, e, cur_pu);
 #pragma unroll
         for (int j = 0; j < kNS; ++j) lsc[j] = cs[j];
       } else {
@@ -1190,7 +1211,7 @@ __global__ __launch_bounds__(64 * WAVES) void stream_resident_kernel(GemmArgs p)
                 for (int t = 0; t < NT; ++t) acc[t] += part[(w2 * NT + t) * 64 + lane];
                 any_bad |= ks_bad[w2] != 0;
               }
-              if (any_bad || (PACKED && cur_flag))
+              if (any_bad || (PACKED && cur_flag != 0u))
                 redo = 1ull;
               else if (my_flat >= 0)
                 epilogue_tile<STAGE, NT>(p, e, acc, col0, my_flat, srow, lq);
@@ -1223,7 +1244,7 @@ __global__ __launch_bounds__(64 * WAVES) void stream_resident_kernel(GemmArgs p)
                   // unit's last K step could run: the pass's mark is complete.)  A unit of a
                   // marked pass, or one that met a code or scale outside the fast path's
                   // domain, is redone after the stream, so the hot loop stays small
-                  if (__ballot(bad != 0u) != 0ull || pass_slow[flag] != 0 || (PACKED && cur_flag))
+                  if (__ballot(bad != 0u) != 0ull || pass_slow[flag] != 0 || (PACKED && cur_flag != 0u))
                     redo |= 1ull << cunit;
                   else if (my_flat >= 0)
                     epilogue_tile<STAGE, NT>(p, e, acc, col0, my_flat, srow, lq);
@@ -1237,7 +1258,7 @@ __global__ __launch_bounds__(64 * WAVES) void stream_resident_kernel(GemmArgs p)
                     }
                     if constexpr (PACKED) {
                       cur_pu += kPackedStride;
-                      cur_flag = packed_unit_flagged(p, e, cur_pu);
+                      cur_flag = packed_unit_flag(p, e, cur_pu);
                     } else {
                       sc_unit += s_unit_stride;
                       if (cunit + 1 < n_my) fetch_scales(s_unit_stride);
@@ -1264,7 +1285,7 @@ __global__ __launch_bounds__(64 * WAVES) void stream_resident_kernel(GemmArgs p)
             redo &= redo - 1ull;
             if constexpr (PACKED) {
               unit_tiles_packed<STAGE, NT>(p, e, first + idx * WAVES, lane, nsteps, cw, cs, shift, col0, cur_pu);
-              exact_unit_packed<NT>(cw, cs, shift, packed_unit_flagged(p, e, cur_pu), a_row, K, lane, acc);
+              exact_unit_packed<NT>(cw, cs, shift, packed_unit_flag(p, e, cur_pu) != 0u, a_row, K, lane, acc);
             } else {
               unit_tiles<STAGE, NT>(p, e, first + idx * WAVES, ln, cw, cs, col0);
               exact_unit_global<NT>(cw, cs, a_row, K, lane, acc);
@@ -2047,8 +2068,8 @@ int num_compute_units() {
 }
 
 constexpr size_t kResidentLdsLimit = 150 * 1024;  // dynamic LDS the resident kernel may ask for
-// ... and its routed forms, whose tables are 10 KB of static LDS over the plain form's
-constexpr size_t kRoutedStaticLds = 10 * 1024;
+// ... and its routed forms, whose tables are 14 KB of static LDS over the plain form's
+constexpr size_t kRoutedStaticLds = 14 * 1024;
 constexpr size_t kRoutedLdsLimit = kResidentLdsLimit - kRoutedStaticLds;
 
 // True when the device grants the kernel its dynamic LDS (asked once per kernel;
