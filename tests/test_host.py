@@ -311,7 +311,7 @@ def test_synth_is_deterministic_and_prefix_stable():
 def test_tile_candidates_and_compiled_in_rules():
     for stage in (0, 1):
         cands = ve.moe_tile_candidates(stage)
-        assert len(cands) == (9 if stage == 0 else 8) and len(set(cands)) == len(cands)
+        assert len(cands) == 8 and len(set(cands)) == 8
         plain = {c[1:] for c in cands if c[0] == 2}
         assert all(c[1:] in plain for c in cands if c[0] == 3)   # a K-split shape has its plain form to fall back to
         assert (0, 4, 4, 0) in cands                      # the tile kernels
@@ -322,8 +322,7 @@ def test_tile_candidates_and_compiled_in_rules():
             # the decode kernels up to 512 routed rows, where a pass's rows fit LDS and registers
             assert (shape[0] in (2, 3)) == (n_flat <= 512 and K <= (4096 if stage == 0 else 3072))
     assert ve.moe_tile_query(0, 2880, 2880, 128)[0] == (2, 8, 2, 2) and ve.moe_tile_query(1, 2880, 2880, 128)[0] == (2, 8, 1, 6)
-    assert ve.moe_tile_query(0, 4096, 1536, 42)[0] == (2, 4, 2, 8)                  # rows of K = 4096
-    assert ve.moe_tile_query(0, 4096, 1536, 6)[0] == (3, 4, 2, 8)                   # ... of one token: K shared
+    assert ve.moe_tile_query(0, 4096, 1536, 6)[0] == (2, 4, 2, 8)                   # rows of K = 4096
     # one token: fewer units than half the device's wavefronts, K shared between them
     assert ve.moe_tile_query(0, 2880, 2880, 4)[0] == (3, 8, 2, 4) and ve.moe_tile_query(1, 2880, 2880, 4)[0] == (3, 8, 1, 8)
     assert ve.moe_tile_query(1, 1536, 4096, 6)[0] == (3, 8, 2, 4)                   # ... with two tiles a unit

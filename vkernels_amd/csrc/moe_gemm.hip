@@ -2374,7 +2374,7 @@ bool prepare_moe_kernels() {
   VK_KSPLIT_VARIANTS(VK_READY)
 #undef VK_READY
   ok = resident_kernel_ready<0, 8, 2, 4, true, 1>() && resident_kernel_ready<0, 8, 2, 2, false, 1>() && ok;
-  ok = resident_kernel_ready<0, 4, 2, 8, true, 1>() && resident_kernel_ready<0, 4, 2, 8, true, 1, true>() && ok;
+  ok = resident_kernel_ready<0, 4, 2, 8, false, 1>() && resident_kernel_ready<0, 4, 2, 8, false, 1, true>() && ok;
   ok = resident_kernel_ready<0, 8, 2, 2, false, 2>() && resident_kernel_ready<0, 4, 2, 8, false, 2>() && ok;
 #define VK_READY(S_, W_, NT_, D_) ok = resident_kernel_ready<S_, W_, NT_, D_, false, 0, true>() && ok;
   VK_RESIDENT_VARIANTS(VK_READY)
@@ -2433,12 +2433,12 @@ bool launch_routed_moe(const FusedMoeArgs& a, const RoutedArgs& r, hipStream_t s
   const int shape = p0.ksplit && p0.waves == 8 && p0.nt == 2 && p0.depth == 4 ? 1
                     : !p0.ksplit && p0.waves == 8 && p0.nt == 2 && p0.depth == 2 ? 2
                     : !p0.ksplit && p0.waves == 4 && p0.nt == 2 && p0.depth == 8 ? 3
-                    : p0.ksplit && p0.waves == 4 && p0.nt == 2 && p0.depth == 8 ? 4 : 0;
+                    : 0;
   bool ready = false;
   if (route_inside) {
     if (shape == 1) ready = p0.packed ? resident_kernel_ready<0, 8, 2, 4, true, 1, true>() : resident_kernel_ready<0, 8, 2, 4, true, 1>();
     if (shape == 2) ready = p0.packed ? resident_kernel_ready<0, 8, 2, 2, false, 1, true>() : resident_kernel_ready<0, 8, 2, 2, false, 1>();
-    if (shape == 4) ready = p0.packed ? resident_kernel_ready<0, 4, 2, 8, true, 1, true>() : resident_kernel_ready<0, 4, 2, 8, true, 1>();
+    if (shape == 3) ready = p0.packed ? resident_kernel_ready<0, 4, 2, 8, false, 1, true>() : resident_kernel_ready<0, 4, 2, 8, false, 1>();
   } else {
     if (shape == 2) ready = p0.packed ? resident_kernel_ready<0, 8, 2, 2, false, 2, true>() : resident_kernel_ready<0, 8, 2, 2, false, 2>();
     if (shape == 3) ready = p0.packed ? resident_kernel_ready<0, 4, 2, 8, false, 2, true>() : resident_kernel_ready<0, 4, 2, 8, false, 2>();
@@ -2448,9 +2448,9 @@ bool launch_routed_moe(const FusedMoeArgs& a, const RoutedArgs& r, hipStream_t s
     if (shape == 1) {
       if (p0.packed) launch_resident<0, 8, 2, 4, true, 1, true>(g0, p0.resident_lds, stream);
       else launch_resident<0, 8, 2, 4, true, 1>(g0, p0.resident_lds, stream);
-    } else if (shape == 4) {
-      if (p0.packed) launch_resident<0, 4, 2, 8, true, 1, true>(g0, p0.resident_lds, stream);
-      else launch_resident<0, 4, 2, 8, true, 1>(g0, p0.resident_lds, stream);
+    } else if (shape == 3) {
+      if (p0.packed) launch_resident<0, 4, 2, 8, false, 1, true>(g0, p0.resident_lds, stream);
+      else launch_resident<0, 4, 2, 8, false, 1>(g0, p0.resident_lds, stream);
     } else {
       if (p0.packed) launch_resident<0, 8, 2, 2, false, 1, true>(g0, p0.resident_lds, stream);
       else launch_resident<0, 8, 2, 2, false, 1>(g0, p0.resident_lds, stream);

@@ -37,7 +37,7 @@ inline bool operator==(const MoeTile& a, const MoeTile& b) {
   X(1, 8, 2, 4) X(1, 8, 1, 4) X(1, 8, 1, 6) X(1, 8, 1, 8) X(1, 8, 1, 12)
 // ... and of its K-split form (every one is also in the list above: a plan that cannot
 // split K falls back to the same shape there).
-#define VK_KSPLIT_VARIANTS(X) X(0, 8, 2, 4) X(0, 8, 2, 6) X(0, 4, 2, 8) X(1, 8, 1, 8) X(1, 8, 2, 4)
+#define VK_KSPLIT_VARIANTS(X) X(0, 8, 2, 4) X(0, 8, 2, 6) X(1, 8, 1, 8) X(1, 8, 2, 4)
 
 struct MoeTileCandidate {
   int stage;
@@ -127,7 +127,9 @@ struct MoeTileRule {
 // A single token or two: when the units of all rows (at most n_flat runs) are fewer than
 // half the wavefronts of the device, a wavefront has one unit or none, and a unit is a chain
 // of K / 128 dependent steps, a few in flight.  The K-split form gives the idle wavefronts a
-// part of K each.
+// part of K each.  Only the shapes whose rows of K values need 8 wavefronts to stage have it
+// (with 4 wavefronts, K up to 4096, all of K takes longer to stage than the shorter chains
+// save: 4096x1536x64x6 at T = 1, 32.0 against 28.4 us).
 constexpr int kMoeComputeUnits = 256;  // of the device the rules were swept on
 
 // packed: the stage reads the prepacked form (its decode kernels have no scale block in
@@ -137,11 +139,6 @@ constexpr int kMoeComputeUnits = 256;  // of the device the rules were swept on
 inline MoeTile pick_moe_tile(int n_flat, int K, int ncols, int stage, bool packed = false,
                              int packed_experts = 0) {
   const int max_rows = moe_decode_max_rows(packed ? packed_experts : 0);
-  // (gate/up rows of 3072 < K <= 4096 run workgroups of 4 wavefronts, and a unit there is a
-  // chain of up to 32 steps: the form pays up to a unit per wavefront)
-  if (stage == 0 && n_flat <= kMoeDecodeMaxRows && K > 3072 && K <= 4096 &&
-      (long long)n_flat * (ncols / 16) <= (long long)kMoeComputeUnits * 4)
-    return MoeTile{kMoeVariantResidentKSplit, 4, 2, 8};
   if (n_flat <= kMoeDecodeMaxRows && K >= 1024 && K <= 3072) {
     const long long spare = (long long)kMoeComputeUnits * 4;  // half of 8 wavefronts per compute unit
     if (stage == 0 && (long long)n_flat * (ncols / 16) <= spare)
