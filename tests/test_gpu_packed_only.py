@@ -32,7 +32,7 @@ def _routed_rows(g, n_flat):
 
 
 @pytest.mark.parametrize("name,T", [("c0", 16), ("c1", 1), ("c1", 2), ("c1", 8), ("c1", 64), ("c2", 64),
-                                    ("c4", 1), ("c4", 7), ("c4", 33)])
+                                    ("c4", 1), ("c4", 2), ("c4", 7), ("c4", 33)])
 def test_decode_sizes_on_the_packed_form_alone(name, T):
     cfg = synth.CONFIGS[name]
     w = cfgs._weights(cfg)
@@ -40,7 +40,14 @@ def test_decode_sizes_on_the_packed_form_alone(name, T):
     g, wn = cfgs._check(cfg, T, w, A, lg, gpu_kw=PACKED_ONLY, tight=True)
     raw = cfgs._run_gpu(cfg, w, A, lg, None, None)
     rows = _routed_rows(g, T * cfg.top_k)
-    assert np.array_equal(g["act"][rows], raw["act"][rows]), "the first stage differs from the raw form's"
+    same_shape = ve.moe_tile_query(0, cfg.H, cfg.I, T * cfg.top_k, packed=True)[0] == \
+        ve.moe_tile_query(0, cfg.H, cfg.I, T * cfg.top_k)[0]
+    if same_shape:   # the same products summed in the same order
+        assert np.array_equal(g["act"][rows], raw["act"][rows]), "the first stage differs from the raw form's"
+    else:            # (K shared between wavefronts in one form only: the sums are ordered differently)
+        a = synth.bf16_bits_to_f32(g["act"][rows]).astype(np.float64)
+        b = synth.bf16_bits_to_f32(raw["act"][rows]).astype(np.float64)
+        assert np.linalg.norm(a - b) <= 2e-3 * np.linalg.norm(b)
     m, l2, nf = error_metrics(g["out"], raw["out"])
     assert nf and l2 <= 1e-5, (m, l2)
 
@@ -141,7 +148,8 @@ def test_a_wide_first_stage_on_the_packed_form_alone():
     assert bool((out == 3.0).all())
 
 
-@pytest.mark.parametrize("name,T", [("c1", 1), ("c1", 8), ("c1", 16), ("c0", 16), ("c1", 40)])
+@pytest.mark.parametrize("name,T", [("c1", 1), ("c1", 8), ("c1", 16), ("c0", 16), ("c1", 40), ("c4", 1), ("c4", 2),
+                                    ("c4", 16)])
 def test_router_alignment_and_layer_in_one_call_on_the_packed_form_alone(name, T):
     cfg = synth.CONFIGS[name]
     w = cfgs._weights(cfg)

@@ -501,7 +501,12 @@ __device__ __forceinline__ void split_bf16x8(u32x4 v, uint32_t sb, uint2& hi, ui
 // stages a pass (every wavefront takes every WAVES-th group of 32 values): workgroups of
 // 8 wavefronts, two to a SIMD, hold K <= 3072; workgroups of 4, with a SIMD's whole
 // register file each, K <= 4096.
-__host__ __device__ constexpr int resident_batch(int waves) { return waves == 4 ? 32 : 96 / waves; }
+// (wide: the K-split form on the prepacked weights, which has the registers for K <= 4096
+// with 8 wavefronts as well: no scale block, and its row registers are free again before
+// the stream starts.)
+__host__ __device__ constexpr int resident_batch(int waves, bool wide = false) {
+  return waves == 4 ? 32 : (wide ? 128 : 96) / waves;
+}
 
 // KSPLIT: the form for a handful of rows (one token), where a workgroup's slice is fewer
 // units than half its wavefronts and a unit, a chain of K / 128 dependent steps with D in
@@ -1030,7 +1035,7 @@ __global__ __launch_bounds__(64 * WAVES) void stream_resident_kernel(GemmArgs p)
         // exactly), then the rest of the rows.  The weights are so asked for as early
         // as the order of the data allows, and both they and the later row pieces
         // stay in flight while the first pieces are split and written.
-        constexpr int kBatch = resident_batch(WAVES);  // pieces per lane, all of K in one batch
+        constexpr int kBatch = resident_batch(WAVES, KSPLIT && PACKED);  // pieces per lane, all of K in one batch
         // pieces of a lane that K steps [0, D) need (K split: all, every part starts at once)
         constexpr int kFirst = KSPLIT ? kBatch : ((D * 4 + WAVES - 1) / WAVES < kBatch ? (D * 4 + WAVES - 1) / WAVES : kBatch);
         const int n_pieces = (nsteps * 4 + WAVES - 1) / WAVES;  // the launcher keeps it <= kBatch
@@ -2128,7 +2133,7 @@ StagePlan plan_stage(const GemmArgs& g) {
   if (pl.resident_lds > kResidentLdsLimit || g.num_blocks > kMaxRuns ||
       (!packed && pl.nt * groups > 64 * resident_scale_pieces(pl.waves)) ||
       (res_units + pl.waves - 1) / pl.waves > 64 ||  // one bit per unit in a wavefront's redo mask
-      nsteps * 4 > resident_batch(pl.waves) * pl.waves)  // the rows are staged in one batch
+      nsteps * 4 > resident_batch(pl.waves, pl.ksplit && packed) * pl.waves)  // the rows are staged in one batch
     pl.variant = kMoeVariantLds;
   return pl;
 }

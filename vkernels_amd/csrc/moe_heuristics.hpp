@@ -139,6 +139,10 @@ constexpr int kMoeComputeUnits = 256;  // of the device the rules were swept on
 inline MoeTile pick_moe_tile(int n_flat, int K, int ncols, int stage, bool packed = false,
                              int packed_experts = 0) {
   const int max_rows = moe_decode_max_rows(packed ? packed_experts : 0);
+  // (on the prepacked form the 8-wavefront K-split shape also holds rows of K up to 4096)
+  if (packed && stage == 0 && n_flat <= kMoeDecodeMaxRows && K > 3072 && K <= 4096 &&
+      (long long)n_flat * (ncols / 16) <= (long long)kMoeComputeUnits * 4)
+    return MoeTile{kMoeVariantResidentKSplit, 8, 2, 4};
   if (n_flat <= kMoeDecodeMaxRows && K >= 1024 && K <= 3072) {
     const long long spare = (long long)kMoeComputeUnits * 4;  // half of 8 wavefronts per compute unit
     if (stage == 0 && (long long)n_flat * (ncols / 16) <= spare)
