@@ -501,9 +501,8 @@ __device__ __forceinline__ void split_bf16x8(u32x4 v, uint32_t sb, uint2& hi, ui
 // stages a pass (every wavefront takes every WAVES-th group of 32 values): workgroups of
 // 8 wavefronts, two to a SIMD, hold K <= 3072; workgroups of 4, with a SIMD's whole
 // register file each, K <= 4096.
-// (wide: the K-split form on the prepacked weights, which has the registers for K <= 4096
-// with 8 wavefronts as well: no scale block, and its row registers are free again before
-// the stream starts.)
+// (wide: the WIDEK instantiations on the prepacked weights, which have the registers for
+// K <= 4096 with 8 wavefronts as well: no scale block to hold.)
 __host__ __device__ constexpr int resident_batch(int waves, bool wide = false) {
   return waves == 4 ? 32 : (wide ? 128 : 96) / waves;
 }
@@ -545,8 +544,13 @@ __device__ __forceinline__ void lds_barrier() {
 // and the scale bytes (already less one) come with the step, four to a lane, so there is
 // no scale block to park in LDS and nothing to check in the loop: a unit that needs the
 // exact path carries a flag, looked up when the unit is begun.
-template <int STAGE, int WAVES, int NT, int D, bool KSPLIT = false, int ROUTE = 0, bool PACKED = false>
+// WIDEK: rows of 3072 < K <= 4096 with 8 wavefronts (16 row pieces a lane instead of 12): the
+// prepacked form has the registers for it; an instantiation of its own, because the four
+// more pieces cost the narrower rows a microsecond a kernel.
+template <int STAGE, int WAVES, int NT, int D, bool KSPLIT = false, int ROUTE = 0, bool PACKED = false,
+          bool WIDEK = false>
 __global__ __launch_bounds__(64 * WAVES) void stream_resident_kernel(GemmArgs p) {
+  static_assert(!WIDEK || (PACKED && WAVES == 8 && STAGE == 0), "the wide rows are the first stage's, prepacked form");
   static_assert(ROUTE == 0 || STAGE == 0, "the routed form is the first stage's");
   static_assert(ROUTE == 0 || 64 * WAVES >= kRouteMaxRows, "a lane per routed row");
   static_assert(!PACKED || (WAVES * (STAGE == 0 ? 8 * NT : 16 * NT)) % (STAGE == 0 ? 64 : 128) == 0,
@@ -1035,7 +1039,7 @@ __global__ __launch_bounds__(64 * WAVES) void stream_resident_kernel(GemmArgs p)
         // exactly), then the rest of the rows.  The weights are so asked for as early
         // as the order of the data allows, and both they and the later row pieces
         // stay in flight while the first pieces are split and written.
-        constexpr int kBatch = resident_batch(WAVES, KSPLIT && PACKED);  // pieces per lane, all of K in one batch
+        constexpr int kBatch = resident_batch(WAVES, WIDEK);  // pieces per lane, all of K in one batch
         // pieces of a lane that K steps [0, D) need (K split: all, every part starts at once)
         constexpr int kFirst = KSPLIT ? kBatch : ((D * 4 + WAVES - 1) / WAVES < kBatch ? (D * 4 + WAVES - 1) / WAVES : kBatch);
         const int n_pieces = (nsteps * 4 + WAVES - 1) / WAVES;  // the launcher keeps it <= kBatch
@@ -2079,11 +2083,12 @@ constexpr size_t kRoutedLdsLimit = kResidentLdsLimit - kRoutedStaticLds;
 
 // True when the device grants the kernel its dynamic LDS (asked once per kernel;
 // a refusal makes the caller take the other variant).
-template <int STAGE, int WAVES, int NT, int D, bool KSPLIT = false, int ROUTE = 0, bool PACKED = false>
+template <int STAGE, int WAVES, int NT, int D, bool KSPLIT = false, int ROUTE = 0, bool PACKED = false,
+          bool WIDEK = false>
 bool resident_kernel_ready() {
   static const bool configured = [] {
     const hipError_t err = hipFuncSetAttribute(
-        reinterpret_cast<const void*>(stream_resident_kernel<STAGE, WAVES, NT, D, KSPLIT, ROUTE, PACKED>),
+        reinterpret_cast<const void*>(stream_resident_kernel<STAGE, WAVES, NT, D, KSPLIT, ROUTE, PACKED, WIDEK>),
         hipFuncAttributeMaxDynamicSharedMemorySize, (int)(ROUTE != 0 ? kRoutedLdsLimit : kResidentLdsLimit));
     if (err != hipSuccess) (void)hipGetLastError();  // not left for the next caller to find
     return err == hipSuccess;
@@ -2091,10 +2096,11 @@ bool resident_kernel_ready() {
   return configured;
 }
 
-template <int STAGE, int WAVES, int NT, int D, bool KSPLIT = false, int ROUTE = 0, bool PACKED = false>
+template <int STAGE, int WAVES, int NT, int D, bool KSPLIT = false, int ROUTE = 0, bool PACKED = false,
+          bool WIDEK = false>
 bool launch_resident(const GemmArgs& g, size_t lds, hipStream_t stream) {
-  if (!resident_kernel_ready<STAGE, WAVES, NT, D, KSPLIT, ROUTE, PACKED>()) return false;
-  hipLaunchKernelGGL((stream_resident_kernel<STAGE, WAVES, NT, D, KSPLIT, ROUTE, PACKED>), dim3(num_compute_units()),
+  if (!resident_kernel_ready<STAGE, WAVES, NT, D, KSPLIT, ROUTE, PACKED, WIDEK>()) return false;
+  hipLaunchKernelGGL((stream_resident_kernel<STAGE, WAVES, NT, D, KSPLIT, ROUTE, PACKED, WIDEK>), dim3(num_compute_units()),
                      dim3(64 * WAVES), lds, stream, g);
   return true;
 }
@@ -2104,6 +2110,7 @@ struct StagePlan {
   int variant, waves, nt, depth;
   bool ksplit;  // the resident kernel with K shared between the wavefronts of a unit
   bool packed;  // ... reading the prepacked form (whenever the caller gives it)
+  bool widek;   // ... its instantiation for rows of 3072 < K <= 4096 with 8 wavefronts
   size_t resident_lds;
 };
 
@@ -2130,10 +2137,13 @@ StagePlan plan_stage(const GemmArgs& g) {
   // (K split: the partial sums of the wavefronts, 1 KB a tile, lie over the operand planes)
   if (pl.ksplit && (size_t)nsteps * 4096 < (size_t)pl.waves * pl.nt * 1024) pl.ksplit = false;
   const int res_units = STAGE == 0 ? g.ncols / (8 * pl.nt) : g.ncols / (16 * pl.nt);
+  // (the wide instantiations exist for the two shapes the rules return at such K)
+  pl.widek = packed && STAGE == 0 && pl.waves == 8 && nsteps * 4 > resident_batch(8) * 8 && pl.nt == 2 &&
+             (pl.ksplit ? pl.depth == 4 : pl.depth == 2);
   if (pl.resident_lds > kResidentLdsLimit || g.num_blocks > kMaxRuns ||
       (!packed && pl.nt * groups > 64 * resident_scale_pieces(pl.waves)) ||
       (res_units + pl.waves - 1) / pl.waves > 64 ||  // one bit per unit in a wavefront's redo mask
-      nsteps * 4 > resident_batch(pl.waves, pl.ksplit && packed) * pl.waves)  // the rows are staged in one batch
+      nsteps * 4 > resident_batch(pl.waves, pl.widek) * pl.waves)  // the rows are staged in one batch
     pl.variant = kMoeVariantLds;
   return pl;
 }
@@ -2159,6 +2169,13 @@ bool wide_kernel_applies(const GemmArgs& g) { return g.Aq != nullptr; }
 template <int STAGE>
 void launch_stage(const GemmArgs& g, const StagePlan& pl, hipStream_t stream) {
   // (a stage without raw weights that is not resident is kept away from here by the callers)
+  if (pl.packed && pl.variant == kMoeVariantResident && pl.widek) {
+    if constexpr (STAGE == 0) {
+      if (pl.ksplit) (void)launch_resident<0, 8, 2, 4, true, 0, true, true>(g, pl.resident_lds, stream);
+      else (void)launch_resident<0, 8, 2, 2, false, 0, true, true>(g, pl.resident_lds, stream);
+    }
+    return;
+  }
   if (pl.packed && pl.variant == kMoeVariantResident) {
 #define VK_RESIDENT(S_, W_, NT_, D_) \
   if constexpr (STAGE == S_) { \
@@ -2380,6 +2397,9 @@ bool prepare_moe_kernels() {
 #undef VK_READY
   ok = resident_kernel_ready<0, 8, 2, 4, true, 1>() && resident_kernel_ready<0, 8, 2, 2, false, 1>() && ok;
   ok = resident_kernel_ready<0, 4, 2, 8, false, 1>() && resident_kernel_ready<0, 4, 2, 8, false, 1, true>() && ok;
+  ok = resident_kernel_ready<0, 8, 2, 2, false, 0, true, true>() && resident_kernel_ready<0, 8, 2, 4, true, 0, true, true>() && ok;
+  ok = resident_kernel_ready<0, 8, 2, 2, false, 1, true, true>() && resident_kernel_ready<0, 8, 2, 4, true, 1, true, true>() && ok;
+  ok = resident_kernel_ready<0, 8, 2, 2, false, 2, true, true>() && ok;
   ok = resident_kernel_ready<0, 8, 2, 2, false, 2>() && resident_kernel_ready<0, 4, 2, 8, false, 2>() && ok;
 #define VK_READY(S_, W_, NT_, D_) ok = resident_kernel_ready<S_, W_, NT_, D_, false, 0, true>() && ok;
   VK_RESIDENT_VARIANTS(VK_READY)
@@ -2440,6 +2460,22 @@ bool launch_routed_moe(const FusedMoeArgs& a, const RoutedArgs& r, hipStream_t s
                     : !p0.ksplit && p0.waves == 4 && p0.nt == 2 && p0.depth == 8 ? 3
                     : 0;
   bool ready = false;
+  if (p0.widek) {  // (shape 1 or 2, prepacked form)
+    if (route_inside) ready = shape == 1 ? resident_kernel_ready<0, 8, 2, 4, true, 1, true, true>()
+                                         : resident_kernel_ready<0, 8, 2, 2, false, 1, true, true>();
+    else ready = shape == 2 && resident_kernel_ready<0, 8, 2, 2, false, 2, true, true>();
+    if (!ready) return false;
+    if (route_inside) {
+      if (shape == 1) launch_resident<0, 8, 2, 4, true, 1, true, true>(g0, p0.resident_lds, stream);
+      else launch_resident<0, 8, 2, 2, false, 1, true, true>(g0, p0.resident_lds, stream);
+    } else {
+      launch_route_topk(r.logits, a.M, r.num_experts, a.top_k, r.renormalize, r.topk_ids, r.topk_w, stream);
+      launch_resident<0, 8, 2, 2, false, 2, true, true>(g0, p0.resident_lds, stream);
+    }
+    g1.topk_w = r.topk_w;
+    launch_stage<1>(g1, p1, stream);
+    return true;
+  }
   if (route_inside) {
     if (shape == 1) ready = p0.packed ? resident_kernel_ready<0, 8, 2, 4, true, 1, true>() : resident_kernel_ready<0, 8, 2, 4, true, 1>();
     if (shape == 2) ready = p0.packed ? resident_kernel_ready<0, 8, 2, 2, false, 1, true>() : resident_kernel_ready<0, 8, 2, 2, false, 1>();

@@ -153,7 +153,7 @@ inline MoeTile pick_moe_tile(int n_flat, int K, int ncols, int stage, bool packe
       return MoeTile{kMoeVariantResidentKSplit, 8, 2, 4};
   }
   const MoeTileRule rules[] = {
-      {0, max_rows, 3072, {kMoeVariantResident, 8, 2, 2}},
+      {0, max_rows, packed ? 4096 : 3072, {kMoeVariantResident, 8, 2, 2}},  // (the prepacked form's rows of a pass: K <= 4096)
       {0, max_rows, 4096, {kMoeVariantResident, 4, 2, 8}},
       {1, max_rows, 1024, {kMoeVariantResident, 8, 1, 4}},
       {1, 24, 3072, {kMoeVariantResident, 8, 2, 4}},
