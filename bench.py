@@ -169,7 +169,6 @@ def run_workload(args, workload, steps, warmup, prepack, split_terms=None, w4a4=
     seed = synth.config_seed(cfg, T)
     dev = torch.device("cuda", 0)
     H, I, k = cfg.H, cfg.I, cfg.top_k
-    prefill = T * k > 512  # the library's own split between its decode and tile kernels
     prepack = prepack and not args.no_workspace   # at every size: the decode kernels read the prepacked form too
     packed_only = prepack and not args.keep_raw
     terms = args.split_terms if split_terms is None else split_terms   # 0 = the library's default
@@ -204,6 +203,8 @@ def run_workload(args, workload, steps, warmup, prepack, split_terms=None, w4a4=
     out = torch.empty((T, H), dtype=torch.float32, device=dev)
     bs = args.block_size or experts[0].block_size_for(T, k)
     lib = ve.load_libvkernels_hip()
+    # the library's own split between its decode and tile kernels
+    prefill = bs > 32 or T * k > int(lib.vk_hip_moe_decode_max_rows(cfg.E if prepack else 0, bs))
     lib.vk_hip_moe_gateup_mxfp4_ex.restype = None
     lib.vk_hip_moe_down_mxfp4_ex.restype = None
 

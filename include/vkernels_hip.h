@@ -274,12 +274,17 @@ int vk_hip_init(void);
  * the decode kernels (blocks of 16) and the tile kernels (blocks of 128) is then rows per
  * expert, and with blocks of 16 the decode kernels also take calls beyond 512 routed
  * rows, up to 9 per expert (where they take the layer's widths at all).
+ * vk_hip_moe_decode_max_rows: the routed rows (M * top_k) up to which a call in blocks of
+ * block_size runs the decode kernels (num_local_experts: of a caller that gives the
+ * prepacked weights, else 0; blocks of 32 are the decode kernels' only on that form).
  *
  * A launch shape is four ints {variant, wavefronts, tiles, depth}: variant 2 =
  * the decode kernel (one workgroup per compute unit, a run's rows resident in
  * LDS), 3 = the same with the K steps of a unit shared between wavefronts (a
- * single token), 0 = the tile kernels; wavefronts per workgroup; 16-row weight
- * tiles per wavefront; K steps in flight per wavefront.
+ * single token), 4 = the decode kernel of the prepacked form that holds the rows a
+ * chunk of K at a time (rows of any K; blocks of 16 or of 32 rows, the 32 rows of a
+ * block in one pass over the expert's weights), 0 = the tile kernels; wavefronts per
+ * workgroup; 16-row weight tiles per wavefront; K steps in flight per wavefront.
  * vk_hip_moe_tile_candidates writes up to `capacity` shapes that stage 0
  * (gate/up) or 1 (down) can be launched at and returns how many there are.
  * vk_hip_moe_tile_query writes the shape a call of this problem size would be
@@ -287,7 +292,7 @@ int vk_hip_init(void);
  * compiled-in rules (a launcher still falls back to the tile kernels where a
  * shape does not fit the device's LDS); stage 2 / 3 ask for stage 0 / 1 of a call
  * that gives the prepacked weights, whose decode kernels have rules of their own
- * (the store's records are shared).
+ * (the store's records are shared), stage 4 / 5 of such a call in blocks of 32 rows.
  * vk_hip_moe_tile_set puts a record for (stage, K, ncols, bucket of n_flat)
  * into the process's store (shape null: removes it); VK_ERROR_INVALID_ARGUMENT
  * for a shape that is not a candidate.  vk_hip_moe_tuning_load reads
@@ -299,6 +304,7 @@ int vk_hip_init(void);
  */
 int vk_hip_moe_default_block_size(int M, int top_k);
 int vk_hip_moe_default_block_size_ex(int M, int top_k, int num_local_experts, int hidden, int ispp);
+int vk_hip_moe_decode_max_rows(int num_local_experts, int block_size);
 int vk_hip_moe_tile_candidates(int stage, int* shapes, int capacity);
 int vk_hip_moe_tile_query(int stage, int K, int ncols, int n_flat, int* shape);
 int vk_hip_moe_tile_set(int stage, int K, int ncols, int n_flat, const int* shape);

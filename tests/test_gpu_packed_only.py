@@ -63,21 +63,23 @@ def test_prefill_sizes_on_the_packed_form_alone(name, T):
     assert np.all(np.isfinite(a["out"]))
 
 
-@pytest.mark.parametrize("name,T", [("c4", 96), ("c2", 256), ("c2", 288)])
+@pytest.mark.parametrize("name,T", [("c4", 96), ("c2", 256), ("c2", 288), ("c4", 255)])
 def test_few_rows_per_expert_beyond_512_rows(name, T):
-    """A caller that gives the prepacked weights gets blocks of 16 and the decode kernels up to
-    9 routed rows per expert (576 rows on 64 experts; 1024 and 1152 on 128 with a few popular
-    ones, where some experts have a dozen passes): the exact-split bounds hold, and the call
-    with blocks of 128 (the prepacked tile kernels) agrees."""
+    """A caller that gives the prepacked weights gets the decode kernels by rows per expert:
+    with blocks of 16 (its own choice) up to 9 per expert (576 rows on 64 experts; 1024 and
+    1152 on 128 with a few popular ones, where some experts have a dozen passes), with the
+    policy's blocks of 32 up to 28 (1530 rows on 64 experts).  The exact-split bounds hold,
+    and the call with blocks of 128 (the prepacked tile kernels) agrees."""
     cfg = synth.CONFIGS[name]
     w = cfgs._weights(cfg)
     A, lg = cfgs._inputs(cfg, T, 6300 + T)
-    g, wn = cfgs._check(cfg, T, w, A, lg, gpu_kw=PACKED_ONLY, tight=True,
-                        block_size=ve.default_block_size(T, cfg.top_k, packed_experts=cfg.E, hidden=cfg.H, ispp=cfg.I))
-    assert g["bs"] == 16 and T * cfg.top_k > 512
+    bs = ve.default_block_size(T, cfg.top_k, packed_experts=cfg.E, hidden=cfg.H, ispp=cfg.I)
+    assert bs == 32 and T * cfg.top_k > 512
     t = cfgs._run_gpu(cfg, w, A, lg, 128, True, **PACKED_ONLY)
-    m, l2, nf = error_metrics(g["out"], t["out"])
-    assert nf and l2 <= 1.5e-3, (m, l2)
+    for bs in ((16, 32) if T < 255 else (32,)):
+        g, wn = cfgs._check(cfg, T, w, A, lg, gpu_kw=PACKED_ONLY, tight=True, block_size=bs, stagewise=(T == 255))
+        m, l2, nf = error_metrics(g["out"], t["out"])
+        assert nf and l2 <= 1.5e-3, (m, l2)
 
 
 @pytest.mark.parametrize("T", [4, 300])
@@ -117,31 +119,34 @@ def test_values_outside_the_range_on_the_packed_form_alone(T):
     assert np.bincount(ids.ravel(), minlength=cfg.E)[:4].min() > 0
 
 
-def test_a_wide_first_stage_on_the_packed_form_alone():
-    """Rows of more than 4096 values do not fit the decode kernels' LDS: with the raw tensors
-    such a call runs the tile kernels on them; without, the prepacked kernels, whatever the
-    batch (they need the workspace)."""
-    cfg = synth.MoEConfig("wide", 4608, 256, 4, 2, (5,), "uniform")
-    T, seed = 5, 6400
+@pytest.mark.parametrize("T", [5, 300])
+def test_a_wide_first_stage_on_the_packed_form_alone(T):
+    """Rows of more than 4096 values do not fit the resident decode kernel's LDS: with the raw
+    tensors such a call runs the tile kernels on them; without, the chunked decode kernel
+    (T = 5) or the prepacked kernels (T = 300: 150 rows per expert), which need the workspace."""
+    cfg = synth.MoEConfig("wide", 4608, 256, 4, 2, (T,), "uniform")
+    seed = 6400
     w = synth.make_weights(cfg.E, cfg.H, cfg.I, seed, device=dev())
     A, lg = cfgs._inputs(cfg, T, seed)
     g = cfgs._run_gpu(cfg, w, A, lg, None, True, **PACKED_ONLY)
     ids, tw = oracle.route_topk(lg, cfg.top_k, True)
     c = cpu_layer(A, w.numpy(), ids, tw, threads=16)
     max_rel, rel_l2, nf = error_metrics(g["out"], c["out"])
-    print(f"wide first stage, packed form alone: max_abs/rms={max_rel:.3e} rel_l2={rel_l2:.3e}")
+    print(f"wide first stage, packed form alone, T={T}: max_abs/rms={max_rel:.3e} rel_l2={rel_l2:.3e}")
     assert nf and max_rel <= MAX_ABS_TOL and rel_l2 <= REL_L2_TOL
-    # and without a workspace the call is refused, not run on weights that are not there
+    if T == 5:
+        return
+    # and without a workspace the prefill-sized call is refused, not run on weights that are not there
     fe = ve.FusedExperts(w.w13, w.w13_scale, w.w2, w.w2_scale, scratch=ve.CaptureSafeScratch(), **PACKED_ONLY)
     d_ids, d_tw = to_dev(ids), to_dev(tw)
-    sids, eids, _, max_em = fe.align(d_ids, 16)
+    sids, eids, _, max_em = fe.align(d_ids, 128)
     act = torch.zeros((max_em, cfg.I), dtype=torch.bfloat16, device=dev())
     out = torch.full((T, cfg.H), 3.0, dtype=torch.float32, device=dev())
     d_A = to_dev(A, torch.bfloat16)
     fe.lib.vk_set_last_error(0, b"")
     fe.moe_prepacked_fn(d_A.data_ptr(), None, None, None, None, d_ids.data_ptr(), d_tw.data_ptr(), act.data_ptr(),
                         out.data_ptr(), T, cfg.H, cfg.I, cfg.top_k, sids.data_ptr(), eids.data_ptr(), max_em,
-                        0.0, 0, 4.0, 25.0, None, None, 16, None, 0, 0, fe.w13_packed.data_ptr(),
+                        0.0, 0, 4.0, 25.0, None, None, 128, None, 0, 0, fe.w13_packed.data_ptr(),
                         fe.w2_packed.data_ptr(), cfg.E, None)
     torch.cuda.synchronize()
     assert fe.lib.vk_last_error_code() == ve.VK_ERROR_INVALID_ARGUMENT

@@ -37,7 +37,7 @@ def _check(cfg, T, w, seed, block_size=None, expert_map=None, local_n=None, **kw
     got = fe.route_layer(A, to_dev(lg), cfg.top_k, block_size=block_size, out_fp32=out)
     torch.cuda.synchronize()
     _, ids, tw, sids, eids, out_em, max_em = got
-    bs = block_size or ve.default_block_size(T, cfg.top_k)
+    bs = block_size or fe.block_size_for(T, cfg.top_k)   # (with the prepacked weights: 32 beyond 256 routed rows)
     rid, rtw = oracle.route_topk(lg, cfg.top_k, True)
     assert np.array_equal(ids.cpu().numpy(), rid), "top-k indices differ from the oracle"
     assert np.array_equal(tw.cpu().numpy().view(np.uint32), rtw.view(np.uint32)), "router weights differ"

@@ -50,17 +50,23 @@ def test_default_block_size():
     assert ve.default_block_size(64, 4) == 16 and ve.default_block_size(128, 4) == 16
     assert ve.default_block_size(129, 4) == 128 and ve.default_block_size(2047, 8) == 128
     assert ve.default_block_size(2048, 8) == 128 and ve.default_block_size(16384, 8) == 128
-    # a caller that gives the prepacked weights: by rows per expert as well (9), as long as
-    # the runs (a block per 16 rows and one more per expert) fit the decode kernels' list of 512
-    # and the decode kernels take the layer's widths
+    # a caller that gives the prepacked weights: blocks of 16 while the first stage's kernel
+    # can align for itself (256 routed rows), then blocks of 32 (a block a pass on the chunked
+    # decode kernel) up to 28 rows per expert, as long as the runs fit the kernels' list of 512
     c4 = dict(packed_experts=64, hidden=4096, ispp=1536)
-    assert ve.default_block_size(96, 6, **c4) == 16 and ve.default_block_size(97, 6, **c4) == 128     # 576 / 582 rows
+    assert ve.default_block_size(42, 6, **c4) == 16 and ve.default_block_size(43, 6, **c4) == 32      # 252 / 258 rows
+    assert ve.default_block_size(298, 6, **c4) == 32 and ve.default_block_size(299, 6, **c4) == 128   # 1788 / 1794 rows
     c2 = dict(packed_experts=128, hidden=2880, ispp=2880)
-    assert ve.default_block_size(288, 4, **c2) == 16 and ve.default_block_size(289, 4, **c2) == 128
-    assert ve.default_block_size(128, 4, packed_experts=8, hidden=2880, ispp=2880) == 16   # 512 rows: decode-sized anyway
+    assert ve.default_block_size(64, 4, **c2) == 16 and ve.default_block_size(896, 4, **c2) == 32
+    assert ve.default_block_size(897, 4, **c2) == 128
+    assert ve.default_block_size(128, 4, packed_experts=8, hidden=2880, ispp=2880) == 32   # 512 rows: decode-sized anyway
     assert ve.default_block_size(129, 4, packed_experts=8, hidden=2880, ispp=2880) == 128
-    assert ve.default_block_size(250, 8, packed_experts=256, hidden=7168, ispp=2048) == 128   # rows too wide for them
+    assert ve.default_block_size(250, 8, packed_experts=256, hidden=7168, ispp=2048) == 32   # rows of any K
     assert ve.default_block_size(512, 8, packed_experts=500, hidden=2880, ispp=2880) == 128   # room for 12 runs only
+    lib = ve.load_libvkernels_hip()
+    assert lib.vk_hip_moe_decode_max_rows(0, 16) == 512 and lib.vk_hip_moe_decode_max_rows(64, 16) == 576
+    assert lib.vk_hip_moe_decode_max_rows(64, 32) == 1792 and lib.vk_hip_moe_decode_max_rows(0, 32) == 0
+    assert lib.vk_hip_moe_decode_max_rows(64, 128) == 512
 
 
 @pytest.mark.parametrize("M,top_k,E,bs", [(1, 1, 8, 16), (4, 2, 8, 16), (64, 4, 32, 64),
@@ -311,7 +317,8 @@ def test_synth_is_deterministic_and_prefix_stable():
 def test_tile_candidates_and_compiled_in_rules():
     for stage in (0, 1):
         cands = ve.moe_tile_candidates(stage)
-        assert len(cands) == 8 and len(set(cands)) == 8
+        assert len(cands) == 10 and len(set(cands)) == 10
+        assert sum(c[0] == 4 for c in cands) == 2         # the chunked decode kernel (prepacked form)
         plain = {c[1:] for c in cands if c[0] == 2}
         assert all(c[1:] in plain for c in cands if c[0] == 3)   # a K-split shape has its plain form to fall back to
         assert (0, 4, 4, 0) in cands                      # the tile kernels
@@ -327,6 +334,12 @@ def test_tile_candidates_and_compiled_in_rules():
     assert ve.moe_tile_query(0, 4096, 1536, 198, packed=True)[0] == (2, 8, 2, 2)
     assert ve.moe_tile_query(0, 4096, 1536, 6, packed=True)[0] == (3, 8, 2, 4)
     assert ve.moe_tile_query(0, 2880, 2880, 256, packed=True)[0] == ve.moe_tile_query(0, 2880, 2880, 256)[0]
+    # the chunked kernel: rows of a K beyond those, and every call in blocks of 32 (prepacked form only)
+    assert ve.moe_tile_query(0, 7168, 2048, 64, packed=True)[0] == (4, 8, 2, 2)
+    assert ve.moe_tile_query(1, 4224, 512, 64, packed=True)[0] == (4, 8, 1, 4)
+    assert ve.moe_tile_query(0, 2880, 2880, 512, packed=True, block_size=32)[0] == (4, 8, 2, 2)
+    assert ve.moe_tile_query(1, 2880, 2880, 512, packed=True, block_size=32)[0] == (4, 8, 1, 4)
+    assert ve.moe_tile_query(0, 7168, 2048, 64)[0] == (0, 4, 4, 0)
     # one token: fewer units than half the device's wavefronts, K shared between them
     assert ve.moe_tile_query(0, 2880, 2880, 4)[0] == (3, 8, 2, 4) and ve.moe_tile_query(1, 2880, 2880, 4)[0] == (3, 8, 1, 8)
     assert ve.moe_tile_query(1, 1536, 4096, 6)[0] == (3, 8, 2, 4)                   # ... with two tiles a unit

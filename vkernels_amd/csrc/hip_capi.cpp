@@ -573,6 +573,12 @@ int vk_hip_moe_default_block_size_ex(int M, int top_k, int num_local_experts, in
                                     num_local_experts < 0 ? 0 : num_local_experts, hidden, ispp);
 }
 
+int vk_hip_moe_decode_max_rows(int num_local_experts, int block_size) {
+  if (block_size == 32) return num_local_experts > 0 ? vk::moe_decode_max_rows32(num_local_experts) : 0;
+  if (block_size != 16) return vk::kMoeDecodeMaxRows;
+  return vk::moe_decode_max_rows(num_local_experts < 0 ? 0 : num_local_experts);
+}
+
 int vk_hip_moe_tile_candidates(int stage, int* shapes, int capacity) {
   size_t n = 0;
   const vk::MoeTileCandidate* table = vk::moe_tile_candidates(&n);
@@ -591,10 +597,12 @@ int vk_hip_moe_tile_candidates(int stage, int* shapes, int capacity) {
 
 int vk_hip_moe_tile_query(int stage, int K, int ncols, int n_flat, int* shape) {
   vk::MoeTile t;
-  const bool packed = stage == 2 || stage == 3;  // the stage on the prepacked form
-  if (packed) stage -= 2;
+  // stage + 2: the stage on the prepacked form; stage + 4: ... with blocks of 32 rows
+  const bool packed = stage >= 2 && stage <= 5;
+  const int block_rows = stage >= 4 && stage <= 5 ? 32 : 16;
+  if (packed) stage &= 1;
   const bool stored = vk::moe_tuning_find(stage, K, ncols, n_flat, &t);
-  if (!stored) t = vk::pick_moe_tile(n_flat, K, ncols, stage, packed);
+  if (!stored) t = vk::pick_moe_tile(n_flat, K, ncols, stage, packed, 0, block_rows);
   if (shape != nullptr) {
     shape[0] = t.variant; shape[1] = t.waves; shape[2] = t.nt; shape[3] = t.depth;
   }

@@ -206,6 +206,61 @@ __device__ __forceinline__ void epilogue_tile(const GemmArgs& p, int e, const f3
   }
 }
 
+// Second stage of the decode kernels: the same tile the other way round,
+// acc[t][r] = C[activation row 4*lq + r][weight row ln of tile t] (the kernels give the
+// matrix cores the rows as the first operand there).  The 16 lanes of a quarter then add
+// into 16 consecutive floats of one row of `out`, a whole 64-byte sector an instruction,
+// where the layout above has four lanes to a sector and sixteen sectors an instruction:
+// the atomic units take a request per sector, and a step's additions cost a tenth.
+// flat4[r] = the flat index of row 4*lq + r of the tile (< 0: padding), w4[r] its routing
+// weight (rows_weights below: asked for when the rows are listed, not here, where a load
+// would have every weight load in flight waited for first), srow0 = the tile's first
+// sorted row.
+__device__ __forceinline__ void rows_weights(const GemmArgs& p, const int (&flat4)[4], float (&w4)[4]) {
+  if (p.topk_w == nullptr) {  // (the linear part alone)
+#pragma unroll
+    for (int r = 0; r < 4; ++r) w4[r] = 0.f;
+    return;
+  }
+  // no load under a condition: one that is skipped by its lanes would still be waited for
+#pragma unroll
+  for (int r = 0; r < 4; ++r) w4[r] = p.topk_w[max(flat4[r], 0)];
+}
+
+template <int NT>
+__device__ __forceinline__ void epilogue_rows(const GemmArgs& p, int e, const f32x4 (&acc)[NT],
+                                              const int (&col0)[NT], const int (&flat4)[4],
+                                              const float (&w4)[4], int srow0, int lane) {
+  const int ln = lane & 15, lq = lane >> 4;
+  if (p.preact != nullptr) {  // the linear part alone, as fp32
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      if (flat4[r] < 0) continue;
+      float* row = p.preact + (size_t)(srow0 + 4 * lq + r) * (size_t)p.ncols;
+#pragma unroll
+      for (int t = 0; t < NT; ++t) row[col0[t] + ln] = acc[t][r];
+    }
+    return;
+  }
+  float b[NT];
+#pragma unroll
+  for (int t = 0; t < NT; ++t) b[t] = 0.f;
+  if (p.bias != nullptr) {  // uniform
+#pragma unroll
+    for (int t = 0; t < NT; ++t) {
+      b[t] = p.bias[(size_t)e * (size_t)p.ncols + col0[t] + ln];
+      __asm__ volatile("" : "+v"(b[t]));  // (waited for here, by every lane)
+    }
+  }
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    if (flat4[r] < 0) continue;
+    float* orow = p.out + (size_t)(flat4[r] / p.top_k) * (size_t)p.ncols + ln;
+#pragma unroll
+    for (int t = 0; t < NT; ++t) unsafeAtomicAdd(orow + col0[t], (acc[t][r] + b[t]) * w4[r]);
+  }
+}
+
 // Weight rows, scale rows and first output column of the NT tiles of `unit`.
 template <int STAGE, int NT>
 __device__ __forceinline__ void unit_tiles(const GemmArgs& p, int e, int unit, int ln,
@@ -399,7 +454,9 @@ constexpr int kStagingUnits = 4;
 // Reference-exact slow path for one unit: one K step at a time, integer-exact
 // dequantisation, the activation row of this lane's column read from global
 // memory (a_row null = padding row).
-template <int NT>
+// ROWS_FIRST: the activation rows as the first operand (the tile the other way round, for
+// epilogue_rows).
+template <int NT, bool ROWS_FIRST = false>
 __device__ __forceinline__ void exact_unit_global(const uint8_t* const (&w_rows)[NT],
                                                   const uint8_t* const (&s_rows)[NT],
                                                   const uint16_t* a_row, int K, int lane,
@@ -423,8 +480,12 @@ __device__ __forceinline__ void exact_unit_global(const uint8_t* const (&w_rows)
           x = *reinterpret_cast<const uint32_t*>(w_rows[t] + (size_t)g * 16 + d * 4);
           sc = s_rows[t][g];
         }
-        acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(dequant8_exact(x, sc)),
-                                                         as_bf16x8(av), acc[t], 0, 0, 0);
+        if constexpr (ROWS_FIRST)
+          acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(av), as_bf16x8(dequant8_exact(x, sc)),
+                                                           acc[t], 0, 0, 0);
+        else
+          acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(dequant8_exact(x, sc)),
+                                                           as_bf16x8(av), acc[t], 0, 0, 0);
       }
     }
   }
@@ -433,7 +494,7 @@ __device__ __forceinline__ void exact_unit_global(const uint8_t* const (&w_rows)
 // The same from the prepacked form (pointers of unit_tiles_packed).  raw: the unit is
 // flagged and holds the raw codes and scale bytes; otherwise the move onto the OCP code
 // points and the decrement of the scale byte are undone (all codes of such a unit are finite).
-template <int NT>
+template <int NT, bool ROWS_FIRST = false>
 __device__ __forceinline__ void exact_unit_packed(const uint8_t* const (&w_rows)[NT],
                                                   const uint8_t* const (&s_rows)[NT],
                                                   const int (&shift)[NT], bool raw, const uint16_t* a_row,
@@ -461,8 +522,12 @@ __device__ __forceinline__ void exact_unit_packed(const uint8_t* const (&w_rows)
             sc = (sc + 1u) & 0xFFu;
           }
         }
-        acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(dequant8_exact(x, sc)),
-                                                         as_bf16x8(av), acc[t], 0, 0, 0);
+        if constexpr (ROWS_FIRST)
+          acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(av), as_bf16x8(dequant8_exact(x, sc)),
+                                                           acc[t], 0, 0, 0);
+        else
+          acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(dequant8_exact(x, sc)),
+                                                           as_bf16x8(av), acc[t], 0, 0, 0);
       }
     }
   }
@@ -526,7 +591,7 @@ __host__ __device__ constexpr int resident_batch(int waves, bool wide = false) {
 // (with more than a handful of tokens every workgroup routing all of them costs more than
 // that launch) and the kernel only aligns, which saves the alignment's launch and this
 // kernel's listing of the runs.
-constexpr int kRouteMaxRows = 256, kRouteMaxExperts = 256, kRoutePer = kRouteMaxExperts / 64;
+constexpr int kRouteMaxRows = kMoeRoutedMaxRows, kRouteMaxExperts = 256, kRoutePer = kRouteMaxExperts / 64;
 constexpr int kRouteMaxTokens = 16;  // ROUTE = 1: tokens every workgroup routes for itself
 
 // A workgroup barrier for LDS alone.  __syncthreads() is a workgroup-wide fence as well,
@@ -1025,6 +1090,11 @@ __global__ __launch_bounds__(64 * WAVES) void stream_resident_kernel(GemmArgs p)
         const int tile = tile0 + tt;
         const int my_flat = __shfl(fl, tt * 16 + ln);         // row of this lane's outputs
         const int st_flat = __shfl(fl, tt * 16 + (lane >> 2));  // row this lane stages
+        int flat4[4];  // second stage: the rows 4 lq + r of this lane's outputs (epilogue_rows)
+#pragma unroll
+        for (int r4 = 0; r4 < 4; ++r4) flat4[r4] = STAGE == 1 ? __shfl(fl, tt * 16 + 4 * lq + r4) : -1;
+        float w4[4] = {0.f, 0.f, 0.f, 0.f};
+        if constexpr (STAGE == 1) rows_weights(p, flat4, w4);
         const int srow = run_row0 + tile * 16 + ln;
         const int flag = pass_no & 1;
         ++pass_no;
@@ -1177,14 +1247,19 @@ __global__ __launch_bounds__(64 * WAVES) void stream_resident_kernel(GemmArgs p)
 #pragma unroll
           for (int t = 0; t < NT; ++t) wa[t] = PACKED ? fp4_operand_packed(sg.w[t]) : fp4_operand(sg.w[t]);
           // the two MFMAs of an accumulator are kept NT instructions apart
+          // (second stage: the rows as the first operand, for epilogue_rows)
 #pragma unroll
           for (int t = 0; t < NT; ++t)
-            acc[t] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wa[t], bh, acc[t], 4, 0, 0,
-                                                                      sa[t], 0, sbh);
+            acc[t] = STAGE == 1 ? __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(bh, wa[t], acc[t], 0, 4, 0,
+                                                                                   sbh, 0, sa[t])
+                                : __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wa[t], bh, acc[t], 4, 0, 0,
+                                                                                   sa[t], 0, sbh);
 #pragma unroll
           for (int t = 0; t < NT; ++t)
-            acc[t] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wa[t], bl, acc[t], 4, 0, 0,
-                                                                      sa[t], 0, sbl);
+            acc[t] = STAGE == 1 ? __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(bl, wa[t], acc[t], 0, 4, 0,
+                                                                                   sbl, 0, sa[t])
+                                : __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wa[t], bl, acc[t], 4, 0, 0,
+                                                                                   sa[t], 0, sbl);
         };
 
         if constexpr (KSPLIT) {
@@ -1222,6 +1297,8 @@ __global__ __launch_bounds__(64 * WAVES) void stream_resident_kernel(GemmArgs p)
               }
               if (any_bad || (PACKED && cur_flag != 0u))
                 redo = 1ull;
+              else if (STAGE == 1)
+                epilogue_rows<NT>(p, e, acc, col0, flat4, w4, run_row0 + tile * 16, lane);
               else if (my_flat >= 0)
                 epilogue_tile<STAGE, NT>(p, e, acc, col0, my_flat, srow, lq);
             }
@@ -1255,6 +1332,8 @@ __global__ __launch_bounds__(64 * WAVES) void stream_resident_kernel(GemmArgs p)
                   // domain, is redone after the stream, so the hot loop stays small
                   if (__ballot(bad != 0u) != 0ull || pass_slow[flag] != 0 || (PACKED && cur_flag != 0u))
                     redo |= 1ull << cunit;
+                  else if (STAGE == 1)
+                    epilogue_rows<NT>(p, e, acc, col0, flat4, w4, run_row0 + tile * 16, lane);
                   else if (my_flat >= 0)
                     epilogue_tile<STAGE, NT>(p, e, acc, col0, my_flat, srow, lq);
                   if (++cunit < n_my) {
@@ -1294,13 +1373,405 @@ __global__ __launch_bounds__(64 * WAVES) void stream_resident_kernel(GemmArgs p)
             redo &= redo - 1ull;
             if constexpr (PACKED) {
               unit_tiles_packed<STAGE, NT>(p, e, first + idx * WAVES, lane, nsteps, cw, cs, shift, col0, cur_pu);
-              exact_unit_packed<NT>(cw, cs, shift, packed_unit_flag(p, e, cur_pu) != 0u, a_row, K, lane, acc);
+              exact_unit_packed<NT, STAGE == 1>(cw, cs, shift, packed_unit_flag(p, e, cur_pu) != 0u, a_row, K, lane, acc);
             } else {
               unit_tiles<STAGE, NT>(p, e, first + idx * WAVES, ln, cw, cs, col0);
-              exact_unit_global<NT>(cw, cs, a_row, K, lane, acc);
+              exact_unit_global<NT, STAGE == 1>(cw, cs, a_row, K, lane, acc);
             }
-            if (my_flat >= 0) epilogue_tile<STAGE, NT>(p, e, acc, col0, my_flat, srow, lq);
+            if (STAGE == 1) epilogue_rows<NT>(p, e, acc, col0, flat4, w4, run_row0 + tile * 16, lane);
+            else if (my_flat >= 0) epilogue_tile<STAGE, NT>(p, e, acc, col0, my_flat, srow, lq);
           }
+        }
+      }
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
+// Decode kernel, chunked form: the prepacked weights, rows of any K, and one or two 16-row
+// tiles of an expert a pass over its weights (blocks of 16 MT rows).
+//
+// The resident kernel above keeps the rows of a pass in LDS for all of K, which bounds K
+// (4096 values) and the rows (16).  Here the rows are in LDS a chunk of kChunkSteps K steps
+// at a time, twice over (the chunk being multiplied and the next one, written while the
+// first runs), and a wavefront keeps the sums of all its units of a segment in registers
+// across the chunks: per chunk it walks its units' K steps of that chunk, one unit after
+// the other, as one stream of loads (D steps in flight, the cursor crossing from unit to
+// unit and from chunk to chunk), with one workgroup barrier a chunk.  A segment is at most
+// kChunkWaves x chunked_max_units units of one run; a slice longer than that stages its rows again
+// per segment (a few per cent of the segment's weight bytes).  With MT = 2 every weight
+// register is multiplied with both row tiles, so an expert with 17 to 32 rows costs one
+// pass over its weights instead of two (a tile without a routed row is skipped).
+// Work split, arithmetic, the exact path and the epilogue are the resident kernel's.
+// ---------------------------------------------------------------------------
+constexpr int kChunkWaves = 8;
+constexpr int kChunkSteps = 8;
+// Units of a wavefront in a segment: their sums (4 registers per tile of weights and of
+// rows) must leave room for the weight steps in flight and a chunk's row pieces; a kernel
+// that spills pays for every reload with a wait for all its loads in flight.
+__host__ __device__ constexpr int chunked_max_units(int nt, int mt) { return (mt == 2 ? 12 : 16) / nt; }
+__host__ __device__ constexpr size_t chunked_lds_bytes(int mt) {
+  return (size_t)2 * kChunkSteps * (size_t)mt * (4096 + 64);
+}
+
+template <int STAGE, int NT, int D, int MT>
+__global__ __launch_bounds__(64 * kChunkWaves) void stream_chunked_kernel(GemmArgs p) {
+  constexpr int WAVES = kChunkWaves, KC = kChunkSteps;
+  constexpr int kMaxU = chunked_max_units(NT, MT);  // units of a wavefront in a segment
+  constexpr int kPieces = KC * 4 / WAVES;  // 16-byte row pieces of a lane per tile and chunk
+  static_assert(KC % D == 0 && (KC * 4) % WAVES == 0, "whole rounds of the pipeline and of the staging per chunk");
+  static_assert((WAVES * (STAGE == 0 ? 8 * NT : 16 * NT)) % (STAGE == 0 ? 64 : 128) == 0,
+                "a wavefront's consecutive units are whole packed units apart");
+  extern __shared__ u32x4 b_lds[];  // [2][KC][MT][2 terms][2 halves][64] operand planes, then the block scales
+  __shared__ int run_block0[kMaxRuns];
+  __shared__ int run_expert[kMaxRuns];
+  __shared__ int n_runs_sh;
+  __shared__ int pass_slow[2];
+  if (STAGE == 0) clear_out_share<64 * WAVES>(p);
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int ln = lane & 15;
+  const int lq = lane >> 4;
+
+  const int K = p.K;
+  const int groups = K / 32;
+  const int nsteps = (groups + 3) / 4;
+  const int nchunks = (nsteps + KC - 1) / KC;
+  const int units = STAGE == 0 ? p.ncols / (8 * NT) : p.ncols / (16 * NT);
+  uint8_t* const bsc_lds = reinterpret_cast<uint8_t*>(b_lds + (size_t)2 * KC * MT * 256);  // [2][KC][MT][64]
+  constexpr int kPackedStride = WAVES * (STAGE == 0 ? 8 * NT : 16 * NT) / (STAGE == 0 ? 64 : 128);
+  const size_t w_unit_stride = (size_t)kPackedStride * (size_t)nsteps * (size_t)kMxStepBytes;
+  constexpr int kNS = STAGE == 0 ? NT / 2 : NT;  // scale words of a K step a lane loads
+
+  // ---- the runs: every block with an expert, in order (a pass each) ----
+  if (wave == 0) {
+    const int nb = p.num_blocks;
+    const unsigned long long below = (1ull << lane) - 1ull;
+    int n = 0;
+    for (int base = 0; base < nb; base += 64) {
+      const int b = base + lane;
+      const int e = b < nb ? p.expert_ids[b] : -1;
+      const unsigned long long mr = __ballot(e >= 0);
+      if (e >= 0) {
+        const int idx = n + (int)__popcll(mr & below);
+        if (idx < kMaxRuns) {
+          run_block0[idx] = b;
+          run_expert[idx] = e;
+        }
+      }
+      n += (int)__popcll(mr);
+    }
+    if (lane == 0) {
+      n_runs_sh = n < kMaxRuns ? n : kMaxRuns;
+      pass_slow[0] = 0;
+      pass_slow[1] = 0;
+    }
+  }
+  lds_barrier();
+  // ---- this workgroup's slice of the (run, unit) space: every run workgroups of its own
+  // where that leaves them balanced (no slice then stages two runs), else cut evenly ----
+  int s0 = 0, s1 = 0;
+  {
+    const int n = n_runs_sh;
+    const int grid = (int)gridDim.x, wg = (int)blockIdx.x;
+    if (n > 0) {
+      bool aligned = n <= grid;
+      if (aligned) {
+        const int limit = (units * n + grid - 1) / grid + kStagingUnits;
+        const int g_min = grid / n;
+        aligned = (units + g_min - 1) / g_min <= limit;
+      }
+      if (aligned) {  // run r has workgroups [grid r / n, grid (r + 1) / n)
+        const int r = ((wg + 1) * n + grid - 1) / grid - 1;
+        const int begin = (int)((unsigned)(grid * r) / (unsigned)n);
+        const int end = (int)((unsigned)(grid * (r + 1)) / (unsigned)n);
+        s0 = r * units + slice_begin(units, wg - begin, end - begin);
+        s1 = r * units + slice_begin(units, wg - begin + 1, end - begin);
+      } else {
+        s0 = slice_begin(n * units, wg, grid);
+        s1 = slice_begin(n * units, wg + 1, grid);
+      }
+    }
+  }
+  if (s0 >= s1) return;  // uniform over the workgroup
+
+  struct Stage {
+    u32x4 w[NT];
+    uint32_t s[kNS];
+  };
+  int seg_no = 0;
+  // what depends on the lane alone: where it writes a row piece and which group it stages
+  const int sd = lane & 3;   // eighth of the group of 32
+  const int sj = lane >> 2;  // row of the tile
+  const int g4 = wave & 3;   // the wavefront's group within a K step (piece `it`: step (wave >> 2) + 2 it)
+  const int plane_lane = (((g4 >> 1) * 64 + ((g4 & 1) * 2 + (sd >> 1)) * 16 + sj) * 16) + (sd & 1) * 8;
+
+  for (int sl = s0; sl < s1;) {
+    const int r = sl / units;
+    const int base_slot = r * units;
+    const int u0 = sl - base_slot;
+    const int u1 = min(min(s1, base_slot + units) - base_slot, u0 + WAVES * kMaxU);
+    sl = base_slot + u1;
+    const int e = run_expert[r];
+    const int run_row0 = run_block0[r] * p.block_size;  // (block_size = 16 MT)
+    const int first = u0 + wave;
+    const int n_my = first < u1 ? (u1 - first + WAVES - 1) / WAVES : 0;
+    const int flag = seg_no & 1;
+    ++seg_no;
+
+    // ---- the rows of the run ----
+    int fl = -1;
+    if (lane < 16 * MT) fl = p.sorted_ids[run_row0 + lane];
+    if (fl < 0 || fl >= p.n_flat) fl = -1;
+    const unsigned long long routed = __ballot(fl >= 0);
+    const bool live1 = MT > 1 && ((routed >> 16) & 0xFFFFull) != 0ull;  // the second tile has a routed row
+    int my_flat[MT], st_flat[MT];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+      my_flat[mt] = __shfl(fl, mt * 16 + ln);   // row of this lane's outputs
+      st_flat[mt] = __shfl(fl, mt * 16 + sj);   // row this lane stages
+    }
+    int flat4[MT][4];  // second stage: the rows 4 lq + r of this lane's outputs (epilogue_rows)
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+      for (int r4 = 0; r4 < 4; ++r4) flat4[mt][r4] = STAGE == 1 ? __shfl(fl, mt * 16 + 4 * lq + r4) : -1;
+    float w4[MT][4];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+#pragma unroll
+      for (int r4 = 0; r4 < 4; ++r4) w4[mt][r4] = 0.f;
+      if constexpr (STAGE == 1) rows_weights(p, flat4[mt], w4[mt]);
+    }
+    uint32_t row_off[MT];  // bytes from A to the lane's eighth of the wavefront's first group
+    bool has_row[MT];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+      has_row[mt] = st_flat[mt] >= 0;
+      row_off[mt] = has_row[mt]
+                        ? ((uint32_t)(STAGE == 0 ? st_flat[mt] / p.top_k : run_row0 + mt * 16 + sj) * (uint32_t)p.a_stride +
+                           (uint32_t)(wave * 32 + sd * 8)) * 2u
+                        : 0u;
+    }
+    const char* const a_base = reinterpret_cast<const char*>(p.A);
+    u32x4 v[MT * kPieces];
+    // piece (mt, it) of chunk c: group c KC 4 + wave + it WAVES of tile mt's rows
+    auto load_rows = [&](int c) {
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) {
+#pragma unroll
+        for (int it = 0; it < kPieces; ++it) {
+          const int gi = c * (KC * 4) + wave + it * WAVES;  // uniform
+          const uint32_t off = gi < groups ? (uint32_t)((c * (KC * 4) + it * WAVES) * 64) + row_off[mt] : 0u;
+          v[mt * kPieces + it] = *reinterpret_cast<const u32x4*>(a_base + off);
+        }
+      }
+    };
+    auto block_scale = [&](const u32x4& x) -> uint32_t {
+      uint32_t emax = bf16x8_max_exponent(x);
+      emax = max(emax, (uint32_t)__builtin_amdgcn_mov_dpp((int)emax, 0xB1, 0xF, 0xF, true));
+      emax = max(emax, (uint32_t)__builtin_amdgcn_mov_dpp((int)emax, 0x4E, 0xF, 0xF, true));
+      if (emax == 0u) return 127u;
+      const uint32_t sb = emax - 7u;
+      return (sb < kScaleLo || sb > kScaleHi) ? 0u : sb;
+    };
+    // split the pieces of chunk c and write them to buffer `buf`
+    auto write_rows = [&](int c, int buf) {
+      bool slow = false;
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) {
+        if (mt > 0 && !live1) continue;  // uniform
+#pragma unroll
+        for (int it = 0; it < kPieces; ++it) {
+          const int gi = c * (KC * 4) + wave + it * WAVES;
+          u32x4 x = v[mt * kPieces + it];
+          if (!(gi < groups && has_row[mt])) x = u32x4{0u, 0u, 0u, 0u};
+          uint32_t sb = block_scale(x);
+          if (sb == 0u) {
+            slow = true;
+            sb = 127u;
+          }
+          uint2 hi, lo;
+          split_bf16x8(x, sb, hi, lo);
+          const int ksl = (wave >> 2) + it * (WAVES / 4);  // step of the chunk
+          const int slot = (buf * KC + ksl) * MT + mt;
+          uint8_t* plane = reinterpret_cast<uint8_t*>(b_lds) + (size_t)slot * 4096 + plane_lane;
+          *reinterpret_cast<uint2*>(plane) = hi;
+          *reinterpret_cast<uint2*>(plane + 2 * 64 * 16) = lo;
+          if (sd == 0) bsc_lds[slot * 64 + g4 * 16 + sj] = (uint8_t)sb;
+        }
+      }
+      if (slow) pass_slow[flag] = 1;
+    };
+
+    // ---- the weight stream's cursor: chunk by chunk, within a chunk unit by unit ----
+    const uint8_t* cw[NT];
+    const uint8_t* cs[NT];
+    int col0[NT];
+    int shift[NT];
+    int pu0 = 0;
+    unit_tiles_packed<STAGE, NT>(p, e, n_my > 0 ? first : u0, lane, nsteps, cw, cs, shift, col0, pu0);
+    const uint8_t* lrow[NT];
+    const uint8_t* lsc[kNS];
+#pragma unroll
+    for (int t = 0; t < NT; ++t) lrow[t] = cw[t];
+#pragma unroll
+    for (int j = 0; j < kNS; ++j) lsc[j] = cs[j];
+    int ld_i = 0;           // position in the current (unit, chunk): 0 .. its steps rounded up to D
+    int ld_u = n_my;        // units of the chunk the cursor has not finished
+    int ld_k0 = 0;          // first step of the cursor's chunk
+    int ld_cs = min(KC, nsteps);  // its steps
+    const size_t rewind = (size_t)(n_my > 0 ? n_my - 1 : 0) * w_unit_stride;
+    auto issue = [&](Stage& st) {
+      const size_t step = (size_t)(ld_k0 + min(ld_i, ld_cs - 1)) * (size_t)kMxStepBytes;
+#pragma unroll
+      for (int t = 0; t < NT; ++t) st.w[t] = *reinterpret_cast<const u32x4*>(lrow[t] + step);
+#pragma unroll
+      for (int j = 0; j < kNS; ++j) st.s[j] = *reinterpret_cast<const uint32_t*>(lsc[j] + step);
+      if (++ld_i >= ((ld_cs + D - 1) / D) * D) {  // uniform, no memory operation inside
+        ld_i = 0;
+        if (--ld_u > 0) {
+#pragma unroll
+          for (int t = 0; t < NT; ++t) lrow[t] += w_unit_stride;
+#pragma unroll
+          for (int j = 0; j < kNS; ++j) lsc[j] += w_unit_stride;
+        } else {  // back to the first unit, next chunk (past the last: the last again, dropped)
+          ld_u = n_my;
+#pragma unroll
+          for (int t = 0; t < NT; ++t) lrow[t] -= rewind;
+#pragma unroll
+          for (int j = 0; j < kNS; ++j) lsc[j] -= rewind;
+          if (ld_k0 + KC < nsteps) {
+            ld_k0 += KC;
+            ld_cs = min(KC, nsteps - ld_k0);
+          }
+        }
+      }
+    };
+
+    lds_barrier();  // the segment before is done with the planes and with its flag
+    if (tid == 0) pass_slow[flag ^ 1] = 0;  // for the next segment; its last reader is behind us
+    load_rows(0);
+    __builtin_amdgcn_sched_barrier(0);
+    Stage st[D];
+    if (n_my > 0) {
+#pragma unroll
+      for (int i = 0; i < D; ++i) issue(st[i]);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    write_rows(0, 0);
+    lds_barrier();
+
+    f32x4 acc[kMaxU][MT][NT];
+#pragma unroll
+    for (int u = 0; u < kMaxU; ++u)
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int t = 0; t < NT; ++t) acc[u][mt][t] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+    auto compute = [&](const Stage& sg, int slot0, f32x4 (&a)[MT][NT]) {
+      int sa[NT];
+      i32x8 wa[NT];
+#pragma unroll
+      for (int t = 0; t < NT; ++t) {
+        sa[t] = (int)((sg.s[t % kNS] >> shift[t]) & 0xFFu);
+        wa[t] = fp4_operand_packed(sg.w[t]);
+      }
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) {
+        if (mt > 0 && !live1) continue;  // uniform
+        const int slot = slot0 + mt;
+        const int sbh = bsc_lds[slot * 64 + lane];
+        const int sbl = sbh - 4;
+        const u32x4 h0 = b_lds[(slot * 4 + 0) * 64 + lane], h1 = b_lds[(slot * 4 + 1) * 64 + lane];
+        const u32x4 l0 = b_lds[(slot * 4 + 2) * 64 + lane], l1 = b_lds[(slot * 4 + 3) * 64 + lane];
+        const i32x8 bh = fp8_operand(h0, h1);
+        const i32x8 bl = fp8_operand(l0, l1);
+#pragma unroll
+        for (int t = 0; t < NT; ++t)
+          a[mt][t] = STAGE == 1
+                         ? __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(bh, wa[t], a[mt][t], 0, 4, 0, sbh, 0, sa[t])
+                         : __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wa[t], bh, a[mt][t], 4, 0, 0, sa[t], 0, sbh);
+#pragma unroll
+        for (int t = 0; t < NT; ++t)
+          a[mt][t] = STAGE == 1
+                         ? __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(bl, wa[t], a[mt][t], 0, 4, 0, sbl, 0, sa[t])
+                         : __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wa[t], bl, a[mt][t], 4, 0, 0, sa[t], 0, sbl);
+      }
+    };
+
+    for (int c = 0; c < nchunks; ++c) {
+      const int steps = min(KC, nsteps - c * KC);
+      const int buf = c & 1;
+      const bool more = c + 1 < nchunks;  // uniform
+      if (more) load_rows(c + 1);
+#pragma unroll
+      for (int u = 0; u < kMaxU; ++u) {
+        if (u < n_my) {  // uniform
+          for (int f0 = 0; f0 < steps; f0 += D) {
+#pragma unroll
+            for (int i = 0; i < D; ++i) {
+              if (f0 + i < steps) compute(st[i], (buf * KC + f0 + i) * MT, acc[u]);
+              issue(st[i]);
+            }
+          }
+        }
+        if (u == 0 && more) write_rows(c + 1, buf ^ 1);  // (their loads have had a unit's steps)
+      }
+      lds_barrier();
+    }
+
+    // ---- epilogue of every unit; those of a marked segment and the flagged ones on the exact path ----
+    // (Here and not with a unit's last steps: inside the unrolled stream the epilogues cost
+    // more registers than the kernel has, and every reload of a spilled one waits for all
+    // the loads in flight.)
+    const bool slow_seg = pass_slow[flag] != 0;
+    unsigned redo = 0u;
+#pragma unroll
+    for (int u = 0; u < kMaxU; ++u) {
+      if (u < n_my) {
+        int pu = 0;
+        unit_tiles_packed<STAGE, NT>(p, e, first + u * WAVES, lane, nsteps, cw, cs, shift, col0, pu);
+        if (slow_seg || packed_unit_flag(p, e, pu) != 0u) {
+          redo |= 1u << u;
+        } else {
+#pragma unroll
+          for (int mt = 0; mt < MT; ++mt) {
+            if (mt > 0 && !live1) continue;
+            if (STAGE == 1) epilogue_rows<NT>(p, e, acc[u][mt], col0, flat4[mt], w4[mt], run_row0 + mt * 16, lane);
+            else if (my_flat[mt] >= 0)
+              epilogue_tile<STAGE, NT>(p, e, acc[u][mt], col0, my_flat[mt], run_row0 + mt * 16 + ln, lq);
+          }
+        }
+      }
+    }
+    while (redo != 0u) {
+      const int u = __builtin_ctz(redo);
+      redo &= redo - 1u;
+      int pu = 0;
+      unit_tiles_packed<STAGE, NT>(p, e, first + u * WAVES, lane, nsteps, cw, cs, shift, col0, pu);
+      const bool raw = packed_unit_flag(p, e, pu) != 0u;
+      for (int mt = 0; mt < MT; ++mt) {
+        if (mt > 0 && !live1) continue;
+        const int flat = mt == 0 ? my_flat[0] : my_flat[MT - 1];
+        const int srow = run_row0 + mt * 16 + ln;
+        const uint16_t* a_row = nullptr;
+        if (flat >= 0) a_row = p.A + (size_t)(STAGE == 0 ? flat / p.top_k : srow) * (size_t)p.a_stride;
+        f32x4 ax[NT];
+        exact_unit_packed<NT, STAGE == 1>(cw, cs, shift, raw, a_row, K, lane, ax);
+        if (STAGE == 1) {
+          int f4[4];
+          float wx[4];
+#pragma unroll
+          for (int r4 = 0; r4 < 4; ++r4) {
+            f4[r4] = mt == 0 ? flat4[0][r4] : flat4[MT - 1][r4];
+            wx[r4] = mt == 0 ? w4[0][r4] : w4[MT - 1][r4];
+          }
+          epilogue_rows<NT>(p, e, ax, col0, f4, wx, run_row0 + mt * 16, lane);
+        } else if (flat >= 0) {
+          epilogue_tile<STAGE, NT>(p, e, ax, col0, flat, srow, lq);
         }
       }
     }
@@ -2105,12 +2576,34 @@ bool launch_resident(const GemmArgs& g, size_t lds, hipStream_t stream) {
   return true;
 }
 
+template <int STAGE, int NT, int D, int MT>
+bool chunked_kernel_ready() {
+  static const bool configured = [] {
+    const hipError_t err = hipFuncSetAttribute(
+        reinterpret_cast<const void*>(stream_chunked_kernel<STAGE, NT, D, MT>),
+        hipFuncAttributeMaxDynamicSharedMemorySize, (int)chunked_lds_bytes(MT));
+    if (err != hipSuccess) (void)hipGetLastError();  // not left for the next caller to find
+    return err == hipSuccess;
+  }();
+  return configured;
+}
+
+template <int STAGE, int NT, int D, int MT>
+bool launch_chunked(const GemmArgs& g, size_t lds, hipStream_t stream) {
+  if (!chunked_kernel_ready<STAGE, NT, D, MT>()) return false;
+  hipLaunchKernelGGL((stream_chunked_kernel<STAGE, NT, D, MT>), dim3(num_compute_units()),
+                     dim3(64 * kChunkWaves), lds, stream, g);
+  return true;
+}
+
 // Launch shape of one stage.  variant kMoeVariantLds = the tile kernel.
 struct StagePlan {
   int variant, waves, nt, depth;
   bool ksplit;  // the resident kernel with K shared between the wavefronts of a unit
   bool packed;  // ... reading the prepacked form (whenever the caller gives it)
   bool widek;   // ... its instantiation for rows of 3072 < K <= 4096 with 8 wavefronts
+  bool chunked; // the chunked decode kernel (prepacked form), `mt` 16-row tiles a pass
+  int mt;
   size_t resident_lds;
 };
 
@@ -2122,9 +2615,28 @@ StagePlan plan_stage(const GemmArgs& g) {
   // ones (no scale block to park, nothing to check or fix in the loop).
   const bool packed = g.Wp != nullptr && !(STAGE == 0 && g.ncols % 64 != 0);
   if (!moe_tuning_find(STAGE, g.K, g.ncols, g.n_flat, &tile))
-    tile = pick_moe_tile(g.n_flat, g.K, g.ncols, STAGE, packed, packed && g.block_size == 16 ? g.p_experts : 0);
+    tile = pick_moe_tile(g.n_flat, g.K, g.ncols, STAGE, packed,
+                         packed && (g.block_size == 16 || g.block_size == 32) ? g.p_experts : 0, g.block_size);
   StagePlan pl;
   pl.packed = packed;
+  pl.chunked = false;
+  pl.mt = 1;
+  if (tile.variant == kMoeVariantChunked) {  // one of the decode kernels for the callers
+    pl.chunked = true;
+    pl.mt = g.block_size / 16;
+    pl.variant = kMoeVariantResident;
+    pl.ksplit = false;
+    pl.widek = false;
+    pl.nt = tile.nt;
+    pl.depth = tile.depth;
+    pl.waves = tile.waves;
+    pl.resident_lds = chunked_lds_bytes(pl.mt);
+    const int c_units = STAGE == 0 ? g.ncols / (8 * pl.nt) : g.ncols / (16 * pl.nt);
+    if (!packed || (g.block_size != 16 && g.block_size != 32) || g.num_blocks > kMaxRuns ||
+        g.ncols % 16 != 0 || c_units < 1 || pl.waves != kChunkWaves)
+      pl.variant = kMoeVariantLds;
+    return pl;
+  }
   pl.ksplit = tile.variant == kMoeVariantResidentKSplit;
   pl.variant = pl.ksplit ? (int)kMoeVariantResident : tile.variant;
   pl.nt = tile.nt;
@@ -2169,6 +2681,19 @@ bool wide_kernel_applies(const GemmArgs& g) { return g.Aq != nullptr; }
 template <int STAGE>
 void launch_stage(const GemmArgs& g, const StagePlan& pl, hipStream_t stream) {
   // (a stage without raw weights that is not resident is kept away from here by the callers)
+  if (pl.variant == kMoeVariantResident && pl.chunked) {
+#define VK_CHUNKED(S_, W_, NT_, D_) \
+  if constexpr (STAGE == S_) { \
+    if (pl.nt == NT_ && pl.depth == D_) { \
+      if (pl.mt == 2 ? launch_chunked<S_, NT_, D_, 2>(g, pl.resident_lds, stream) \
+                     : launch_chunked<S_, NT_, D_, 1>(g, pl.resident_lds, stream)) \
+        return; \
+    } \
+  }
+    VK_CHUNKED_VARIANTS(VK_CHUNKED)
+#undef VK_CHUNKED
+    return;
+  }
   if (pl.packed && pl.variant == kMoeVariantResident && pl.widek) {
     if constexpr (STAGE == 0) {
       if (pl.ksplit) (void)launch_resident<0, 8, 2, 4, true, 0, true, true>(g, pl.resident_lds, stream);
@@ -2337,7 +2862,7 @@ bool fused_moe_packed_only_ok(const FusedMoeArgs& a) {
   if (a.M <= 0 || a.EM <= 0 || a.block_size <= 0) return true;  // nothing will run
   const GemmArgs g0 = gateup_args(a), g1 = down_args(a);
   const StagePlan p0 = plan_stage<0>(g0), p1 = plan_stage<1>(g1);
-  if (p0.variant == kMoeVariantResident && p1.variant == kMoeVariantResident) return true;
+  if (p0.variant == kMoeVariantResident && p1.variant == kMoeVariantResident && p0.packed && p1.packed) return true;
   return fused_moe_prepacked_takes(a, true);
 }
 
@@ -2353,7 +2878,8 @@ bool moe_down_packed_only_ok(const FusedMoeArgs& a) {
   if (a.w2_packed == nullptr || a.num_experts <= 0) return false;
   if (a.M <= 0 || a.EM <= 0 || a.block_size <= 0) return true;
   const GemmArgs g = down_args(a);
-  if (plan_stage<1>(g).variant == kMoeVariantResident) return true;
+  const StagePlan pl = plan_stage<1>(g);
+  if (pl.variant == kMoeVariantResident && pl.packed) return true;
   return fused_moe_prepacked_takes(a, false);
 }
 
@@ -2409,6 +2935,10 @@ bool prepare_moe_kernels() {
 #undef VK_READY
   ok = resident_kernel_ready<0, 8, 2, 4, true, 1, true>() && resident_kernel_ready<0, 8, 2, 2, false, 1, true>() && ok;
   ok = resident_kernel_ready<0, 8, 2, 2, false, 2, true>() && resident_kernel_ready<0, 4, 2, 8, false, 2, true>() && ok;
+#define VK_READY(S_, W_, NT_, D_) \
+  ok = chunked_kernel_ready<S_, NT_, D_, 1>() && chunked_kernel_ready<S_, NT_, D_, 2>() && ok;
+  VK_CHUNKED_VARIANTS(VK_READY)
+#undef VK_READY
   MoeTile unused;
   (void)moe_tuning_find(0, 64, 64, 1, &unused);  // reads the tuning store now rather than on the first launch
   return ok;
@@ -2434,6 +2964,7 @@ bool launch_routed_moe(const FusedMoeArgs& a, const RoutedArgs& r, hipStream_t s
   GemmArgs g1 = down_args(b);
   const StagePlan p0 = plan_stage<0>(g0), p1 = plan_stage<1>(g1);
   if (p0.variant != kMoeVariantResident || p1.variant != kMoeVariantResident) return false;
+  if (p0.chunked) return false;              // (the chunked kernel has no routed form)
   if (p0.packed != p1.packed) return false;  // (both packed forms or neither)
   if (p0.resident_lds > kRoutedLdsLimit) return false;
   g0.rt_logits = r.logits;

@@ -11,13 +11,16 @@
 
 namespace vk {
 
-enum { kMoeVariantLds = 0, kMoeVariantResident = 2, kMoeVariantResidentKSplit = 3 };
+enum { kMoeVariantLds = 0, kMoeVariantResident = 2, kMoeVariantResidentKSplit = 3, kMoeVariantChunked = 4 };
 
 struct MoeTile {
   int variant;  // kMoeVariantResident: one workgroup per compute unit, the
                 // activation rows of a run resident in LDS (decode);
                 // kMoeVariantResidentKSplit: the same, the K steps of a unit shared between
                 // the wavefronts that would otherwise have none (a handful of rows);
+                // kMoeVariantChunked: the decode kernel of the prepacked form that holds the
+                // rows a chunk of K at a time (rows of any K; blocks of 16 or of 32 rows,
+                // the 32 rows of a block in one pass over the expert's weights);
                 // kMoeVariantLds: the tile kernels (rows staged through LDS)
   int waves;    // wavefronts per workgroup
   int nt;       // 16-row weight tiles per wavefront
@@ -38,6 +41,8 @@ inline bool operator==(const MoeTile& a, const MoeTile& b) {
 // ... and of its K-split form (every one is also in the list above: a plan that cannot
 // split K falls back to the same shape there).
 #define VK_KSPLIT_VARIANTS(X) X(0, 8, 2, 4) X(0, 8, 2, 6) X(1, 8, 1, 8) X(1, 8, 2, 4)
+// ... and of the chunked kernel (prepacked form only; 8 wavefronts).
+#define VK_CHUNKED_VARIANTS(X) X(0, 8, 2, 2) X(0, 8, 2, 4) X(1, 8, 1, 2) X(1, 8, 1, 4)
 
 struct MoeTileCandidate {
   int stage;
@@ -51,6 +56,9 @@ inline const MoeTileCandidate* moe_tile_candidates(size_t* count) {
 #undef VK_CANDIDATE
 #define VK_CANDIDATE(S_, W_, NT_, D_) {S_, {kMoeVariantResidentKSplit, W_, NT_, D_}},
       VK_KSPLIT_VARIANTS(VK_CANDIDATE)
+#undef VK_CANDIDATE
+#define VK_CANDIDATE(S_, W_, NT_, D_) {S_, {kMoeVariantChunked, W_, NT_, D_}},
+      VK_CHUNKED_VARIANTS(VK_CANDIDATE)
 #undef VK_CANDIDATE
       {0, {kMoeVariantLds, 4, 4, 0}},
       {1, {kMoeVariantLds, 4, 4, 0}},
@@ -87,6 +95,27 @@ inline int moe_decode_max_rows(int packed_experts) {
   if (packed_experts <= 0) return kMoeDecodeMaxRows;
   const long long by_expert = (long long)kMoeDecodeRowsPerExpert * packed_experts;
   const long long by_runs = 16ll * (kMoeMaxRuns - packed_experts);
+  const long long m = by_expert < by_runs ? by_expert : by_runs;
+  return m > kMoeDecodeMaxRows ? (int)m : kMoeDecodeMaxRows;
+}
+
+// Blocks of 32 rows on the prepacked form (the chunked decode kernel multiplies both 16-row
+// tiles of a block with every weight register): up to this many routed rows per expert
+// (measured against the prepacked tile kernels in blocks of 128, us a step: 32 experts,
+// 1024 rows, 32 each, 144 against 160, and 1200 rows, 37.5 each, 175 against 168; 64
+// experts, 1800 rows, 28 each, 193 against 207, 2100 rows, 33 each, 214 against 216, 2520
+// rows, 39 each, 248 against 227; 128 experts with a few popular ones, 2048 rows, 269
+// against 277; 256 experts of 7168 x 2048, 4000 rows, 16 each, 1157 against 1304, but 8000
+// rows, 31 each, where four experts in ten have a second block, 1687 against 1397).
+constexpr int kMoeDecodeRowsPerExpert32 = 28;
+// Routed rows up to which the first stage's decode kernel routes or aligns for itself
+// (blocks of 16 only).
+constexpr int kMoeRoutedMaxRows = 256;
+
+inline int moe_decode_max_rows32(int packed_experts) {
+  if (packed_experts <= 0) return kMoeDecodeMaxRows;
+  const long long by_expert = (long long)kMoeDecodeRowsPerExpert32 * packed_experts;
+  const long long by_runs = 32ll * (kMoeMaxRuns - packed_experts);
   const long long m = by_expert < by_runs ? by_expert : by_runs;
   return m > kMoeDecodeMaxRows ? (int)m : kMoeDecodeMaxRows;
 }
@@ -134,10 +163,15 @@ constexpr int kMoeComputeUnits = 256;  // of the device the rules were swept on
 
 // packed: the stage reads the prepacked form (its decode kernels have no scale block in
 // LDS and fewer registers in use, so their best shapes are swept separately).
-// packed_experts: their number when the call also comes in blocks of 16 (else 0): the
+// packed_experts: their number when the call also comes in blocks of 16 or 32 (else 0): the
 // decode range then follows moe_decode_max_rows.
+// block_rows: the alignment's block size.  Blocks of 32 on the prepacked form go to the
+// chunked kernel, a block a pass; so do rows of a K the resident kernel cannot hold.
 inline MoeTile pick_moe_tile(int n_flat, int K, int ncols, int stage, bool packed = false,
-                             int packed_experts = 0) {
+                             int packed_experts = 0, int block_rows = 16) {
+  const MoeTile chunked = MoeTile{kMoeVariantChunked, 8, stage == 0 ? 2 : 1, stage == 0 ? 2 : 4};
+  if (packed && block_rows == 32)
+    return n_flat <= moe_decode_max_rows32(packed_experts) ? chunked : MoeTile{kMoeVariantLds, 4, 4, 0};
   const int max_rows = moe_decode_max_rows(packed ? packed_experts : 0);
   // (on the prepacked form the 8-wavefront K-split shape also holds rows of K up to 4096)
   if (packed && stage == 0 && n_flat <= kMoeDecodeMaxRows && K > 3072 && K <= 4096 &&
@@ -161,6 +195,7 @@ inline MoeTile pick_moe_tile(int n_flat, int K, int ncols, int stage, bool packe
   };
   for (const MoeTileRule& r : rules)
     if (r.stage == stage && n_flat <= r.max_rows && K <= r.max_k) return r.tile;
+  if (packed && n_flat <= max_rows) return chunked;  // rows of any K
   return MoeTile{kMoeVariantLds, 4, 4, 0};
 }
 
@@ -170,15 +205,19 @@ inline MoeTile pick_moe_tile(int n_flat, int K, int ncols, int stage, bool packe
 // window of 128 sorted rows of one expert, so blocks of 128 give every expert windows of
 // its own (0.5 to 8 % faster than blocks of 64 from 16 to 770 rows per expert).
 // packed_experts, hidden, ispp: the number of (local) experts and the layer's widths when
-// the caller gives the prepacked weights, 0 otherwise: beyond kMoeDecodeMaxRows rows the
-// blocks are 16 only where the decode kernels take both stages.
+// the caller gives the prepacked weights, 0 otherwise.  On that form, beyond the rows of
+// the routed forms (which want blocks of 16), blocks of 32 and the chunked decode kernel
+// up to kMoeDecodeRowsPerExpert32 rows per expert: an expert with 17 to 32 rows costs one
+// pass over its weights, not two (us a step, blocks of 16 / 32 / 128: 32 experts, 512
+// rows, 124 / 111 / 142; 64 experts, 510 rows, 139 / 138 / 144, and 1530 rows, - / 181 /
+// 201; 128 experts with a few popular ones, 1152 rows, 244 / 205 / 246).
 inline int moe_default_block_size(int M, int top_k, int packed_experts = 0, int hidden = 0, int ispp = 0) {
   const long long n = (long long)M * (long long)top_k;
-  if (n <= kMoeDecodeMaxRows) return 16;
-  if (packed_experts <= 0 || hidden <= 0 || ispp <= 0 || n > moe_decode_max_rows(packed_experts)) return 128;
-  const bool decode = pick_moe_tile((int)n, hidden, ispp, 0, true, packed_experts).variant != kMoeVariantLds &&
-                      pick_moe_tile((int)n, ispp, hidden, 1, true, packed_experts).variant != kMoeVariantLds;
-  return decode ? 16 : 128;
+  if (n <= kMoeRoutedMaxRows) return 16;
+  if (packed_experts > 0 && hidden > 0 && ispp > 0 && n <= moe_decode_max_rows32(packed_experts) &&
+      hidden % 64 == 0 && ispp % 64 == 0)
+    return 32;
+  return n <= kMoeDecodeMaxRows ? 16 : 128;
 }
 
 }  // namespace vk

@@ -76,6 +76,9 @@ def main() -> None:
     ap.add_argument("--packed", action="store_true",
                     help="sweep the decode kernels that read the prepacked form (the weights are prepacked "
                          "and the raw tensors let go of); shapes they do not take are skipped")
+    ap.add_argument("--block-size", type=int, default=0,
+                    help="alignment block of the calls (default: the library's policy, and only batches of "
+                         "up to 512 routed rows); 32 with --packed: the chunked decode kernel's two-tile passes")
     args = ap.parse_args()
 
     import numpy as np
@@ -100,15 +103,16 @@ def main() -> None:
                                            keep_raw=not args.packed))
             del w
         for T in args.tokens:
-            if T * k > 512:
+            if T * k > 512 and not args.block_size:
                 continue   # the tile kernels' side of the split: nothing to choose between
             A = torch.from_numpy(synth.make_activations(T, H, 7).view(np.int16)).view(torch.bfloat16).to(dev)
             logits = torch.from_numpy(synth.make_logits("uniform", T, E, 7)).to(dev)
             ids, tw = fe_sets[0].route(logits, k, True)
             out = torch.zeros((T, H), dtype=torch.float32, device=dev)
-            bs = ve.default_block_size(T, k)
+            bs = args.block_size or ve.default_block_size(T, k)
             for stage, K, ncols in ((0, H, I), (1, I, H)):
-                rule, _ = ve.moe_tile_query(stage, K, ncols, T * k, packed=args.packed)
+                rule, _ = ve.moe_tile_query(stage, K, ncols, min(T * k, 512) if args.block_size else T * k,
+                                            packed=args.packed, block_size=bs)
                 times = {}
                 for cand in ve.moe_tile_candidates(stage):
                     if args.packed and cand[0] == 0:

@@ -386,14 +386,15 @@ def moe_tile_candidates(stage: int, lib=None) -> list[tuple[int, int, int, int]]
     return [tuple(buf[4 * i:4 * i + 4]) for i in range(n)]
 
 
-def moe_tile_query(stage: int, K: int, ncols: int, n_flat: int, lib=None, packed: bool = False):
+def moe_tile_query(stage: int, K: int, ncols: int, n_flat: int, lib=None, packed: bool = False,
+                   block_size: int = 16):
     """((variant, wavefronts, tiles, depth), from_store) a call of this size is planned with
-    (packed: when the caller gives the prepacked weights)."""
+    (packed: when the caller gives the prepacked weights; block_size 32: ... in blocks of 32)."""
     lib = load_libvkernels_hip() if lib is None else lib
     fn = lib.vk_hip_moe_tile_query
     fn.restype, fn.argtypes = _I, [_I, _I, _I, _I, _P]
     buf = (ctypes.c_int * 4)()
-    stored = int(fn(stage + (2 if packed else 0), K, ncols, n_flat, buf))
+    stored = int(fn(stage + ((4 if block_size == 32 else 2) if packed else 0), K, ncols, n_flat, buf))
     return tuple(buf), bool(stored)
 
 
