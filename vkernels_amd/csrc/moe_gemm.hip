@@ -1992,14 +1992,19 @@ __global__ __launch_bounds__(64 * kTileWaves, 2) void tile_gemm_kernel(GemmArgs 
           const i32x8 bh = fp8_operand(h0, h1);
           const i32x8 bl = fp8_operand(l0, l1);
           // the two MFMAs of an accumulator are kept NT instructions apart
+          // (second stage: the rows as the first operand, for epilogue_rows)
 #pragma unroll
           for (int t = 0; t < NT; ++t)
-            acc[m][t] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wa[t], bh, acc[m][t], 4, 0,
-                                                                         0, sa[t], 0, sbh);
+            acc[m][t] = STAGE == 1 ? __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(bh, wa[t], acc[m][t], 0, 4,
+                                                                                      0, sbh, 0, sa[t])
+                                   : __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wa[t], bh, acc[m][t], 4, 0,
+                                                                                      0, sa[t], 0, sbh);
 #pragma unroll
           for (int t = 0; t < NT; ++t)
-            acc[m][t] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wa[t], bl, acc[m][t], 4, 0,
-                                                                         0, sa[t], 0, sbl);
+            acc[m][t] = STAGE == 1 ? __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(bl, wa[t], acc[m][t], 0, 4,
+                                                                                      0, sbl, 0, sa[t])
+                                   : __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wa[t], bl, acc[m][t], 4, 0,
+                                                                                      0, sa[t], 0, sbl);
         }
       }
     }
@@ -2020,12 +2025,20 @@ __global__ __launch_bounds__(64 * kTileWaves, 2) void tile_gemm_kernel(GemmArgs 
     if (redo) {
       const uint16_t* a_row = nullptr;
       if (flat >= 0) a_row = p.A + (size_t)(STAGE == 0 ? flat / p.top_k : srow) * (size_t)p.a_stride;
-      exact_unit_global<NT>(w_rows, s_rows, a_row, K, lane, acc[m]);
+      exact_unit_global<NT, STAGE == 1>(w_rows, s_rows, a_row, K, lane, acc[m]);
     }
-    uint2 packed[NT / 2] = {};
-    if (flat >= 0) epilogue_tile<STAGE, NT>(p, e, acc[m], col0, flat, srow, lq, packed);
-    if (STAGE == 0 && p.actq != nullptr)
-      store_split_act(p, col0[0], col0[1], flat, srow, lane, packed[0], packed[1]);
+    if constexpr (STAGE == 1) {
+      int flat4[4];
+      float w4[4];
+#pragma unroll
+      for (int r = 0; r < 4; ++r) flat4[r] = row_flat[m * 16 + 4 * lq + r];
+      rows_weights(p, flat4, w4);
+      epilogue_rows<NT>(p, e, acc[m], col0, flat4, w4, row0 + m * 16, lane);
+    } else {
+      uint2 packed[NT / 2] = {};
+      if (flat >= 0) epilogue_tile<STAGE, NT>(p, e, acc[m], col0, flat, srow, lq, packed);
+      if (p.actq != nullptr) store_split_act(p, col0[0], col0[1], flat, srow, lane, packed[0], packed[1]);
+    }
   }
 }
 
