@@ -137,3 +137,26 @@ def test_epilogues_on_the_chunked_kernel(variant):
         gpu_kw.update(activation="situ", beta=3.0, linear_beta=20.0)
         cpu_kw.update(activation=1, beta=3.0, linear_beta=20.0)
     cfgs._check(cfg, T, w, A, lg, gpu_kw=gpu_kw, cpu_kw=cpu_kw, block_size=32)
+
+
+@pytest.mark.parametrize("name,T", [("c4", 33), ("c1", 64)])
+def test_chunked_shapes_forced_in_blocks_of_16(name, T):
+    """The tuning store may name the chunked kernel for calls the rules give to the resident
+    one: blocks of 16, a tile a pass (second stage of c4: rows of 1536 values, its
+    single-chunk form)."""
+    cfg = synth.CONFIGS[name]
+    n_flat = T * cfg.top_k
+    w = cfgs._weights(cfg)
+    A, lg = cfgs._inputs(cfg, T, 7000 + T)
+    keys = ((0, cfg.H, cfg.I), (1, cfg.I, cfg.H))
+    try:
+        for stage, K, ncols in keys:
+            ve.moe_tile_set(stage, K, ncols, n_flat, (CHUNKED, 8, 2, 2) if stage == 0 else (CHUNKED, 8, 1, 4))
+        g, _ = cfgs._check(cfg, T, w, A, lg, gpu_kw=PACKED_ONLY, tight=True, block_size=16, stagewise=(name == "c4"))
+    finally:
+        for stage, K, ncols in keys:
+            ve.moe_tile_set(stage, K, ncols, n_flat, None)
+    b = cfgs._run_gpu(cfg, w, A, lg, 16, None, **PACKED_ONLY)
+    assert np.array_equal(_act_by_flat_row(g, n_flat), _act_by_flat_row(b, n_flat))
+    m, l2, nf = error_metrics(g["out"], b["out"])
+    assert nf and l2 <= 1e-5, (m, l2)

@@ -1414,10 +1414,15 @@ __host__ __device__ constexpr size_t chunked_lds_bytes(int mt) {
   return (size_t)2 * kChunkSteps * (size_t)mt * (4096 + 64);
 }
 
-template <int STAGE, int NT, int D, int MT>
+// ONE: rows of K <= 128 x 2 kChunkSteps, which are one chunk (the two buffers as one):
+// nothing to keep across chunks, so a wavefront walks its units one after the other as the
+// resident kernel does, every unit's epilogue under the loads of the next (where all
+// epilogues of a segment come after its stream, the second stage's atomic additions of all
+// workgroups fall together, with no load in flight).
+template <int STAGE, int NT, int D, int MT, bool ONE = false>
 __global__ __launch_bounds__(64 * kChunkWaves) void stream_chunked_kernel(GemmArgs p) {
-  constexpr int WAVES = kChunkWaves, KC = kChunkSteps;
-  constexpr int kMaxU = chunked_max_units(NT, MT);  // units of a wavefront in a segment
+  constexpr int WAVES = kChunkWaves, KC = ONE ? 2 * kChunkSteps : kChunkSteps;
+  constexpr int kMaxU = ONE ? 32 : chunked_max_units(NT, MT);  // units of a wavefront in a segment
   constexpr int kPieces = KC * 4 / WAVES;  // 16-byte row pieces of a lane per tile and chunk
   static_assert(KC % D == 0 && (KC * 4) % WAVES == 0, "whole rounds of the pipeline and of the staging per chunk");
   static_assert((WAVES * (STAGE == 0 ? 8 * NT : 16 * NT)) % (STAGE == 0 ? 64 : 128) == 0,
@@ -1439,7 +1444,7 @@ __global__ __launch_bounds__(64 * kChunkWaves) void stream_chunked_kernel(GemmAr
   const int nsteps = (groups + 3) / 4;
   const int nchunks = (nsteps + KC - 1) / KC;
   const int units = STAGE == 0 ? p.ncols / (8 * NT) : p.ncols / (16 * NT);
-  uint8_t* const bsc_lds = reinterpret_cast<uint8_t*>(b_lds + (size_t)2 * KC * MT * 256);  // [2][KC][MT][64]
+  uint8_t* const bsc_lds = reinterpret_cast<uint8_t*>(b_lds + (size_t)(ONE ? 1 : 2) * KC * MT * 256);  // [2][KC][MT][64]
   constexpr int kPackedStride = WAVES * (STAGE == 0 ? 8 * NT : 16 * NT) / (STAGE == 0 ? 64 : 128);
   const size_t w_unit_stride = (size_t)kPackedStride * (size_t)nsteps * (size_t)kMxStepBytes;
   constexpr int kNS = STAGE == 0 ? NT / 2 : NT;  // scale words of a K step a lane loads
@@ -1663,14 +1668,6 @@ __global__ __launch_bounds__(64 * kChunkWaves) void stream_chunked_kernel(GemmAr
     write_rows(0, 0);
     lds_barrier();
 
-    f32x4 acc[kMaxU][MT][NT];
-#pragma unroll
-    for (int u = 0; u < kMaxU; ++u)
-#pragma unroll
-      for (int mt = 0; mt < MT; ++mt)
-#pragma unroll
-        for (int t = 0; t < NT; ++t) acc[u][mt][t] = f32x4{0.f, 0.f, 0.f, 0.f};
-
     auto compute = [&](const Stage& sg, int slot0, f32x4 (&a)[MT][NT]) {
       int sa[NT];
       i32x8 wa[NT];
@@ -1701,6 +1698,51 @@ __global__ __launch_bounds__(64 * kChunkWaves) void stream_chunked_kernel(GemmAr
                          : __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wa[t], bl, a[mt][t], 4, 0, 0, sa[t], 0, sbl);
       }
     };
+    unsigned redo = 0u;
+
+    if constexpr (ONE) {
+      // (all rows are written, so the segment's mark is complete)
+      int cur_pu = pu0;
+      uint32_t cur_flag = n_my > 0 ? packed_unit_flag(p, e, cur_pu) : 0u;
+      for (int j = 0; j < n_my; ++j) {
+        f32x4 a1[MT][NT];
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+          for (int t = 0; t < NT; ++t) a1[mt][t] = f32x4{0.f, 0.f, 0.f, 0.f};
+        for (int f0 = 0; f0 < nsteps; f0 += D) {
+#pragma unroll
+          for (int i = 0; i < D; ++i) {
+            if (f0 + i < nsteps) compute(st[i], (f0 + i) * MT, a1);
+            issue(st[i]);
+          }
+        }
+        if (pass_slow[flag] != 0 || cur_flag != 0u) {
+          redo |= 1u << j;
+        } else {
+#pragma unroll
+          for (int mt = 0; mt < MT; ++mt) {
+            if (mt > 0 && !live1) continue;
+            if (STAGE == 1) epilogue_rows<NT>(p, e, a1[mt], col0, flat4[mt], w4[mt], run_row0 + mt * 16, lane);
+            else if (my_flat[mt] >= 0)
+              epilogue_tile<STAGE, NT>(p, e, a1[mt], col0, my_flat[mt], run_row0 + mt * 16 + ln, lq);
+          }
+        }
+        if (j + 1 < n_my) {
+#pragma unroll
+          for (int t = 0; t < NT; ++t) col0[t] += WAVES * (STAGE == 0 ? 8 * NT : 16 * NT);
+          cur_pu += kPackedStride;
+          cur_flag = packed_unit_flag(p, e, cur_pu);
+        }
+      }
+    } else {
+    f32x4 acc[kMaxU][MT][NT];
+#pragma unroll
+    for (int u = 0; u < kMaxU; ++u)
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int t = 0; t < NT; ++t) acc[u][mt][t] = f32x4{0.f, 0.f, 0.f, 0.f};
 
     for (int c = 0; c < nchunks; ++c) {
       const int steps = min(KC, nsteps - c * KC);
@@ -1728,7 +1770,6 @@ __global__ __launch_bounds__(64 * kChunkWaves) void stream_chunked_kernel(GemmAr
     // more registers than the kernel has, and every reload of a spilled one waits for all
     // the loads in flight.)
     const bool slow_seg = pass_slow[flag] != 0;
-    unsigned redo = 0u;
 #pragma unroll
     for (int u = 0; u < kMaxU; ++u) {
       if (u < n_my) {
@@ -1747,6 +1788,7 @@ __global__ __launch_bounds__(64 * kChunkWaves) void stream_chunked_kernel(GemmAr
         }
       }
     }
+    }  // (not ONE)
     while (redo != 0u) {
       const int u = __builtin_ctz(redo);
       redo &= redo - 1u;
@@ -2589,11 +2631,11 @@ bool launch_resident(const GemmArgs& g, size_t lds, hipStream_t stream) {
   return true;
 }
 
-template <int STAGE, int NT, int D, int MT>
+template <int STAGE, int NT, int D, int MT, bool ONE = false>
 bool chunked_kernel_ready() {
   static const bool configured = [] {
     const hipError_t err = hipFuncSetAttribute(
-        reinterpret_cast<const void*>(stream_chunked_kernel<STAGE, NT, D, MT>),
+        reinterpret_cast<const void*>(stream_chunked_kernel<STAGE, NT, D, MT, ONE>),
         hipFuncAttributeMaxDynamicSharedMemorySize, (int)chunked_lds_bytes(MT));
     if (err != hipSuccess) (void)hipGetLastError();  // not left for the next caller to find
     return err == hipSuccess;
@@ -2601,12 +2643,18 @@ bool chunked_kernel_ready() {
   return configured;
 }
 
-template <int STAGE, int NT, int D, int MT>
+template <int STAGE, int NT, int D, int MT, bool ONE = false>
 bool launch_chunked(const GemmArgs& g, size_t lds, hipStream_t stream) {
-  if (!chunked_kernel_ready<STAGE, NT, D, MT>()) return false;
-  hipLaunchKernelGGL((stream_chunked_kernel<STAGE, NT, D, MT>), dim3(num_compute_units()),
+  if (!chunked_kernel_ready<STAGE, NT, D, MT, ONE>()) return false;
+  hipLaunchKernelGGL((stream_chunked_kernel<STAGE, NT, D, MT, ONE>), dim3(num_compute_units()),
                      dim3(64 * kChunkWaves), lds, stream, g);
   return true;
+}
+
+// The chunked kernel's single-chunk form: the second stage's, for rows of up to 2048 values.
+template <int STAGE>
+bool chunked_one_applies(const GemmArgs& g) {
+  return STAGE == 1 && (g.K / 32 + 3) / 4 <= 2 * kChunkSteps;
 }
 
 // Launch shape of one stage.  variant kMoeVariantLds = the tile kernel.
@@ -2698,6 +2746,12 @@ void launch_stage(const GemmArgs& g, const StagePlan& pl, hipStream_t stream) {
 #define VK_CHUNKED(S_, W_, NT_, D_) \
   if constexpr (STAGE == S_) { \
     if (pl.nt == NT_ && pl.depth == D_) { \
+      if constexpr (S_ == 1) { \
+        if (chunked_one_applies<S_>(g) && \
+            (pl.mt == 2 ? launch_chunked<S_, NT_, D_, 2, true>(g, pl.resident_lds, stream) \
+                        : launch_chunked<S_, NT_, D_, 1, true>(g, pl.resident_lds, stream))) \
+          return; \
+      } \
       if (pl.mt == 2 ? launch_chunked<S_, NT_, D_, 2>(g, pl.resident_lds, stream) \
                      : launch_chunked<S_, NT_, D_, 1>(g, pl.resident_lds, stream)) \
         return; \
@@ -2949,7 +3003,9 @@ bool prepare_moe_kernels() {
   ok = resident_kernel_ready<0, 8, 2, 4, true, 1, true>() && resident_kernel_ready<0, 8, 2, 2, false, 1, true>() && ok;
   ok = resident_kernel_ready<0, 8, 2, 2, false, 2, true>() && resident_kernel_ready<0, 4, 2, 8, false, 2, true>() && ok;
 #define VK_READY(S_, W_, NT_, D_) \
-  ok = chunked_kernel_ready<S_, NT_, D_, 1>() && chunked_kernel_ready<S_, NT_, D_, 2>() && ok;
+  ok = chunked_kernel_ready<S_, NT_, D_, 1>() && chunked_kernel_ready<S_, NT_, D_, 2>() && ok; \
+  if constexpr (S_ == 1) \
+    ok = chunked_kernel_ready<S_, NT_, D_, 1, true>() && chunked_kernel_ready<S_, NT_, D_, 2, true>() && ok;
   VK_CHUNKED_VARIANTS(VK_READY)
 #undef VK_READY
   MoeTile unused;
