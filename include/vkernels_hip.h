@@ -199,8 +199,9 @@ void vk_hip_fused_moe_mxfp4_ex(
  * and nothing is checked or moved in the loop), and both exact paths read it as
  * well.  The raw tensors are therefore optional: w13, w13_scale, w2 and w2_scale
  * may all be NULL (one copy of the weights), provided the call is one the decode
- * kernels take (up to 512 routed rows, hidden <= 4096 for the first stage and
- * ispp <= 3072 for the second) or the workspace is given; otherwise the call is
+ * kernels take (vk_hip_moe_decode_max_rows routed rows: 512, or a number of rows per
+ * expert in blocks of 16 or 32; rows of any width) or the workspace is given; otherwise
+ * the call is
  * refused with VK_ERROR_INVALID_ARGUMENT in the error state.  On the packed path of
  * prefill-sized calls the bf16
  * activations are multiplied as a sum of FP6 (E2M3) terms per block of 32 along K,
@@ -271,9 +272,11 @@ int vk_hip_init(void);
  * vk_hip_moe_align_block_size and on to the layer).  Any multiple of 16 works.
  * vk_hip_moe_default_block_size_ex: the same for a caller that gives the prepacked
  * weights of num_local_experts experts of a hidden x ispp layer: what decides between
- * the decode kernels (blocks of 16) and the tile kernels (blocks of 128) is then rows per
- * expert, and with blocks of 16 the decode kernels also take calls beyond 512 routed
- * rows, up to 9 per expert (where they take the layer's widths at all).
+ * the decode kernels and the tile kernels (blocks of 128) is then rows per expert.  16 up
+ * to 256 routed rows (where the first stage's kernel can align for itself); beyond, 32 up
+ * to 28 rows per expert: the decode kernel of that form takes a block of 32 rows in one
+ * pass over the expert's weights.  (A caller who passes blocks of 16 beyond 512 routed
+ * rows still gets the decode kernels up to 9 rows per expert.)
  * vk_hip_moe_decode_max_rows: the routed rows (M * top_k) up to which a call in blocks of
  * block_size runs the decode kernels (num_local_experts: of a caller that gives the
  * prepacked weights, else 0; blocks of 32 are the decode kernels' only on that form).
@@ -517,8 +520,7 @@ int vk_hip_moe_combine(const float* partial, const float* b2, const float* topk_
  * (K = hidden_k / ispp_k) of num_experts experts.  With it the raw shard (w13 /
  * w13_scale, w2 / w2_scale) may be NULL: the exact paths read the packed form, and calls
  * of up to 512 routed rows run the decode kernels on it; a call that would need the raw
- * shard (no workspace at prefill sizes, a slice too wide for the decode kernels) is then
- * refused with VK_ERROR_INVALID_ARGUMENT.  workspace:
+ * shard (no workspace at prefill sizes) is then refused with VK_ERROR_INVALID_ARGUMENT.  workspace:
  * vk_hip_moe_preact_workspace_bytes(stage, M, EM, k_dim) bytes, 16-byte aligned (the
  * split rows of the K slice).  flags: VK_HIP_MOE_SPLIT2 / _SPLIT3 as for the layer
  * (default: three FP6 terms per activation in the first stage, two in the second).

@@ -328,7 +328,7 @@ def test_tile_candidates_and_compiled_in_rules():
             assert not stored and shape in cands, (stage, n_flat, shape)   # selectors return table entries only
             # the decode kernels up to 512 routed rows, where a pass's rows fit LDS and registers
             assert (shape[0] in (2, 3)) == (n_flat <= 512 and K <= (4096 if stage == 0 else 3072))
-    assert ve.moe_tile_query(0, 2880, 2880, 128)[0] == (2, 8, 2, 2) and ve.moe_tile_query(1, 2880, 2880, 128)[0] == (2, 8, 1, 6)
+    assert ve.moe_tile_query(0, 2880, 2880, 128)[0] == (2, 8, 2, 2) and ve.moe_tile_query(1, 2880, 2880, 128)[0] == (2, 8, 1, 4)
     assert ve.moe_tile_query(0, 4096, 1536, 6)[0] == (2, 4, 2, 8)                   # rows of K = 4096
     # ... which the kernels on the prepacked form take with 8 wavefronts (and K shared for one token)
     assert ve.moe_tile_query(0, 4096, 1536, 198, packed=True)[0] == (2, 8, 2, 2)

@@ -139,15 +139,18 @@ struct MoeTileRule {
 // ispp / 16 units per expert); the down stage, with half the weight rows, takes single
 // tiles (nt = 1) and keeps the bytes in flight per wavefront with a deeper pipeline.
 // Rows (each from the sweep table profiles/moe_decode_tile_sweep.md):
-//  - K <= 1024: a unit is a few steps long, and steps in flight past its end are
-//    wasted loads: the shallowest pipelines (256x512x8x2 at T = 64: 10.7 against 11.4 us);
+//  - the shallowest pipelines of the table (with K <= 1024 a unit is a few steps long, and
+//    steps in flight past its end are wasted loads: 256x512x8x2 at T = 64, 8.7 against 9.2 us;
+//    with longer rows the depth hardly matters);
 //  - 3072 < K <= 4096 (4096x1536x64x6 gate/up): the rows of a pass fit LDS and registers
 //    only with 4 wavefronts per workgroup (34 against 69 us at T = 1, 97 against 185 us
 //    at T = 32 for the tile kernel, which is what runs beyond K = 4096);
-//  - down stage, up to 24 rows (2 to 4 tokens): units of two tiles, 4 to 5 % faster than
-//    single tiles there (2880x2880x32x4 at T = 4: 23.5 against 24.6 us; 4096x1536x64x6 at
-//    T = 2: 17.7 against 18.6 us), level or behind from 32 rows on;
-//  - otherwise (8, 2, 4) / (8, 1, 8), within 5 % of the best of every other point swept:
+//  - down stage: single tiles, four K steps in flight, at every size (units of two tiles
+//    were 4 to 5 % faster up to 24 rows while a lane's epilogue held four columns of one row;
+//    with the rows as the matrix cores' first operand a lane holds one column of four rows,
+//    and two tiles are 5 to 20 % behind there: 2880x2880x32x4 at T = 3, 20.2 against 16.7 us
+//    on the prepacked form; six steps in flight are 1 to 3 % behind four at most points);
+//  - otherwise (8, 2, 2) / (8, 1, 4), within 5 % of the best of every other point swept:
 //    with 128 experts and 32 tokens or more, uniformly routed, the 4-wavefront shapes
 //    are 3 to 5 % faster for gate/up; the number of runs that makes it so is not known
 //    here, and with skewed routing (27 active experts of 128) the same shape is much
@@ -189,9 +192,7 @@ inline MoeTile pick_moe_tile(int n_flat, int K, int ncols, int stage, bool packe
   const MoeTileRule rules[] = {
       {0, max_rows, packed ? 4096 : 3072, {kMoeVariantResident, 8, 2, 2}},  // (the prepacked form's rows of a pass: K <= 4096)
       {0, max_rows, 4096, {kMoeVariantResident, 4, 2, 8}},
-      {1, max_rows, 1024, {kMoeVariantResident, 8, 1, 4}},
-      {1, 24, 3072, {kMoeVariantResident, 8, 2, 4}},
-      {1, max_rows, 3072, {kMoeVariantResident, 8, 1, 6}},
+      {1, max_rows, 3072, {kMoeVariantResident, 8, 1, 4}},
   };
   for (const MoeTileRule& r : rules)
     if (r.stage == stage && n_flat <= r.max_rows && K <= r.max_k) return r.tile;
