@@ -245,14 +245,16 @@ PREPACKED2_MAX_TOL, PREPACKED2_L2_TOL = 2e-2, 2e-3
 
 @pytest.mark.parametrize("name,T,bs,tp,raw", [("c1", 300, 128, 1, True), ("c1", 600, 128, 2, True),
                                               ("c4", 255, 64, 3, True), ("c1", 600, 128, 2, False),
-                                              ("c4", 255, 64, 3, False), ("c1", 48, 16, 2, False)])
+                                              ("c4", 255, 64, 3, False), ("c1", 48, 16, 2, False),
+                                              ("c1", 48, 32, 2, False), ("c4", 100, 32, 2, False)])
 def test_prepacked_stages_against_the_oracle_and_in_composition(hip_lib, name, T, bs, tp, raw):
     """vk_hip_moe_gateup_preact_prepacked / _down_preact_prepacked: every rank's K slice of the
     weights prepacked as its own shard, the A / act slice addressed inside the full rows; each
     stage against the oracle's function of the same name on the same slice (rows that are not
     routed left as they were), and the composition (slices summed, epilogues once) against
     the fused oracle.  raw = False: the shard's raw tensors are not passed (one copy of the
-    weights; decode-sized calls then run the decode kernels on the prepacked shard)."""
+    weights; decode-sized calls then run the decode kernels on the prepacked shard: in blocks
+    of 32 the chunked kernel, whose linear part goes through the same two epilogues)."""
     lib = _prepacked_fns(hip_lib)
     cfg = synth.CONFIGS[name]
     H, I, k = cfg.H, cfg.I, cfg.top_k
