@@ -335,9 +335,9 @@ def test_tile_candidates_and_compiled_in_rules():
     assert ve.moe_tile_query(0, 4096, 1536, 6, packed=True)[0] == (3, 8, 2, 4)
     assert ve.moe_tile_query(0, 2880, 2880, 256, packed=True)[0] == ve.moe_tile_query(0, 2880, 2880, 256)[0]
     # the chunked kernel: rows of a K beyond those, and every call in blocks of 32 (prepacked form only)
-    assert ve.moe_tile_query(0, 7168, 2048, 64, packed=True)[0] == (4, 8, 2, 2)
+    assert ve.moe_tile_query(0, 7168, 2048, 64, packed=True)[0] == (4, 8, 2, 4)
     assert ve.moe_tile_query(1, 4224, 512, 64, packed=True)[0] == (4, 8, 1, 4)
-    assert ve.moe_tile_query(0, 2880, 2880, 512, packed=True, block_size=32)[0] == (4, 8, 2, 2)
+    assert ve.moe_tile_query(0, 2880, 2880, 512, packed=True, block_size=32)[0] == (4, 8, 2, 4)
     assert ve.moe_tile_query(1, 2880, 2880, 512, packed=True, block_size=32)[0] == (4, 8, 1, 4)
     assert ve.moe_tile_query(0, 7168, 2048, 64)[0] == (0, 4, 4, 0)
     # one token: fewer units than half the device's wavefronts, K shared between them
