@@ -55,3 +55,46 @@ def test_random_small_layers(seed):
     print(f"seed {seed}: worst max_abs/rms={worst[0]:.3e} rel_l2={worst[1]:.3e}")
     # measured: 1e-2 / 8e-4 at most; the contract is 2e-2 / 5e-3
     assert worst[0] <= 1.2e-2 and worst[1] <= 1.5e-3
+
+
+def test_random_layers_on_the_chunked_decode_kernel():
+    """The same on the prepacked form alone, drawn where the chunked decode kernel runs: blocks
+    of 32 rows at any width, or blocks of 16 with rows the resident kernel cannot hold (more than
+    4096 values in the first stage, more than 3072 in the second)."""
+    rng = np.random.default_rng(11)
+    worst = [0.0, 0.0]
+    for case in range(24):
+        E = int(rng.choice([2, 4, 8, 17, 32, 64, 128]))
+        k = int(rng.integers(1, min(8, E) + 1))
+        bs = int(rng.choice([16, 32, 32, 32]))
+        if bs == 16:
+            H, I = [(4160, 128), (5120, 256), (256, 3136), (4608, 3200)][int(rng.integers(0, 4))]
+        else:
+            H = int(rng.choice([64, 128, 512, 1024, 2880, 4160]))
+            I = int(rng.choice([64, 256, 512, 1024, 3136]))
+        T = int(rng.choice([1, 2, 3, 5, 8, 13, 16, 17, 31, 40, 64, 96, 128]))
+        kind = str(rng.choice(["uniform", "zipf", "router"]))
+        s = int(rng.integers(1, 1 << 30))
+        what = dict(case=case, E=E, k=k, H=H, I=I, T=T, bs=bs, routing=kind, seed=s)
+        print(what, flush=True)
+        stages = [ve.moe_tile_query(st, K, n, min(T * k, 512), packed=True, block_size=bs)[0][0]
+                  for st, K, n in ((0, H, I), (1, I, H))]
+        assert 4 in stages, (what, stages)     # at least one stage is the chunked kernel's
+        w = synth.make_weights(E, H, I, s, device=dev())
+        A_bits = synth.make_activations(T, H, s)
+        lg = synth.make_logits(kind, T, E, s, A_bits, H)
+        wn = w.numpy()
+        fe = ve.FusedExperts(w.w13, w.w13_scale, w.w2, w.w2_scale, scratch=ve.CaptureSafeScratch(),
+                             prepack=True, keep_raw=False)
+        del w
+        ids, tw, sids, eids, out_em, max_em, _ = fe.route_align(to_dev(lg), k, True, bs)
+        out = fe.apply(to_dev(A_bits, torch.bfloat16), ids, tw, block_size=bs, aligned=(sids, eids, max_em))
+        torch.cuda.synchronize()
+        rid, rw = oracle.route_topk(lg, k, True)
+        assert np.array_equal(ids.cpu().numpy(), rid), what
+        c = cpu_layer(A_bits, wn, rid, rw, threads=16)
+        m, l2, nf = error_metrics(out.cpu().numpy(), c["out"])
+        assert nf and m <= MAX_ABS_TOL and l2 <= REL_L2_TOL, (what, m, l2)
+        worst = [max(worst[0], m), max(worst[1], l2)]
+    print(f"chunked kernel: worst max_abs/rms={worst[0]:.3e} rel_l2={worst[1]:.3e}")
+    assert worst[0] <= 1.2e-2 and worst[1] <= 1.5e-3
