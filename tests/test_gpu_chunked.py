@@ -160,3 +160,21 @@ def test_chunked_shapes_forced_in_blocks_of_16(name, T):
     assert np.array_equal(_act_by_flat_row(g, n_flat), _act_by_flat_row(b, n_flat))
     m, l2, nf = error_metrics(g["out"], b["out"])
     assert nf and l2 <= 1e-5, (m, l2)
+
+
+def test_more_runs_than_workgroups():
+    """384 experts, 800 routed rows in blocks of 32: more runs (blocks with rows) than the launch
+    has workgroups, so the (run, unit) space is cut evenly and a workgroup's slice spans runs,
+    segment after segment with different rows."""
+    cfg = synth.MoEConfig("many", 256, 128, 384, 4, (200,), "uniform")
+    T, seed = 200, 7100
+    w = synth.make_weights(cfg.E, cfg.H, cfg.I, seed, device=dev())
+    A, lg = cfgs._inputs(cfg, T, seed)
+    g = cfgs._run_gpu(cfg, w, A, lg, 32, None, **PACKED_ONLY)
+    runs = int((g["eids"] >= 0).sum())
+    assert runs > 304, runs       # (more than the compute units of the device)
+    ids, tw = oracle.route_topk(lg, cfg.top_k, True)
+    c = cpu_layer(A, w.numpy(), ids, tw, threads=16)
+    max_rel, rel_l2, nf = error_metrics(g["out"], c["out"])
+    print(f"{runs} runs: max_abs/rms={max_rel:.3e} rel_l2={rel_l2:.3e}")
+    assert nf and max_rel <= EXACT_SPLIT_MAX_ABS_TOL and rel_l2 <= EXACT_SPLIT_REL_L2_TOL
