@@ -134,7 +134,7 @@ struct MoeTileRule {
 // split between the kernel families is on the routed rows alone.
 //
 // Decode: the units of a run are shared by (compute units / runs) workgroups of 8
-// wavefronts, so a stage wants at least ~3 units per wavefront or the last round leaves
+// wavefronts, so a stage wants at least ~3 units per wavefront or the last of them leaves
 // most wavefronts idle.  Gate/up units are a gate tile and its up tile (nt = 2,
 // ispp / 16 units per expert); the down stage, with half the weight rows, takes single
 // tiles (nt = 1) and keeps the bytes in flight per wavefront with a deeper pipeline.
