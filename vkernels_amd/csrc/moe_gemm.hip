@@ -432,6 +432,16 @@ __device__ __forceinline__ i32x8 fp4_operand_packed(u32x4 w) {
   return __builtin_shufflevector(y, y, 0, 1, 2, 3, -1, -1, -1, -1);
 }
 
+// Position of a workgroup in the decode kernels' split of the work.  The hardware hands
+// consecutive workgroup ids to the 8 XCDs in turn, each with an L2 of its own.  Taking the
+// ids of one XCD as one consecutive range of positions puts the workgroups of a run, and of
+// the runs next to it, behind one L2: the passes of an expert with several blocks are runs
+// side by side whose workgroups stream the same weights at the same time, so what the first
+// of them fetches the others find there.
+__device__ __forceinline__ int xcd_major_index(int id, int grid) {
+  return (grid & 7) == 0 ? (id & 7) * (grid >> 3) + (id >> 3) : id;
+}
+
 // First item of part `i` when `total` items are cut into `parts` contiguous
 // slices whose sizes differ by at most one.
 __device__ __forceinline__ int slice_begin(int total, int i, int parts) {
@@ -819,7 +829,7 @@ __global__ __launch_bounds__(64 * WAVES) void stream_resident_kernel(GemmArgs p)
   // ---- list the runs (first and last block of every run, in order) ---------
   if (wave == 0) {
     const int nb = p.num_blocks;
-    const int grid = (int)gridDim.x, wg = (int)blockIdx.x;
+    const int grid = (int)gridDim.x, wg = xcd_major_index((int)blockIdx.x, (int)gridDim.x);
     const unsigned long long below = (1ull << lane) - 1ull;
     // Every block with an expert is a run of its own: the blocks of an expert then go to
     // different workgroups side by side, each staging once, where a run of several blocks
@@ -1479,7 +1489,7 @@ __global__ __launch_bounds__(64 * kChunkWaves) void stream_chunked_kernel(GemmAr
   int s0 = 0, s1 = 0;
   {
     const int n = n_runs_sh;
-    const int grid = (int)gridDim.x, wg = (int)blockIdx.x;
+    const int grid = (int)gridDim.x, wg = xcd_major_index((int)blockIdx.x, (int)gridDim.x);
     if (n > 0) {
       bool aligned = n <= grid;
       if (aligned) {
